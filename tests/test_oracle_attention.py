@@ -1,0 +1,205 @@
+"""Pins the CPU oracle's attention functions without the reference being runnable:
+closed forms, a library cross-check, invariants and an independent scalar brute force."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import attention as A
+
+
+def _rand(B, Hq, Hkv, Nq, Nk, D, seed, scale=1.0, dtype=torch.bfloat16):
+    g = torch.Generator().manual_seed(seed)
+    q = (torch.randn(B, Hq, Nq, D, generator=g) * scale).to(dtype)
+    k = (torch.randn(B, Hkv, Nk, D, generator=g) * scale).to(dtype)
+    v = (torch.randn(B, Hkv, Nk, D, generator=g) * scale).to(dtype)
+    return q, k, v
+
+
+def _cos(a, b):
+    a, b = a.double().flatten(), b.double().flatten()
+    return float(a @ b / (a.norm() * b.norm()))
+
+
+def test_exact_attention_matches_torch_sdpa():
+    q, k, v = _rand(2, 4, 2, 96, 96, 32, 0)
+    out, lse2 = A.exact_attention(q, k, v)
+    ref = torch.nn.functional.scaled_dot_product_attention(
+        q.double(), k.double().repeat_interleave(2, 1), v.double().repeat_interleave(2, 1), is_causal=True)
+    assert torch.allclose(out, ref, rtol=1e-10, atol=1e-12)
+    # a transposed GQA mapping (tiled instead of blocked heads) must fail this check
+    bad = torch.nn.functional.scaled_dot_product_attention(
+        q.double(), k.double().repeat(1, 2, 1, 1), v.double().repeat(1, 2, 1, 1), is_causal=True)
+    assert not torch.allclose(out, bad, rtol=1e-3, atol=1e-3)
+    # lse2 is base 2 of the natural-scaled scores
+    s = (q.double() @ k.double().repeat_interleave(2, 1).transpose(-1, -2)) / math.sqrt(32)
+    s = s.masked_fill(torch.triu(torch.ones(96, 96, dtype=torch.bool), 1), float("-inf"))
+    assert torch.allclose(lse2, torch.logsumexp(s, -1) / math.log(2), rtol=1e-12)
+
+
+def test_fold_scale_is_bf16_rounding_of_fp32_product():
+    q = torch.tensor([[1.0, 0.3333, -2.5, 7.0]], dtype=torch.bfloat16)
+    sm = np.float32(1.0 / 128 ** 0.5 * 1.44269504)
+    exp = torch.tensor((q.float().numpy() * sm).astype(np.float32)).to(torch.bfloat16)
+    assert torch.equal(A.fold_scale(q, 128), exp)
+
+
+@pytest.mark.parametrize("scale", [1.0, 1.0 / 128 ** 0.5])
+def test_blockwise_no_quant_equals_closed_form(scale):
+    q, k, v = _rand(1, 4, 2, 200, 200, 128, 1, scale)
+    out, lse = A.prefill_blockwise(q, k, v, out_dtype=torch.float32)
+    # closed form on the query that already carries the folded factor: isolates the blockwise algorithm
+    ref, lse_ref = A.exact_attention(A.fold_scale(q, 128), k, v, score_scale=math.log(2.0))
+    rms = ref.pow(2).mean().sqrt()
+    assert float((out.double() - ref).abs().max() / rms) < 4e-3   # fp16 P/V rounding + fp32 sums
+    assert torch.allclose(lse.double(), lse_ref, atol=1e-4, rtol=1e-5)
+    # against the unfolded closed form the bf16 fold dominates (documented ~4e-2 of rms for N(0,1))
+    ref2, _ = A.exact_attention(q, k, v)
+    assert _cos(out, ref2) > 0.9999
+
+
+def test_blockwise_independent_of_row_tile():
+    q, k, v = _rand(1, 2, 1, 256, 256, 64, 2)
+    for mode in (A.P_NONE, A.P_STATIC448, A.P_BLOCK_ABSMAX):
+        o128, l128 = A.prefill_blockwise(q, k, v, p_quant=mode, block_m=128, out_dtype=torch.float32)
+        o64, l64 = A.prefill_blockwise(q, k, v, p_quant=mode, block_m=64, out_dtype=torch.float32)
+        assert torch.equal(o128, o64) and torch.equal(l128, l64)
+
+
+def _scalar_fp8_prefill(q, k, v, D):
+    """Independent scalar restatement of attn_triton.py:64-86 + :208-213 for ONE head, row by row."""
+    f32 = np.float32
+    qf = A.fold_scale(q, D).float().numpy()
+    kf = k.float().numpy()
+    vf = v.to(torch.float16).float().numpy()
+    N = qf.shape[0]
+    out = np.zeros((N, D), dtype=f32)
+    lse = np.zeros(N, dtype=f32)
+    grid = torch.arange(256, dtype=torch.uint8).view(torch.float8_e4m3fn).float().numpy()
+    grid = np.sort(grid[np.isfinite(grid) & (grid >= 0)])
+    for i in range(N):
+        m, l, acc = f32(-np.inf), f32(1.0), np.zeros(D, dtype=f32)
+        tile0 = (i // 128) * 128
+        for j0 in range(0, tile0 + 128, 64):
+            if j0 >= N:
+                break
+            s = np.zeros(64, dtype=f32)
+            for c in range(64):
+                if j0 + c < N:
+                    s[c] = np.dot(qf[i].astype(np.float64), kf[j0 + c].astype(np.float64))
+                if j0 >= tile0 and j0 + c > i:
+                    s[c] += f32(-1000000.0)
+            m_new = max(m, s.max())
+            p = np.exp2((s - m_new).astype(np.float64)).astype(f32)
+            alpha = f32(np.exp2(np.float64(m - m_new)))
+            l = f32(l * alpha + p.sum(dtype=f32))
+            acc = acc * alpha
+            # e4m3 round-to-nearest-even by search on the value grid, then fp16(x/448)
+            x = (p * f32(448.0)).astype(np.float64)
+            idx = np.searchsorted(grid, x)
+            lo = grid[np.clip(idx - 1, 0, len(grid) - 1)]
+            hi = grid[np.clip(idx, 0, len(grid) - 1)]
+            pick_hi = (hi - x < x - lo) | ((hi - x == x - lo) & ((np.clip(idx, 0, len(grid) - 1) % 2) == 0))
+            p8 = np.where(pick_hi, hi, lo)
+            pq = (p8 / 448.0).astype(np.float16).astype(f32)
+            for c in range(64):
+                if j0 + c < N:
+                    acc = acc + pq[c] * vf[j0 + c]
+            m = m_new
+        out[i] = acc / l
+        lse[i] = np.log2(l) + m
+    return out, lse
+
+
+def test_fp8_static_matches_scalar_bruteforce():
+    D = 32
+    q, k, v = _rand(1, 1, 1, 160, 160, D, 3)
+    out, lse = A.prefill_blockwise(q, k, v, p_quant=A.P_STATIC448, out_dtype=torch.float32)
+    ref, lse_ref = _scalar_fp8_prefill(q[0, 0], k[0, 0], v[0, 0], D)
+    d = np.abs(out[0, 0].numpy() - ref)
+    rms = np.sqrt((ref ** 2).mean())
+    # fp32 summation order differs (matmul vs sequential); an e4m3 flip would show as ~6e-2*|v|
+    assert np.quantile(d, 0.999) < 2e-5 * max(rms, 1.0)
+    assert d.max() < 0.05
+    assert np.allclose(lse[0, 0].numpy(), lse_ref, atol=2e-5)
+
+
+def test_fp8_error_levels_against_exact():
+    q, k, v = _rand(1, 4, 1, 1024, 1024, 128, 4)
+    ref, lse_ref = A.exact_attention(q, k, v)
+    rms = float(ref.pow(2).mean().sqrt())
+    for mode in (A.P_STATIC448, A.P_BLOCK_ABSMAX):
+        out, lse = A.prefill_blockwise(q, k, v, p_quant=mode, out_dtype=torch.float32)
+        assert _cos(out, ref) > 0.9995
+        mean_rel = float((out.double() - ref).abs().mean()) / rms
+        assert 5e-3 < mean_rel < 3e-2  # e4m3 has a 3-bit mantissa: about 1.35e-2 expected
+        # the denominator uses the unquantised p, so lse2 is unaffected by the P quantisation
+        assert torch.allclose(lse.double(), lse_ref, atol=5e-2)
+
+
+def test_window_invariants_and_explicit_mask():
+    N, D = 512, 64
+    q, k, v = _rand(1, 2, 1, N, N, D, 5)
+    full, _ = A.prefill_blockwise(q, k, v, out_dtype=torch.float32, block_m=64)
+    big = [N + 256, N + 256]
+    w, _ = A.prefill_blockwise(q, k, v, out_dtype=torch.float32, block_m=64, sink=128, w8=big, w4=big)
+    assert torch.equal(w, full)  # window >= N  =>  full causal
+    # N <= block_m => full causal whatever the windows are
+    qs, ks, vs = q[:, :, :64], k[:, :, :64], v[:, :, :64]
+    a, _ = A.prefill_blockwise(qs, ks, vs, out_dtype=torch.float32, block_m=128, sink=0, w8=[0, 0], w4=[0, 0])
+    b, _ = A.prefill_blockwise(qs, ks, vs, out_dtype=torch.float32, block_m=128)
+    assert torch.equal(a, b)
+    # general case against the closed form under an explicit mask built from the four ranges
+    for bm, sink, w8, w4 in ((64, 128, 128, 256), (128, 64, 128, 128), (64, 0, 0, 0), (128, 256, 256, 384)):
+        out, lse = A.prefill_blockwise(q, k, v, out_dtype=torch.float32, block_m=bm, sink=sink,
+                                       w8=[w8, w8 + 128], w4=[w4, w4 + 128])
+        for h, extra in ((0, 0), (1, 128)):
+            mask = A.window_mask(N, N, q_offset=0, block_m=bm, sink=sink, w8=w8 + extra, w4=w4 + extra)
+            ref, lse_ref = A.exact_attention(A.fold_scale(q[:, h:h + 1], D), k, v, mask=mask[None, None],
+                                             score_scale=math.log(2.0))
+            rms = ref.pow(2).mean().sqrt()
+            assert float((out[:, h:h + 1].double() - ref).abs().max() / rms) < 5e-3
+            assert torch.allclose(lse[:, h:h + 1].double(), lse_ref, atol=1e-4)
+    # window 0 => sink + diagonal block only: row 300 (block_m 64) sees [0,128) and [256,300]
+    m = A.window_mask(N, N, q_offset=0, block_m=64, sink=128, w8=0, w4=0)
+    assert m[300].nonzero().flatten().tolist() == list(range(0, 128)) + list(range(256, 301))
+
+
+def test_relative_window_size():
+    assert A.window_size_relative(0.1, 131072) == 13184      # ceil128(13107)
+    assert A.window_size_relative(0.1, 4096) == 512          # ceil128(409)
+    assert A.window_size_relative(0.0, 4096) == 0
+    assert A.window_size_relative(1.0, 4096) == 4096
+
+
+def test_chunked_prefill_offset_matches_full():
+    N, D = 384, 64
+    q, k, v = _rand(1, 2, 2, N, N, D, 6)
+    full, lf = A.prefill_blockwise(q, k, v, out_dtype=torch.float32)
+    part, lp = A.prefill_blockwise(q[:, :, 256:], k, v, q_offset=256, out_dtype=torch.float32)
+    assert torch.equal(part, full[:, :, 256:]) and torch.equal(lp, lf[:, :, 256:])
+
+
+def test_decode_closed_form_and_split_combine():
+    B, Hq, Hkv, L, D = 2, 8, 2, 1000, 64
+    g = torch.Generator().manual_seed(7)
+    q = torch.randn(B, Hq, 1, D, generator=g).bfloat16()
+    k = torch.randn(B, Hkv, L, D, generator=g).bfloat16()
+    v = torch.randn(B, Hkv, L, D, generator=g).bfloat16()
+    lens = [777, 1000]
+    out, lse = A.decode_blockwise(q, k, v, lens)
+    ref, lse_ref = A.exact_attention(A.fold_scale(q, D), k, v, causal=False, kv_lens=lens, score_scale=math.log(2.0))
+    assert torch.allclose(out.double(), ref[:, :, 0], atol=2e-5, rtol=1e-4)
+    assert torch.allclose(lse.double(), lse_ref[:, :, 0], atol=1e-4)
+    # split-KV combine identity, with ragged and one empty split for batch 0
+    cuts = [(0, 256), (256, 640), (640, 832), (832, 1000)]
+    outs, lses = zip(*[A.decode_blockwise(q, k, v, lens, token_range=c) for c in cuts])
+    assert torch.isinf(lses[3][0]).all()
+    o2, l2 = A.combine_splits(torch.stack(outs), torch.stack(lses))
+    assert torch.allclose(o2, out, atol=1e-5, rtol=1e-5) and torch.allclose(l2, lse, atol=1e-5)
+    # K mean-centring (attn_triton_decode.py:268-269) leaves the result unchanged
+    kc = (k.float() - k.float().mean(dim=2, keepdim=True))
+    oc, _ = A.exact_attention(q, kc, v, causal=False, kv_lens=lens)
+    o0, _ = A.exact_attention(q, k.float(), v, causal=False, kv_lens=lens)
+    assert torch.allclose(oc, o0, atol=1e-9)
