@@ -1,0 +1,142 @@
+/*
+ * libsqattn_hip.so -- C ABI of the MI355X (gfx950) implementation of SQAttn's attention hot path.
+ *
+ * Every entry point takes borrowed DLPack tensors (device pointers, shapes, strides in elements), plain
+ * scalars and a HIP stream handle (`hipStream_t` passed as `void*`, NULL = the null stream); it enqueues
+ * work on that stream and returns without synchronising unless stated otherwise.  Nothing is retained
+ * after the call returns; outputs and workspaces are allocated by the caller.  Return value: SQ_OK or a
+ * negative SQ_E* code; `sq_last_error()` then holds a message (thread-local).  No entry point throws or
+ * aborts.  Tensors must live on one ROCm device (DLPack device type kDLROCM, or kDLCUDA as some
+ * PyTorch-ROCm builds report), have a contiguous last dimension and a 16-byte aligned base address.
+ *
+ * Reference interfaces replaced (paths relative to the reference repository):
+ *   sq_prefill_fwd            sqattn/attn_triton.py:216-315 (attn_causal -> _attn_fwd launch :279-310),
+ *                             sqattn/attn_triton_mix_relative.py:309-483 (launch :439-475),
+ *                             sqattn/attn_triton_mix_bad.py:285-426 (launch :388-424)
+ *   sq_decode_fwd             sqattn/attn_triton_decode.py:244-361 (decode launch :293-324)
+ *   sq_kmeans_train           cache_hub/kmeans.py:127-196 (assign launch :147-173, update launch :175-193)
+ *   sq_reverse_index          cache_hub/kmeans.py:233-262
+ *   sq_index_add              cache_hub/kmeans.py:307-329
+ *   sq_topk_select            no reference counterpart (defined by this build's benchmark configuration)
+ */
+#ifndef SQATTN_H_
+#define SQATTN_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#include "sq_dlpack.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SQ_ABI_VERSION 1
+
+enum {
+  SQ_OK = 0,
+  SQ_EINVAL = -1,       /* bad argument value (layout, head_dim > 128, sink, mode, null pointer)  */
+  SQ_ESHAPE = -2,       /* shapes/strides inconsistent with each other                            */
+  SQ_EDEVICE = -3,      /* tensor not on a ROCm device, or tensors on different devices           */
+  SQ_EDTYPE = -4,       /* unsupported element type                                               */
+  SQ_EUNSUPPORTED = -5, /* valid in the reference but outside what the kernels implement          */
+  SQ_EHIP = -6,         /* a HIP runtime call failed (message carries hipGetErrorString)          */
+  SQ_EWORKSPACE = -7    /* workspace missing or too small                                         */
+};
+
+enum { SQ_LAYOUT_HND = 0, SQ_LAYOUT_NHD = 1 };
+
+/* Quantisation of the softmax probabilities before P.V */
+enum {
+  SQ_P_NONE = 0,         /* p.to(fp16)                               attn_triton.py:83           */
+  SQ_P_E4M3_STATIC = 1,  /* fp16(fp16(e4m3(p*448))/448)              attn_triton.py:81-82        */
+  SQ_P_E4M3_BLOCK = 2    /* per (64 rows x 64 keys) absmax scale a: e4m3(p*448/a)*a/448 (no ref.) */
+};
+
+enum { SQ_WINDOW_NONE = 0, SQ_WINDOW_SIZES = 1 };
+
+int sq_abi_version(void);
+const char* sq_last_error(void);
+
+/* ---------------------------------------------------------------------------------------- prefill */
+typedef struct sq_prefill_params {
+  int32_t layout;        /* SQ_LAYOUT_*: q/out [B,Hq,Nq,D] + k/v [B,Hkv,Nk,D], or [B,N,H,D]               */
+  int32_t p_quant;       /* SQ_P_*                                                                        */
+  int32_t head_dim_og;   /* head_dim before zero-padding to 128: softmax scale = log2e/sqrt(head_dim_og); */
+                         /* 0 = the tensors' D (attn_triton.py:236-250)                                   */
+  int64_t q_offset;      /* absolute position of query row 0 (0 in the reference, which needs Nq == Nk)   */
+  int32_t window_mode;   /* SQ_WINDOW_NONE: full causal (attn_triton.py). SQ_WINDOW_SIZES: sink + windows */
+  int32_t block_m;       /* query-block size that defines the window ranges: 64 (relative wrapper,        */
+                         /* attn_triton_mix_relative.py:423) or 128 (absolute, attn_triton_mix_bad.py:386) */
+  int32_t sink;          /* sink size in tokens, multiple of 64                                           */
+  int32_t num_heads_w;   /* number of entries of w8/w4 (== Hq)                                            */
+  const int32_t* w8;     /* HOST arrays: per-head 8-bit / 4-bit window sizes in tokens (multiples of 64). */
+  const int32_t* w4;     /* The relative wrapper converts ratios with ceil128(int(f32(ratio)*kv_len)).    */
+} sq_prefill_params;
+
+/* Bytes of device workspace sq_prefill_fwd needs (fp16 transposed V tiles). */
+size_t sq_prefill_workspace_bytes(int64_t batch, int64_t num_kv_heads, int64_t kv_len, int64_t head_dim);
+
+/*
+ * out = softmax2(q~ k^T) v per the reference's blockwise algorithm, q~ = q * log2e/sqrt(D) rounded to q's
+ * dtype.  q, k, v: bf16 or fp16 (same type), D == 128 (the host zero-pads smaller heads).  q4/k4 (may be NULL = alias of q/k) are the
+ * operands used inside the 4-bit window range.  out: bf16/fp16/fp32, same shape as q.
+ * lse (may be NULL): fp32 [B,Hq,Nq], base-2 log-sum-exp (attn_triton.py:210-213).
+ */
+int sq_prefill_fwd(const DLTensor* q, const DLTensor* k, const DLTensor* v, const DLTensor* q4,
+                   const DLTensor* k4, DLTensor* out, DLTensor* lse, DLTensor* workspace,
+                   const sq_prefill_params* params, void* stream);
+
+/* ----------------------------------------------------------------------------------------- decode */
+typedef struct sq_decode_params {
+  int32_t layout;      /* SQ_LAYOUT_HND: q [B,Hq,1,D], caches [B,Hkv,L,D]; SQ_LAYOUT_NHD: [B,1,Hq,D], [B,L,Hkv,D] */
+  int32_t p_quant;     /* SQ_P_NONE or SQ_P_E4M3_STATIC (attn_triton_decode.py:232-233)                        */
+  int32_t num_splits;  /* KV splits per (batch, kv head); 0 = let the library choose                            */
+  int32_t head_dim_og; /* head_dim before zero-padding to 128 (0 = the tensors' D)                             */
+} sq_decode_params;
+
+/* Number of splits the library would choose, and the workspace needed for a given number of splits. */
+int32_t sq_decode_num_splits(int64_t batch, int64_t num_kv_heads, int64_t max_len);
+size_t sq_decode_workspace_bytes(int64_t batch, int64_t num_q_heads, int64_t head_dim, int32_t num_splits);
+
+/*
+ * One query token per sequence against a KV cache; seqlens (int32 [B], may be NULL = L) gives the valid
+ * prefix of each sequence.  The K-mean subtraction of attn_unified (attn_triton_decode.py:268-269) is
+ * omitted: it cannot change a softmax.  out same shape as q; lse (may be NULL) fp32 [B,Hq,1].
+ */
+int sq_decode_fwd(const DLTensor* q, const DLTensor* kcache, const DLTensor* vcache, const DLTensor* seqlens,
+                  DLTensor* out, DLTensor* lse, DLTensor* workspace, const sq_decode_params* params,
+                  void* stream);
+
+/* ---------------------------------------------------------------------------------------- k-means */
+size_t sq_kmeans_workspace_bytes(int64_t groups, int64_t num_tokens, int64_t num_centroids, int64_t dim);
+
+/*
+ * One Lloyd step: idx[g,n] = argmax_c <data[g,n], centroids[g,c]> (lowest index on ties); cnt = cluster
+ * sizes; centroids[g,c] <- mean of its tokens (L2-normalised if `normalize`), stored only where cnt > 0.
+ * data, centroids: bf16 [G,N,D] / [G,C,D], D == 128, C % 32 == 0 (kmeans.py:146); idx int32 [G,N];
+ * cnt int32 [G,C].  Cluster sums are exact (fp64 accumulation), hence independent of summation order.
+ */
+int sq_kmeans_train(const DLTensor* data, DLTensor* centroids, DLTensor* idx, DLTensor* cnt,
+                    DLTensor* workspace, int32_t normalize, void* stream);
+
+/* clusters[g,c,0:cnt] = token ids with idx == c in ascending order (rest 0); cluster_size = counts. */
+int sq_reverse_index(const DLTensor* idx, DLTensor* clusters, DLTensor* cluster_size, DLTensor* workspace,
+                     void* stream);
+
+/* out[g,c,:] = sum of value[g,n,:] over idx[g,n] == c, cast to value's dtype; out [G,C,D]. */
+int sq_index_add(const DLTensor* value, const DLTensor* idx, DLTensor* out, DLTensor* workspace, void* stream);
+
+/*
+ * Centroid-scored token selection: per group g = b*Hkv + kvh, clusters ranked by
+ * max_{h in group} <query[b,h], centroids[g,c]> (ties -> lower c); whole clusters taken in rank order
+ * until k tokens are emitted; missing tail = -1.  query bf16 [B,Hq,D]; out int32 [G,k].
+ */
+int sq_topk_select(const DLTensor* query, const DLTensor* centroids, const DLTensor* clusters,
+                   const DLTensor* cluster_size, DLTensor* out, DLTensor* workspace, int32_t num_kv_groups,
+                   void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SQATTN_H_ */

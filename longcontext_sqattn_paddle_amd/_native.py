@@ -1,0 +1,147 @@
+"""ctypes binding of libsqattn_hip.so: DLPack capsules in, error codes out.
+
+The library is the only compute path of this package.  If it is missing, or a call fails, an exception
+is raised -- there is no eager/PyTorch fallback.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Optional
+
+import torch
+
+_PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG_DIR, "libsqattn_hip.so")
+
+SQ_OK, SQ_EINVAL, SQ_ESHAPE, SQ_EDEVICE, SQ_EDTYPE, SQ_EUNSUPPORTED, SQ_EHIP, SQ_EWORKSPACE = 0, -1, -2, -3, -4, -5, -6, -7
+LAYOUT = {"HND": 0, "NHD": 1}
+P_NONE, P_E4M3_STATIC, P_E4M3_BLOCK = 0, 1, 2
+WINDOW_NONE, WINDOW_SIZES = 0, 1
+
+
+class DLDevice(ctypes.Structure):
+    _fields_ = [("device_type", ctypes.c_int32), ("device_id", ctypes.c_int32)]
+
+
+class DLDataType(ctypes.Structure):
+    _fields_ = [("code", ctypes.c_uint8), ("bits", ctypes.c_uint8), ("lanes", ctypes.c_uint16)]
+
+
+class DLTensor(ctypes.Structure):
+    _fields_ = [
+        ("data", ctypes.c_void_p),
+        ("device", DLDevice),
+        ("ndim", ctypes.c_int32),
+        ("dtype", DLDataType),
+        ("shape", ctypes.POINTER(ctypes.c_int64)),
+        ("strides", ctypes.POINTER(ctypes.c_int64)),
+        ("byte_offset", ctypes.c_uint64),
+    ]
+
+
+class PrefillParams(ctypes.Structure):
+    _fields_ = [
+        ("layout", ctypes.c_int32),
+        ("p_quant", ctypes.c_int32),
+        ("head_dim_og", ctypes.c_int32),
+        ("q_offset", ctypes.c_int64),
+        ("window_mode", ctypes.c_int32),
+        ("block_m", ctypes.c_int32),
+        ("sink", ctypes.c_int32),
+        ("num_heads_w", ctypes.c_int32),
+        ("w8", ctypes.POINTER(ctypes.c_int32)),
+        ("w4", ctypes.POINTER(ctypes.c_int32)),
+    ]
+
+
+class DecodeParams(ctypes.Structure):
+    _fields_ = [
+        ("layout", ctypes.c_int32),
+        ("p_quant", ctypes.c_int32),
+        ("num_splits", ctypes.c_int32),
+        ("head_dim_og", ctypes.c_int32),
+    ]
+
+
+_P = ctypes.POINTER(DLTensor)
+
+# every symbol include/sqattn.h declares: name -> (restype, argtypes)
+SYMBOLS = {
+    "sq_abi_version": (ctypes.c_int, []),
+    "sq_last_error": (ctypes.c_char_p, []),
+    "sq_prefill_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int64] * 4),
+    "sq_prefill_fwd": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, _P, _P, ctypes.POINTER(PrefillParams), ctypes.c_void_p]),
+    "sq_decode_num_splits": (ctypes.c_int32, [ctypes.c_int64] * 3),
+    "sq_decode_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int32]),
+    "sq_decode_fwd": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, _P, ctypes.POINTER(DecodeParams), ctypes.c_void_p]),
+    "sq_kmeans_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int64] * 4),
+    "sq_kmeans_train": (ctypes.c_int, [_P, _P, _P, _P, _P, ctypes.c_int32, ctypes.c_void_p]),
+    "sq_reverse_index": (ctypes.c_int, [_P, _P, _P, _P, ctypes.c_void_p]),
+    "sq_index_add": (ctypes.c_int, [_P, _P, _P, _P, ctypes.c_void_p]),
+    "sq_topk_select": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, ctypes.c_int32, ctypes.c_void_p]),
+}
+
+_lib: Optional[ctypes.CDLL] = None
+
+
+def lib() -> ctypes.CDLL:
+    """Load the shared library once; raise if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `python -m longcontext_sqattn_paddle_amd.build` "
+                "(there is no fallback path)")
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SYMBOLS.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        if handle.sq_abi_version() != 1:
+            raise RuntimeError("libsqattn_hip.so ABI version mismatch")
+        _lib = handle
+    return _lib
+
+
+_capsule_ptr = ctypes.pythonapi.PyCapsule_GetPointer
+_capsule_ptr.restype = ctypes.c_void_p
+_capsule_ptr.argtypes = [ctypes.py_object, ctypes.c_char_p]
+
+
+class Borrowed:
+    """A DLTensor borrowed from a torch tensor through its DLPack capsule.
+
+    The capsule is kept alive (and never consumed) for the lifetime of this object; dropping it runs
+    the producer's deleter, so the library only ever sees borrowed memory.
+    """
+
+    def __init__(self, t: torch.Tensor):
+        self.tensor = t
+        self.capsule = torch.utils.dlpack.to_dlpack(t)
+        addr = _capsule_ptr(self.capsule, b"dltensor")
+        self.ptr = ctypes.cast(addr, _P)  # DLManagedTensor starts with its DLTensor
+
+
+def dl(t: Optional[torch.Tensor]):
+    return None if t is None else Borrowed(t)
+
+
+def ptr(b: Optional[Borrowed]):
+    return None if b is None else b.ptr
+
+
+def check(code: int) -> None:
+    """Map a library error code to the exception type the reference raises for the same mistake."""
+    if code == SQ_OK:
+        return
+    msg = lib().sq_last_error().decode("utf-8", "replace")
+    if code in (SQ_EINVAL, SQ_EUNSUPPORTED, SQ_EDTYPE):
+        raise ValueError(msg)
+    if code == SQ_ESHAPE:
+        raise AssertionError(msg)
+    raise RuntimeError(f"libsqattn_hip error {code}: {msg}")
+
+
+def current_stream(device) -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)

@@ -1,0 +1,107 @@
+// Shared host/device helpers of libsqattn_hip.so (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "sqattn.h"
+
+namespace sq {
+
+// ------------------------------------------------------------------------------------------ errors
+void set_error(const char* fmt, ...);  // stores a thread-local message, defined in capi.hip
+
+#define SQ_FAIL(code, ...)        \
+  do {                            \
+    ::sq::set_error(__VA_ARGS__); \
+    return (code);                \
+  } while (0)
+
+#define SQ_REQUIRE(cond, code, ...)          \
+  do {                                       \
+    if (!(cond)) SQ_FAIL(code, __VA_ARGS__); \
+  } while (0)
+
+#define SQ_HIP(call)                                                                        \
+  do {                                                                                      \
+    hipError_t e__ = (call);                                                                \
+    if (e__ != hipSuccess) SQ_FAIL(SQ_EHIP, "%s failed: %s", #call, hipGetErrorString(e__)); \
+  } while (0)
+
+// ------------------------------------------------------------------------------------ tensor views
+enum class DType { BF16, F16, F32, I32, OTHER };
+
+inline DType dtype_of(const DLTensor* t) {
+  if (t->dtype.lanes != 1) return DType::OTHER;
+  if (t->dtype.code == kDLBfloat && t->dtype.bits == 16) return DType::BF16;
+  if (t->dtype.code == kDLFloat && t->dtype.bits == 16) return DType::F16;
+  if (t->dtype.code == kDLFloat && t->dtype.bits == 32) return DType::F32;
+  if (t->dtype.code == kDLInt && t->dtype.bits == 32) return DType::I32;
+  return DType::OTHER;
+}
+
+inline int dtype_bytes(DType d) { return (d == DType::BF16 || d == DType::F16) ? 2 : 4; }
+
+inline bool on_gpu(const DLTensor* t) {
+  return t->device.device_type == kDLROCM || t->device.device_type == kDLCUDA;
+}
+
+inline int64_t stride_of(const DLTensor* t, int dim) {
+  if (t->strides) return t->strides[dim];
+  int64_t s = 1;
+  for (int i = t->ndim - 1; i > dim; --i) s *= t->shape[i];
+  return s;
+}
+
+inline char* data_of(const DLTensor* t) { return static_cast<char*>(t->data) + t->byte_offset; }
+
+inline int64_t numel_of(const DLTensor* t) {
+  int64_t n = 1;
+  for (int i = 0; i < t->ndim; ++i) n *= t->shape[i];
+  return n;
+}
+
+inline bool is_compact(const DLTensor* t) {
+  int64_t s = 1;
+  for (int i = t->ndim - 1; i >= 0; --i) {
+    if (t->shape[i] != 1 && stride_of(t, i) != s) return false;
+    s *= t->shape[i];
+  }
+  return true;
+}
+
+// Common checks of one tensor argument: non-null, on a GPU, expected rank, last dim contiguous,
+// 16-byte aligned base.  Returns SQ_OK or an error code with the message set.
+int check_tensor(const DLTensor* t, const char* name, int ndim, int device_id);
+
+// ------------------------------------------------------------------------------------ device utils
+#if defined(__HIPCC__)
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
+typedef __attribute__((ext_vector_type(4))) _Float16 f16x4_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+typedef __attribute__((ext_vector_type(4))) int i32x4_t;
+typedef __attribute__((ext_vector_type(2))) int i32x2_t;
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t bits16) { return __uint_as_float(bits16 << 16); }
+
+// round-to-nearest-even fp32 -> bf16 bit pattern (finite inputs)
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float x) {
+  uint32_t u = __float_as_uint(x);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return u >> 16;
+}
+
+// e4m3 (OCP, max 448) round trip of a non-negative value <= 448: fp32 -> fp8 (RNE) -> fp32
+__device__ __forceinline__ float e4m3_roundtrip(float x) {
+  int pk = __builtin_amdgcn_cvt_pk_fp8_f32(x, x, 0, false);
+  return __builtin_amdgcn_cvt_f32_fp8(pk, 0);
+}
+
+__device__ __forceinline__ float wave_xor_max(float v, int mask) { return fmaxf(v, __shfl_xor(v, mask)); }
+#endif
+
+}  // namespace sq

@@ -1,0 +1,392 @@
+// Split-KV decode attention for gfx950 (MI355X): one query token per sequence against a GQA KV cache.
+//
+// Replaces the reference's `_attn_decode_fwd` + `attn_unified` decode branch
+// (sqattn/attn_triton_decode.py:175-241, 244-324).  The reference runs one program per (batch, q-head)
+// and streams the whole cache serially, re-reading each KV head once per q-head of its group.  Here a
+// workgroup owns one (batch, kv-head, token range): it streams that range ONCE for all q-heads of the
+// group, writes a normalised partial output with its base-2 log-sum-exp, and a second tiny kernel merges
+// the partials (lse = log2 sum_s 2^lse_s, o = sum_s 2^(lse_s-lse) o_s).
+//
+// Data path per wave and 16-token tile (HBM-bound; everything else is sized to stay out of the way):
+//   K : 4 x 16-byte loads per lane, lane (r=lane%16, g=lane/16) reads K[n0+r][32kk+8g .. +7]  -> A operand
+//   S^T[token, head] = K . Q~^T  on v_mfma_f32_16x16x32 (bf16/f16 in, fp32 acc); Q~ (16 padded heads) lives
+//        in registers as the B operand; lane (r,g) ends up with head r, tokens n0+4g+i, i<4.
+//   V : 4 x 16-byte loads per lane, load i reads V[n0+4g+i][8r .. 8r+7] (full 256-byte rows per 16 lanes)
+//   O^T[d, head] += V^T . P^T  on v_mfma_f32_16x16x4_f32 with k = the 4 lane groups g: the A operand is
+//        the fp32 value of one loaded V element, the B operand is the lane's own p -- no transposition,
+//        no LDS, products in fp32 exactly as the reference's `p * v.to(float32)` (:234).
+#include "common.hpp"
+
+namespace sq {
+namespace {
+
+constexpr int kD = 128;          // head_dim handled by the kernels (the host pads smaller heads with zeros)
+constexpr int kWaves = 4;
+constexpr int kTile = 16;        // tokens per MFMA tile
+constexpr int kOStride = 132;    // padded row of the cross-wave merge buffer (floats)
+
+struct DecodeArgs {
+  const void* q;
+  const void* k;
+  const void* v;
+  const int32_t* seqlens;
+  float* part_o;    // [B, Hq, S, D] normalised partial outputs
+  float* part_lse;  // [B, Hq, S]    base-2 LSE of each partial (-inf = empty)
+  int64_t q_sb, q_sh;
+  int64_t k_sb, k_sh, k_sn;
+  int64_t v_sb, v_sh, v_sn;
+  int32_t B, Hq, Hkv, L, group, head_chunks, num_splits, chunk, p_quant;
+  float sm;  // log2e / sqrt(D_original), rounded to fp32
+};
+
+template <bool BF16>
+__device__ __forceinline__ float elem_to_f32(uint32_t bits16) {
+  if constexpr (BF16) {
+    return bf16_bits_to_f32(bits16);
+  } else {
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)bits16);
+  }
+}
+
+template <bool BF16>
+__device__ __forceinline__ uint32_t f32_to_elem(float x) {
+  if constexpr (BF16) {
+    return f32_to_bf16_bits(x);
+  } else {
+    return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)x);
+  }
+}
+
+template <bool BF16>
+__device__ __forceinline__ f32x4_t mfma_qk(const uint4& a, const uint4& b, f32x4_t c) {
+  if constexpr (BF16) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b),
+                                                   c, 0, 0, 0);
+  } else {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c,
+                                                  0, 0, 0);
+  }
+}
+
+template <bool BF16>
+__global__ __launch_bounds__(kWaves * 64) void decode_splitkv_kernel(DecodeArgs a) {
+  __shared__ float s_o[kWaves][16][kOStride];
+  __shared__ float s_m[kWaves][16];
+  __shared__ float s_l[kWaves][16];
+
+  const int split = blockIdx.x;
+  const int kvh = blockIdx.y / a.head_chunks;
+  const int hc = blockIdx.y % a.head_chunks;
+  const int b = blockIdx.z;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int r = lane & 15;
+  const int g = lane >> 4;
+
+  int Lb = a.seqlens ? a.seqlens[b] : a.L;
+  Lb = min(max(Lb, 0), a.L);
+  const int t0 = split * a.chunk;
+  const int t1 = min(t0 + a.chunk, Lb);
+  const int h0 = hc * 16;                    // first head of this chunk inside the kv group
+  const int nh = min(16, a.group - h0);      // heads handled here
+  const int hq0 = kvh * a.group + h0;        // absolute first q head
+
+  if (t1 <= t0) {  // empty split: weight 0 in the merge
+    for (int i = threadIdx.x; i < nh * kD; i += blockDim.x) {
+      const int h = i / kD, d = i % kD;
+      a.part_o[(((int64_t)b * a.Hq + hq0 + h) * a.num_splits + split) * kD + d] = 0.f;
+    }
+    if (threadIdx.x < nh)
+      a.part_lse[((int64_t)b * a.Hq + hq0 + threadIdx.x) * a.num_splits + split] = -INFINITY;
+    return;
+  }
+
+  // Q~ fragments (B operand): lane (col head r, k-group g) holds q~[r][32kk+8g .. +7]
+  uint4 qf[4];
+  {
+    const uint16_t* qp = (const uint16_t*)a.q + (int64_t)b * a.q_sb + (int64_t)(hq0 + r) * a.q_sh;
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      uint32_t w[4] = {0, 0, 0, 0};
+      if (r < nh) {
+        const uint4 raw = *(const uint4*)(qp + 32 * kk + 8 * g);
+        const uint32_t in[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float lo = elem_to_f32<BF16>(in[j] & 0xffffu) * a.sm;
+          const float hi = elem_to_f32<BF16>(in[j] >> 16) * a.sm;
+          w[j] = f32_to_elem<BF16>(lo) | (f32_to_elem<BF16>(hi) << 16);
+        }
+      }
+      qf[kk] = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+  }
+
+  const uint16_t* kbase = (const uint16_t*)a.k + (int64_t)b * a.k_sb + (int64_t)kvh * a.k_sh;
+  const uint16_t* vbase = (const uint16_t*)a.v + (int64_t)b * a.v_sb + (int64_t)kvh * a.v_sh;
+
+  float m = -INFINITY;   // running max of head r (identical in the 4 lanes that share r)
+  float l = 0.f;         // this lane's share of the running denominator
+  f32x4_t acc[8];        // acc[e][i] = O^T[d = 32g + 8i + e][head r]
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+  const int ntiles = (t1 - t0 + kTile - 1) / kTile;
+  for (int tile = wave; tile < ntiles; tile += kWaves) {
+    const int n0 = t0 + tile * kTile;
+    // loads are clamped to the last valid token so that nothing past the valid prefix is touched
+    uint4 kf[4], vf[4];
+    {
+      const int tk = min(n0 + r, t1 - 1);
+      const uint16_t* kp = kbase + (int64_t)tk * a.k_sn + 8 * g;
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) kf[kk] = *(const uint4*)(kp + 32 * kk);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int tv = min(n0 + 4 * g + i, t1 - 1);
+        vf[i] = *(const uint4*)(vbase + (int64_t)tv * a.v_sn + 8 * r);
+      }
+    }
+    f32x4_t s = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) s = mfma_qk<BF16>(kf[kk], qf[kk], s);
+
+    float p[4];
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      p[i] = (n0 + 4 * g + i < t1) ? s[i] : -INFINITY;
+      tmax = fmaxf(tmax, p[i]);
+    }
+    tmax = wave_xor_max(tmax, 16);
+    tmax = wave_xor_max(tmax, 32);
+    const float m_new = fmaxf(m, tmax);      // finite: the tile holds at least one valid token
+    const float alpha = exp2f(m - m_new);    // exp2(-inf) = 0 on the first tile
+    float psum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      p[i] = exp2f(p[i] - m_new);
+      psum += p[i];
+    }
+    l = l * alpha + psum;
+    if (a.p_quant == SQ_P_E4M3_STATIC) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) p[i] = (float)(_Float16)(e4m3_roundtrip(p[i] * 448.f) / 448.f);
+    }
+    if (__any(alpha != 1.f)) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] *= alpha;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t w[4] = {vf[i].x, vf[i].y, vf[i].z, vf[i].w};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const uint32_t bits = (e & 1) ? (w[e >> 1] >> 16) : (w[e >> 1] & 0xffffu);
+        acc[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(elem_to_f32<BF16>(bits), p[i], acc[e], 0, 0, 0);
+      }
+    }
+    m = m_new;
+  }
+
+  // fold the 4 lane groups' shares of l, then merge the 4 waves through LDS
+  l += __shfl_xor(l, 16);
+  l += __shfl_xor(l, 32);
+#pragma unroll
+  for (int e = 0; e < 8; ++e)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) s_o[wave][r][32 * g + 8 * i + e] = acc[e][i];
+  if (g == 0) {
+    s_m[wave][r] = m;
+    s_l[wave][r] = l;
+  }
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < nh * kD; idx += blockDim.x) {
+    const int h = idx / kD, d = idx % kD;
+    float mm = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) mm = fmaxf(mm, s_m[w][h]);
+    float lt = 0.f, o = 0.f;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+      const float sc = exp2f(s_m[w][h] - mm);  // 0 for a wave that saw no tile (m = -inf)
+      lt += s_l[w][h] * sc;
+      o += s_o[w][h][d] * sc;
+    }
+    const int64_t row = ((int64_t)b * a.Hq + hq0 + h) * a.num_splits + split;
+    a.part_o[row * kD + d] = o / lt;
+    if (d == 0) a.part_lse[row] = mm + log2f(lt);
+  }
+}
+
+struct CombineArgs {
+  const float* part_o;
+  const float* part_lse;
+  void* out;
+  float* lse;  // may be null
+  int64_t o_sb, o_sh;
+  int32_t Hq, num_splits, out_dtype;  // 0 bf16, 1 f16, 2 f32
+};
+
+__global__ __launch_bounds__(kD) void decode_combine_kernel(CombineArgs a) {
+  const int h = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
+  const int64_t row0 = ((int64_t)b * a.Hq + h) * a.num_splits;
+  float mx = -INFINITY;
+  for (int s = 0; s < a.num_splits; ++s) mx = fmaxf(mx, a.part_lse[row0 + s]);
+  float tot = 0.f, o = 0.f;
+  if (mx > -INFINITY) {
+    for (int s = 0; s < a.num_splits; ++s) {
+      const float w = exp2f(a.part_lse[row0 + s] - mx);
+      if (w > 0.f) {
+        tot += w;
+        o += w * a.part_o[(row0 + s) * kD + d];
+      }
+    }
+    o /= tot;
+  }
+  const int64_t off = (int64_t)b * a.o_sb + (int64_t)h * a.o_sh + d;
+  if (a.out_dtype == 0) {
+    ((uint16_t*)a.out)[off] = (uint16_t)f32_to_bf16_bits(o);
+  } else if (a.out_dtype == 1) {
+    ((_Float16*)a.out)[off] = (_Float16)o;
+  } else {
+    ((float*)a.out)[off] = o;
+  }
+  if (a.lse && d == 0) a.lse[(int64_t)b * a.Hq + h] = (mx > -INFINITY) ? mx + log2f(tot) : -INFINITY;
+}
+
+}  // namespace
+}  // namespace sq
+
+using namespace sq;
+
+extern "C" int32_t sq_decode_num_splits(int64_t batch, int64_t num_kv_heads, int64_t max_len) {
+  if (batch <= 0 || num_kv_heads <= 0 || max_len <= 0) return 1;
+  // about 4 workgroups per CU over 256 CUs, at least 256 tokens (4 waves x 4 tiles) per workgroup
+  const int64_t target_blocks = 1024;
+  int64_t s = (target_blocks + batch * num_kv_heads - 1) / (batch * num_kv_heads);
+  const int64_t max_s = (max_len + 255) / 256;
+  if (s > max_s) s = max_s;
+  if (s < 1) s = 1;
+  if (s > 4096) s = 4096;
+  return (int32_t)s;
+}
+
+extern "C" size_t sq_decode_workspace_bytes(int64_t batch, int64_t num_q_heads, int64_t head_dim, int32_t num_splits) {
+  (void)head_dim;
+  if (batch <= 0 || num_q_heads <= 0 || num_splits <= 0) return 0;
+  return (size_t)batch * num_q_heads * num_splits * (kD + 1) * sizeof(float);
+}
+
+extern "C" int sq_decode_fwd(const DLTensor* q, const DLTensor* kcache, const DLTensor* vcache, const DLTensor* seqlens,
+                             DLTensor* out, DLTensor* lse, DLTensor* workspace, const sq_decode_params* params,
+                             void* stream) {
+  SQ_REQUIRE(params, SQ_EINVAL, "sq_decode_fwd: params is null");
+  SQ_REQUIRE(q && kcache && vcache && out, SQ_EINVAL, "sq_decode_fwd: q, kcache, vcache and out must be non-null");
+  SQ_REQUIRE(params->layout == SQ_LAYOUT_HND || params->layout == SQ_LAYOUT_NHD, SQ_EINVAL,
+             "tensor_layout %d not supported", params->layout);
+  SQ_REQUIRE(params->p_quant == SQ_P_NONE || params->p_quant == SQ_P_E4M3_STATIC, SQ_EINVAL,
+             "sq_decode_fwd: p_quant %d not supported", params->p_quant);
+  int rc;
+  const int dev = q->device.device_id;
+  if ((rc = check_tensor(q, "q", 4, dev)) || (rc = check_tensor(kcache, "kcache", 4, dev)) ||
+      (rc = check_tensor(vcache, "vcache", 4, dev)) || (rc = check_tensor(out, "out", 4, dev)))
+    return rc;
+  const DType dt = dtype_of(q);
+  SQ_REQUIRE(dt == DType::BF16 || dt == DType::F16, SQ_EDTYPE, "sq_decode_fwd: q must be bf16 or fp16");
+  SQ_REQUIRE(dtype_of(kcache) == dt && dtype_of(vcache) == dt, SQ_EDTYPE, "sq_decode_fwd: q, kcache, vcache dtypes differ");
+  const DType odt = dtype_of(out);
+  SQ_REQUIRE(odt == DType::BF16 || odt == DType::F16 || odt == DType::F32, SQ_EDTYPE,
+             "sq_decode_fwd: out must be bf16, fp16 or fp32");
+  const bool hnd = params->layout == SQ_LAYOUT_HND;
+  const int hdim = hnd ? 1 : 2, ndim = hnd ? 2 : 1;
+  const int64_t B = q->shape[0], Hq = q->shape[hdim], Nq = q->shape[ndim], D = q->shape[3];
+  const int64_t Hkv = kcache->shape[hdim], L = kcache->shape[ndim];
+  SQ_REQUIRE(D == kD, SQ_EINVAL, "Unsupported head_dim: %lld (the kernels take 128; pad smaller heads with zeros)", (long long)D);
+  SQ_REQUIRE(Nq == 1, SQ_ESHAPE, "sq_decode_fwd: query length must be 1, got %lld", (long long)Nq);
+  SQ_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && L > 0, SQ_ESHAPE, "sq_decode_fwd: empty tensor");
+  SQ_REQUIRE(Hq % Hkv == 0, SQ_ESHAPE, "sq_decode_fwd: Hq=%lld not a multiple of Hkv=%lld", (long long)Hq, (long long)Hkv);
+  SQ_REQUIRE(kcache->shape[0] == B && kcache->shape[3] == D, SQ_ESHAPE, "sq_decode_fwd: kcache shape mismatch");
+  for (int i = 0; i < 4; ++i)
+    SQ_REQUIRE(vcache->shape[i] == kcache->shape[i], SQ_ESHAPE, "sq_decode_fwd: vcache shape differs from kcache");
+  for (int i = 0; i < 4; ++i) SQ_REQUIRE(out->shape[i] == q->shape[i], SQ_ESHAPE, "sq_decode_fwd: out shape differs from q");
+  SQ_REQUIRE(L < (1ll << 31) - 65536, SQ_EUNSUPPORTED, "sq_decode_fwd: cache longer than 2^31 tokens");
+  SQ_REQUIRE(stride_of(kcache, ndim) % 8 == 0 && stride_of(vcache, ndim) % 8 == 0 && stride_of(kcache, hdim) % 8 == 0 &&
+                 stride_of(vcache, hdim) % 8 == 0 && stride_of(kcache, 0) % 8 == 0 && stride_of(vcache, 0) % 8 == 0 &&
+                 stride_of(q, hdim) % 8 == 0 && stride_of(q, 0) % 8 == 0,
+             SQ_ESHAPE, "sq_decode_fwd: strides must be multiples of 8 elements (16-byte vector loads)");
+  if (seqlens) {
+    SQ_REQUIRE(on_gpu(seqlens) && seqlens->device.device_id == dev, SQ_EDEVICE, "sq_decode_fwd: seqlens not on the same device");
+    SQ_REQUIRE(dtype_of(seqlens) == DType::I32 && seqlens->ndim == 1 && seqlens->shape[0] == B && stride_of(seqlens, 0) == 1,
+               SQ_ESHAPE, "sq_decode_fwd: seqlens must be a contiguous int32 [B]");
+  }
+  if (lse) {
+    SQ_REQUIRE(on_gpu(lse) && lse->device.device_id == dev, SQ_EDEVICE, "sq_decode_fwd: lse not on the same device");
+    SQ_REQUIRE(dtype_of(lse) == DType::F32 && numel_of(lse) == B * Hq && is_compact(lse), SQ_ESHAPE,
+               "sq_decode_fwd: lse must be a compact fp32 tensor of B*Hq elements");
+  }
+  int32_t S = params->num_splits > 0 ? params->num_splits : sq_decode_num_splits(B, Hkv, L);
+  if (S > L) S = (int32_t)L;
+  int64_t chunk = (L + S - 1) / S;
+  chunk = (chunk + kTile * kWaves - 1) / (kTile * kWaves) * (kTile * kWaves);
+  const size_t need = sq_decode_workspace_bytes(B, Hq, D, S);
+  SQ_REQUIRE(workspace && on_gpu(workspace) && workspace->device.device_id == dev, SQ_EWORKSPACE,
+             "sq_decode_fwd: workspace missing or not on the device");
+  SQ_REQUIRE((size_t)numel_of(workspace) * (workspace->dtype.bits / 8) >= need && is_compact(workspace), SQ_EWORKSPACE,
+             "sq_decode_fwd: workspace too small: need %zu bytes", need);
+  SQ_REQUIRE(((uintptr_t)data_of(workspace) & 15) == 0, SQ_EWORKSPACE, "sq_decode_fwd: workspace not 16-byte aligned");
+
+  const int64_t group = Hq / Hkv;
+  DecodeArgs a;
+  a.q = data_of(q);
+  a.k = data_of(kcache);
+  a.v = data_of(vcache);
+  a.seqlens = seqlens ? (const int32_t*)data_of(seqlens) : nullptr;
+  a.part_o = (float*)data_of(workspace);
+  a.part_lse = a.part_o + (size_t)B * Hq * S * kD;
+  a.q_sb = stride_of(q, 0);
+  a.q_sh = stride_of(q, hdim);
+  a.k_sb = stride_of(kcache, 0);
+  a.k_sh = stride_of(kcache, hdim);
+  a.k_sn = stride_of(kcache, ndim);
+  a.v_sb = stride_of(vcache, 0);
+  a.v_sh = stride_of(vcache, hdim);
+  a.v_sn = stride_of(vcache, ndim);
+  a.B = (int32_t)B;
+  a.Hq = (int32_t)Hq;
+  a.Hkv = (int32_t)Hkv;
+  a.L = (int32_t)L;
+  a.group = (int32_t)group;
+  a.head_chunks = (int32_t)((group + 15) / 16);
+  a.num_splits = S;
+  a.chunk = (int32_t)chunk;
+  a.p_quant = params->p_quant;
+  const int64_t d_og = params->head_dim_og > 0 ? params->head_dim_og : D;
+  SQ_REQUIRE(d_og <= kD, SQ_EINVAL, "Unsupported head_dim: %lld", (long long)d_og);
+  a.sm = (float)(1.0 / sqrt((double)d_og) * 1.44269504);
+
+  hipStream_t st = (hipStream_t)stream;
+  int cur = -1;
+  SQ_HIP(hipGetDevice(&cur));
+  SQ_REQUIRE(cur == dev, SQ_EDEVICE, "sq_decode_fwd: tensors live on device %d but the current device is %d", dev, cur);
+  const dim3 grid((unsigned)S, (unsigned)(Hkv * a.head_chunks), (unsigned)B);
+  if (dt == DType::BF16) {
+    hipLaunchKernelGGL(decode_splitkv_kernel<true>, grid, dim3(kWaves * 64), 0, st, a);
+  } else {
+    hipLaunchKernelGGL(decode_splitkv_kernel<false>, grid, dim3(kWaves * 64), 0, st, a);
+  }
+  SQ_HIP(hipGetLastError());
+  CombineArgs c;
+  c.part_o = a.part_o;
+  c.part_lse = a.part_lse;
+  c.out = data_of(out);
+  c.lse = lse ? (float*)data_of(lse) : nullptr;
+  c.o_sb = stride_of(out, 0);
+  c.o_sh = stride_of(out, hdim);
+  c.Hq = (int32_t)Hq;
+  c.num_splits = S;
+  c.out_dtype = odt == DType::BF16 ? 0 : (odt == DType::F16 ? 1 : 2);
+  hipLaunchKernelGGL(decode_combine_kernel, dim3((unsigned)Hq, (unsigned)B), dim3(kD), 0, st, c);
+  SQ_HIP(hipGetLastError());
+  return SQ_OK;
+}

@@ -1,0 +1,68 @@
+"""`attn_unified` / `attn_causal` of the reference's sqattn/attn_triton_decode.py:244-375 on the HIP kernels.
+
+`qo_len == 1` runs the split-KV decode kernel (one pass over the cache for all q-heads of a KV group,
+LSE combine); anything else runs the prefill kernel.  The module keeps the reference's file name so that
+imports keep working; nothing here uses Triton.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from .. import _native as N
+from ._common import pad_head_dim, require_gpu
+
+
+def attn_decode(q, k, v, tensor_layout="HND", output_dtype=torch.float16, return_lse=False, is_P_fp8_quant=False,
+                seqlens: Optional[torch.Tensor] = None, num_splits: int = 0, workspace: Optional[torch.Tensor] = None,
+                out: Optional[torch.Tensor] = None):
+    """Decode attention: q [B,Hq,1,D] (HND) or [B,1,Hq,D] (NHD) against caches [B,Hkv,L,D] / [B,L,Hkv,D].
+
+    Extensions over the reference (all optional): `seqlens` int32 [B] valid prefix per sequence,
+    `num_splits` KV splits, caller-provided `workspace`/`out` so that a serving loop allocates nothing.
+    """
+    if tensor_layout not in N.LAYOUT:
+        raise ValueError(f"tensor_layout {tensor_layout} not supported")
+    require_gpu(q, k, v)
+    head_dim_og = q.size(-1)
+    q, k, v = pad_head_dim((q, k, v), head_dim_og)
+    assert q.stride(-1) == 1 and k.stride(-1) == 1 and v.stride(-1) == 1
+    hdim, ndim = (1, 2) if tensor_layout == "HND" else (2, 1)
+    B, Hq, Hkv, L = q.size(0), q.size(hdim), k.size(hdim), k.size(ndim)
+    lib = N.lib()
+    S = num_splits if num_splits > 0 else lib.sq_decode_num_splits(B, Hkv, L)
+    need = lib.sq_decode_workspace_bytes(B, Hq, 128, S)
+    if workspace is None:
+        workspace = torch.empty(need // 4, dtype=torch.float32, device=q.device)
+    o = out if out is not None else torch.empty(q.shape, dtype=output_dtype, device=q.device)
+    lse = torch.empty([B, Hq, 1], dtype=torch.float32, device=q.device) if return_lse else None
+    params = N.DecodeParams(N.LAYOUT[tensor_layout], N.P_E4M3_STATIC if is_P_fp8_quant else N.P_NONE, S, head_dim_og)
+    bq, bk, bv, bs, bo, bl, bw = (N.dl(t) for t in (q, k, v, seqlens, o, lse, workspace))
+    N.check(lib.sq_decode_fwd(N.ptr(bq), N.ptr(bk), N.ptr(bv), N.ptr(bs), N.ptr(bo), N.ptr(bl), N.ptr(bw),
+                              params, N.current_stream(q.device)))
+    o = o[..., :head_dim_og]
+    return (o, lse) if return_lse else o
+
+
+def attn_unified(q, k, v, tensor_layout="HND", output_dtype=torch.float16, return_lse=False, is_P_fp8_quant=False):
+    """Unified interface (attn_triton_decode.py:244-361).
+
+    Decode: the per-channel K-mean subtraction of the reference (:268-269) is skipped, it shifts all
+    scores of a row equally and cannot change the softmax.  Prefill: K is centred with tensor ops as in
+    the reference (the bf16 rounding of the centred K is part of its result), then the prefill kernel runs.
+    """
+    if tensor_layout not in N.LAYOUT:
+        raise ValueError(f"tensor_layout {tensor_layout} not supported")
+    seq_dim = 1 if tensor_layout == "NHD" else 2
+    if q.size(seq_dim) == 1:
+        return attn_decode(q, k, v, tensor_layout, output_dtype, return_lse, is_P_fp8_quant)
+    from .attn_triton import attn_causal as _prefill
+
+    k = k - k.mean(dim=seq_dim, keepdim=True)
+    return _prefill(q, k, v, tensor_layout, output_dtype, return_lse, is_P_fp8_quant)
+
+
+def attn_causal(q, k, v, tensor_layout="HND", output_dtype=torch.float16, return_lse=False, is_P_fp8_quant=False):
+    """Alias kept by the reference (attn_triton_decode.py:364-375)."""
+    return attn_unified(q, k, v, tensor_layout, output_dtype, return_lse, is_P_fp8_quant)
