@@ -1,7 +1,652 @@
+// Causal / sink+window prefill attention for gfx950 (MI355X).
+//
+// Replaces the reference's Triton prefill kernels and their wrappers:
+//   full causal      sqattn/attn_triton.py:10-87 (_attn_fwd_inner), :90-213 (_attn_fwd), :216-315 (attn_causal)
+//   relative window  sqattn/attn_triton_mix_relative.py:8-99, :102-306, :309-483
+//   absolute window  sqattn/attn_triton_mix_bad.py:9-98, :101-282, :285-426
+// All three run the same KV-block step (S = q~.k, running max, p = exp2(S-m), l += sum p, optional e4m3
+// round trip of p, acc += fp16(p).fp16(v)); they differ only in which 64-key blocks a query block visits.
+//
+// Design (CDNA4, 64-wide waves, 1 wave per SIMD, 512 registers per lane):
+//   * workgroup = WAVES waves x 64 query rows of one q-head; K and V^T tiles of 64 keys are staged once per
+//     workgroup in LDS (double buffered, padded rows) and shared by all its rows;
+//   * S^T = K . Q~^T on v_mfma_f32_32x32x16 (bf16 or f16): K rows are the A operand straight out of LDS, Q~
+//     stays in registers as the B operand for the whole kernel.  The accumulator then holds, per lane,
+//     one query row and 32 of the 64 keys, so the row max needs one cross-lane exchange and the row sum none;
+//   * P^T in that accumulator layout *is* the B-operand layout of O^T += V^T . P^T (f16 MFMA), provided V^T is
+//     stored with the matching key permutation -- a one-off pre-pass writes V as fp16, transposed, permuted
+//     tiles into the workspace (O(N) work against the O(N^2) main loop);
+//   * blockIdx -> (kv head, q head, q block) mapping keeps the q-heads of one KV head on the same XCD(s) so
+//     their K/V tiles are shared in that XCD's L2, and issues the longest (last) query blocks first.
 #include "common.hpp"
+
+namespace sq {
+namespace {
+
+constexpr int kD = 128;
+constexpr int kBN = 64;                  // keys per tile (BLOCK_N of every reference kernel)
+constexpr int kRowsPerWave = 64;
+constexpr int kKStride = 272;            // bytes per K row in LDS (256 + 16 pad)
+constexpr int kVStride = 144;            // bytes per V^T row in LDS (128 + 16 pad)
+constexpr int kKTileBytes = kBN * kKStride;
+constexpr int kVTileBytes = kD * kVStride;
+constexpr int kStageBytes = kKTileBytes + kVTileBytes;
+constexpr int kMaxHeads = 128;
+
+struct PrefillArgs {
+  const void* q;
+  const void* k;
+  const void* q4;   // operands of the 4-bit window range (null: same as q/k)
+  const void* k4;
+  const _Float16* vt;  // [B, Hkv, nT, 128, 64] fp16 transposed, permuted V tiles
+  void* out;
+  float* lse;
+  int64_t q_sb, q_sh, q_sn;
+  int64_t k_sb, k_sh, k_sn;
+  int64_t o_sb, o_sh, o_sn;
+  int32_t B, Hq, Hkv, group, Nq, Nk, nT, nQB;
+  int32_t q_offset, p_quant, window_mode, block_m, sink, out_dtype;
+  int32_t sched_mode, sched_xpp, sched_items, sched_pairs;
+  float sm;
+  int32_t w8[kMaxHeads];
+  int32_t w4[kMaxHeads];
+};
+
+struct PrepArgs {
+  const void* v;
+  _Float16* vt;
+  int64_t v_sb, v_sh, v_sn;
+  int32_t Nk, nT, Hkv, is_bf16;
+};
+
+// position of key u (0..15) inside its group of 16 in the V^T tile: bits 2 and 3 swapped, so that the 8
+// keys a lane owns in one half of the S^T accumulator are 8 consecutive halfs.
+__device__ __forceinline__ int perm16(int u) { return (u & 3) | ((u & 4) << 1) | ((u & 8) >> 1); }
+
+__global__ __launch_bounds__(256) void prefill_prep_v_kernel(PrepArgs a) {
+  const int j = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+  const int o = threadIdx.x & 15;    // channel octet
+  const int tq = threadIdx.x >> 4;   // key quad
+  const uint16_t* vb = (const uint16_t*)a.v + (int64_t)b * a.v_sb + (int64_t)kvh * a.v_sh;
+  _Float16 h[4][8];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int n = j * kBN + 4 * tq + i;
+    uint4 raw = make_uint4(0, 0, 0, 0);
+    if (n < a.Nk) raw = *(const uint4*)(vb + (int64_t)n * a.v_sn + 8 * o);
+    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const uint32_t bits = (e & 1) ? (w[e >> 1] >> 16) : (w[e >> 1] & 0xffffu);
+      h[i][e] = a.is_bf16 ? (_Float16)bf16_bits_to_f32(bits) : __builtin_bit_cast(_Float16, (uint16_t)bits);
+    }
+  }
+  _Float16* tile = a.vt + (((int64_t)b * a.Hkv + kvh) * a.nT + j) * (int64_t)(kD * kBN);
+  const int pos = (4 * tq & ~15) | perm16(4 * tq & 15);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    f16x4_t val = {h[0][e], h[1][e], h[2][e], h[3][e]};
+    *(f16x4_t*)(tile + (8 * o + e) * kBN + pos) = val;
+  }
+}
+
+template <bool BF16>
+__device__ __forceinline__ f32x16_t mfma_qk32(const uint4& a, const uint4& b, f32x16_t c) {
+  if constexpr (BF16) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b),
+                                                   c, 0, 0, 0);
+  } else {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c,
+                                                  0, 0, 0);
+  }
+}
+
+__device__ __forceinline__ f32x16_t mfma_pv32(const uint4& a, const uint4& b, f32x16_t c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0,
+                                                0, 0);
+}
+
+__device__ __forceinline__ uint32_t pack_f16(float lo, float hi) {
+  typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+  typedef __attribute__((ext_vector_type(2))) _Float16 f16x2_t;
+  f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2_t));
+}
+
+template <bool BF16>
+__device__ __forceinline__ uint32_t scale_pair(uint32_t w, float sm) {
+  if constexpr (BF16) {
+    const float lo = bf16_bits_to_f32(w & 0xffffu) * sm;
+    const float hi = bf16_bits_to_f32(w >> 16) * sm;
+    return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+  } else {
+    const float lo = (float)__builtin_bit_cast(_Float16, (uint16_t)(w & 0xffffu)) * sm;
+    const float hi = (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> 16)) * sm;
+    return pack_f16(lo, hi);
+  }
+}
+
+// The KV tiles one 64-row wave visits, in tile units (multiples of 64 keys).
+struct WaveRanges {
+  int sink_hi;    // [0, sink_hi)
+  int win_lo;     // [win_lo, win_hi): window tiles strictly before the query block
+  int win_hi;
+  int r4_lo;      // [r4_lo, r4_hi): tiles of the 4-bit window range (subset of the window tiles)
+  int r4_hi;
+  int diag_lo;    // [diag_lo, diag_hi]: tiles of the query block itself up to this wave's own diagonal tile
+  int diag_hi;
+  __device__ __forceinline__ bool visits(int j) const {
+    return j < sink_hi || (j >= win_lo && j < win_hi) || (j >= diag_lo && j <= diag_hi);
+  }
+};
+
+__device__ __forceinline__ WaveRanges wave_ranges(const PrefillArgs& a, int pos0, int head) {
+  WaveRanges r;
+  if (a.window_mode == SQ_WINDOW_NONE) {  // attn_triton.py:57-63
+    r.sink_hi = 0;
+    r.win_lo = 0;
+    r.win_hi = pos0 / kBN;
+    r.r4_lo = r.r4_hi = 0;
+    r.diag_lo = r.diag_hi = pos0 / kBN;
+    return r;
+  }
+  // attn_triton_mix_relative.py:36-75 / attn_triton_mix_bad.py:37-74
+  const int qs = pos0 / a.block_m * a.block_m;
+  const int qe = qs + a.block_m;
+  const int w8 = a.w8[head], w4 = a.w4[head];
+  const int left4 = max(a.sink, qe - w4);
+  const int left8 = max(a.sink, qe - w8);
+  r.sink_hi = min(a.sink, qs) / kBN;
+  int lo = qs, hi = qs;
+  r.r4_lo = r.r4_hi = 0;
+  if (left8 < qs) lo = left8;
+  if (left4 < left8) {  // range 2 non-empty; the host guarantees left8 <= qs here
+    r.r4_lo = left4 / kBN;
+    r.r4_hi = left8 / kBN;
+    lo = left4;
+  }
+  r.win_lo = lo / kBN;
+  r.win_hi = hi / kBN;
+  r.diag_lo = qs / kBN;
+  r.diag_hi = pos0 / kBN;
+  return r;
+}
+
+template <bool BF16, int WAVES>
+__global__ __launch_bounds__(WAVES * 64, 1) void prefill_kernel(PrefillArgs a) {
+  constexpr int NT = WAVES * 64;
+  constexpr int CH = (kBN * kD * 2 / 16) / NT;  // 16-byte chunks per thread and tile operand
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+
+  // ---- schedule: blockIdx -> (pair = (b, kvh), item = (q block descending, head in group))
+  int pair, item;
+  {
+    const int id = blockIdx.x;
+    if (a.sched_mode == 0) {  // pairs share the 8 XCDs evenly: sched_xpp XCDs per pair
+      const int xcd = id & 7, s = id >> 3;
+      pair = xcd / a.sched_xpp;
+      item = s * a.sched_xpp + xcd % a.sched_xpp;
+    } else if (a.sched_mode == 1) {  // one XCD works through pairs xcd, xcd+8, ...
+      const int xcd = id & 7, s = id >> 3;
+      pair = (s / a.sched_items) * 8 + xcd;
+      item = s % a.sched_items;
+    } else {
+      pair = id % a.sched_pairs;
+      item = id / a.sched_pairs;
+    }
+    if (item >= a.sched_items || pair >= a.sched_pairs) return;
+  }
+  const int b = pair / a.Hkv, kvh = pair % a.Hkv;
+  const int hg = item % a.group;
+  const int qb = a.nQB - 1 - item / a.group;
+  const int head = kvh * a.group + hg;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int c32 = lane & 31, g = lane >> 5;
+
+  const int row_wg0 = qb * (WAVES * kRowsPerWave);          // first query row of the workgroup
+  const int row_w0 = row_wg0 + wave * kRowsPerWave;         // first query row of this wave
+  const int pos0 = a.q_offset + row_w0;                     // its absolute position
+  const bool wave_active = row_w0 < a.Nq;
+  const WaveRanges wr = wave_ranges(a, pos0, head);
+
+  // ---- workgroup-level tile schedule: segment A = sink tiles, segment B = window .. last diagonal
+  int segA_hi = 0, segB_lo = 1 << 30, segB_hi = 0;
+#pragma unroll
+  for (int w = 0; w < WAVES; ++w) {
+    const int rw = row_wg0 + w * kRowsPerWave;
+    if (rw < a.Nq) {
+      const WaveRanges o = wave_ranges(a, a.q_offset + rw, head);
+      segA_hi = max(segA_hi, o.sink_hi);
+      segB_lo = min(segB_lo, min(o.win_lo, o.diag_lo));
+      segB_hi = max(segB_hi, o.diag_hi + 1);
+    }
+  }
+  segB_hi = min(segB_hi, a.nT);
+  if (segB_lo <= segA_hi) {  // contiguous: one segment
+    segA_hi = 0;
+    segB_lo = 0;
+  }
+  const bool distinct4 = a.q4 != nullptr;  // host guarantees WAVES*64 <= block_m in that case
+
+  // ---- Q~ fragments (B operand of S^T = K.Q~^T): lane (column = row c32 of block bm, k-group g)
+  uint4 qf[2][8];
+  auto load_q = [&](const void* qbase) {
+    const uint16_t* qp = (const uint16_t*)qbase + (int64_t)b * a.q_sb + (int64_t)head * a.q_sh;
+#pragma unroll
+    for (int bm = 0; bm < 2; ++bm) {
+      const int row = min(row_w0 + 32 * bm + c32, a.Nq - 1);
+      const uint16_t* rp = qp + (int64_t)max(row, 0) * a.q_sn + 8 * g;
+#pragma unroll
+      for (int kk = 0; kk < 8; ++kk) {
+        const uint4 raw = *(const uint4*)(rp + 16 * kk);
+        qf[bm][kk] = make_uint4(scale_pair<BF16>(raw.x, a.sm), scale_pair<BF16>(raw.y, a.sm),
+                                scale_pair<BF16>(raw.z, a.sm), scale_pair<BF16>(raw.w, a.sm));
+      }
+    }
+  };
+  load_q(a.q);
+  bool q_is4 = false;
+
+  f32x16_t O[4][2];
+#pragma unroll
+  for (int bd = 0; bd < 4; ++bd)
+#pragma unroll
+    for (int bm = 0; bm < 2; ++bm)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) O[bd][bm][i] = 0.f;
+  float m_run[2] = {-INFINITY, -INFINITY};
+  float l_run[2] = {0.f, 0.f};
+
+  const _Float16* vt_base = a.vt + ((int64_t)b * a.Hkv + kvh) * (int64_t)a.nT * (kD * kBN);
+
+  // ---- tile staging helpers
+  uint4 kreg[CH], vreg[CH];
+  auto tile_uses4 = [&](int j) { return distinct4 && j >= wr.r4_lo && j < wr.r4_hi; };
+  auto gload = [&](int j) {
+    const void* ksrc = tile_uses4(j) ? a.k4 : a.k;
+    const uint16_t* kb = (const uint16_t*)ksrc + (int64_t)b * a.k_sb + (int64_t)kvh * a.k_sh;
+    const uint4* vsrc = (const uint4*)(vt_base + (int64_t)j * (kD * kBN));
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const int ch = c * NT + tid;            // chunk id 0..1023
+      const int n = min(j * kBN + (ch >> 4), a.Nk - 1);
+      kreg[c] = *(const uint4*)(kb + (int64_t)n * a.k_sn + 8 * (ch & 15));
+      vreg[c] = vsrc[ch];
+    }
+  };
+  auto lstore = [&](int stage) {
+    char* kbuf = smem + stage * kStageBytes;
+    char* vbuf = kbuf + kKTileBytes;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const int ch = c * NT + tid;
+      *(uint4*)(kbuf + (ch >> 4) * kKStride + (ch & 15) * 16) = kreg[c];
+      *(uint4*)(vbuf + (ch >> 3) * kVStride + (ch & 7) * 16) = vreg[c];
+    }
+  };
+  auto next_tile = [&](int j) {
+    int n = j + 1;
+    if (n >= segA_hi && n < segB_lo) n = segB_lo;
+    return n;
+  };
+
+  int j = (segA_hi > 0) ? 0 : segB_lo;
+  if (j < segB_hi) {
+    gload(j);
+    lstore(0);
+  }
+  __syncthreads();
+
+  for (int it = 0; j < segB_hi; ++it) {
+    const int jn = next_tile(j);
+    const bool have_next = jn < segB_hi;
+    if (have_next) gload(jn);
+
+    if (wave_active && wr.visits(j)) {
+      if (distinct4) {  // switch the Q~ operand set when entering/leaving the 4-bit window range
+        const bool want4 = tile_uses4(j);
+        if (want4 != q_is4) {
+          load_q(want4 ? a.q4 : a.q);
+          q_is4 = want4;
+        }
+      }
+      const char* kbuf = smem + (it & 1) * kStageBytes;
+      const char* vbuf = kbuf + kKTileBytes;
+
+      // S^T[key, row] for 2 key blocks x 2 row blocks of 32
+      f32x16_t S[2][2];
+#pragma unroll
+      for (int bn = 0; bn < 2; ++bn)
+#pragma unroll
+        for (int bm = 0; bm < 2; ++bm)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) S[bn][bm][i] = 0.f;
+#pragma unroll
+      for (int kk = 0; kk < 8; ++kk) {
+        const uint4 a0 = *(const uint4*)(kbuf + c32 * kKStride + (16 * kk + 8 * g) * 2);
+        const uint4 a1 = *(const uint4*)(kbuf + (32 + c32) * kKStride + (16 * kk + 8 * g) * 2);
+        S[0][0] = mfma_qk32<BF16>(a0, qf[0][kk], S[0][0]);
+        S[0][1] = mfma_qk32<BF16>(a0, qf[1][kk], S[0][1]);
+        S[1][0] = mfma_qk32<BF16>(a1, qf[0][kk], S[1][0]);
+        S[1][1] = mfma_qk32<BF16>(a1, qf[1][kk], S[1][1]);
+      }
+      if (j >= wr.diag_lo) {  // causal mask inside the query block's own tiles (attn_triton.py:69-71)
+#pragma unroll
+        for (int bn = 0; bn < 2; ++bn)
+#pragma unroll
+          for (int bm = 0; bm < 2; ++bm)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+              const int col = j * kBN + 32 * bn + 8 * (i >> 2) + 4 * g + (i & 3);
+              const int row = pos0 + 32 * bm + c32;
+              if (col > row) S[bn][bm][i] = -INFINITY;
+            }
+      }
+      // online softmax per query row (= lane column); keys of a row live in this lane and lane^32
+      float alpha[2];
+#pragma unroll
+      for (int bm = 0; bm < 2; ++bm) {
+        float tmax = -INFINITY;
+#pragma unroll
+        for (int bn = 0; bn < 2; ++bn)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) tmax = fmaxf(tmax, S[bn][bm][i]);
+        tmax = wave_xor_max(tmax, 32);
+        const float m_new = fmaxf(m_run[bm], tmax);
+        alpha[bm] = exp2f(m_run[bm] - m_new);
+        m_run[bm] = m_new;
+        float psum = 0.f;
+#pragma unroll
+        for (int bn = 0; bn < 2; ++bn)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            const float p = exp2f(S[bn][bm][i] - m_new);
+            S[bn][bm][i] = p;
+            psum += p;
+          }
+        l_run[bm] = l_run[bm] * alpha[bm] + psum;
+      }
+      // quantise P and pack to fp16 in the B-operand layout of the P.V MFMA
+      if (a.p_quant == SQ_P_E4M3_BLOCK) {
+        float amax = 0.f;
+#pragma unroll
+        for (int bn = 0; bn < 2; ++bn)
+#pragma unroll
+          for (int bm = 0; bm < 2; ++bm)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) amax = fmaxf(amax, S[bn][bm][i]);
+#pragma unroll
+        for (int sh = 1; sh < 64; sh <<= 1) amax = wave_xor_max(amax, sh);
+        const float sc = 448.f / amax;   // amax > 0: every visited tile has an unmasked key per row
+        const float inv = amax / 448.f;
+#pragma unroll
+        for (int bn = 0; bn < 2; ++bn)
+#pragma unroll
+          for (int bm = 0; bm < 2; ++bm)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) S[bn][bm][i] = e4m3_roundtrip(fminf(S[bn][bm][i] * sc, 448.f)) * inv;
+      } else if (a.p_quant == SQ_P_E4M3_STATIC) {
+#pragma unroll
+        for (int bn = 0; bn < 2; ++bn)
+#pragma unroll
+          for (int bm = 0; bm < 2; ++bm)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) S[bn][bm][i] = e4m3_roundtrip(S[bn][bm][i] * 448.f) * (1.0f / 448.0f);
+      }
+      uint4 P[2][2][2];  // [bm][bn][t]
+#pragma unroll
+      for (int bm = 0; bm < 2; ++bm)
+#pragma unroll
+        for (int bn = 0; bn < 2; ++bn)
+#pragma unroll
+          for (int t = 0; t < 2; ++t) {
+            const f32x16_t& s = S[bn][bm];
+            P[bm][bn][t] = make_uint4(pack_f16(s[8 * t + 0], s[8 * t + 1]), pack_f16(s[8 * t + 2], s[8 * t + 3]),
+                                      pack_f16(s[8 * t + 4], s[8 * t + 5]), pack_f16(s[8 * t + 6], s[8 * t + 7]));
+          }
+      if (__any(alpha[0] != 1.f || alpha[1] != 1.f)) {
+#pragma unroll
+        for (int bd = 0; bd < 4; ++bd)
+#pragma unroll
+          for (int bm = 0; bm < 2; ++bm) O[bd][bm] *= alpha[bm];
+      }
+      // O^T[d, row] += V^T[d, key] . P^T[key, row]
+#pragma unroll
+      for (int bd = 0; bd < 4; ++bd)
+#pragma unroll
+        for (int bn = 0; bn < 2; ++bn)
+#pragma unroll
+          for (int t = 0; t < 2; ++t) {
+            const uint4 av = *(const uint4*)(vbuf + (32 * bd + c32) * kVStride + (32 * bn + 16 * t + 8 * g) * 2);
+            O[bd][0] = mfma_pv32(av, P[0][bn][t], O[bd][0]);
+            O[bd][1] = mfma_pv32(av, P[1][bn][t], O[bd][1]);
+          }
+    }
+
+    if (have_next) lstore((it + 1) & 1);
+    __syncthreads();
+    j = jn;
+  }
+
+  // ---- epilogue: out = acc / l (attn_triton.py:208-209), lse2 = log2(l) + m (:210-213)
+  if (!wave_active) return;
+#pragma unroll
+  for (int bm = 0; bm < 2; ++bm) {
+    const float l = l_run[bm] + __shfl_xor(l_run[bm], 32);
+    const int row = row_w0 + 32 * bm + c32;
+    if (row >= a.Nq) continue;
+    const int64_t obase = (int64_t)b * a.o_sb + (int64_t)head * a.o_sh + (int64_t)row * a.o_sn;
+#pragma unroll
+    for (int bd = 0; bd < 4; ++bd)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4) {
+        const int d = 32 * bd + 8 * i4 + 4 * g;
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = O[bd][bm][4 * i4 + e] / l;
+        if (a.out_dtype == 0) {
+          uint2 w = make_uint2(f32_to_bf16_bits(v[0]) | (f32_to_bf16_bits(v[1]) << 16),
+                               f32_to_bf16_bits(v[2]) | (f32_to_bf16_bits(v[3]) << 16));
+          *(uint2*)((uint16_t*)a.out + obase + d) = w;
+        } else if (a.out_dtype == 1) {
+          uint2 w = make_uint2(pack_f16(v[0], v[1]), pack_f16(v[2], v[3]));
+          *(uint2*)((uint16_t*)a.out + obase + d) = w;
+        } else {
+          *(float4*)((float*)a.out + obase + d) = make_float4(v[0], v[1], v[2], v[3]);
+        }
+      }
+    if (a.lse && g == 0) a.lse[((int64_t)b * a.Hq + head) * a.Nq + row] = log2f(l) + m_run[bm];
+  }
+}
+
+}  // namespace
+}  // namespace sq
+
 using namespace sq;
-extern "C" size_t sq_prefill_workspace_bytes(int64_t, int64_t, int64_t, int64_t) { return 0; }
-extern "C" int sq_prefill_fwd(const DLTensor*, const DLTensor*, const DLTensor*, const DLTensor*, const DLTensor*,
-                              DLTensor*, DLTensor*, DLTensor*, const sq_prefill_params*, void*) {
-  SQ_FAIL(SQ_EUNSUPPORTED, "sq_prefill_fwd: not built yet");
+
+extern "C" size_t sq_prefill_workspace_bytes(int64_t batch, int64_t num_kv_heads, int64_t kv_len, int64_t head_dim) {
+  (void)head_dim;
+  if (batch <= 0 || num_kv_heads <= 0 || kv_len <= 0) return 0;
+  const int64_t nT = (kv_len + kBN - 1) / kBN;
+  return (size_t)(batch * num_kv_heads * nT) * (size_t)(kD * kBN) * sizeof(_Float16);
+}
+
+extern "C" int sq_prefill_fwd(const DLTensor* q, const DLTensor* k, const DLTensor* v, const DLTensor* q4,
+                              const DLTensor* k4, DLTensor* out, DLTensor* lse, DLTensor* workspace,
+                              const sq_prefill_params* p, void* stream) {
+  SQ_REQUIRE(p, SQ_EINVAL, "sq_prefill_fwd: params is null");
+  SQ_REQUIRE(q && k && v && out, SQ_EINVAL, "sq_prefill_fwd: q, k, v and out must be non-null");
+  SQ_REQUIRE(p->layout == SQ_LAYOUT_HND || p->layout == SQ_LAYOUT_NHD, SQ_EINVAL, "tensor_layout %d not supported", p->layout);
+  SQ_REQUIRE(p->p_quant >= SQ_P_NONE && p->p_quant <= SQ_P_E4M3_BLOCK, SQ_EINVAL, "sq_prefill_fwd: p_quant %d not supported", p->p_quant);
+  SQ_REQUIRE((q4 == nullptr) == (k4 == nullptr), SQ_EINVAL, "sq_prefill_fwd: q4 and k4 must be given together");
+  int rc;
+  const int dev = q->device.device_id;
+  if ((rc = check_tensor(q, "q", 4, dev)) || (rc = check_tensor(k, "k", 4, dev)) || (rc = check_tensor(v, "v", 4, dev)) ||
+      (rc = check_tensor(out, "out", 4, dev)))
+    return rc;
+  if (q4 && ((rc = check_tensor(q4, "q4", 4, dev)) || (rc = check_tensor(k4, "k4", 4, dev)))) return rc;
+  const DType dt = dtype_of(q);
+  SQ_REQUIRE(dt == DType::BF16 || dt == DType::F16, SQ_EDTYPE, "sq_prefill_fwd: q must be bf16 or fp16");
+  SQ_REQUIRE(dtype_of(k) == dt && dtype_of(v) == dt, SQ_EDTYPE, "sq_prefill_fwd: q, k, v dtypes differ");
+  if (q4) SQ_REQUIRE(dtype_of(q4) == dt && dtype_of(k4) == dt, SQ_EDTYPE, "sq_prefill_fwd: q4/k4 dtype differs from q");
+  const DType odt = dtype_of(out);
+  SQ_REQUIRE(odt == DType::BF16 || odt == DType::F16 || odt == DType::F32, SQ_EDTYPE, "sq_prefill_fwd: out must be bf16, fp16 or fp32");
+  const bool hnd = p->layout == SQ_LAYOUT_HND;
+  const int hdim = hnd ? 1 : 2, ndim = hnd ? 2 : 1;
+  const int64_t B = q->shape[0], Hq = q->shape[hdim], Nq = q->shape[ndim], D = q->shape[3];
+  const int64_t Hkv = k->shape[hdim], Nk = k->shape[ndim];
+  SQ_REQUIRE(D == kD, SQ_EINVAL, "Unsupported head_dim: %lld (the kernels take 128; pad smaller heads with zeros)", (long long)D);
+  SQ_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && Nq > 0 && Nk > 0, SQ_ESHAPE, "sq_prefill_fwd: empty tensor");
+  SQ_REQUIRE(Hq % Hkv == 0, SQ_ESHAPE, "sq_prefill_fwd: Hq=%lld not a multiple of Hkv=%lld", (long long)Hq, (long long)Hkv);
+  SQ_REQUIRE(Hq <= kMaxHeads, SQ_EUNSUPPORTED, "sq_prefill_fwd: more than %d q heads", kMaxHeads);
+  SQ_REQUIRE(k->shape[0] == B && k->shape[3] == D, SQ_ESHAPE, "sq_prefill_fwd: k shape mismatch");
+  for (int i = 0; i < 4; ++i) {
+    SQ_REQUIRE(v->shape[i] == k->shape[i], SQ_ESHAPE, "sq_prefill_fwd: v shape differs from k");
+    SQ_REQUIRE(out->shape[i] == q->shape[i], SQ_ESHAPE, "sq_prefill_fwd: out shape differs from q");
+    if (q4) {
+      SQ_REQUIRE(q4->shape[i] == q->shape[i] && k4->shape[i] == k->shape[i], SQ_ESHAPE, "sq_prefill_fwd: q4/k4 shapes differ from q/k");
+      SQ_REQUIRE(stride_of(q4, i) == stride_of(q, i) && stride_of(k4, i) == stride_of(k, i), SQ_ESHAPE,
+                 "sq_prefill_fwd: q4/k4 strides differ from q/k");
+    }
+  }
+  SQ_REQUIRE(p->q_offset >= 0 && p->q_offset % kBN == 0, SQ_EINVAL, "sq_prefill_fwd: q_offset must be a non-negative multiple of 64");
+  SQ_REQUIRE(p->q_offset + Nq == Nk, SQ_ESHAPE,
+             "qo_len and kv_len must be equal for causal attention (q_offset + qo_len = %lld, kv_len = %lld)",
+             (long long)(p->q_offset + Nq), (long long)Nk);
+  SQ_REQUIRE(Nk < (1ll << 31) - 65536, SQ_EUNSUPPORTED, "sq_prefill_fwd: more than 2^31 keys");
+  const DLTensor* ts[5] = {q, k, v, out, nullptr};
+  for (int t = 0; t < 4; ++t)
+    for (int i = 0; i < 3; ++i)
+      SQ_REQUIRE(stride_of(ts[t], i) % (t == 3 && odt == DType::F32 ? 4 : 8) == 0 || ts[t]->shape[i] == 1, SQ_ESHAPE,
+                 "sq_prefill_fwd: strides must keep rows 16-byte aligned");
+  if (lse) {
+    SQ_REQUIRE(on_gpu(lse) && lse->device.device_id == dev, SQ_EDEVICE, "sq_prefill_fwd: lse not on the same device");
+    SQ_REQUIRE(dtype_of(lse) == DType::F32 && numel_of(lse) == B * Hq * Nq && is_compact(lse), SQ_ESHAPE,
+               "sq_prefill_fwd: lse must be a compact fp32 [B,Hq,Nq]");
+  }
+  int waves = 4;
+  if (p->window_mode == SQ_WINDOW_SIZES) {
+    SQ_REQUIRE(p->block_m == 64 || p->block_m == 128, SQ_EINVAL, "sq_prefill_fwd: block_m must be 64 or 128");
+    SQ_REQUIRE(p->sink >= 0, SQ_EINVAL, "sink_size must be a non-negative integer, got %d", p->sink);
+    SQ_REQUIRE(p->sink % kBN == 0, SQ_EUNSUPPORTED, "sq_prefill_fwd: sink_size %d is not a multiple of 64", p->sink);
+    SQ_REQUIRE(p->w8 && p->w4 && p->num_heads_w == Hq, SQ_EINVAL, "sq_prefill_fwd: w8/w4 must hold one window per q head");
+    SQ_REQUIRE(p->q_offset % p->block_m == 0, SQ_EINVAL, "sq_prefill_fwd: q_offset must be a multiple of block_m");
+    for (int h = 0; h < Hq; ++h) {
+      SQ_REQUIRE(p->w8[h] >= 0 && p->w4[h] >= 0, SQ_EINVAL, "sq_prefill_fwd: negative window size for head %d", h);
+      SQ_REQUIRE(p->w8[h] % kBN == 0 && p->w4[h] % kBN == 0, SQ_EUNSUPPORTED,
+                 "sq_prefill_fwd: window sizes must be multiples of 64 (head %d: %d / %d)", h, p->w8[h], p->w4[h]);
+      // with w4 > w8 and w8 < block_m the reference's 4-bit range overlaps the diagonal block unmasked
+      SQ_REQUIRE(!(p->w4[h] > p->w8[h] && p->w8[h] < p->block_m), SQ_EUNSUPPORTED,
+                 "sq_prefill_fwd: head %d: a 4-bit window wider than an 8-bit window smaller than block_m reads future keys "
+                 "in the reference and is not supported", h);
+    }
+    if (q4) waves = p->block_m / kRowsPerWave;  // all waves of a workgroup must agree on the operand set of a tile
+    SQ_REQUIRE(waves >= 2, SQ_EUNSUPPORTED, "sq_prefill_fwd: separate 4-bit operands need block_m = 128");
+  } else {
+    SQ_REQUIRE(p->window_mode == SQ_WINDOW_NONE, SQ_EINVAL, "sq_prefill_fwd: window_mode %d not supported", p->window_mode);
+    SQ_REQUIRE(!q4, SQ_EINVAL, "sq_prefill_fwd: q4/k4 only apply to window mode");
+  }
+  const size_t need = sq_prefill_workspace_bytes(B, Hkv, Nk, D);
+  SQ_REQUIRE(workspace && on_gpu(workspace) && workspace->device.device_id == dev, SQ_EWORKSPACE,
+             "sq_prefill_fwd: workspace missing or not on the device");
+  SQ_REQUIRE((size_t)numel_of(workspace) * (workspace->dtype.bits / 8) >= need && is_compact(workspace), SQ_EWORKSPACE,
+             "sq_prefill_fwd: workspace too small: need %zu bytes", need);
+  SQ_REQUIRE(((uintptr_t)data_of(workspace) & 15) == 0, SQ_EWORKSPACE, "sq_prefill_fwd: workspace not 16-byte aligned");
+
+  hipStream_t st = (hipStream_t)stream;
+  int cur = -1;
+  SQ_HIP(hipGetDevice(&cur));
+  SQ_REQUIRE(cur == dev, SQ_EDEVICE, "sq_prefill_fwd: tensors live on device %d but the current device is %d", dev, cur);
+
+  const int nT = (int)((Nk + kBN - 1) / kBN);
+  PrepArgs pa;
+  pa.v = data_of(v);
+  pa.vt = (_Float16*)data_of(workspace);
+  pa.v_sb = stride_of(v, 0);
+  pa.v_sh = stride_of(v, hdim);
+  pa.v_sn = stride_of(v, ndim);
+  pa.Nk = (int)Nk;
+  pa.nT = nT;
+  pa.Hkv = (int)Hkv;
+  pa.is_bf16 = dt == DType::BF16;
+  hipLaunchKernelGGL(prefill_prep_v_kernel, dim3(nT, (unsigned)Hkv, (unsigned)B), dim3(256), 0, st, pa);
+  SQ_HIP(hipGetLastError());
+
+  PrefillArgs local;  // passed to the kernel by value (about 1.2 KB with the per-head windows)
+  memset(&local, 0, sizeof(local));
+  local.q = data_of(q);
+  local.k = data_of(k);
+  local.q4 = q4 ? data_of(q4) : nullptr;
+  local.k4 = k4 ? data_of(k4) : nullptr;
+  local.vt = pa.vt;
+  local.out = data_of(out);
+  local.lse = lse ? (float*)data_of(lse) : nullptr;
+  local.q_sb = stride_of(q, 0);
+  local.q_sh = stride_of(q, hdim);
+  local.q_sn = stride_of(q, ndim);
+  local.k_sb = stride_of(k, 0);
+  local.k_sh = stride_of(k, hdim);
+  local.k_sn = stride_of(k, ndim);
+  local.o_sb = stride_of(out, 0);
+  local.o_sh = stride_of(out, hdim);
+  local.o_sn = stride_of(out, ndim);
+  local.B = (int)B;
+  local.Hq = (int)Hq;
+  local.Hkv = (int)Hkv;
+  local.group = (int)(Hq / Hkv);
+  local.Nq = (int)Nq;
+  local.Nk = (int)Nk;
+  local.nT = nT;
+  const int rows_wg = waves * kRowsPerWave;
+  local.nQB = (int)((Nq + rows_wg - 1) / rows_wg);
+  local.q_offset = (int)p->q_offset;
+  local.p_quant = p->p_quant;
+  local.window_mode = p->window_mode;
+  local.block_m = p->window_mode == SQ_WINDOW_SIZES ? p->block_m : 128;
+  local.sink = p->sink;
+  local.out_dtype = odt == DType::BF16 ? 0 : (odt == DType::F16 ? 1 : 2);
+  const int64_t d_og = p->head_dim_og > 0 ? p->head_dim_og : D;
+  SQ_REQUIRE(d_og <= kD, SQ_EINVAL, "Unsupported head_dim: %lld", (long long)d_og);
+  local.sm = (float)(1.0 / sqrt((double)d_og) * 1.44269504);
+  if (p->window_mode == SQ_WINDOW_SIZES)
+    for (int h = 0; h < Hq; ++h) {
+      local.w8[h] = p->w8[h];
+      local.w4[h] = p->w4[h];
+    }
+  const int pairs = (int)(B * Hkv);
+  const int items = local.group * local.nQB;
+  local.sched_pairs = pairs;
+  local.sched_items = items;
+  unsigned blocks;
+  if (pairs <= 8 && 8 % pairs == 0) {
+    local.sched_mode = 0;
+    local.sched_xpp = 8 / pairs;
+    blocks = 8u * (unsigned)((items + local.sched_xpp - 1) / local.sched_xpp);
+  } else if (pairs % 8 == 0) {
+    local.sched_mode = 1;
+    local.sched_xpp = 1;
+    blocks = (unsigned)pairs * (unsigned)items;
+  } else {
+    local.sched_mode = 2;
+    local.sched_xpp = 1;
+    blocks = (unsigned)pairs * (unsigned)items;
+  }
+  const size_t smem = 2 * kStageBytes;
+  const bool bf = dt == DType::BF16;
+#define SQ_LAUNCH_PREFILL(BF, W)                                                                              \
+  do {                                                                                                        \
+    SQ_HIP(hipFuncSetAttribute((const void*)prefill_kernel<BF, W>, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                               (int)smem));                                                                   \
+    hipLaunchKernelGGL((prefill_kernel<BF, W>), dim3(blocks), dim3(W * 64), smem, st, local);                 \
+  } while (0)
+  if (waves == 4) {
+    if (bf) SQ_LAUNCH_PREFILL(true, 4); else SQ_LAUNCH_PREFILL(false, 4);
+  } else {
+    if (bf) SQ_LAUNCH_PREFILL(true, 2); else SQ_LAUNCH_PREFILL(false, 2);
+  }
+#undef SQ_LAUNCH_PREFILL
+  SQ_HIP(hipGetLastError());
+  return SQ_OK;
 }

@@ -1,0 +1,172 @@
+"""GPU parity: prefill kernel (through the C ABI) against the CPU oracle.
+
+Stated tolerances.  Kernel vs the same-algorithm oracle (identical quantisation points; only v_exp_f32 and
+fp32 summation order differ): without P quantisation max|d| <= 2e-3 * rms(out); with e4m3 P a few
+probabilities sit within an ulp of a rounding boundary and flip to the neighbouring e4m3 value, so the
+check is cosine >= 0.99999, 99.9 % of elements within 2e-3 * rms and every element within 0.25 * rms.
+Kernel vs exact attention: cosine >= 0.999 (the bar of the benchmark configuration).
+"""
+import math
+
+import pytest
+import torch
+
+from oracle import attention as A
+from oracle import inputs
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _cos(a, b):
+    a, b = a.double().flatten(), b.double().flatten()
+    return float(a @ b / (a.norm() * b.norm()))
+
+
+def _check(out, ref, quantised):
+    out, ref = out.double().cpu(), ref.double()
+    rms = float(ref.pow(2).mean().sqrt())
+    d = (out - ref).abs()
+    if not quantised:
+        assert float(d.max()) <= 2e-3 * rms, (float(d.max()), rms)
+    else:
+        assert _cos(out, ref) >= 0.99999
+        assert float(torch.quantile(d.flatten()[:: max(1, d.numel() // 1000000)], 0.999)) <= 2e-3 * rms
+        assert float(d.max()) <= 0.25 * rms, (float(d.max()), rms)
+
+
+def _rand(B, Hq, Hkv, N, D, seed, dtype=torch.bfloat16, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    q = (torch.randn(B, Hq, N, D, generator=g) * scale).to(dtype)
+    k = (torch.randn(B, Hkv, N, D, generator=g) * scale).to(dtype)
+    v = (torch.randn(B, Hkv, N, D, generator=g) * scale).to(dtype)
+    return q, k, v
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,N", [(1, 4, 2, 512), (2, 14, 2, 700), (1, 2, 1, 64), (1, 3, 3, 1000)])
+@pytest.mark.parametrize("mode", [A.P_NONE, A.P_STATIC448, A.P_BLOCK_ABSMAX])
+def test_causal_matches_oracle(B, Hq, Hkv, N, mode):
+    from longcontext_sqattn_paddle_amd.sqattn.attn_triton import attn_causal
+
+    print(f"case prefill causal B={B} Hq={Hq} Hkv={Hkv} N={N} p_quant={mode}", flush=True)
+    q, k, v = _rand(B, Hq, Hkv, N, 128, 100 + N)
+    ref, lse_ref = A.prefill_blockwise(q, k, v, p_quant=mode, out_dtype=torch.float32)
+    out, lse = attn_causal(q.to(DEV), k.to(DEV), v.to(DEV), "HND", torch.float32, return_lse=True, p_quant=mode)
+    torch.cuda.synchronize()
+    _check(out, ref, mode != A.P_NONE)
+    assert torch.allclose(lse.cpu(), lse_ref, atol=2e-4)
+    exact, _ = A.exact_attention(q, k, v)
+    assert _cos(out.cpu(), exact) >= 0.999
+
+
+def test_nhd_layout_bf16_out_and_gqa_7():
+    from longcontext_sqattn_paddle_amd.sqattn.attn_triton import attn_causal
+
+    q, k, v = _rand(1, 28, 4, 384, 128, 7)
+    ref, _ = A.prefill_blockwise(q, k, v, p_quant=A.P_STATIC448, out_dtype=torch.float32)
+    qn, kn, vn = (t.permute(0, 2, 1, 3).contiguous().to(DEV) for t in (q, k, v))
+    out = attn_causal(qn, kn, vn, "NHD", torch.bfloat16, is_P_fp8_quant=True)
+    torch.cuda.synchronize()
+    assert out.shape == (1, 384, 28, 128) and out.dtype == torch.bfloat16
+    o = out.permute(0, 2, 1, 3).float().cpu()
+    assert _cos(o, ref) >= 0.9999
+    assert float((o - ref).abs().max()) <= 2 ** -7 * float(ref.abs().max()) + 0.25 * float(ref.pow(2).mean().sqrt())
+
+
+def test_fp16_inputs_and_head_dim_64():
+    from longcontext_sqattn_paddle_amd.sqattn.attn_triton import attn_causal
+
+    q, k, v = _rand(1, 4, 2, 320, 64, 9, dtype=torch.float16)
+    ref, lse_ref = A.prefill_blockwise(q, k, v, out_dtype=torch.float32)
+    out, lse = attn_causal(q.to(DEV), k.to(DEV), v.to(DEV), "HND", torch.float32, return_lse=True)
+    torch.cuda.synchronize()
+    assert out.shape == (1, 4, 320, 64)
+    _check(out, ref, False)
+    assert torch.allclose(lse.cpu(), lse_ref, atol=2e-4)
+
+
+def test_config2_style_inputs_with_k_outliers():
+    from longcontext_sqattn_paddle_amd.sqattn.attn_triton import attn_causal
+
+    q, k, v = inputs.prefill_inputs(1, 7, 1, 2048, 128, seed=2)
+    ref, _ = A.prefill_blockwise(q, k, v, p_quant=A.P_STATIC448, out_dtype=torch.float32)
+    out = attn_causal(q.to(DEV), k.to(DEV), v.to(DEV), "HND", torch.float32, is_P_fp8_quant=True)
+    torch.cuda.synchronize()
+    _check(out, ref, True)
+    exact, _ = A.exact_attention(q, k, v)
+    assert _cos(out.cpu(), exact) >= 0.999
+
+
+def test_chunked_prefill_offset():
+    from longcontext_sqattn_paddle_amd.sqattn.attn_triton import attn_causal
+
+    q, k, v = _rand(1, 4, 2, 768, 128, 11)
+    ref, lse_ref = A.prefill_blockwise(q, k, v, out_dtype=torch.float32)
+    out, lse = attn_causal(q[:, :, 512:].contiguous().to(DEV), k.to(DEV), v.to(DEV), "HND", torch.float32,
+                           return_lse=True, q_offset=512)
+    torch.cuda.synchronize()
+    _check(out, ref[:, :, 512:], False)
+    assert torch.allclose(lse.cpu(), lse_ref[:, :, 512:], atol=2e-4)
+
+
+@pytest.mark.parametrize("sink,r8,r4", [(128, 0.25, 0.25), (256, [0.125, 0.5], [0.5, 0.5]), (0, 0.0, 0.0), (64, 2.0, 2.0)])
+def test_relative_window_matches_oracle(sink, r8, r4):
+    from longcontext_sqattn_paddle_amd.sqattn.attn_triton_mix_relative import attn_hierarchical_relative_window
+
+    N = 1024
+    q, k, v = _rand(1, 2, 1, N, 128, 13)
+    l8 = r8 if isinstance(r8, list) else [r8, r8]
+    l4 = r4 if isinstance(r4, list) else [r4, r4]
+    w8 = [A.window_size_relative(x, N) for x in l8]
+    w4 = [A.window_size_relative(x, N) for x in l4]
+    ref, lse_ref = A.prefill_blockwise(q, k, v, block_m=64, sink=sink, w8=w8, w4=w4, out_dtype=torch.float32)
+    qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
+    out, lse = attn_hierarchical_relative_window(qd, kd, qd, kd, vd, r8, r4, sink, "HND", torch.float32, return_lse=True)
+    torch.cuda.synchronize()
+    _check(out, ref, False)
+    assert torch.allclose(lse.cpu(), lse_ref, atol=2e-4)
+
+
+@pytest.mark.parametrize("sink,w8,w4,distinct", [(128, 256, 512, True), (64, 128, 128, True), (256, [128, 384], [640, 384], True),
+                                                 (128, 256, 512, False), (0, 0, 0, False)])
+def test_absolute_window_matches_oracle(sink, w8, w4, distinct):
+    from longcontext_sqattn_paddle_amd.sqattn.attn_triton_mix_bad import attn_hierarchical_window
+    from oracle import fake_quant as FQ
+
+    N = 1152
+    q, k, v = _rand(1, 2, 1, N, 128, 17)
+    q4 = FQ.int_fake_quant(q, 4, True, "per_token") if distinct else q
+    k4 = FQ.int_fake_quant(k, 4, True, "per_token") if distinct else k
+    l8 = w8 if isinstance(w8, list) else [w8, w8]
+    l4 = w4 if isinstance(w4, list) else [w4, w4]
+    ref, lse_ref = A.prefill_blockwise(q, k, v, block_m=128, sink=sink, w8=l8, w4=l4, q4=q4, k4=k4, out_dtype=torch.float32)
+    qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
+    q4d, k4d = (q4.to(DEV), k4.to(DEV)) if distinct else (qd, kd)
+    arg8 = torch.tensor(l8, dtype=torch.int32) if isinstance(w8, list) else w8
+    arg4 = torch.tensor(l4, dtype=torch.int32) if isinstance(w4, list) else w4
+    out, lse = attn_hierarchical_window(qd, kd, q4d, k4d, vd, arg8, arg4, sink, "HND", torch.float32, return_lse=True)
+    torch.cuda.synchronize()
+    _check(out, ref, False)
+    assert torch.allclose(lse.cpu(), lse_ref, atol=2e-4)
+
+
+def test_prefill_argument_errors():
+    from longcontext_sqattn_paddle_amd.sqattn.attn_triton import attn_causal
+    from longcontext_sqattn_paddle_amd.sqattn.attn_triton_mix_relative import attn_hierarchical_relative_window
+
+    q = torch.zeros(1, 2, 128, 128, dtype=torch.bfloat16, device=DEV)
+    k = torch.zeros(1, 1, 128, 128, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(ValueError):
+        attn_causal(q, k, k, "DNH")
+    with pytest.raises(ValueError):
+        attn_causal(torch.zeros(1, 2, 128, 256, dtype=torch.bfloat16, device=DEV), k, k)
+    with pytest.raises(AssertionError):   # qo_len != kv_len (attn_triton.py:272)
+        attn_causal(q, k[:, :, :64].contiguous(), k[:, :, :64].contiguous())
+    with pytest.raises(AssertionError):   # last dim not contiguous (attn_triton.py:245-247)
+        attn_causal(q.transpose(2, 3).contiguous().transpose(2, 3), k, k)
+    with pytest.raises(ValueError):       # sink must be a non-negative int (attn_triton_mix_relative.py:367-368)
+        attn_hierarchical_relative_window(q, k, q, k, k, 0.1, 0.1, -1)
+    with pytest.raises(ValueError):
+        attn_hierarchical_relative_window(q, k, q, k, k, 0.1, 0.1, 2.5)
+    with pytest.raises(RuntimeError):     # no CPU path
+        attn_causal(q.cpu(), k.cpu(), k.cpu())
