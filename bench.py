@@ -1,0 +1,177 @@
+#!/usr/bin/env python3
+"""Headline benchmark: SQAttn prefill attention at 128K (Qwen2.5-7B layer shape, FP8-e4m3 P) on one MI355X,
+with the 1M-token split-KV decode as the second half of the metric, a roofline object for the dominant
+kernel and the reference's fake-quant + SDPA path timed on the host cores.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--seq-len N] [--no-cpu-baseline] [--no-decode]
+
+Prints ONE JSON line on stdout.  A "step" is one full prefill attention call (V pre-pass + main kernel) on
+inputs already resident in HBM.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+METRIC = "prefill attn TFLOP/s @128K + decode HBM GB/s @1M, Qwen2.5-7B GQA 28/4 heads"
+PEAK_MFMA_BF16_TFLOPS = 2500.0   # MI355X dense bf16/fp16 MFMA
+PEAK_HBM_GBS = 8000.0            # MI355X HBM3E
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def time_prefill(torch, N, steps, warmup, p_quant):
+    from longcontext_sqattn_paddle_amd import workloads
+    from longcontext_sqattn_paddle_amd.sqattn._prefill import prefill_workspace
+    from longcontext_sqattn_paddle_amd.sqattn.attn_triton import attn_causal
+
+    dev = torch.device("cuda:0")
+    Hq, Hkv, D = 28, 4, 128
+    t0 = time.time()
+    q, k, v = workloads.prefill_inputs(1, Hq, Hkv, N, D, seed=2)
+    q, k, v = q.to(dev), k.to(dev), v.to(dev)
+    log(f"[bench] prefill inputs N={N} generated and uploaded in {time.time() - t0:.1f}s")
+    ws = prefill_workspace(1, Hkv, N, dev)
+    out = torch.empty_like(q)
+    stream = torch.cuda.current_stream(dev)
+
+    def step():
+        attn_causal(q, k, v, "HND", torch.bfloat16, p_quant=p_quant, workspace=ws, out=out)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    for _ in range(steps):
+        step()
+    e1.record(stream)
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / steps
+    flops = 4.0 * N * N * D * Hq / 2   # causal half, FlashAttention convention
+    # a finite, non-trivial output guards against timing a launch that did nothing
+    chk = out[0, :, -1, :].float()
+    assert bool(torch.isfinite(chk).all()) and float(chk.abs().sum()) > 0
+    return ms, flops
+
+
+def time_decode(torch, B, L, iters=20, warmup=5):
+    from longcontext_sqattn_paddle_amd.sqattn.attn_triton_decode import DecodePlan
+
+    dev = torch.device("cuda:0")
+    Hq, Hkv, D = 28, 4, 128
+    g = torch.Generator(device=dev).manual_seed(3)
+    nset = 2   # rotate buffer sets so that the 256 MB Infinity Cache cannot serve a re-read
+    plans, total = [], 0
+    for _ in range(nset):
+        q = torch.randn(B, 1, Hq, D, device=dev, generator=g).bfloat16()
+        kc = torch.randn(B, L, Hkv, D, device=dev, generator=g, dtype=torch.bfloat16)
+        vc = torch.randn(B, L, Hkv, D, device=dev, generator=g, dtype=torch.bfloat16)
+        lens = torch.randint((3 * L) // 4, L + 1, (B,), device=dev, generator=g, dtype=torch.int32) if B > 1 else \
+            torch.full((B,), L, device=dev, dtype=torch.int32)
+        plans.append(DecodePlan(q, kc, vc, "NHD", torch.bfloat16, seqlens=lens))
+        total = int(lens.sum().item())
+    stream = torch.cuda.current_stream(dev)
+    for i in range(warmup):
+        plans[i % nset].run()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    for i in range(iters):
+        plans[i % nset].run()
+    e1.record(stream)
+    torch.cuda.synchronize()
+    us = e0.elapsed_time(e1) / iters * 1e3
+    nbytes = 2048.0 * total   # K+V bf16, 4 kv heads x 128, read once for all 7 q-heads of a group
+    return us, nbytes
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--seq-len", type=int, default=131072)
+    ap.add_argument("--p-quant", type=int, default=1, help="0 none, 1 e4m3 static 448 (reference), 2 e4m3 block absmax")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-decode", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py needs an MI355X (torch.cuda.is_available() is False)", file=sys.stderr)
+        sys.exit(3)
+    N = args.seq_len
+    ms, flops = time_prefill(torch, N, args.steps, args.warmup, args.p_quant)
+    tflops = flops / ms / 1e9
+    log(f"[bench] prefill N={N}: {ms:.2f} ms/step, {tflops:.1f} TFLOP/s")
+
+    result = {
+        "metric": METRIC,
+        "value": round(tflops, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": f"prefill attention, batch 1, 28 q heads / 4 kv heads, head_dim 128, seq {N}, causal, "
+                        f"bf16 N(0,1)/sqrt(128) with 2% K outlier channels x8, P quant mode {args.p_quant} (e4m3), fp32 accumulate",
+            "flops_per_step": flops,
+        },
+        "roofline": {
+            "bound": "mfma",
+            "kernel": "prefill_kernel",
+            "achieved": round(tflops, 2),
+            "peak": PEAK_MFMA_BF16_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": round(tflops / PEAK_MFMA_BF16_TFLOPS, 4),
+            "traffic": None,
+        },
+    }
+    if not args.no_decode:
+        dec = {}
+        for name, B, L in (("1M_b1", 1, 1048576), ("128K_b1", 1, 131072), ("128K_b8", 8, 131072)):
+            us, nbytes = time_decode(torch, B, L)
+            gbs = nbytes / us / 1e3
+            dec[name] = {"us_per_call": round(us, 2), "GB_per_s": round(gbs, 1), "frac_of_hbm_peak": round(gbs / PEAK_HBM_GBS, 4),
+                         "bytes": nbytes}
+            log(f"[bench] decode {name}: {us:.1f} us, {gbs:.0f} GB/s")
+            torch.cuda.empty_cache()
+        result["decode"] = dec
+    if not args.no_cpu_baseline:
+        from oracle.cpu_baseline import time_cpu_baseline   # the checker's CPU path, timed as the baseline only
+
+        cpu_tflops, threads, dt, n = time_cpu_baseline(budget_s=12.0)
+        result["cpu_baseline"] = {
+            "value": round(cpu_tflops, 4),
+            "unit": "TFLOP/s",
+            "cores": threads,
+            "kind": "port",
+            "sample": f"config-1 shape (batch 1, 4 q heads on 1 kv head, head_dim 128, seq 4096, causal): GQA expand, K centring, "
+                      f"int8/int4 fake-quant, torch CPU SDPA in bf16; {n} passes of {dt * 1e3:.1f} ms on {threads} threads "
+                      f"({os.cpu_count()} logical CPUs)",
+        }
+        log(f"[bench] cpu baseline: {cpu_tflops:.3f} TFLOP/s on {threads} threads")
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

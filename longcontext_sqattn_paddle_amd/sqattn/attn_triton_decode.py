@@ -45,6 +45,38 @@ def attn_decode(q, k, v, tensor_layout="HND", output_dtype=torch.float16, return
     return (o, lse) if return_lse else o
 
 
+class DecodePlan:
+    """A decode launch prepared once and replayed: every tensor (query, caches, seqlens, output, LSE,
+    workspace) is borrowed up front, so `run()` is one C call that allocates nothing.  For serving loops
+    whose buffers stay in place between steps (the KV cache grows in place; `seqlens` is updated on device).
+    """
+
+    def __init__(self, q, k, v, tensor_layout="NHD", output_dtype=torch.bfloat16, return_lse=False,
+                 is_P_fp8_quant=False, seqlens=None, num_splits: int = 0):
+        if tensor_layout not in N.LAYOUT:
+            raise ValueError(f"tensor_layout {tensor_layout} not supported")
+        require_gpu(q, k, v)
+        if q.size(-1) != 128:
+            raise ValueError("DecodePlan needs head_dim 128 tensors (pad once, outside the loop)")
+        hdim, ndim = (1, 2) if tensor_layout == "HND" else (2, 1)
+        B, Hq, Hkv, L = q.size(0), q.size(hdim), k.size(hdim), k.size(ndim)
+        self._lib = N.lib()
+        S = num_splits if num_splits > 0 else self._lib.sq_decode_num_splits(B, Hkv, L)
+        self.workspace = torch.empty(self._lib.sq_decode_workspace_bytes(B, Hq, 128, S) // 4, dtype=torch.float32,
+                                     device=q.device)
+        self.out = torch.empty(q.shape, dtype=output_dtype, device=q.device)
+        self.lse = torch.empty([B, Hq, 1], dtype=torch.float32, device=q.device) if return_lse else None
+        self._params = N.DecodeParams(N.LAYOUT[tensor_layout], N.P_E4M3_STATIC if is_P_fp8_quant else N.P_NONE, S, 128)
+        self._b = [N.dl(t) for t in (q, k, v, seqlens, self.out, self.lse, self.workspace)]
+        self._ptrs = [N.ptr(x) for x in self._b]
+        self._device = q.device
+
+    def run(self, stream=None):
+        st = N.current_stream(self._device) if stream is None else stream
+        N.check(self._lib.sq_decode_fwd(*self._ptrs, self._params, st))
+        return self.out
+
+
 def attn_unified(q, k, v, tensor_layout="HND", output_dtype=torch.float16, return_lse=False, is_P_fp8_quant=False):
     """Unified interface (attn_triton_decode.py:244-361).
 

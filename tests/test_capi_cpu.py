@@ -1,0 +1,92 @@
+"""CPU-side checks of the C ABI: the library loads, exports every symbol the header declares, and
+rejects bad arguments with error codes (no compute call is made here)."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from longcontext_sqattn_paddle_amd import _native as N
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "sqattn.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(sq_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = _declared_symbols()
+    assert "sq_prefill_fwd" in names and "sq_decode_fwd" in names and "sq_kmeans_train" in names
+    handle = ctypes.CDLL(N.LIB_PATH)
+    for n in names:
+        assert hasattr(handle, n), f"{n} declared in include/sqattn.h but not exported"
+    assert set(names) == set(N.SYMBOLS), "ctypes table and header disagree"
+    assert N.lib().sq_abi_version() == 1
+
+
+def test_sizes_and_split_heuristic():
+    lib = N.lib()
+    assert lib.sq_prefill_workspace_bytes(1, 4, 131072, 128) == 4 * 131072 * 128 * 2
+    assert lib.sq_prefill_workspace_bytes(1, 4, 100, 128) == 4 * 2 * 64 * 128 * 2     # rounded up to 64-key tiles
+    s = lib.sq_decode_num_splits(1, 4, 131072)
+    assert 1 <= s <= 131072 // 256
+    assert lib.sq_decode_num_splits(8, 4, 131072) <= s
+    assert lib.sq_decode_workspace_bytes(2, 28, 128, 16) == 2 * 28 * 16 * 129 * 4
+    assert lib.sq_decode_num_splits(1, 4, 10) == 1
+
+
+def _dec(q, k, v, out, ws, layout=0, p_quant=0):
+    lib = N.lib()
+    b = [N.dl(t) for t in (q, k, v, None, out, None, ws)]
+    return lib.sq_decode_fwd(*[N.ptr(x) for x in b], N.DecodeParams(layout, p_quant, 0, 0), None), \
+        lib.sq_last_error().decode()
+
+
+def test_decode_rejects_cpu_tensors_and_bad_arguments():
+    q = torch.zeros(1, 4, 1, 128, dtype=torch.bfloat16)
+    k = torch.zeros(1, 2, 64, 128, dtype=torch.bfloat16)
+    ws = torch.zeros(4096)
+    rc, msg = _dec(q, k, k, q.clone(), ws)
+    assert rc == N.SQ_EDEVICE and "ROCm" in msg
+    rc, msg = _dec(q, k, k, q.clone(), ws, layout=7)
+    assert rc == N.SQ_EINVAL and "tensor_layout" in msg
+    rc, _ = _dec(q, k, k, q.clone(), ws, p_quant=2)
+    assert rc == N.SQ_EINVAL
+    lib = N.lib()
+    assert lib.sq_decode_fwd(None, None, None, None, None, None, None, N.DecodeParams(0, 0, 0, 0), None) == N.SQ_EINVAL
+    assert lib.sq_decode_fwd(None, None, None, None, None, None, None, None, None) == N.SQ_EINVAL
+
+
+def test_prefill_rejects_cpu_tensors_and_bad_arguments():
+    lib = N.lib()
+    q = torch.zeros(1, 2, 64, 128, dtype=torch.bfloat16)
+    b = [N.dl(t) for t in (q, q, q, None, None, q.clone(), None, torch.zeros(64))]
+    p = N.PrefillParams()
+    assert lib.sq_prefill_fwd(*[N.ptr(x) for x in b], ctypes.byref(p), None) == N.SQ_EDEVICE
+    p.layout = 5
+    assert lib.sq_prefill_fwd(*[N.ptr(x) for x in b], ctypes.byref(p), None) == N.SQ_EINVAL
+    p.layout, p.p_quant = 0, 9
+    assert lib.sq_prefill_fwd(*[N.ptr(x) for x in b], ctypes.byref(p), None) == N.SQ_EINVAL
+    assert lib.sq_prefill_fwd(None, None, None, None, None, None, None, None, None, None) == N.SQ_EINVAL
+
+
+def test_error_mapping():
+    with pytest.raises(ValueError):
+        _ = N.check(N.SQ_EINVAL)
+    with pytest.raises(AssertionError):
+        N.check(N.SQ_ESHAPE)
+    with pytest.raises(RuntimeError):
+        N.check(N.SQ_EHIP)
+    N.check(N.SQ_OK)
+
+
+def test_wrappers_refuse_cpu_tensors():
+    from longcontext_sqattn_paddle_amd.sqattn.attn_triton import attn_causal
+
+    q = torch.zeros(1, 2, 64, 128, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        attn_causal(q, q, q)
