@@ -1,16 +1,604 @@
+// KV k-means clustering and centroid-scored token selection for gfx950 (MI355X).
+//
+// Replaces the reference's Triton kernels in cache_hub/kmeans.py:
+//   _triton_assign_kernel :7-79, _triton_update_kernel :82-124, _triton_k_means_train :127-196,
+//   _triton_reverse_index_kernel :199-262, _triton_index_add_kernel :265-329.
+// The reference scatters every token into its cluster sum with fp32 atomics (16.8 M atomics per head and
+// iteration at 131072 x 128).  Here the assignment is a dense bf16 MFMA contraction with an arg-max
+// epilogue in registers, tokens are then counting-sorted by cluster (deterministic, ascending inside a
+// cluster) and every cluster is summed by one workgroup in fp64, which is exact for bf16 data and therefore
+// independent of order.  The same sort yields the reverse index.
 #include "common.hpp"
+
+namespace sq {
+namespace {
+
+constexpr int kD = 128;
+constexpr int kCB = 64;            // centroids per LDS stage
+constexpr int kCStride = 272;      // bytes per centroid row in LDS (256 + 16 pad)
+constexpr int kStage = kCB * kCStride;
+constexpr int kTileTok = 256;      // tokens per workgroup in assign / sort kernels
+constexpr int kMaxC = 8192;
+
+// ------------------------------------------------------------------------------------------ fill
+__global__ void fill_i32_kernel(int32_t* p, int64_t n, int32_t v) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = v;
+}
+
+// ---------------------------------------------------------------------------------------- assign
+struct AssignArgs {
+  const uint16_t* data;  // [G,N,128] bf16
+  const uint16_t* cent;  // [G,C,128] bf16
+  int32_t* idx;          // [G,N]
+  int32_t* cnt;          // [G,C] (pre-zeroed)
+  int64_t d_sg, d_sn, c_sg, c_sc, i_sg, n_sg;
+  int32_t N, C;
+};
+
+__global__ __launch_bounds__(256, 2) void kmeans_assign_kernel(AssignArgs a) {
+  __shared__ __attribute__((aligned(16))) char smem[2 * kStage];
+  const int g_id = blockIdx.y;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int c32 = lane & 31, g = lane >> 5;
+  const int tok0 = blockIdx.x * kTileTok + wave * 64;
+
+  // token fragments (B operand of S^T = Cent . Data^T): lane (column = token c32 of block bm, k-group g)
+  const uint16_t* db = a.data + (int64_t)g_id * a.d_sg;
+  uint4 tf[2][8];
+#pragma unroll
+  for (int bm = 0; bm < 2; ++bm) {
+    const int n = min(tok0 + 32 * bm + c32, a.N - 1);
+    const uint16_t* rp = db + (int64_t)n * a.d_sn + 8 * g;
+#pragma unroll
+    for (int kk = 0; kk < 8; ++kk) tf[bm][kk] = *(const uint4*)(rp + 16 * kk);
+  }
+  float best[2] = {-INFINITY, -INFINITY};
+  int bidx[2] = {0, 0};
+
+  const uint16_t* cb = a.cent + (int64_t)g_id * a.c_sg;
+  uint4 creg[4];
+  auto gload = [&](int chunk) {
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int ch = c * 256 + tid;
+      const int row = min(chunk * kCB + (ch >> 4), a.C - 1);
+      creg[c] = *(const uint4*)(cb + (int64_t)row * a.c_sc + 8 * (ch & 15));
+    }
+  };
+  auto lstore = [&](int stage) {
+    char* buf = smem + stage * kStage;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int ch = c * 256 + tid;
+      *(uint4*)(buf + (ch >> 4) * kCStride + (ch & 15) * 16) = creg[c];
+    }
+  };
+  const int nchunks = (a.C + kCB - 1) / kCB;
+  gload(0);
+  lstore(0);
+  __syncthreads();
+  for (int chunk = 0; chunk < nchunks; ++chunk) {
+    const bool have_next = chunk + 1 < nchunks;
+    if (have_next) gload(chunk + 1);
+    const char* buf = smem + (chunk & 1) * kStage;
+    f32x16_t S[2][2];
+#pragma unroll
+    for (int bn = 0; bn < 2; ++bn)
+#pragma unroll
+      for (int bm = 0; bm < 2; ++bm)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) S[bn][bm][i] = 0.f;
+#pragma unroll
+    for (int kk = 0; kk < 8; ++kk) {
+      const uint4 a0 = *(const uint4*)(buf + c32 * kCStride + (16 * kk + 8 * g) * 2);
+      const uint4 a1 = *(const uint4*)(buf + (32 + c32) * kCStride + (16 * kk + 8 * g) * 2);
+      S[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a0), __builtin_bit_cast(bf16x8_t, tf[0][kk]), S[0][0], 0, 0, 0);
+      S[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a0), __builtin_bit_cast(bf16x8_t, tf[1][kk]), S[0][1], 0, 0, 0);
+      S[1][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a1), __builtin_bit_cast(bf16x8_t, tf[0][kk]), S[1][0], 0, 0, 0);
+      S[1][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a1), __builtin_bit_cast(bf16x8_t, tf[1][kk]), S[1][1], 0, 0, 0);
+    }
+    // running arg-max in ascending centroid order with strict '>' = lowest index on ties (kmeans.py:62-65)
+    const bool tail = (chunk + 1) * kCB > a.C;
+#pragma unroll
+    for (int bm = 0; bm < 2; ++bm)
+#pragma unroll
+      for (int bn = 0; bn < 2; ++bn)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int c = chunk * kCB + 32 * bn + 8 * (i >> 2) + 4 * g + (i & 3);
+          float s = S[bn][bm][i];
+          if (tail && c >= a.C) s = -INFINITY;
+          if (s > best[bm]) {
+            best[bm] = s;
+            bidx[bm] = c;
+          }
+        }
+    if (have_next) lstore((chunk + 1) & 1);
+    __syncthreads();
+  }
+#pragma unroll
+  for (int bm = 0; bm < 2; ++bm) {
+    const float ob = __shfl_xor(best[bm], 32);
+    const int oi = __shfl_xor(bidx[bm], 32);
+    if (ob > best[bm] || (ob == best[bm] && oi < bidx[bm])) {
+      best[bm] = ob;
+      bidx[bm] = oi;
+    }
+    const int n = tok0 + 32 * bm + c32;
+    if (g == 0 && n < a.N) {
+      a.idx[(int64_t)g_id * a.i_sg + n] = bidx[bm];
+      atomicAdd(a.cnt + (int64_t)g_id * a.n_sg + bidx[bm], 1);
+    }
+  }
+}
+
+// ------------------------------------------------------------------------- counting sort by cluster
+struct SortArgs {
+  const int32_t* idx;     // [G,N]
+  int32_t* tile_hist;     // [G,nT,C]  in: per-tile histogram, after scan: exclusive prefix over tiles
+  int32_t* total;         // [G,C]     cluster sizes (written by the scan)
+  int32_t* off;           // [G,C+1]   exclusive prefix over clusters (train only)
+  int32_t* dst;           // order [G,N] (train) or clusters [G,C,M] (reverse index)
+  int64_t i_sg, dst_sg, dst_sc;
+  int32_t N, C, nT, M, use_off;
+};
+
+__global__ __launch_bounds__(kTileTok) void sort_hist_kernel(SortArgs a) {
+  extern __shared__ int32_t hist[];
+  const int tile = blockIdx.x, g = blockIdx.y;
+  for (int c = threadIdx.x; c < a.C; c += blockDim.x) hist[c] = 0;
+  __syncthreads();
+  const int n = tile * kTileTok + threadIdx.x;
+  if (n < a.N) {
+    const int c = a.idx[(int64_t)g * a.i_sg + n];
+    if (c >= 0 && c < a.C) atomicAdd(&hist[c], 1);
+  }
+  __syncthreads();
+  int32_t* out = a.tile_hist + ((int64_t)g * a.nT + tile) * a.C;
+  for (int c = threadIdx.x; c < a.C; c += blockDim.x) out[c] = hist[c];
+}
+
+__global__ __launch_bounds__(256) void sort_scan_tiles_kernel(SortArgs a) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x, g = blockIdx.y;
+  if (c >= a.C) return;
+  int32_t* h = a.tile_hist + (int64_t)g * a.nT * a.C + c;
+  int run = 0;
+  for (int t = 0; t < a.nT; ++t) {
+    const int v = h[(int64_t)t * a.C];
+    h[(int64_t)t * a.C] = run;
+    run += v;
+  }
+  a.total[(int64_t)g * a.C + c] = run;
+}
+
+__global__ __launch_bounds__(1024) void sort_scan_clusters_kernel(SortArgs a) {
+  __shared__ int32_t part[1024];
+  const int g = blockIdx.x, t = threadIdx.x;
+  const int per = (a.C + 1023) / 1024;
+  const int32_t* tot = a.total + (int64_t)g * a.C;
+  int s = 0;
+  for (int i = 0; i < per; ++i) {
+    const int c = t * per + i;
+    if (c < a.C) s += tot[c];
+  }
+  part[t] = s;
+  __syncthreads();
+  for (int d = 1; d < 1024; d <<= 1) {  // Hillis-Steele inclusive scan
+    const int v = (t >= d) ? part[t - d] : 0;
+    __syncthreads();
+    part[t] += v;
+    __syncthreads();
+  }
+  int run = part[t] - s;
+  int32_t* off = a.off + (int64_t)g * (a.C + 1);
+  for (int i = 0; i < per; ++i) {
+    const int c = t * per + i;
+    if (c < a.C) {
+      off[c] = run;
+      run += tot[c];
+    }
+  }
+  if (t == 1023) off[a.C] = part[1023];
+}
+
+__global__ __launch_bounds__(kTileTok) void sort_scatter_kernel(SortArgs a) {
+  __shared__ int32_t cl[kTileTok];
+  const int tile = blockIdx.x, g = blockIdx.y, t = threadIdx.x;
+  const int n = tile * kTileTok + t;
+  const int c = (n < a.N) ? a.idx[(int64_t)g * a.i_sg + n] : -1;
+  cl[t] = c;
+  __syncthreads();
+  if (c < 0 || c >= a.C) return;
+  int rank = 0;
+  for (int u = 0; u < t; ++u) rank += (cl[u] == c);   // tokens of a tile keep their ascending order
+  const int base = a.tile_hist[((int64_t)g * a.nT + tile) * a.C + c] + rank;
+  if (a.use_off) {
+    a.dst[(int64_t)g * a.dst_sg + a.off[(int64_t)g * (a.C + 1) + c] + base] = n;
+  } else if (base < a.M) {
+    a.dst[(int64_t)g * a.dst_sg + (int64_t)c * a.dst_sc + base] = n;
+  }
+}
+
+// ------------------------------------------------------------------------- per-cluster sum + update
+struct SumArgs {
+  const uint16_t* src;    // [G,N,128] bf16 rows to sum (keys for the update, values for index_add)
+  const int32_t* order;   // [G,N] tokens sorted by cluster
+  const int32_t* off;     // [G,C+1]
+  uint16_t* dst;          // [G,C,128] bf16: centroids (update) or value sums (index_add)
+  int64_t s_sg, s_sn, o_sg, d_sg, d_sc;
+  int32_t C, mode;        // mode 0: plain sum cast to bf16; 1: mean; 2: mean + L2 normalise (1,2: only where cnt > 0)
+};
+
+__global__ __launch_bounds__(256) void cluster_sum_kernel(SumArgs a) {
+  __shared__ double red[16][kD];
+  __shared__ double ss_red[kD];
+  const int c = blockIdx.x, g = blockIdx.y, t = threadIdx.x;
+  const int o = t & 15, r = t >> 4;
+  const int32_t* off = a.off + (int64_t)g * (a.C + 1);
+  const int beg = off[c], cnt = off[c + 1] - beg;
+  const int32_t* ord = a.order + (int64_t)g * a.o_sg + beg;
+  const uint16_t* sb = a.src + (int64_t)g * a.s_sg + 8 * o;
+  double acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  for (int i0 = r; i0 < cnt; i0 += 64) {  // 4 rows in flight per thread
+    uint4 raw[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int i = i0 + 16 * u;
+      raw[u] = make_uint4(0, 0, 0, 0);
+      if (i < cnt) raw[u] = *(const uint4*)(sb + (int64_t)ord[i] * a.s_sn);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const uint32_t w[4] = {raw[u].x, raw[u].y, raw[u].z, raw[u].w};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const uint32_t bits = (e & 1) ? (w[e >> 1] >> 16) : (w[e >> 1] & 0xffffu);
+        acc[e] += (double)bf16_bits_to_f32(bits);
+      }
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) red[r][8 * o + e] = acc[e];
+  __syncthreads();
+  float x = 0.f;
+  if (t < kD) {
+    double s = 0;
+#pragma unroll
+    for (int rr = 0; rr < 16; ++rr) s += red[rr][t];
+    x = (float)s;                                   // exact sum rounded once to fp32
+    if (a.mode >= 1) x = x / (float)cnt;            // kmeans.py:121
+    ss_red[t] = (double)x * (double)x;
+  }
+  __syncthreads();
+  if (a.mode == 2) {
+    for (int d = kD / 2; d > 0; d >>= 1) {
+      if (t < d) ss_red[t] += ss_red[t + d];
+      __syncthreads();
+    }
+    if (t < kD) x = x / sqrtf((float)ss_red[0]);    // kmeans.py:122-123
+  }
+  if (t < kD && (a.mode == 0 || cnt > 0))           // empty clusters keep the old centroid (kmeans.py:120,124)
+    a.dst[(int64_t)g * a.d_sg + (int64_t)c * a.d_sc + t] = (uint16_t)f32_to_bf16_bits(x);
+}
+
+// ---------------------------------------------------------------------------------- top-k selection
+struct TopkArgs {
+  const uint16_t* query;   // [B,Hq,128] bf16
+  const uint16_t* cent;    // [G,C,128] bf16
+  const int32_t* clusters; // [G,C,M]
+  const int32_t* size;     // [G,C]
+  int32_t* out;            // [G,k]
+  float* score;            // workspace [G,C]
+  int32_t* start;          // workspace [G,C] start position of each cluster in rank order
+  int64_t q_sb, q_sh, c_sg, c_sc, cl_sg, cl_sc;
+  int32_t C, M, k, Hkv, group;
+};
+
+__global__ __launch_bounds__(256) void topk_score_kernel(TopkArgs a) {
+  const int g = blockIdx.y, b = g / a.Hkv, kvh = g % a.Hkv;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= a.C) return;
+  const uint16_t* cp = a.cent + (int64_t)g * a.c_sg + (int64_t)c * a.c_sc;
+  float best = -INFINITY;
+  for (int h = 0; h < a.group; ++h) {
+    const uint16_t* qp = a.query + (int64_t)b * a.q_sb + (int64_t)(kvh * a.group + h) * a.q_sh;
+    float s = 0.f;
+    for (int d = 0; d < kD; ++d) s += bf16_bits_to_f32(qp[d]) * bf16_bits_to_f32(cp[d]);
+    best = fmaxf(best, s);
+  }
+  a.score[(int64_t)g * a.C + c] = best;
+}
+
+// rank clusters by (score desc, index asc), prefix-sum their sizes in rank order, copy token ids.
+__global__ __launch_bounds__(1024) void topk_emit_kernel(TopkArgs a) {
+  extern __shared__ int32_t sh[];          // [C] size in rank order, then exclusive prefix
+  const int g = blockIdx.x, t = threadIdx.x;
+  const float* sc = a.score + (int64_t)g * a.C;
+  const int32_t* size = a.size + (int64_t)g * a.C;
+  int32_t* start = a.start + (int64_t)g * a.C;
+  for (int c = t; c < a.C; c += blockDim.x) {
+    const float s = sc[c];
+    int rank = 0;
+    for (int u = 0; u < a.C; ++u) {
+      const float v = sc[u];
+      rank += (v > s) || (v == s && u < c);
+    }
+    start[c] = rank;            // temporarily the rank
+    sh[rank] = size[c];
+  }
+  __syncthreads();
+  if (t == 0) {                 // C <= 8192: a serial prefix is a few microseconds
+    int run = 0;
+    for (int r = 0; r < a.C; ++r) {
+      const int v = sh[r];
+      sh[r] = run;
+      run += v;
+    }
+  }
+  __syncthreads();
+  int32_t* out = a.out + (int64_t)g * a.k;
+  for (int c = t; c < a.C; c += blockDim.x) {
+    const int st = sh[start[c]];
+    const int n = min(size[c], a.M);
+    const int32_t* src = a.clusters + (int64_t)g * a.cl_sg + (int64_t)c * a.cl_sc;
+    for (int i = 0; i < n && st + i < a.k; ++i) out[st + i] = src[i];
+  }
+}
+
+__global__ void topk_tail_kernel(TopkArgs a) {
+  // positions past the total number of tokens stay -1
+  const int g = blockIdx.y;
+  const int32_t* size = a.size + (int64_t)g * a.C;
+  __shared__ int tot;
+  if (threadIdx.x == 0) {
+    int s = 0;
+    for (int c = 0; c < a.C; ++c) s += min(size[c], a.M);
+    tot = s;
+  }
+  __syncthreads();
+  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < a.k; i += gridDim.x * blockDim.x)
+    if (i >= tot) a.out[(int64_t)g * a.k + i] = -1;
+}
+
+struct WsLayout {
+  size_t off_bytes, hist_bytes, order_bytes, score_bytes, start_bytes, total_bytes;
+  int nT;
+  size_t all() const { return off_bytes + hist_bytes + order_bytes + score_bytes + start_bytes + total_bytes; }
+};
+
+WsLayout ws_layout(int64_t G, int64_t N, int64_t C) {
+  WsLayout w;
+  auto up = [](size_t x) { return (x + 255) / 256 * 256; };
+  w.nT = (int)((N + kTileTok - 1) / kTileTok);
+  w.off_bytes = up((size_t)G * (C + 1) * 4);
+  w.hist_bytes = up((size_t)G * w.nT * C * 4);
+  w.order_bytes = up((size_t)G * N * 4);
+  w.score_bytes = up((size_t)G * C * 4);
+  w.start_bytes = up((size_t)G * C * 4);
+  w.total_bytes = up((size_t)G * C * 4);
+  return w;
+}
+
+int check_ws(const DLTensor* ws, size_t need, int dev, const char* who) {
+  SQ_REQUIRE(ws && on_gpu(ws) && ws->device.device_id == dev, SQ_EWORKSPACE, "%s: workspace missing or not on the device", who);
+  SQ_REQUIRE((size_t)numel_of(ws) * (ws->dtype.bits / 8) >= need && is_compact(ws), SQ_EWORKSPACE,
+             "%s: workspace too small: need %zu bytes", who, need);
+  SQ_REQUIRE(((uintptr_t)data_of(ws) & 255) == 0, SQ_EWORKSPACE, "%s: workspace not 256-byte aligned", who);
+  return SQ_OK;
+}
+
+int check_current_device(int dev, const char* who) {
+  int cur = -1;
+  SQ_HIP(hipGetDevice(&cur));
+  SQ_REQUIRE(cur == dev, SQ_EDEVICE, "%s: tensors live on device %d but the current device is %d", who, dev, cur);
+  return SQ_OK;
+}
+
+// sorts tokens by cluster into `dst`; shared by train / index_add (order + offsets) and reverse_index
+int run_sort(const DLTensor* idx, char* wsp, const WsLayout& w, int32_t* dst, int64_t dst_sg, int64_t dst_sc, int M,
+             bool use_off, int32_t* total_out, int C, hipStream_t st) {
+  const int64_t G = idx->shape[0], N = idx->shape[1];
+  SortArgs s;
+  s.idx = (const int32_t*)data_of(idx);
+  s.off = (int32_t*)wsp;
+  s.tile_hist = (int32_t*)(wsp + w.off_bytes);
+  s.total = total_out ? total_out : (int32_t*)(wsp + w.off_bytes + w.hist_bytes + w.order_bytes + w.score_bytes + w.start_bytes);
+  s.dst = dst;
+  s.i_sg = stride_of(idx, 0);
+  s.dst_sg = dst_sg;
+  s.dst_sc = dst_sc;
+  s.N = (int)N;
+  s.C = C;
+  s.nT = w.nT;
+  s.M = M;
+  s.use_off = use_off;
+  hipLaunchKernelGGL(sort_hist_kernel, dim3(w.nT, (unsigned)G), dim3(kTileTok), (size_t)C * 4, st, s);
+  hipLaunchKernelGGL(sort_scan_tiles_kernel, dim3((C + 255) / 256, (unsigned)G), dim3(256), 0, st, s);
+  if (use_off) hipLaunchKernelGGL(sort_scan_clusters_kernel, dim3((unsigned)G), dim3(1024), 0, st, s);
+  hipLaunchKernelGGL(sort_scatter_kernel, dim3(w.nT, (unsigned)G), dim3(kTileTok), 0, st, s);
+  SQ_HIP(hipGetLastError());
+  return SQ_OK;
+}
+
+int check_gnd(const DLTensor* t, const char* name, int dev) {
+  int rc = check_tensor(t, name, 3, dev);
+  if (rc) return rc;
+  SQ_REQUIRE(dtype_of(t) == DType::BF16, SQ_EDTYPE, "%s must be bf16", name);
+  SQ_REQUIRE(t->shape[2] == kD, SQ_EUNSUPPORTED, "%s: last dimension must be 128, got %lld", name, (long long)t->shape[2]);
+  SQ_REQUIRE(stride_of(t, 0) % 8 == 0 && stride_of(t, 1) % 8 == 0, SQ_ESHAPE, "%s: strides must be multiples of 8 elements", name);
+  return SQ_OK;
+}
+
+int check_i32(const DLTensor* t, const char* name, int ndim, int dev) {
+  SQ_REQUIRE(t != nullptr, SQ_EINVAL, "%s is null", name);
+  SQ_REQUIRE(on_gpu(t) && t->device.device_id == dev, SQ_EDEVICE, "%s is not on the same ROCm device", name);
+  SQ_REQUIRE(dtype_of(t) == DType::I32 && t->ndim == ndim && is_compact(t), SQ_ESHAPE, "%s must be a compact int32 tensor of rank %d", name, ndim);
+  return SQ_OK;
+}
+
+}  // namespace
+}  // namespace sq
+
 using namespace sq;
-extern "C" size_t sq_kmeans_workspace_bytes(int64_t, int64_t, int64_t, int64_t) { return 0; }
-extern "C" int sq_kmeans_train(const DLTensor*, DLTensor*, DLTensor*, DLTensor*, DLTensor*, int32_t, void*) {
-  SQ_FAIL(SQ_EUNSUPPORTED, "sq_kmeans_train: not built yet");
+
+extern "C" size_t sq_kmeans_workspace_bytes(int64_t groups, int64_t num_tokens, int64_t num_centroids, int64_t dim) {
+  (void)dim;
+  if (groups <= 0 || num_tokens <= 0 || num_centroids <= 0) return 0;
+  return ws_layout(groups, num_tokens, num_centroids).all();
 }
-extern "C" int sq_reverse_index(const DLTensor*, DLTensor*, DLTensor*, DLTensor*, void*) {
-  SQ_FAIL(SQ_EUNSUPPORTED, "sq_reverse_index: not built yet");
+
+extern "C" int sq_kmeans_train(const DLTensor* data, DLTensor* centroids, DLTensor* idx, DLTensor* cnt, DLTensor* workspace,
+                               int32_t normalize, void* stream) {
+  SQ_REQUIRE(data && centroids && idx && cnt, SQ_EINVAL, "sq_kmeans_train: data, centroids, idx and cnt must be non-null");
+  const int dev = data->device.device_id;
+  int rc;
+  if ((rc = check_gnd(data, "data", dev)) || (rc = check_gnd(centroids, "centroids", dev)) || (rc = check_i32(idx, "idx", 2, dev)) ||
+      (rc = check_i32(cnt, "cnt", 2, dev)))
+    return rc;
+  const int64_t G = data->shape[0], N = data->shape[1], C = centroids->shape[1];
+  SQ_REQUIRE(G > 0 && N > 0 && C > 0, SQ_ESHAPE, "sq_kmeans_train: empty tensor");
+  SQ_REQUIRE(centroids->shape[0] == G && idx->shape[0] == G && idx->shape[1] == N && cnt->shape[0] == G && cnt->shape[1] == C,
+             SQ_ESHAPE, "sq_kmeans_train: shapes of data/centroids/idx/cnt disagree");
+  SQ_REQUIRE(C % 32 == 0, SQ_ESHAPE, "num_centroids %% 32 != 0 (num_centroids = %lld)", (long long)C);
+  SQ_REQUIRE(C <= kMaxC, SQ_EUNSUPPORTED, "sq_kmeans_train: more than %d centroids", kMaxC);
+  SQ_REQUIRE(N < (1ll << 31) - 65536, SQ_EUNSUPPORTED, "sq_kmeans_train: too many tokens");
+  const WsLayout w = ws_layout(G, N, C);
+  if ((rc = check_ws(workspace, w.all(), dev, "sq_kmeans_train")) || (rc = check_current_device(dev, "sq_kmeans_train"))) return rc;
+  hipStream_t st = (hipStream_t)stream;
+  char* wsp = data_of(workspace);
+
+  hipLaunchKernelGGL(fill_i32_kernel, dim3(64), dim3(256), 0, st, (int32_t*)data_of(cnt), G * C, 0);
+  AssignArgs a;
+  a.data = (const uint16_t*)data_of(data);
+  a.cent = (const uint16_t*)data_of(centroids);
+  a.idx = (int32_t*)data_of(idx);
+  a.cnt = (int32_t*)data_of(cnt);
+  a.d_sg = stride_of(data, 0);
+  a.d_sn = stride_of(data, 1);
+  a.c_sg = stride_of(centroids, 0);
+  a.c_sc = stride_of(centroids, 1);
+  a.i_sg = stride_of(idx, 0);
+  a.n_sg = stride_of(cnt, 0);
+  a.N = (int)N;
+  a.C = (int)C;
+  hipLaunchKernelGGL(kmeans_assign_kernel, dim3((unsigned)((N + kTileTok - 1) / kTileTok), (unsigned)G), dim3(256), 0, st, a);
+  SQ_HIP(hipGetLastError());
+  int32_t* order = (int32_t*)(wsp + w.off_bytes + w.hist_bytes);
+  if ((rc = run_sort(idx, wsp, w, order, N, 0, 0, true, nullptr, (int)C, st))) return rc;
+  SumArgs s;
+  s.src = a.data;
+  s.order = order;
+  s.off = (const int32_t*)wsp;
+  s.dst = (uint16_t*)data_of(centroids);
+  s.s_sg = a.d_sg;
+  s.s_sn = a.d_sn;
+  s.o_sg = N;
+  s.d_sg = a.c_sg;
+  s.d_sc = a.c_sc;
+  s.C = (int)C;
+  s.mode = normalize ? 2 : 1;
+  hipLaunchKernelGGL(cluster_sum_kernel, dim3((unsigned)C, (unsigned)G), dim3(256), 0, st, s);
+  SQ_HIP(hipGetLastError());
+  return SQ_OK;
 }
-extern "C" int sq_index_add(const DLTensor*, const DLTensor*, DLTensor*, DLTensor*, void*) {
-  SQ_FAIL(SQ_EUNSUPPORTED, "sq_index_add: not built yet");
+
+extern "C" int sq_reverse_index(const DLTensor* idx, DLTensor* clusters, DLTensor* cluster_size, DLTensor* workspace, void* stream) {
+  SQ_REQUIRE(idx && clusters && cluster_size, SQ_EINVAL, "sq_reverse_index: idx, clusters and cluster_size must be non-null");
+  const int dev = idx->device.device_id;
+  int rc;
+  if ((rc = check_i32(idx, "idx", 2, dev)) || (rc = check_i32(clusters, "clusters", 3, dev)) ||
+      (rc = check_i32(cluster_size, "cluster_size", 2, dev)))
+    return rc;
+  const int64_t G = idx->shape[0], N = idx->shape[1], C = clusters->shape[1], M = clusters->shape[2];
+  SQ_REQUIRE(G > 0 && N > 0 && C > 0 && M > 0, SQ_ESHAPE, "sq_reverse_index: empty tensor");
+  SQ_REQUIRE(clusters->shape[0] == G && cluster_size->shape[0] == G && cluster_size->shape[1] == C, SQ_ESHAPE,
+             "sq_reverse_index: shapes of idx/clusters/cluster_size disagree");
+  SQ_REQUIRE(C <= kMaxC, SQ_EUNSUPPORTED, "sq_reverse_index: more than %d centroids", kMaxC);
+  const WsLayout w = ws_layout(G, N, C);
+  if ((rc = check_ws(workspace, w.all(), dev, "sq_reverse_index")) || (rc = check_current_device(dev, "sq_reverse_index"))) return rc;
+  hipStream_t st = (hipStream_t)stream;
+  hipLaunchKernelGGL(fill_i32_kernel, dim3(256), dim3(256), 0, st, (int32_t*)data_of(clusters), G * C * M, 0);
+  return run_sort(idx, data_of(workspace), w, (int32_t*)data_of(clusters), C * M, M, (int)M, false,
+                  (int32_t*)data_of(cluster_size), (int)C, st);
 }
-extern "C" int sq_topk_select(const DLTensor*, const DLTensor*, const DLTensor*, const DLTensor*, DLTensor*, DLTensor*,
-                              int32_t, void*) {
-  SQ_FAIL(SQ_EUNSUPPORTED, "sq_topk_select: not built yet");
+
+extern "C" int sq_index_add(const DLTensor* value, const DLTensor* idx, DLTensor* out, DLTensor* workspace, void* stream) {
+  SQ_REQUIRE(value && idx && out, SQ_EINVAL, "sq_index_add: value, idx and out must be non-null");
+  const int dev = value->device.device_id;
+  int rc;
+  if ((rc = check_gnd(value, "value", dev)) || (rc = check_gnd(out, "out", dev)) || (rc = check_i32(idx, "idx", 2, dev))) return rc;
+  const int64_t G = value->shape[0], N = value->shape[1], C = out->shape[1];
+  SQ_REQUIRE(G > 0 && N > 0 && C > 0, SQ_ESHAPE, "sq_index_add: empty tensor");
+  SQ_REQUIRE(out->shape[0] == G && idx->shape[0] == G && idx->shape[1] == N, SQ_ESHAPE, "sq_index_add: shapes disagree");
+  SQ_REQUIRE(C <= kMaxC, SQ_EUNSUPPORTED, "sq_index_add: more than %d centroids", kMaxC);
+  const WsLayout w = ws_layout(G, N, C);
+  if ((rc = check_ws(workspace, w.all(), dev, "sq_index_add")) || (rc = check_current_device(dev, "sq_index_add"))) return rc;
+  hipStream_t st = (hipStream_t)stream;
+  char* wsp = data_of(workspace);
+  int32_t* order = (int32_t*)(wsp + w.off_bytes + w.hist_bytes);
+  if ((rc = run_sort(idx, wsp, w, order, N, 0, 0, true, nullptr, (int)C, st))) return rc;
+  SumArgs s;
+  s.src = (const uint16_t*)data_of(value);
+  s.order = order;
+  s.off = (const int32_t*)wsp;
+  s.dst = (uint16_t*)data_of(out);
+  s.s_sg = stride_of(value, 0);
+  s.s_sn = stride_of(value, 1);
+  s.o_sg = N;
+  s.d_sg = stride_of(out, 0);
+  s.d_sc = stride_of(out, 1);
+  s.C = (int)C;
+  s.mode = 0;
+  hipLaunchKernelGGL(cluster_sum_kernel, dim3((unsigned)C, (unsigned)G), dim3(256), 0, st, s);
+  SQ_HIP(hipGetLastError());
+  return SQ_OK;
+}
+
+extern "C" int sq_topk_select(const DLTensor* query, const DLTensor* centroids, const DLTensor* clusters,
+                              const DLTensor* cluster_size, DLTensor* out, DLTensor* workspace, int32_t num_kv_groups,
+                              void* stream) {
+  SQ_REQUIRE(query && centroids && clusters && cluster_size && out, SQ_EINVAL, "sq_topk_select: null tensor argument");
+  const int dev = query->device.device_id;
+  int rc;
+  if ((rc = check_gnd(query, "query", dev)) || (rc = check_gnd(centroids, "centroids", dev)) ||
+      (rc = check_i32(clusters, "clusters", 3, dev)) || (rc = check_i32(cluster_size, "cluster_size", 2, dev)) ||
+      (rc = check_i32(out, "out", 2, dev)))
+    return rc;
+  const int64_t B = query->shape[0], Hq = query->shape[1], G = centroids->shape[0], C = centroids->shape[1];
+  const int64_t M = clusters->shape[2], k = out->shape[1];
+  SQ_REQUIRE(num_kv_groups > 0 && Hq % num_kv_groups == 0, SQ_EINVAL, "sq_topk_select: num_kv_groups %d does not divide Hq", num_kv_groups);
+  const int64_t Hkv = Hq / num_kv_groups;
+  SQ_REQUIRE(G == B * Hkv, SQ_ESHAPE, "sq_topk_select: centroids has %lld groups, expected B*Hkv = %lld", (long long)G, (long long)(B * Hkv));
+  SQ_REQUIRE(clusters->shape[0] == G && clusters->shape[1] == C && cluster_size->shape[0] == G && cluster_size->shape[1] == C &&
+                 out->shape[0] == G && k > 0 && M > 0,
+             SQ_ESHAPE, "sq_topk_select: shapes disagree");
+  SQ_REQUIRE(C <= kMaxC, SQ_EUNSUPPORTED, "sq_topk_select: more than %d centroids", kMaxC);
+  const WsLayout w = ws_layout(G, 1, C);
+  if ((rc = check_ws(workspace, w.all(), dev, "sq_topk_select")) || (rc = check_current_device(dev, "sq_topk_select"))) return rc;
+  hipStream_t st = (hipStream_t)stream;
+  char* wsp = data_of(workspace);
+  TopkArgs a;
+  a.query = (const uint16_t*)data_of(query);
+  a.cent = (const uint16_t*)data_of(centroids);
+  a.clusters = (const int32_t*)data_of(clusters);
+  a.size = (const int32_t*)data_of(cluster_size);
+  a.out = (int32_t*)data_of(out);
+  a.score = (float*)(wsp + w.off_bytes + w.hist_bytes + w.order_bytes);
+  a.start = (int32_t*)(wsp + w.off_bytes + w.hist_bytes + w.order_bytes + w.score_bytes);
+  a.q_sb = stride_of(query, 0);
+  a.q_sh = stride_of(query, 1);
+  a.c_sg = stride_of(centroids, 0);
+  a.c_sc = stride_of(centroids, 1);
+  a.cl_sg = C * M;
+  a.cl_sc = M;
+  a.C = (int)C;
+  a.M = (int)M;
+  a.k = (int)k;
+  a.Hkv = (int)Hkv;
+  a.group = num_kv_groups;
+  hipLaunchKernelGGL(topk_score_kernel, dim3((unsigned)((C + 255) / 256), (unsigned)G), dim3(256), 0, st, a);
+  hipLaunchKernelGGL(topk_emit_kernel, dim3((unsigned)G), dim3(1024), (size_t)C * 4, st, a);
+  hipLaunchKernelGGL(topk_tail_kernel, dim3(8, (unsigned)G), dim3(256), 0, st, a);
+  SQ_HIP(hipGetLastError());
+  return SQ_OK;
 }
