@@ -1,0 +1,185 @@
+"""Drop-in for the reference's sqattn/attn_replacer.py: same entry points, HIP kernels underneath.
+
+`process_model(model, "SQAttn", window_sizes, args)` binds `mp_triton_wrapper(...)` as
+`layer.prefill_attention` exactly like the reference (:12-34); the closure does what the reference's does
+(:323-452) -- GQA handling, K mean-centring, 8-/4-bit fake-quant of Q/K, 8-bit fake-quant of V, sink +
+hierarchical-window prefill, reshape to [B, N, Hq*D] -- with two deliberate differences:
+  * K and V are never expanded to the 28 q-heads (`repeat_kv`, :335-336): the kernel maps q-head -> kv-head
+    itself.  Every per-token / per-(token, channel) quantisation range is unchanged by the expansion
+    (per-token ranges are per head; the "per_channel" range reduces over batch and heads, fake_quant.py:30-32,
+    and duplicated heads add nothing to a min/max), so the results are identical at 1/7 of the traffic;
+  * the dead `seq_len == 1` branch (:369-420, it uses names deleted three lines earlier) is replaced by the
+    split-KV decode kernel.
+"""
+from __future__ import annotations
+
+import math
+import types
+
+import torch
+
+from .attn_triton_decode import attn_decode
+from .attn_triton_mix_bad import attn_hierarchical_window
+from .attn_triton_mix_relative import attn_hierarchical_relative_window
+from .fake_quant import FloatQuantizer, IntegerQuantizer
+from .sdpa_attention import sdpa_attention_forward
+
+
+def process_model(model, method, window_sizes=None, args=None, patch_decode=False):
+    """attn_replacer.py:12-34.  `patch_decode=True` (extension) also binds the split-KV decode kernel as
+    `layer.decode_attention` on every layer."""
+    if method == "SQAttn":
+        for i in range(len(model.layers)):
+            if i in window_sizes.keys():
+                layer = model.layers[i]
+                bit8_window_sizes = window_sizes[i]["bit8"]
+                bit4_window_sizes = window_sizes[i]["bit4"]
+                sink_size = window_sizes[i]["sink"]  # read and, as in the reference (:19,24), overridden by 256
+                layer.prefill_attention = types.MethodType(
+                    mp_triton_wrapper(i, args=args, bit8_window_sizes=bit8_window_sizes,
+                                      bit4_window_sizes=bit4_window_sizes, sink_window_size=256), layer)
+                model.layers[i] = layer
+        if patch_decode:
+            for layer in model.layers:
+                layer.decode_attention = types.MethodType(decode_attention_fn, layer)
+    elif method == "SDPA":
+        print("use sdpa")
+    elif method == "FlashAttn":
+        print("use full flash attn")
+    else:
+        raise ValueError(f"Unsupported attention type: {method}")
+    return model
+
+
+def decode_attention_fn(module, query_states, key_states, value_states, layer_idx=None, seqlens=None):
+    """`layer.decode_attention(q [B,1,Hq,D], Kcache, Vcache [B,L,Hkv,D], None)[0]` slot (model_hub/LLM.py:105):
+    returns a 1-tuple so that the caller's `[0]` picks the [B,1,Hq*D] output."""
+    out = attn_decode(query_states, key_states, value_states, "NHD", query_states.dtype, seqlens=seqlens)
+    b, n, h, d = out.shape
+    return (out.reshape(b, n, h * d),)
+
+
+def _normalise_windows(bit8_window_sizes, bit4_window_sizes):
+    """attn_replacer.py:299-321."""
+    is_per_head = isinstance(bit8_window_sizes, list) or isinstance(bit4_window_sizes, list)
+    if is_per_head:
+        num_heads = len(bit8_window_sizes) if isinstance(bit8_window_sizes, list) else len(bit4_window_sizes)
+        if isinstance(bit8_window_sizes, int):
+            bit8_window_sizes = [bit8_window_sizes] * num_heads
+        if isinstance(bit4_window_sizes, int):
+            bit4_window_sizes = [bit4_window_sizes] * num_heads
+        if bit8_window_sizes is None:
+            bit8_window_sizes = [0] * num_heads
+        if bit4_window_sizes is None:
+            bit4_window_sizes = [0] * num_heads
+    else:
+        bit8_window_sizes = bit8_window_sizes or 0
+        bit4_window_sizes = bit4_window_sizes or 0
+    return bit8_window_sizes, bit4_window_sizes
+
+
+def _quantizers(args):
+    """attn_replacer.py:340-358."""
+    if args.qk_qtype == "int":
+        bit8_qk = IntegerQuantizer(8, True, "per_token")
+    elif args.qk_qtype in ("e4m3", "e5m2"):
+        bit8_qk = FloatQuantizer(args.qk_qtype, True, "per_token")
+    else:
+        raise ValueError(f"Invalid quantization type: {args.qk_qtype}")
+    bit4_qk = IntegerQuantizer(4, True, "per_token")
+    if args.v_qtype == "int":
+        bit8_v = IntegerQuantizer(8, True, "per_channel")
+    elif args.v_qtype in ("e4m3", "e5m2"):
+        bit8_v = FloatQuantizer(args.v_qtype, True, "per_channel")
+    else:
+        raise ValueError(f"Invalid quantization type: {args.v_qtype}")
+    return bit8_qk, bit4_qk, bit8_v
+
+
+def mp_triton_wrapper(layer_idx, bit8_window_sizes=0, bit4_window_sizes=0, sink_window_size=0, args=None):
+    """attn_replacer.py:296-454: builds the `prefill_attention` closure of one layer."""
+    bit8_window_sizes, bit4_window_sizes = _normalise_windows(bit8_window_sizes, bit4_window_sizes)
+
+    def attention_fn(module, query, key, value, attention_mask, dropout=0.0, scaling=1.0, sliding_window=None, **kwargs):
+        # query [B,N,Hq,D], key/value [B,N,Hkv,D]  ->  HND views without expanding the kv heads
+        if hasattr(module, "num_key_value_groups"):
+            key = key.permute(0, 2, 1, 3)
+            value = value.permute(0, 2, 1, 3)
+            query = query.permute(0, 2, 1, 3)
+        bit8_qk, bit4_qk, bit8_v = _quantizers(args)
+        seq_len = query.shape[2]
+        if seq_len == 1:
+            q_nhd = query.permute(0, 2, 1, 3)
+            out = attn_decode(q_nhd, key.permute(0, 2, 1, 3), value.permute(0, 2, 1, 3), "NHD", torch.bfloat16)
+            b, n, h, d = out.shape
+            return out.reshape(b, n, h * d)
+        key = key - key.mean(dim=2, keepdim=True)
+        q_bit8 = bit8_qk.fake_quant_tensor(query)
+        k_bit8 = bit8_qk.fake_quant_tensor(key)
+        v_bit8 = bit8_v.fake_quant_tensor(value)
+        p_quant = kwargs.get("p_quant", None)
+        if args.use_relative_distance:
+            # the relative launch aliases the 4-bit operands to the 8-bit ones (attn_triton_mix_relative.py:441-444),
+            # so the two 4-bit passes of the reference (:362,364) would be dead work and are skipped
+            del query, key, value
+            attn_output = attn_hierarchical_relative_window(
+                q_bit8, k_bit8, q_bit8, k_bit8, v_bit8, int8_window_ratios=bit8_window_sizes,
+                int4_window_ratios=bit4_window_sizes, sink_size=sink_window_size, tensor_layout="HND",
+                output_dtype=torch.bfloat16, p_quant=p_quant)
+        else:
+            q_bit4 = bit4_qk.fake_quant_tensor(query)
+            k_bit4 = bit4_qk.fake_quant_tensor(key)
+            del query, key, value
+            attn_output = attn_hierarchical_window(
+                q_bit8, k_bit8, q_bit4, k_bit4, v_bit8, int8_window_sizes=bit8_window_sizes,
+                int4_window_sizes=bit4_window_sizes, sink_size=sink_window_size, tensor_layout="HND",
+                output_dtype=torch.bfloat16, p_quant=p_quant)
+        attn_output = attn_output.transpose(1, 2).contiguous()
+        bs, seq_len, head, head_dim = attn_output.shape
+        return attn_output.view(bs, seq_len, head * head_dim)
+
+    return attention_fn
+
+
+def delayed_sdpa_wrapper(layer_idx, bit8_window_sizes=0, bit4_window_sizes=0, sink_window_size=0, args=None):
+    """attn_replacer.py:36-250: the masked-SDPA emulation.  The reference's quantised branch is unfinished
+    (it stops in a debugger, :187-189); only its plain branch (`args.quant` false) is meaningful and kept."""
+
+    def attention_fn(module, q, k, v, attn_mask, dropout=0.0, scaling=1.0, sliding_window=None, **kwargs):
+        if getattr(args, "quant", False):
+            raise NotImplementedError("the reference's quantised masked-SDPA emulation is unfinished (pdb.set_trace)")
+        return sdpa_attention_forward(module, q, k, v, attention_mask=attn_mask, dropout=dropout, scaling=scaling, **kwargs)
+
+    return attention_fn
+
+
+def cal_attn_weight(module, query, key, is_causal=True, attn_mask=None):
+    """Dense softmax attention map used by calibration (attn_replacer.py:253-278)."""
+    if hasattr(module, "num_key_value_groups"):
+        key = repeat_kv(key, module.num_key_value_groups)
+        query = query.permute(0, 2, 1, 3)
+    query, key = query.contiguous(), key.contiguous()
+    L, S = query.shape[-2], key.shape[-2]
+    attn_bias = torch.zeros(L, S, dtype=query.dtype, device=query.device)
+    if is_causal:
+        assert attn_mask is None
+        keep = torch.ones(L, S, dtype=torch.bool, device=query.device).tril(diagonal=0)
+        attn_bias.masked_fill_(keep.logical_not(), float("-inf"))
+    if attn_mask is not None:
+        if attn_mask.dtype == torch.bool:
+            attn_bias.masked_fill_(attn_mask.logical_not(), float("-inf"))
+        else:
+            attn_bias = attn_mask + attn_bias
+    attn_weight = query @ key.transpose(-2, -1) * (1 / math.sqrt(query.shape[-1]))
+    attn_weight += attn_bias
+    return torch.softmax(attn_weight, dim=-1)
+
+
+def repeat_kv(hidden_states: torch.Tensor, n_rep: int) -> torch.Tensor:
+    """[B,N,Hkv,D] -> [B,Hkv*n_rep,N,D], each kv head repeated n_rep times (attn_replacer.py:281-293)."""
+    batch, slen, num_key_value_heads, head_dim = hidden_states.shape
+    hidden_states = hidden_states.permute(0, 2, 1, 3)
+    if n_rep == 1:
+        return hidden_states
+    hidden_states = hidden_states[:, :, None, :, :].expand(batch, num_key_value_heads, n_rep, slen, head_dim)
+    return hidden_states.reshape(batch, num_key_value_heads * n_rep, slen, head_dim)

@@ -1,0 +1,140 @@
+"""Fake quantisers with the reference's class names and arguments (sqattn/fake_quant.py), on torch tensors.
+
+`IntegerQuantizer(bit, symmetric, granularity)` / `FloatQuantizer("e4m3"|"e5m2", True, granularity)` and
+their `fake_quant_tensor` / `real_quant_tensor` behave like the reference's: ranges per tensor, per
+"channel" (reduced over dims 0 and 1, fake_quant.py:30-32) or per token (last dim), rounding half away
+from zero as `paddle.round` does, and the home-made float simulation of fake_quant.py:151-204 including
+its quirks (largest e4m3 output 240, no subnormals).  These are elementwise tensor passes that feed the
+HIP attention kernels; they run wherever the tensor lives.
+"""
+from __future__ import annotations
+
+import torch
+
+
+def _round(x: torch.Tensor) -> torch.Tensor:
+    return torch.sign(x) * torch.floor(torch.abs(x) + 0.5)
+
+
+class BaseQuantizer(object):
+    def __init__(self, bit, symmetric, granularity, **kwargs):
+        self.bit = bit
+        self.sym = symmetric
+        self.granularity = granularity
+        self.kwargs = kwargs
+        if self.granularity == "per_group":
+            self.group_size = self.kwargs["group_size"]
+        self.calib_algo = self.kwargs.get("calib_algo", "minmax")
+
+    def get_tensor_range(self, tensor):
+        if self.calib_algo == "minmax":
+            return self.get_minmax_range(tensor)
+        if self.calib_algo == "mse":
+            raise NotImplementedError
+        raise ValueError(f"Unsupported calibration algorithm: {self.calib_algo}")
+
+    def get_minmax_range(self, tensor):
+        if tensor.dtype in (torch.bfloat16, torch.float16):
+            tensor = tensor.float()
+        if self.granularity == "per_tensor":
+            return tensor.min(), tensor.max()
+        if self.granularity == "per_channel":
+            return tensor.amin(dim=(0, 1), keepdim=True), tensor.amax(dim=(0, 1), keepdim=True)
+        return tensor.amin(dim=-1, keepdim=True), tensor.amax(dim=-1, keepdim=True)
+
+    def get_qparams(self, tensor_range, device):
+        min_val, max_val = tensor_range
+        qmin, qmax = self.qmin.to(device), self.qmax.to(device)
+        if self.sym:
+            abs_max = torch.maximum(max_val.abs(), min_val.abs()).clamp(min=1e-05)
+            scales = abs_max / qmax
+            zeros = torch.tensor(0.0, device=device)
+        else:
+            scales = (max_val - min_val).clamp(min=1e-05) / (qmax - qmin)
+            zeros = torch.minimum(torch.maximum(qmin - _round(min_val / scales), qmin), qmax)
+        return scales, zeros, qmax, qmin
+
+    def reshape_tensor(self, tensor, allow_padding=False):
+        return tensor.reshape(-1, self.group_size) if self.granularity == "per_group" else tensor
+
+    def restore_tensor(self, tensor, shape):
+        return tensor if tensor.shape == shape else tensor.reshape(shape)
+
+    def get_tensor_qparams(self, tensor):
+        tensor = self.reshape_tensor(tensor)
+        tensor_range = self.get_tensor_range(tensor)
+        scales, zeros, qmax, qmin = self.get_qparams(tensor_range, tensor.device)
+        return tensor, scales, zeros, qmax, qmin
+
+    def fake_quant_tensor(self, tensor):
+        org_shape, org_dtype = tensor.shape, tensor.dtype
+        tensor, scales, zeros, qmax, qmin = self.get_tensor_qparams(tensor)
+        tensor = self.quant_dequant(tensor.float(), scales, zeros, qmax, qmin)
+        return self.restore_tensor(tensor, org_shape).to(org_dtype)
+
+    def real_quant_tensor(self, tensor):
+        org_shape = tensor.shape
+        tensor, scales, zeros, qmax, qmin = self.get_tensor_qparams(tensor)
+        tensor = self.quant(tensor.float(), scales, zeros, qmax, qmin)
+        tensor = self.restore_tensor(tensor, org_shape)
+        return tensor, scales, (None if self.sym else zeros)
+
+    def quant_dequant(self, tensor, scales, zeros, qmax, qmin):
+        return self.dequant(self.quant(tensor, scales, zeros, qmax, qmin), scales, zeros)
+
+    def dequant(self, tensor, scales, zeros):
+        return (tensor - zeros) * scales
+
+
+class IntegerQuantizer(BaseQuantizer):
+    def __init__(self, bit, symmetric, granularity, **kwargs):
+        super().__init__(bit, symmetric, granularity, **kwargs)
+        if "int_range" in self.kwargs:
+            qmin, qmax = self.kwargs["int_range"]
+        elif self.sym:
+            qmin, qmax = -(2 ** (self.bit - 1)), 2 ** (self.bit - 1) - 1
+        else:
+            qmin, qmax = 0.0, 2 ** self.bit - 1
+        self.qmin = torch.tensor(float(qmin))
+        self.qmax = torch.tensor(float(qmax))
+        self.dst_nbins = 2 ** bit
+
+    def quant(self, tensor, scales, zeros, qmax, qmin):
+        return torch.minimum(torch.maximum(_round(tensor / scales) + zeros, qmin), qmax)
+
+
+def float_quantize(x, e_bits=5, m_bits=10, rounding="nearest"):
+    """Float simulation of fake_quant.py:151-204 (nearest or stochastic mantissa rounding)."""
+    assert rounding in ["nearest", "stochastic"]
+    bias = 2 ** (e_bits - 1) - 1
+    eps = 2.0 ** (-m_bits)
+    max_exp = 2 ** (e_bits - 1) - 1
+    min_exp = 1 - bias
+    sign = torch.sign(x)
+    x = torch.abs(x)
+    zero_mask = x == 0
+    exp = torch.floor(torch.log2(x + 1e-30))
+    frac = x / (2.0 ** exp) - 1.0
+    exp_clamped = exp.clamp(min_exp, max_exp)
+    if rounding == "nearest":
+        frac_q = _round(frac / eps) * eps
+    else:
+        frac_q = torch.floor(frac / eps + torch.rand_like(frac)) * eps
+    frac_q = frac_q.clamp(0.0, 1.0 - eps)
+    x_q = (1.0 + frac_q) * (2.0 ** exp_clamped) * sign
+    max_val = (2 - 2 ** (-m_bits)) * (2.0 ** max_exp)
+    x_q = x_q.clamp(-max_val, max_val)
+    return torch.where(zero_mask, torch.zeros_like(x_q), x_q)
+
+
+class FloatQuantizer(BaseQuantizer):
+    def __init__(self, bit, symmetric, granularity, **kwargs):
+        super().__init__(bit, symmetric, granularity, **kwargs)
+        assert self.bit in ["e4m3", "e5m2"], f"Unsupported bit configuration: {self.bit}"
+        assert self.sym
+        self.e_bits, self.m_bits, fmax = (4, 3, 448.0) if self.bit == "e4m3" else (5, 2, 57344.0)
+        self.qmin, self.qmax = torch.tensor(-fmax), torch.tensor(fmax)
+
+    def quant(self, tensor, scales, zeros, qmax, qmin):
+        scaled = torch.minimum(torch.maximum(tensor / scales + zeros, qmin), qmax)
+        return float_quantize(scaled.float(), self.e_bits, self.m_bits, rounding="nearest")

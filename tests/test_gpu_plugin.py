@@ -1,0 +1,116 @@
+"""GPU parity of the drop-in boundary: `process_model` / `mp_triton_wrapper` closures against the oracle's
+restatement of the reference closure (sqattn/attn_replacer.py:296-454), plus the fake quantisers."""
+import types
+
+import pytest
+import torch
+
+from oracle import attention as A
+from oracle import fake_quant as FQ
+from oracle import inputs, plugin
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+class _Layer:
+    def __init__(self, groups):
+        self.num_key_value_groups = groups
+
+    def prefill_attention(self, q, k, v, layer_idx=None):
+        raise AssertionError("not patched")
+
+
+class _Model:
+    def __init__(self, n, groups):
+        self.layers = [_Layer(groups) for _ in range(n)]
+
+
+def _args(relative, qk="int", v="int"):
+    return types.SimpleNamespace(qk_qtype=qk, v_qtype=v, use_relative_distance=relative)
+
+
+def _cos(a, b):
+    a, b = a.double().flatten(), b.double().flatten()
+    return float(a @ b / (a.norm() * b.norm()))
+
+
+@pytest.mark.parametrize("qtype", ["int", "e4m3"])
+def test_fake_quantisers_match_oracle(qtype):
+    from longcontext_sqattn_paddle_amd.sqattn.fake_quant import FloatQuantizer, IntegerQuantizer
+
+    x = torch.randn(2, 3, 50, 128, generator=torch.Generator().manual_seed(0)).bfloat16()
+    xd = x.to(DEV)
+    if qtype == "int":
+        for bit, sym, gran in ((8, True, "per_token"), (4, True, "per_token"), (8, True, "per_channel"), (8, False, "per_channel")):
+            got = IntegerQuantizer(bit, sym, gran).fake_quant_tensor(xd).cpu()
+            assert torch.equal(got, FQ.int_fake_quant(x, bit, sym, gran)), (bit, sym, gran)
+    else:
+        for fmt, gran in (("e4m3", "per_token"), ("e5m2", "per_channel")):
+            got = FloatQuantizer(fmt, True, gran).fake_quant_tensor(xd).cpu()
+            ref = FQ.float_fake_quant(x, fmt, gran)
+            # log2/exp2 on the device may differ by an ulp from the host's: allow rare one-step differences
+            assert float((got.float() - ref.float()).abs().max()) <= float(ref.float().abs().max()) * 0.13
+            assert float((got != ref).float().mean()) < 1e-3
+
+
+def test_process_model_binds_and_skips_like_the_reference():
+    from longcontext_sqattn_paddle_amd.sqattn.attn_replacer import process_model
+
+    m = _Model(4, 4)
+    ws = {1: {"bit8": 0.1, "bit4": 0.1, "sink": 64}, 2: {"bit8": [0.1] * 4, "bit4": [0.2] * 4, "sink": 64}}
+    process_model(m, "SQAttn", ws, _args(True))
+    assert "prefill_attention" not in vars(m.layers[0]) and "prefill_attention" in vars(m.layers[1])
+    assert process_model(m, "SDPA") is m and process_model(m, "FlashAttn") is m
+    with pytest.raises(ValueError):
+        process_model(m, "Other")
+
+
+@pytest.mark.parametrize("relative,bit8,bit4", [(True, 0.1, 0.1), (True, [0.05, 0.1, 0.2, 0.3], [0.4, 0.1, 0.2, 0.5]),
+                                                (False, 256, 512), (False, [128, 256, 384, 2048], [256, 256, 640, 2048])])
+def test_plugin_closure_matches_oracle(relative, bit8, bit4):
+    from longcontext_sqattn_paddle_amd.sqattn.attn_replacer import process_model
+
+    q, k, v = inputs.plugin_inputs(1, 4, 1, 2048, 128, seed=1)
+    m = _Model(2, 4)
+    process_model(m, "SQAttn", {1: {"bit8": bit8, "bit4": bit4, "sink": 0}}, _args(relative))
+    out = m.layers[1].prefill_attention(q.to(DEV), k.to(DEV), v.to(DEV), None)
+    torch.cuda.synchronize()
+    assert out.shape == (1, 2048, 512) and out.dtype == torch.bfloat16
+    ref = plugin.plugin_attention(q, k, v, num_kv_groups=4, bit8=bit8, bit4=bit4, sink=256, relative=relative)
+    o, r = out.float().cpu(), ref.float()
+    rms = float(r.pow(2).mean().sqrt())
+    assert _cos(o, r) >= 0.99999
+    # both sides round the same fp32 result to bf16: one bf16 ulp of the largest output plus kernel noise
+    assert float((o - r).abs().max()) <= 2 ** -7 * float(r.abs().max()) + 2e-3 * rms
+
+
+def test_config1_full_causal_with_block_fp8_p():
+    """Benchmark configuration 1: seq 4096, 4 q-heads on 1 kv head, int8 fake-quant, windows >= N (full causal),
+    P quantised to e4m3 with per-64x64-block absmax scales (a mode the reference closure itself never enables)."""
+    from longcontext_sqattn_paddle_amd import _native as N
+    from longcontext_sqattn_paddle_amd.sqattn.attn_replacer import mp_triton_wrapper
+
+    q, k, v = inputs.plugin_inputs(1, 4, 1, 4096, 128, seed=1)
+    fn = mp_triton_wrapper(0, bit8_window_sizes=2.0, bit4_window_sizes=2.0, sink_window_size=256, args=_args(True))
+    out = fn(_Layer(4), q.to(DEV), k.to(DEV), v.to(DEV), None, p_quant=N.P_E4M3_BLOCK)
+    torch.cuda.synchronize()
+    ref = plugin.plugin_attention(q, k, v, num_kv_groups=4, bit8=2.0, bit4=2.0, sink=256, relative=True, p_quant=A.P_BLOCK_ABSMAX)
+    o, r = out.float().cpu(), ref.float()
+    assert _cos(o, r) >= 0.99995
+    exact, _ = A.exact_attention(q.permute(0, 2, 1, 3), k.permute(0, 2, 1, 3), v.permute(0, 2, 1, 3))
+    e = exact.permute(0, 2, 1, 3).reshape(1, 4096, 512)
+    assert _cos(o, e) >= 0.999   # int8 Q/K/V + e4m3 P against exact attention: the benchmark's stated bar
+
+
+def test_decode_slot():
+    from longcontext_sqattn_paddle_amd.sqattn.attn_replacer import decode_attention_fn
+
+    q, kc, vc, lens = inputs.decode_inputs(2, 8, 2, 1024, 128, seed=9)
+    lens_d = lens.to(DEV)
+    out = decode_attention_fn(_Layer(4), q.to(DEV), kc.to(DEV), vc.to(DEV), None, seqlens=lens_d)[0]
+    torch.cuda.synchronize()
+    ref, _ = A.exact_attention(q.permute(0, 2, 1, 3), kc.permute(0, 2, 1, 3), vc.permute(0, 2, 1, 3), causal=False,
+                               kv_lens=[int(x) for x in lens])
+    assert out.shape == (2, 1, 8 * 128)
+    assert _cos(out.float().cpu(), ref.permute(0, 2, 1, 3).reshape(2, 1, 1024)) >= 0.9999
