@@ -25,7 +25,6 @@ namespace {
 
 constexpr int kD = 128;
 constexpr int kBN = 64;                  // keys per tile (BLOCK_N of every reference kernel)
-constexpr int kRowsPerWave = 64;
 constexpr int kKStride = 272;            // bytes per K row in LDS (256 + 16 pad)
 constexpr int kVStride = 144;            // bytes per V^T row in LDS (128 + 16 pad)
 constexpr int kKTileBytes = kBN * kKStride;
@@ -172,11 +171,67 @@ __device__ __forceinline__ WaveRanges wave_ranges(const PrefillArgs& a, int pos0
   return r;
 }
 
-template <bool BF16, int WAVES>
-__global__ __launch_bounds__(WAVES * 64, 1) void prefill_kernel(PrefillArgs a) {
+// exchange with the lane 32 away (the other half of the keys of the same query row)
+__device__ __forceinline__ float xor32_max(float v) {
+  const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+}
+__device__ __forceinline__ float xor32_sum(float v) {
+  const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
+}
+
+constexpr float kLog2_448 = 8.807354922057604f;  // log2(448)
+
+// Quantise 8 probabilities (one k-step of the P.V MFMA) and pack them as fp16 B-operand registers.
+//   MODE 0  p.to(fp16)
+//   MODE 1  fp16(e4m3(p*448)/448)   reference static scale (attn_triton.py:81-82): sc = 448, inv = 1/448
+//   MODE 2  fp16(e4m3(p*sc)*inv)    block absmax scale a: sc = 448/a, inv = a/448
+//   MODE 3  fp16(e4m3(p448))        p448 = 448*p, the factor folded into the exponent; the 1/448 cancels in
+//                                   acc/l because l is accumulated from p448 as well
+template <int MODE>
+__device__ __forceinline__ uint4 quant_pack8(const f32x16_t& s, int t, float sc, float inv) {
+  uint32_t w[4];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const float p0 = s[8 * t + 4 * h + 0], p1 = s[8 * t + 4 * h + 1], p2 = s[8 * t + 4 * h + 2], p3 = s[8 * t + 4 * h + 3];
+    if constexpr (MODE == 0) {
+      w[2 * h] = pack_f16(p0, p1);
+      w[2 * h + 1] = pack_f16(p2, p3);
+    } else if constexpr (MODE == 3) {
+      int pk = __builtin_amdgcn_cvt_pk_fp8_f32(p0, p1, 0, false);
+      pk = __builtin_amdgcn_cvt_pk_fp8_f32(p2, p3, pk, true);
+      w[2 * h] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(pk, 1.0f, false));
+      w[2 * h + 1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(pk, 1.0f, true));
+    } else {
+      float q0 = p0 * sc, q1 = p1 * sc, q2 = p2 * sc, q3 = p3 * sc;
+      if constexpr (MODE == 2) {
+        q0 = fminf(q0, 448.f);
+        q1 = fminf(q1, 448.f);
+        q2 = fminf(q2, 448.f);
+        q3 = fminf(q3, 448.f);
+      }
+      int pk = __builtin_amdgcn_cvt_pk_fp8_f32(q0, q1, 0, false);
+      pk = __builtin_amdgcn_cvt_pk_fp8_f32(q2, q3, pk, true);
+      typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+      const f32x2_t lo = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(pk, 1.0f, false);
+      const f32x2_t hi = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(pk, 1.0f, true);
+      w[2 * h] = pack_f16(lo[0] * inv, lo[1] * inv);
+      w[2 * h + 1] = pack_f16(hi[0] * inv, hi[1] * inv);
+    }
+  }
+  return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+// One workgroup = WAVES waves x 32 query rows of one q-head (2 waves per SIMD when WAVES == 8, so that one
+// wave's MFMA phase overlaps the other's softmax phase).  MODE as in quant_pack8.
+template <bool BF16, int WAVES, int MODE>
+__global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
   constexpr int NT = WAVES * 64;
   constexpr int CH = (kBN * kD * 2 / 16) / NT;  // 16-byte chunks per thread and tile operand
+  constexpr int ROWS = 32;                      // query rows per wave
   extern __shared__ __attribute__((aligned(16))) char smem[];
+  __shared__ float s_amax[2][WAVES];            // MODE 2: tile maxima of the two waves of a 64-row group
 
   // ---- schedule: blockIdx -> (pair = (b, kvh), item = (q block descending, head in group))
   int pair, item;
@@ -205,9 +260,9 @@ __global__ __launch_bounds__(WAVES * 64, 1) void prefill_kernel(PrefillArgs a) {
   const int lane = tid & 63, wave = tid >> 6;
   const int c32 = lane & 31, g = lane >> 5;
 
-  const int row_wg0 = qb * (WAVES * kRowsPerWave);          // first query row of the workgroup
-  const int row_w0 = row_wg0 + wave * kRowsPerWave;         // first query row of this wave
-  const int pos0 = a.q_offset + row_w0;                     // its absolute position
+  const int row_wg0 = qb * (WAVES * ROWS);          // first query row of the workgroup
+  const int row_w0 = row_wg0 + wave * ROWS;         // first query row of this wave
+  const int pos0 = a.q_offset + row_w0;             // its absolute position
   const bool wave_active = row_w0 < a.Nq;
   const WaveRanges wr = wave_ranges(a, pos0, head);
 
@@ -215,7 +270,7 @@ __global__ __launch_bounds__(WAVES * 64, 1) void prefill_kernel(PrefillArgs a) {
   int segA_hi = 0, segB_lo = 1 << 30, segB_hi = 0;
 #pragma unroll
   for (int w = 0; w < WAVES; ++w) {
-    const int rw = row_wg0 + w * kRowsPerWave;
+    const int rw = row_wg0 + w * ROWS;
     if (rw < a.Nq) {
       const WaveRanges o = wave_ranges(a, a.q_offset + rw, head);
       segA_hi = max(segA_hi, o.sink_hi);
@@ -228,36 +283,31 @@ __global__ __launch_bounds__(WAVES * 64, 1) void prefill_kernel(PrefillArgs a) {
     segA_hi = 0;
     segB_lo = 0;
   }
-  const bool distinct4 = a.q4 != nullptr;  // host guarantees WAVES*64 <= block_m in that case
+  const bool distinct4 = a.q4 != nullptr;  // host guarantees WAVES*32 == block_m in that case
 
-  // ---- Q~ fragments (B operand of S^T = K.Q~^T): lane (column = row c32 of block bm, k-group g)
-  uint4 qf[2][8];
+  // ---- Q~ fragments (B operand of S^T = K.Q~^T): lane (column = query row c32, k-group g)
+  uint4 qf[8];
   auto load_q = [&](const void* qbase) {
     const uint16_t* qp = (const uint16_t*)qbase + (int64_t)b * a.q_sb + (int64_t)head * a.q_sh;
+    const int row = max(min(row_w0 + c32, a.Nq - 1), 0);
+    const uint16_t* rp = qp + (int64_t)row * a.q_sn + 8 * g;
 #pragma unroll
-    for (int bm = 0; bm < 2; ++bm) {
-      const int row = min(row_w0 + 32 * bm + c32, a.Nq - 1);
-      const uint16_t* rp = qp + (int64_t)max(row, 0) * a.q_sn + 8 * g;
-#pragma unroll
-      for (int kk = 0; kk < 8; ++kk) {
-        const uint4 raw = *(const uint4*)(rp + 16 * kk);
-        qf[bm][kk] = make_uint4(scale_pair<BF16>(raw.x, a.sm), scale_pair<BF16>(raw.y, a.sm),
-                                scale_pair<BF16>(raw.z, a.sm), scale_pair<BF16>(raw.w, a.sm));
-      }
+    for (int kk = 0; kk < 8; ++kk) {
+      const uint4 raw = *(const uint4*)(rp + 16 * kk);
+      qf[kk] = make_uint4(scale_pair<BF16>(raw.x, a.sm), scale_pair<BF16>(raw.y, a.sm), scale_pair<BF16>(raw.z, a.sm),
+                          scale_pair<BF16>(raw.w, a.sm));
     }
   };
   load_q(a.q);
   bool q_is4 = false;
 
-  f32x16_t O[4][2];
+  f32x16_t O[4];
 #pragma unroll
   for (int bd = 0; bd < 4; ++bd)
 #pragma unroll
-    for (int bm = 0; bm < 2; ++bm)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) O[bd][bm][i] = 0.f;
-  float m_run[2] = {-INFINITY, -INFINITY};
-  float l_run[2] = {0.f, 0.f};
+    for (int i = 0; i < 16; ++i) O[bd][i] = 0.f;
+  float m_run = -INFINITY;
+  float l_run = 0.f;   // this lane's share of the denominator (times 448 in MODE 3)
 
   const _Float16* vt_base = a.vt + ((int64_t)b * a.Hkv + kvh) * (int64_t)a.nT * (kD * kBN);
 
@@ -303,8 +353,13 @@ __global__ __launch_bounds__(WAVES * 64, 1) void prefill_kernel(PrefillArgs a) {
     const int jn = next_tile(j);
     const bool have_next = jn < segB_hi;
     if (have_next) gload(jn);
+    const bool visit = wave_active && wr.visits(j);
+    const char* kbuf = smem + (it & 1) * kStageBytes;
+    const char* vbuf = kbuf + kKTileBytes;
+    f32x16_t S[2];
+    float alpha = 1.f;
 
-    if (wave_active && wr.visits(j)) {
+    if (visit) {
       if (distinct4) {  // switch the Q~ operand set when entering/leaving the 4-bit window range
         const bool want4 = tile_uses4(j);
         if (want4 != q_is4) {
@@ -312,105 +367,79 @@ __global__ __launch_bounds__(WAVES * 64, 1) void prefill_kernel(PrefillArgs a) {
           q_is4 = want4;
         }
       }
-      const char* kbuf = smem + (it & 1) * kStageBytes;
-      const char* vbuf = kbuf + kKTileBytes;
-
-      // S^T[key, row] for 2 key blocks x 2 row blocks of 32
-      f32x16_t S[2][2];
+      // S^T[key, row] for the 2 key blocks of 32
 #pragma unroll
       for (int bn = 0; bn < 2; ++bn)
 #pragma unroll
-        for (int bm = 0; bm < 2; ++bm)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) S[bn][bm][i] = 0.f;
+        for (int i = 0; i < 16; ++i) S[bn][i] = 0.f;
 #pragma unroll
       for (int kk = 0; kk < 8; ++kk) {
         const uint4 a0 = *(const uint4*)(kbuf + c32 * kKStride + (16 * kk + 8 * g) * 2);
         const uint4 a1 = *(const uint4*)(kbuf + (32 + c32) * kKStride + (16 * kk + 8 * g) * 2);
-        S[0][0] = mfma_qk32<BF16>(a0, qf[0][kk], S[0][0]);
-        S[0][1] = mfma_qk32<BF16>(a0, qf[1][kk], S[0][1]);
-        S[1][0] = mfma_qk32<BF16>(a1, qf[0][kk], S[1][0]);
-        S[1][1] = mfma_qk32<BF16>(a1, qf[1][kk], S[1][1]);
+        S[0] = mfma_qk32<BF16>(a0, qf[kk], S[0]);
+        S[1] = mfma_qk32<BF16>(a1, qf[kk], S[1]);
       }
       if (j >= wr.diag_lo) {  // causal mask inside the query block's own tiles (attn_triton.py:69-71)
-#pragma unroll
-        for (int bn = 0; bn < 2; ++bn)
-#pragma unroll
-          for (int bm = 0; bm < 2; ++bm)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-              const int col = j * kBN + 32 * bn + 8 * (i >> 2) + 4 * g + (i & 3);
-              const int row = pos0 + 32 * bm + c32;
-              if (col > row) S[bn][bm][i] = -INFINITY;
-            }
-      }
-      // online softmax per query row (= lane column); keys of a row live in this lane and lane^32
-      float alpha[2];
-#pragma unroll
-      for (int bm = 0; bm < 2; ++bm) {
-        float tmax = -INFINITY;
-#pragma unroll
-        for (int bn = 0; bn < 2; ++bn)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) tmax = fmaxf(tmax, S[bn][bm][i]);
-        tmax = wave_xor_max(tmax, 32);
-        const float m_new = fmaxf(m_run[bm], tmax);
-        alpha[bm] = exp2f(m_run[bm] - m_new);
-        m_run[bm] = m_new;
-        float psum = 0.f;
+        const int row = pos0 + c32;
 #pragma unroll
         for (int bn = 0; bn < 2; ++bn)
 #pragma unroll
           for (int i = 0; i < 16; ++i) {
-            const float p = exp2f(S[bn][bm][i] - m_new);
-            S[bn][bm][i] = p;
-            psum += p;
+            const int col = j * kBN + 32 * bn + 8 * (i >> 2) + 4 * g + (i & 3);
+            if (col > row) S[bn][i] = -INFINITY;
           }
-        l_run[bm] = l_run[bm] * alpha[bm] + psum;
       }
-      // quantise P and pack to fp16 in the B-operand layout of the P.V MFMA
-      if (a.p_quant == SQ_P_E4M3_BLOCK) {
-        float amax = 0.f;
+      // online softmax of this lane's query row; the row's other 32 keys live in lane^32
+      float tmax = fmaxf(S[0][0], S[1][0]);
 #pragma unroll
-        for (int bn = 0; bn < 2; ++bn)
+      for (int i = 1; i < 16; ++i) tmax = fmaxf(tmax, fmaxf(S[0][i], S[1][i]));
+      tmax = xor32_max(tmax);
+      const float m_new = fmaxf(m_run, tmax);
+      alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+      m_run = m_new;
+      const float shift = (MODE == 3) ? m_new - kLog2_448 : m_new;
+      float psum = 0.f;
 #pragma unroll
-          for (int bm = 0; bm < 2; ++bm)
+      for (int bn = 0; bn < 2; ++bn)
 #pragma unroll
-            for (int i = 0; i < 16; ++i) amax = fmaxf(amax, S[bn][bm][i]);
+        for (int i = 0; i < 16; ++i) {
+          const float p = __builtin_amdgcn_exp2f(S[bn][i] - shift);
+          S[bn][i] = p;
+          psum += p;
+        }
+      l_run = l_run * alpha + psum;
+    }
+
+    float sc = 448.f, inv = 1.0f / 448.0f;
+    if constexpr (MODE == 2) {  // block absmax over the 64-row group: this wave and its neighbour (wave ^ 1)
+      float amax = 0.f;
+      if (visit) {
+        amax = fmaxf(S[0][0], S[1][0]);
 #pragma unroll
-        for (int sh = 1; sh < 64; sh <<= 1) amax = wave_xor_max(amax, sh);
-        const float sc = 448.f / amax;   // amax > 0: every visited tile has an unmasked key per row
-        const float inv = amax / 448.f;
+        for (int i = 1; i < 16; ++i) amax = fmaxf(amax, fmaxf(S[0][i], S[1][i]));
+        if (row_w0 + c32 >= a.Nq) amax = 0.f;   // rows past the end are clamped copies, not part of the block
 #pragma unroll
-        for (int bn = 0; bn < 2; ++bn)
-#pragma unroll
-          for (int bm = 0; bm < 2; ++bm)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) S[bn][bm][i] = e4m3_roundtrip(fminf(S[bn][bm][i] * sc, 448.f)) * inv;
-      } else if (a.p_quant == SQ_P_E4M3_STATIC) {
-#pragma unroll
-        for (int bn = 0; bn < 2; ++bn)
-#pragma unroll
-          for (int bm = 0; bm < 2; ++bm)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) S[bn][bm][i] = e4m3_roundtrip(S[bn][bm][i] * 448.f) * (1.0f / 448.0f);
+        for (int sh = 1; sh < 32; sh <<= 1) amax = wave_xor_max(amax, sh);
+        amax = xor32_max(amax);
       }
-      uint4 P[2][2][2];  // [bm][bn][t]
+      if (lane == 0) s_amax[it & 1][wave] = amax;  // 0 from a wave that does not visit this tile
+      __syncthreads();  // every wave of the workgroup passes here once per tile, visiting or not
+      if (visit) {
+        if constexpr (WAVES > 1) amax = fmaxf(amax, s_amax[it & 1][wave ^ 1]);
+        sc = 448.f / amax;   // amax > 0: every visited tile has an unmasked key in every row
+        inv = amax / 448.f;
+      }
+    }
+
+    if (visit) {
+      uint4 P[2][2];  // [bn][t]
 #pragma unroll
-      for (int bm = 0; bm < 2; ++bm)
+      for (int bn = 0; bn < 2; ++bn)
 #pragma unroll
-        for (int bn = 0; bn < 2; ++bn)
+        for (int t = 0; t < 2; ++t) P[bn][t] = quant_pack8<MODE>(S[bn], t, sc, inv);
+      if (__any(alpha != 1.f)) {
 #pragma unroll
-          for (int t = 0; t < 2; ++t) {
-            const f32x16_t& s = S[bn][bm];
-            P[bm][bn][t] = make_uint4(pack_f16(s[8 * t + 0], s[8 * t + 1]), pack_f16(s[8 * t + 2], s[8 * t + 3]),
-                                      pack_f16(s[8 * t + 4], s[8 * t + 5]), pack_f16(s[8 * t + 6], s[8 * t + 7]));
-          }
-      if (__any(alpha[0] != 1.f || alpha[1] != 1.f)) {
-#pragma unroll
-        for (int bd = 0; bd < 4; ++bd)
-#pragma unroll
-          for (int bm = 0; bm < 2; ++bm) O[bd][bm] *= alpha[bm];
+        for (int bd = 0; bd < 4; ++bd) O[bd] *= alpha;
       }
       // O^T[d, row] += V^T[d, key] . P^T[key, row]
 #pragma unroll
@@ -420,8 +449,7 @@ __global__ __launch_bounds__(WAVES * 64, 1) void prefill_kernel(PrefillArgs a) {
 #pragma unroll
           for (int t = 0; t < 2; ++t) {
             const uint4 av = *(const uint4*)(vbuf + (32 * bd + c32) * kVStride + (32 * bn + 16 * t + 8 * g) * 2);
-            O[bd][0] = mfma_pv32(av, P[0][bn][t], O[bd][0]);
-            O[bd][1] = mfma_pv32(av, P[1][bn][t], O[bd][1]);
+            O[bd] = mfma_pv32(av, P[bn][t], O[bd]);
           }
     }
 
@@ -432,32 +460,32 @@ __global__ __launch_bounds__(WAVES * 64, 1) void prefill_kernel(PrefillArgs a) {
 
   // ---- epilogue: out = acc / l (attn_triton.py:208-209), lse2 = log2(l) + m (:210-213)
   if (!wave_active) return;
+  const float l = xor32_sum(l_run);
+  const int row = row_w0 + c32;
+  if (row >= a.Nq) return;
+  const int64_t obase = (int64_t)b * a.o_sb + (int64_t)head * a.o_sh + (int64_t)row * a.o_sn;
 #pragma unroll
-  for (int bm = 0; bm < 2; ++bm) {
-    const float l = l_run[bm] + __shfl_xor(l_run[bm], 32);
-    const int row = row_w0 + 32 * bm + c32;
-    if (row >= a.Nq) continue;
-    const int64_t obase = (int64_t)b * a.o_sb + (int64_t)head * a.o_sh + (int64_t)row * a.o_sn;
+  for (int bd = 0; bd < 4; ++bd)
 #pragma unroll
-    for (int bd = 0; bd < 4; ++bd)
+    for (int i4 = 0; i4 < 4; ++i4) {
+      const int d = 32 * bd + 8 * i4 + 4 * g;
+      float v[4];
 #pragma unroll
-      for (int i4 = 0; i4 < 4; ++i4) {
-        const int d = 32 * bd + 8 * i4 + 4 * g;
-        float v[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] = O[bd][bm][4 * i4 + e] / l;
-        if (a.out_dtype == 0) {
-          uint2 w = make_uint2(f32_to_bf16_bits(v[0]) | (f32_to_bf16_bits(v[1]) << 16),
-                               f32_to_bf16_bits(v[2]) | (f32_to_bf16_bits(v[3]) << 16));
-          *(uint2*)((uint16_t*)a.out + obase + d) = w;
-        } else if (a.out_dtype == 1) {
-          uint2 w = make_uint2(pack_f16(v[0], v[1]), pack_f16(v[2], v[3]));
-          *(uint2*)((uint16_t*)a.out + obase + d) = w;
-        } else {
-          *(float4*)((float*)a.out + obase + d) = make_float4(v[0], v[1], v[2], v[3]);
-        }
+      for (int e = 0; e < 4; ++e) v[e] = O[bd][4 * i4 + e] / l;
+      if (a.out_dtype == 0) {
+        uint2 w = make_uint2(f32_to_bf16_bits(v[0]) | (f32_to_bf16_bits(v[1]) << 16),
+                             f32_to_bf16_bits(v[2]) | (f32_to_bf16_bits(v[3]) << 16));
+        *(uint2*)((uint16_t*)a.out + obase + d) = w;
+      } else if (a.out_dtype == 1) {
+        uint2 w = make_uint2(pack_f16(v[0], v[1]), pack_f16(v[2], v[3]));
+        *(uint2*)((uint16_t*)a.out + obase + d) = w;
+      } else {
+        *(float4*)((float*)a.out + obase + d) = make_float4(v[0], v[1], v[2], v[3]);
       }
-    if (a.lse && g == 0) a.lse[((int64_t)b * a.Hq + head) * a.Nq + row] = log2f(l) + m_run[bm];
+    }
+  if (a.lse && g == 0) {
+    const float lt = (MODE == 3) ? l * (1.0f / 448.0f) : l;
+    a.lse[((int64_t)b * a.Hq + head) * a.Nq + row] = log2f(lt) + m_run;
   }
 }
 
@@ -479,7 +507,7 @@ extern "C" int sq_prefill_fwd(const DLTensor* q, const DLTensor* k, const DLTens
   SQ_REQUIRE(p, SQ_EINVAL, "sq_prefill_fwd: params is null");
   SQ_REQUIRE(q && k && v && out, SQ_EINVAL, "sq_prefill_fwd: q, k, v and out must be non-null");
   SQ_REQUIRE(p->layout == SQ_LAYOUT_HND || p->layout == SQ_LAYOUT_NHD, SQ_EINVAL, "tensor_layout %d not supported", p->layout);
-  SQ_REQUIRE(p->p_quant >= SQ_P_NONE && p->p_quant <= SQ_P_E4M3_BLOCK, SQ_EINVAL, "sq_prefill_fwd: p_quant %d not supported", p->p_quant);
+  SQ_REQUIRE(p->p_quant >= SQ_P_NONE && p->p_quant <= SQ_P_E4M3_STATIC_FAST, SQ_EINVAL, "sq_prefill_fwd: p_quant %d not supported", p->p_quant);
   SQ_REQUIRE((q4 == nullptr) == (k4 == nullptr), SQ_EINVAL, "sq_prefill_fwd: q4 and k4 must be given together");
   int rc;
   const int dev = q->device.device_id;
@@ -526,7 +554,7 @@ extern "C" int sq_prefill_fwd(const DLTensor* q, const DLTensor* k, const DLTens
     SQ_REQUIRE(dtype_of(lse) == DType::F32 && numel_of(lse) == B * Hq * Nq && is_compact(lse), SQ_ESHAPE,
                "sq_prefill_fwd: lse must be a compact fp32 [B,Hq,Nq]");
   }
-  int waves = 4;
+  int waves = 8;
   if (p->window_mode == SQ_WINDOW_SIZES) {
     SQ_REQUIRE(p->block_m == 64 || p->block_m == 128, SQ_EINVAL, "sq_prefill_fwd: block_m must be 64 or 128");
     SQ_REQUIRE(p->sink >= 0, SQ_EINVAL, "sink_size must be a non-negative integer, got %d", p->sink);
@@ -542,8 +570,7 @@ extern "C" int sq_prefill_fwd(const DLTensor* q, const DLTensor* k, const DLTens
                  "sq_prefill_fwd: head %d: a 4-bit window wider than an 8-bit window smaller than block_m reads future keys "
                  "in the reference and is not supported", h);
     }
-    if (q4) waves = p->block_m / kRowsPerWave;  // all waves of a workgroup must agree on the operand set of a tile
-    SQ_REQUIRE(waves >= 2, SQ_EUNSUPPORTED, "sq_prefill_fwd: separate 4-bit operands need block_m = 128");
+    if (q4) waves = p->block_m / 32;  // all waves of a workgroup must agree on the operand set of a tile
   } else {
     SQ_REQUIRE(p->window_mode == SQ_WINDOW_NONE, SQ_EINVAL, "sq_prefill_fwd: window_mode %d not supported", p->window_mode);
     SQ_REQUIRE(!q4, SQ_EINVAL, "sq_prefill_fwd: q4/k4 only apply to window mode");
@@ -599,7 +626,7 @@ extern "C" int sq_prefill_fwd(const DLTensor* q, const DLTensor* k, const DLTens
   local.Nq = (int)Nq;
   local.Nk = (int)Nk;
   local.nT = nT;
-  const int rows_wg = waves * kRowsPerWave;
+  const int rows_wg = waves * 32;
   local.nQB = (int)((Nq + rows_wg - 1) / rows_wg);
   local.q_offset = (int)p->q_offset;
   local.p_quant = p->p_quant;
@@ -635,17 +662,29 @@ extern "C" int sq_prefill_fwd(const DLTensor* q, const DLTensor* k, const DLTens
   }
   const size_t smem = 2 * kStageBytes;
   const bool bf = dt == DType::BF16;
-#define SQ_LAUNCH_PREFILL(BF, W)                                                                              \
-  do {                                                                                                        \
-    SQ_HIP(hipFuncSetAttribute((const void*)prefill_kernel<BF, W>, hipFuncAttributeMaxDynamicSharedMemorySize, \
-                               (int)smem));                                                                   \
-    hipLaunchKernelGGL((prefill_kernel<BF, W>), dim3(blocks), dim3(W * 64), smem, st, local);                 \
+#define SQ_LAUNCH_PREFILL(BF, W, M)                                                                              \
+  do {                                                                                                           \
+    SQ_HIP(hipFuncSetAttribute((const void*)prefill_kernel<BF, W, M>, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                               (int)smem));                                                                      \
+    hipLaunchKernelGGL((prefill_kernel<BF, W, M>), dim3(blocks), dim3(W * 64), smem, st, local);                 \
   } while (0)
-  if (waves == 4) {
-    if (bf) SQ_LAUNCH_PREFILL(true, 4); else SQ_LAUNCH_PREFILL(false, 4);
+#define SQ_LAUNCH_MODE(BF, W)                                   \
+  do {                                                          \
+    switch (p->p_quant) {                                       \
+      case SQ_P_NONE: SQ_LAUNCH_PREFILL(BF, W, 0); break;        \
+      case SQ_P_E4M3_STATIC: SQ_LAUNCH_PREFILL(BF, W, 1); break; \
+      case SQ_P_E4M3_BLOCK: SQ_LAUNCH_PREFILL(BF, W, 2); break;  \
+      default: SQ_LAUNCH_PREFILL(BF, W, 3); break;               \
+    }                                                           \
+  } while (0)
+  if (waves == 8) {
+    if (bf) SQ_LAUNCH_MODE(true, 8); else SQ_LAUNCH_MODE(false, 8);
+  } else if (waves == 4) {
+    if (bf) SQ_LAUNCH_MODE(true, 4); else SQ_LAUNCH_MODE(false, 4);
   } else {
-    if (bf) SQ_LAUNCH_PREFILL(true, 2); else SQ_LAUNCH_PREFILL(false, 2);
+    if (bf) SQ_LAUNCH_MODE(true, 2); else SQ_LAUNCH_MODE(false, 2);
   }
+#undef SQ_LAUNCH_MODE
 #undef SQ_LAUNCH_PREFILL
   SQ_HIP(hipGetLastError());
   return SQ_OK;

@@ -44,13 +44,14 @@ def _rand(B, Hq, Hkv, N, D, seed, dtype=torch.bfloat16, scale=1.0):
 
 
 @pytest.mark.parametrize("B,Hq,Hkv,N", [(1, 4, 2, 512), (2, 14, 2, 700), (1, 2, 1, 64), (1, 3, 3, 1000)])
-@pytest.mark.parametrize("mode", [A.P_NONE, A.P_STATIC448, A.P_BLOCK_ABSMAX])
+@pytest.mark.parametrize("mode", [A.P_NONE, A.P_STATIC448, A.P_BLOCK_ABSMAX, 3])
 def test_causal_matches_oracle(B, Hq, Hkv, N, mode):
     from longcontext_sqattn_paddle_amd.sqattn.attn_triton import attn_causal
 
     print(f"case prefill causal B={B} Hq={Hq} Hkv={Hkv} N={N} p_quant={mode}", flush=True)
     q, k, v = _rand(B, Hq, Hkv, N, 128, 100 + N)
-    ref, lse_ref = A.prefill_blockwise(q, k, v, p_quant=mode, out_dtype=torch.float32)
+    # kernel mode 3 is the static-448 grid with the scale folded into the exponent: same oracle, same tolerance
+    ref, lse_ref = A.prefill_blockwise(q, k, v, p_quant=A.P_STATIC448 if mode == 3 else mode, out_dtype=torch.float32)
     out, lse = attn_causal(q.to(DEV), k.to(DEV), v.to(DEV), "HND", torch.float32, return_lse=True, p_quant=mode)
     torch.cuda.synchronize()
     _check(out, ref, mode != A.P_NONE)
