@@ -18,6 +18,8 @@
 //     tiles into the workspace (O(N) work against the O(N^2) main loop);
 //   * blockIdx -> (kv head, q head, q block) mapping keeps the q-heads of one KV head on the same XCD(s) so
 //     their K/V tiles are shared in that XCD's L2, and issues the longest (last) query blocks first.
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace sq {
@@ -25,8 +27,12 @@ namespace {
 
 constexpr int kD = 128;
 constexpr int kBN = 64;                  // keys per tile (BLOCK_N of every reference kernel)
-constexpr int kKStride = 272;            // bytes per K row in LDS (256 + 16 pad)
-constexpr int kVStride = 144;            // bytes per V^T row in LDS (128 + 16 pad)
+// LDS tiles are unpadded and XOR-swizzled at 16-byte granularity (they are filled by global_load_lds, which
+// writes 64 consecutive 16-byte slots per wave instruction): chunk c of K row n sits in slot c ^ (n & 15),
+// chunk c of V^T row d in slot c ^ ((d >> 1) & 7).  The 16 rows a quarter-wave reads at one chunk index then
+// fall into 16 different 16-byte bank groups.
+constexpr int kKStride = 256;            // bytes per K row in LDS
+constexpr int kVStride = 128;            // bytes per V^T row in LDS
 constexpr int kKTileBytes = kBN * kKStride;
 constexpr int kVTileBytes = kD * kVStride;
 constexpr int kStageBytes = kKTileBytes + kVTileBytes;
@@ -171,6 +177,13 @@ __device__ __forceinline__ WaveRanges wave_ranges(const PrefillArgs& a, int pos0
   return r;
 }
 
+// v_max3_f32 without the canonicalising self-max the compiler adds around fmaxf of MFMA results
+__device__ __forceinline__ float max3(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+
 // exchange with the lane 32 away (the other half of the keys of the same query row)
 __device__ __forceinline__ float xor32_max(float v) {
   const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
@@ -257,7 +270,8 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
   const int head = kvh * a.group + hg;
 
   const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: keep it (and all it feeds) in SGPRs
   const int c32 = lane & 31, g = lane >> 5;
 
   const int row_wg0 = qb * (WAVES * ROWS);          // first query row of the workgroup
@@ -283,7 +297,8 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
     segA_hi = 0;
     segB_lo = 0;
   }
-  const bool distinct4 = a.q4 != nullptr;  // host guarantees WAVES*32 == block_m in that case
+  // separate 4-bit operands only ever run with WAVES*32 == block_m <= 128 (all waves agree on a tile's operand set)
+  const bool distinct4 = (WAVES < 8) && a.q4 != nullptr;
 
   // ---- Q~ fragments (B operand of S^T = K.Q~^T): lane (column = query row c32, k-group g)
   uint4 qf[8];
@@ -306,34 +321,38 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
   for (int bd = 0; bd < 4; ++bd)
 #pragma unroll
     for (int i = 0; i < 16; ++i) O[bd][i] = 0.f;
-  float m_run = -INFINITY;
-  float l_run = 0.f;   // this lane's share of the denominator (times 448 in MODE 3)
+  // Online-softmax state of this lane's query row.  The score accumulators are *initialised* with
+  // cinit = kC - m_run (kC = log2(448) in MODE 3, else 0), so the MFMA chain delivers S - m_run + kC and, as
+  // long as the running maximum does not move, p (or 448 p) is a bare exp2 of the accumulator.
+  constexpr float kC = (MODE == 3) ? kLog2_448 : 0.f;
+  float m_run = 0.f;       // reference point of the exponent; the first visited tile replaces it by the row maximum
+  float l_run = 0.f;       // this lane's share of the denominator (times 448 in MODE 3)
+  bool first = true;       // wave-uniform: no tile visited yet
+  f32x16_t Cinit;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) Cinit[i] = kC;
 
   const _Float16* vt_base = a.vt + ((int64_t)b * a.Hkv + kvh) * (int64_t)a.nT * (kD * kBN);
 
-  // ---- tile staging helpers
-  uint4 kreg[CH], vreg[CH];
+  // ---- tile staging: global -> LDS directly (no registers), CH wave instructions of 64 x 16 bytes per operand
+  typedef __attribute__((address_space(3))) void* lds_ptr_t;
   auto tile_uses4 = [&](int j) { return distinct4 && j >= wr.r4_lo && j < wr.r4_hi; };
-  auto gload = [&](int j) {
-    const void* ksrc = tile_uses4(j) ? a.k4 : a.k;
-    const uint16_t* kb = (const uint16_t*)ksrc + (int64_t)b * a.k_sb + (int64_t)kvh * a.k_sh;
-    const uint4* vsrc = (const uint4*)(vt_base + (int64_t)j * (kD * kBN));
-#pragma unroll
-    for (int c = 0; c < CH; ++c) {
-      const int ch = c * NT + tid;            // chunk id 0..1023
-      const int n = min(j * kBN + (ch >> 4), a.Nk - 1);
-      kreg[c] = *(const uint4*)(kb + (int64_t)n * a.k_sn + 8 * (ch & 15));
-      vreg[c] = vsrc[ch];
-    }
-  };
-  auto lstore = [&](int stage) {
+  const int64_t k_head_off = (int64_t)b * a.k_sb + (int64_t)kvh * a.k_sh;
+  auto stage_tile = [&](int j, int stage) {
     char* kbuf = smem + stage * kStageBytes;
     char* vbuf = kbuf + kKTileBytes;
+    const uint16_t* kb = (const uint16_t*)(tile_uses4(j) ? a.k4 : a.k) + k_head_off;
+    const _Float16* vsrc = vt_base + (int64_t)j * (kD * kBN);
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
-      const int ch = c * NT + tid;
-      *(uint4*)(kbuf + (ch >> 4) * kKStride + (ch & 15) * 16) = kreg[c];
-      *(uint4*)(vbuf + (ch >> 3) * kVStride + (ch & 7) * 16) = vreg[c];
+      const int q = wave * CH + c;                       // wave instruction index 0..15 -> 1 KB of each tile
+      const int kr = 4 * q + (lane >> 4);                // K row in the tile
+      const int kc = (lane & 15) ^ (kr & 15);            // global chunk that lands in this lane's slot
+      const int n = min(j * kBN + kr, a.Nk - 1);
+      __builtin_amdgcn_global_load_lds((const void*)(kb + (int64_t)n * a.k_sn + 8 * kc), (lds_ptr_t)(kbuf + q * 1024), 16, 0, 0);
+      const int vr = 8 * q + (lane >> 3);                // V^T row (channel)
+      const int vc = (lane & 7) ^ ((vr >> 1) & 7);
+      __builtin_amdgcn_global_load_lds((const void*)(vsrc + vr * kBN + 8 * vc), (lds_ptr_t)(vbuf + q * 1024), 16, 0, 0);
     }
   };
   auto next_tile = [&](int j) {
@@ -342,118 +361,132 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
     return n;
   };
 
+  // ---- one KV tile for this wave.  `masked`: the tile lies in the query block's own (diagonal) range.
+  auto tile_body = [&](int j, int it, const char* kbuf, const char* vbuf, bool masked) {
+    const int ksw = c32 & 15;          // swizzle of this lane's K rows (c32 and c32 + 32 share it)
+    const int vsw = (c32 >> 1) & 7;    // swizzle of this lane's V^T rows (32 bd + c32)
+    f32x16_t S[2];
+    {
+      const uint4 a0 = *(const uint4*)(kbuf + c32 * kKStride + ((g ^ ksw) << 4));
+      const uint4 a1 = *(const uint4*)(kbuf + (32 + c32) * kKStride + ((g ^ ksw) << 4));
+      S[0] = mfma_qk32<BF16>(a0, qf[0], Cinit);
+      S[1] = mfma_qk32<BF16>(a1, qf[0], Cinit);
+    }
+#pragma unroll
+    for (int kk = 1; kk < 8; ++kk) {
+      const uint4 a0 = *(const uint4*)(kbuf + c32 * kKStride + (((2 * kk + g) ^ ksw) << 4));
+      const uint4 a1 = *(const uint4*)(kbuf + (32 + c32) * kKStride + (((2 * kk + g) ^ ksw) << 4));
+      S[0] = mfma_qk32<BF16>(a0, qf[kk], S[0]);
+      S[1] = mfma_qk32<BF16>(a1, qf[kk], S[1]);
+    }
+    if (masked) {  // causal mask inside the query block's own tiles (attn_triton.py:69-71)
+      asm volatile("; causal mask" ::: "memory");   // keeps this a real branch: one tile in thousands takes it
+      const int row = pos0 + c32;
+#pragma unroll
+      for (int bn = 0; bn < 2; ++bn)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int col = j * kBN + 32 * bn + 8 * (i >> 2) + 4 * g + (i & 3);
+          if (col > row) S[bn][i] = -INFINITY;
+        }
+    }
+    // row maximum of S - m_run + kC; the row's other 32 keys live in lane^32
+    float tmax = max3(S[0][0], S[1][0], S[0][1]);
+#pragma unroll
+    for (int i = 1; i < 15; ++i) tmax = max3(tmax, S[1][i], S[0][i + 1]);
+    tmax = max3(tmax, S[1][15], S[1][15]);
+    tmax = xor32_max(tmax);
+    if (first || __any(tmax > kC)) {
+      // some row's maximum moved by d (on the first tile: from the arbitrary reference 0 to the row maximum):
+      // shift the scores, rescale the accumulators, re-centre the accumulator initialiser
+      asm volatile("; new row maximum" ::: "memory");
+      const float d = first ? (tmax - kC) : fmaxf(tmax - kC, 0.f);
+      const float alpha = first ? 0.f : __builtin_amdgcn_exp2f(-d);
+      m_run += d;
+      l_run *= alpha;
+#pragma unroll
+      for (int bn = 0; bn < 2; ++bn)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) S[bn][i] -= d;
+#pragma unroll
+      for (int bd = 0; bd < 4; ++bd) O[bd] *= alpha;
+      const float c = kC - m_run;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) Cinit[i] = c;
+      first = false;
+    }
+    float psum = 0.f;
+#pragma unroll
+    for (int bn = 0; bn < 2; ++bn)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const float p = __builtin_amdgcn_exp2f(S[bn][i]);
+        S[bn][i] = p;
+        psum += p;
+      }
+    l_run += psum;
+
+    float sc = 448.f, inv = 1.0f / 448.0f;
+    if constexpr (MODE == 2) {  // block absmax over the 64-row group: this wave and its neighbour (wave ^ 1)
+      float amax = fmaxf(S[0][0], S[1][0]);
+#pragma unroll
+      for (int i = 1; i < 16; ++i) amax = fmaxf(amax, fmaxf(S[0][i], S[1][i]));
+      if (row_w0 + c32 >= a.Nq) amax = 0.f;   // rows past the end are clamped copies, not part of the block
+#pragma unroll
+      for (int sh = 1; sh < 32; sh <<= 1) amax = wave_xor_max(amax, sh);
+      amax = xor32_max(amax);
+      if (lane == 0) s_amax[it & 1][wave] = amax;
+      __syncthreads();  // see the matching barrier for waves that skip this tile
+      if constexpr (WAVES > 1) amax = fmaxf(amax, s_amax[it & 1][wave ^ 1]);
+      sc = 448.f / amax;   // amax > 0: every visited tile has an unmasked key in every row
+      inv = amax / 448.f;
+    }
+    uint4 P[2][2];  // [bn][t]
+#pragma unroll
+    for (int bn = 0; bn < 2; ++bn)
+#pragma unroll
+      for (int t = 0; t < 2; ++t) P[bn][t] = quant_pack8<MODE>(S[bn], t, sc, inv);
+    // O^T[d, row] += V^T[d, key] . P^T[key, row]
+#pragma unroll
+    for (int bd = 0; bd < 4; ++bd)
+#pragma unroll
+      for (int bn = 0; bn < 2; ++bn)
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          const uint4 av = *(const uint4*)(vbuf + (32 * bd + c32) * kVStride + (((4 * bn + 2 * t + g) ^ vsw) << 4));
+          O[bd] = mfma_pv32(av, P[bn][t], O[bd]);
+        }
+  };
+
   int j = (segA_hi > 0) ? 0 : segB_lo;
-  if (j < segB_hi) {
-    gload(j);
-    lstore(0);
-  }
+  if (j < segB_hi) stage_tile(j, 0);
+  __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
 
   for (int it = 0; j < segB_hi; ++it) {
     const int jn = next_tile(j);
     const bool have_next = jn < segB_hi;
-    if (have_next) gload(jn);
-    const bool visit = wave_active && wr.visits(j);
+    if (have_next) stage_tile(jn, (it + 1) & 1);   // the other stage was last read before the previous barrier
     const char* kbuf = smem + (it & 1) * kStageBytes;
     const char* vbuf = kbuf + kKTileBytes;
-    f32x16_t S[2];
-    float alpha = 1.f;
 
-    if (visit) {
-      if (distinct4) {  // switch the Q~ operand set when entering/leaving the 4-bit window range
-        const bool want4 = tile_uses4(j);
-        if (want4 != q_is4) {
-          load_q(want4 ? a.q4 : a.q);
-          q_is4 = want4;
+    if (wave_active && wr.visits(j)) {
+      if constexpr (WAVES < 8) {
+        if (distinct4) {  // switch the Q~ operand set when entering/leaving the 4-bit window range
+          const bool want4 = tile_uses4(j);
+          if (want4 != q_is4) {
+            load_q(want4 ? a.q4 : a.q);
+            q_is4 = want4;
+          }
         }
       }
-      // S^T[key, row] for the 2 key blocks of 32
-#pragma unroll
-      for (int bn = 0; bn < 2; ++bn)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) S[bn][i] = 0.f;
-#pragma unroll
-      for (int kk = 0; kk < 8; ++kk) {
-        const uint4 a0 = *(const uint4*)(kbuf + c32 * kKStride + (16 * kk + 8 * g) * 2);
-        const uint4 a1 = *(const uint4*)(kbuf + (32 + c32) * kKStride + (16 * kk + 8 * g) * 2);
-        S[0] = mfma_qk32<BF16>(a0, qf[kk], S[0]);
-        S[1] = mfma_qk32<BF16>(a1, qf[kk], S[1]);
-      }
-      if (j >= wr.diag_lo) {  // causal mask inside the query block's own tiles (attn_triton.py:69-71)
-        const int row = pos0 + c32;
-#pragma unroll
-        for (int bn = 0; bn < 2; ++bn)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) {
-            const int col = j * kBN + 32 * bn + 8 * (i >> 2) + 4 * g + (i & 3);
-            if (col > row) S[bn][i] = -INFINITY;
-          }
-      }
-      // online softmax of this lane's query row; the row's other 32 keys live in lane^32
-      float tmax = fmaxf(S[0][0], S[1][0]);
-#pragma unroll
-      for (int i = 1; i < 16; ++i) tmax = fmaxf(tmax, fmaxf(S[0][i], S[1][i]));
-      tmax = xor32_max(tmax);
-      const float m_new = fmaxf(m_run, tmax);
-      alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-      m_run = m_new;
-      const float shift = (MODE == 3) ? m_new - kLog2_448 : m_new;
-      float psum = 0.f;
-#pragma unroll
-      for (int bn = 0; bn < 2; ++bn)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const float p = __builtin_amdgcn_exp2f(S[bn][i] - shift);
-          S[bn][i] = p;
-          psum += p;
-        }
-      l_run = l_run * alpha + psum;
+      tile_body(j, it, kbuf, vbuf, j >= wr.diag_lo);
+    } else if constexpr (MODE == 2) {
+      if (lane == 0) s_amax[it & 1][wave] = 0.f;  // a wave that skips the tile contributes nothing to the block maximum
+      __syncthreads();                            // every wave passes one such barrier per tile
     }
 
-    float sc = 448.f, inv = 1.0f / 448.0f;
-    if constexpr (MODE == 2) {  // block absmax over the 64-row group: this wave and its neighbour (wave ^ 1)
-      float amax = 0.f;
-      if (visit) {
-        amax = fmaxf(S[0][0], S[1][0]);
-#pragma unroll
-        for (int i = 1; i < 16; ++i) amax = fmaxf(amax, fmaxf(S[0][i], S[1][i]));
-        if (row_w0 + c32 >= a.Nq) amax = 0.f;   // rows past the end are clamped copies, not part of the block
-#pragma unroll
-        for (int sh = 1; sh < 32; sh <<= 1) amax = wave_xor_max(amax, sh);
-        amax = xor32_max(amax);
-      }
-      if (lane == 0) s_amax[it & 1][wave] = amax;  // 0 from a wave that does not visit this tile
-      __syncthreads();  // every wave of the workgroup passes here once per tile, visiting or not
-      if (visit) {
-        if constexpr (WAVES > 1) amax = fmaxf(amax, s_amax[it & 1][wave ^ 1]);
-        sc = 448.f / amax;   // amax > 0: every visited tile has an unmasked key in every row
-        inv = amax / 448.f;
-      }
-    }
-
-    if (visit) {
-      uint4 P[2][2];  // [bn][t]
-#pragma unroll
-      for (int bn = 0; bn < 2; ++bn)
-#pragma unroll
-        for (int t = 0; t < 2; ++t) P[bn][t] = quant_pack8<MODE>(S[bn], t, sc, inv);
-      if (__any(alpha != 1.f)) {
-#pragma unroll
-        for (int bd = 0; bd < 4; ++bd) O[bd] *= alpha;
-      }
-      // O^T[d, row] += V^T[d, key] . P^T[key, row]
-#pragma unroll
-      for (int bd = 0; bd < 4; ++bd)
-#pragma unroll
-        for (int bn = 0; bn < 2; ++bn)
-#pragma unroll
-          for (int t = 0; t < 2; ++t) {
-            const uint4 av = *(const uint4*)(vbuf + (32 * bd + c32) * kVStride + (32 * bn + 16 * t + 8 * g) * 2);
-            O[bd] = mfma_pv32(av, P[bn][t], O[bd]);
-          }
-    }
-
-    if (have_next) lstore((it + 1) & 1);
+    __builtin_amdgcn_s_waitcnt(0);   // this wave's share of the next tile has landed in LDS
     __syncthreads();
     j = jn;
   }
