@@ -334,22 +334,31 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
 
   const _Float16* vt_base = a.vt + ((int64_t)b * a.Hkv + kvh) * (int64_t)a.nT * (kD * kBN);
 
-  // ---- tile staging: global -> LDS directly (no registers), CH wave instructions of 64 x 16 bytes per operand
+  // ---- tile staging: global -> LDS directly (no registers), CH wave instructions of 64 x 16 bytes per operand.
+  // K and V^T have their own double buffers because the K tile runs one step ahead of the V^T tile (below).
   typedef __attribute__((address_space(3))) void* lds_ptr_t;
   auto tile_uses4 = [&](int j) { return distinct4 && j >= wr.r4_lo && j < wr.r4_hi; };
   const int64_t k_head_off = (int64_t)b * a.k_sb + (int64_t)kvh * a.k_sh;
-  auto stage_tile = [&](int j, int stage) {
-    char* kbuf = smem + stage * kStageBytes;
-    char* vbuf = kbuf + kKTileBytes;
+  char* const kbase_lds = smem;                     // 2 x 16 KB
+  char* const vbase_lds = smem + 2 * kKTileBytes;   // 2 x 16 KB
+  auto stage_k = [&](int j, int stage) {
+    char* kbuf = kbase_lds + stage * kKTileBytes;
     const uint16_t* kb = (const uint16_t*)(tile_uses4(j) ? a.k4 : a.k) + k_head_off;
-    const _Float16* vsrc = vt_base + (int64_t)j * (kD * kBN);
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
-      const int q = wave * CH + c;                       // wave instruction index 0..15 -> 1 KB of each tile
+      const int q = wave * CH + c;                       // wave instruction index 0..15 -> 1 KB of the tile
       const int kr = 4 * q + (lane >> 4);                // K row in the tile
       const int kc = (lane & 15) ^ (kr & 15);            // global chunk that lands in this lane's slot
       const int n = min(j * kBN + kr, a.Nk - 1);
       __builtin_amdgcn_global_load_lds((const void*)(kb + (int64_t)n * a.k_sn + 8 * kc), (lds_ptr_t)(kbuf + q * 1024), 16, 0, 0);
+    }
+  };
+  auto stage_v = [&](int j, int stage) {
+    char* vbuf = vbase_lds + stage * kVTileBytes;
+    const _Float16* vsrc = vt_base + (int64_t)j * (kD * kBN);
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const int q = wave * CH + c;
       const int vr = 8 * q + (lane >> 3);                // V^T row (channel)
       const int vc = (lane & 7) ^ ((vr >> 1) & 7);
       __builtin_amdgcn_global_load_lds((const void*)(vsrc + vr * kBN + 8 * vc), (lds_ptr_t)(vbuf + q * 1024), 16, 0, 0);
@@ -361,11 +370,11 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
     return n;
   };
 
-  // ---- one KV tile for this wave.  `masked`: the tile lies in the query block's own (diagonal) range.
-  auto tile_body = [&](int j, int it, const char* kbuf, const char* vbuf, bool masked) {
-    const int ksw = c32 & 15;          // swizzle of this lane's K rows (c32 and c32 + 32 share it)
-    const int vsw = (c32 >> 1) & 7;    // swizzle of this lane's V^T rows (32 bd + c32)
-    f32x16_t S[2];
+  const int ksw = c32 & 15;          // swizzle of this lane's K rows (c32 and c32 + 32 share it)
+  const int vsw = (c32 >> 1) & 7;    // swizzle of this lane's V^T rows (32 bd + c32)
+
+  // S^T = K . Q~^T + Cinit for one tile: 16 MFMAs that nothing below depends on until the next step
+  auto qk_tile = [&](const char* kbuf, f32x16_t (&S)[2]) {
     {
       const uint4 a0 = *(const uint4*)(kbuf + c32 * kKStride + ((g ^ ksw) << 4));
       const uint4 a1 = *(const uint4*)(kbuf + (32 + c32) * kKStride + ((g ^ ksw) << 4));
@@ -379,16 +388,24 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
       S[0] = mfma_qk32<BF16>(a0, qf[kk], S[0]);
       S[1] = mfma_qk32<BF16>(a1, qf[kk], S[1]);
     }
+  };
+
+  // softmax update + P.V for the tile whose scores are in S.  Once the running maximum of this tile is settled,
+  // the Q.K^T MFMAs of the following tile (K in knext, result in Snext) are issued in the same straight-line
+  // block as the exponentials, conversions and P.V MFMAs, so that the matrix pipe and the vector ALU of this
+  // wave work side by side.
+  auto softmax_pv = [&](int j, int it, const char* vbuf, bool masked, f32x16_t (&S)[2], const char* knext, f32x16_t (&Snext)[2]) {
     if (masked) {  // causal mask inside the query block's own tiles (attn_triton.py:69-71)
-      asm volatile("; causal mask" ::: "memory");   // keeps this a real branch: one tile in thousands takes it
-      const int row = pos0 + c32;
+      // One tile in thousands takes this branch.  The laundered copy of g keeps the branch a branch and stops
+      // the compiler from hoisting 32 per-lane column constants out of the loop into precious registers.
+      int gm = g;
+      asm volatile("; causal mask" : "+v"(gm));
+      const int rel = pos0 + c32 - j * kBN - 4 * gm;   // key index (within the tile, minus 4g) of the diagonal
 #pragma unroll
       for (int bn = 0; bn < 2; ++bn)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int col = j * kBN + 32 * bn + 8 * (i >> 2) + 4 * g + (i & 3);
-          if (col > row) S[bn][i] = -INFINITY;
-        }
+        for (int i = 0; i < 16; ++i)
+          if (32 * bn + 8 * (i >> 2) + (i & 3) > rel) S[bn][i] = -INFINITY;
     }
     // row maximum of S - m_run + kC; the row's other 32 keys live in lane^32
     float tmax = max3(S[0][0], S[1][0], S[0][1]);
@@ -415,6 +432,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
       for (int i = 0; i < 16; ++i) Cinit[i] = c;
       first = false;
     }
+    qk_tile(knext, Snext);   // scores of the next tile, relative to the maximum just settled
     float psum = 0.f;
 #pragma unroll
     for (int bn = 0; bn < 2; ++bn)
@@ -458,37 +476,64 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
         }
   };
 
-  int j = (segA_hi > 0) ? 0 : segB_lo;
-  if (j < segB_hi) stage_tile(j, 0);
+  // ---- main loop, software pipelined inside each wave: in step `it` the wave issues the Q.K^T MFMAs of tile
+  // t[it+1] and, while the matrix pipe works on them, runs the softmax of tile t[it] on the vector ALU, then the
+  // P.V MFMAs of tile t[it].  LDS therefore holds K(t[it+1]) and V^T(t[it]) while K(t[it+2]) and V^T(t[it+1])
+  // stream in.
+  int j = (segA_hi > 0) ? 0 : segB_lo;         // t[it]
+  int j1 = next_tile(j);                       // t[it+1]
+  if (j < segB_hi) {
+    stage_k(j, 0);
+    stage_v(j, 0);
+    if (j1 < segB_hi) stage_k(j1, 1);
+  }
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
-
-  for (int it = 0; j < segB_hi; ++it) {
-    const int jn = next_tile(j);
-    const bool have_next = jn < segB_hi;
-    if (have_next) stage_tile(jn, (it + 1) & 1);   // the other stage was last read before the previous barrier
-    const char* kbuf = smem + (it & 1) * kStageBytes;
-    const char* vbuf = kbuf + kKTileBytes;
-
-    if (wave_active && wr.visits(j)) {
-      if constexpr (WAVES < 8) {
-        if (distinct4) {  // switch the Q~ operand set when entering/leaving the 4-bit window range
-          const bool want4 = tile_uses4(j);
-          if (want4 != q_is4) {
-            load_q(want4 ? a.q4 : a.q);
-            q_is4 = want4;
-          }
+  auto switch_q = [&](int jt) {
+    if constexpr (WAVES < 8) {
+      if (distinct4) {  // switch the Q~ operand set when entering/leaving the 4-bit window range
+        const bool want4 = tile_uses4(jt);
+        if (want4 != q_is4) {
+          load_q(want4 ? a.q4 : a.q);
+          q_is4 = want4;
         }
       }
-      tile_body(j, it, kbuf, vbuf, j >= wr.diag_lo);
-    } else if constexpr (MODE == 2) {
-      if (lane == 0) s_amax[it & 1][wave] = 0.f;  // a wave that skips the tile contributes nothing to the block maximum
-      __syncthreads();                            // every wave passes one such barrier per tile
     }
-
-    __builtin_amdgcn_s_waitcnt(0);   // this wave's share of the next tile has landed in LDS
+  };
+  f32x16_t Sa[2], Sb[2];
+  bool vis_cur = wave_active && j < segB_hi && wr.visits(j);
+  if (vis_cur) {
+    switch_q(j);
+    qk_tile(kbase_lds, Sa);
+  }
+  auto step = [&](int it, f32x16_t (&Scur)[2], f32x16_t (&Snxt)[2]) {
+    const int j2 = next_tile(j1);
+    if (j2 < segB_hi) stage_k(j2, it & 1);             // K(t[it]) in that buffer was consumed in the previous step
+    if (j1 < segB_hi) stage_v(j1, (it + 1) & 1);       // so was V^T(t[it-1])
+    const bool vis_nxt = wave_active && j1 < segB_hi && wr.visits(j1);
+    const char* knext = kbase_lds + ((it + 1) & 1) * kKTileBytes;
+    if (vis_nxt) switch_q(j1);
+    if (vis_cur) {
+      // Q.K^T of the next tile is computed even if this wave will not use it (the buffer then holds an older
+      // tile or nothing meaningful; the result is dropped): the common path stays free of branches
+      softmax_pv(j, it, vbase_lds + (it & 1) * kVTileBytes, j >= wr.diag_lo, Scur, knext, Snxt);
+    } else {
+      if (vis_nxt) qk_tile(knext, Snxt);
+      if constexpr (MODE == 2) {
+        if (lane == 0) s_amax[it & 1][wave] = 0.f;  // a wave that skips the tile contributes nothing to the block maximum
+        __syncthreads();                            // every wave passes one such barrier per tile
+      }
+    }
+    __builtin_amdgcn_s_waitcnt(0);   // this wave's share of the staged tiles has landed in LDS
     __syncthreads();
-    j = jn;
+    vis_cur = vis_nxt;
+    j = j1;
+    j1 = j2;
+  };
+  for (int it = 0; j < segB_hi; it += 2) {
+    step(it, Sa, Sb);
+    if (j >= segB_hi) break;
+    step(it + 1, Sb, Sa);
   }
 
   // ---- epilogue: out = acc / l (attn_triton.py:208-209), lse2 = log2(l) + m (:210-213)
@@ -693,7 +738,7 @@ extern "C" int sq_prefill_fwd(const DLTensor* q, const DLTensor* k, const DLTens
     local.sched_xpp = 1;
     blocks = (unsigned)pairs * (unsigned)items;
   }
-  const size_t smem = 2 * kStageBytes;
+  const size_t smem = 2 * (size_t)kStageBytes;
   const bool bf = dt == DType::BF16;
 #define SQ_LAUNCH_PREFILL(BF, W, M)                                                                              \
   do {                                                                                                           \
