@@ -36,8 +36,16 @@ struct DecodeArgs {
   int64_t k_sb, k_sh, k_sn;
   int64_t v_sb, v_sh, v_sn;
   int32_t B, Hq, Hkv, L, group, head_chunks, num_splits, chunk, p_quant;
+  int32_t hpw;  // kv heads per workgroup (1, 2 or 4): 4/hpw waves share one kv head and interleave its tiles
   float sm;  // log2e / sqrt(D_original), rounded to fp32
 };
+
+// 16-byte load of cache data that is read exactly once: non-temporal, so it does not displace useful lines
+__device__ __forceinline__ uint4 stream_load(const uint16_t* p) {
+  typedef __attribute__((ext_vector_type(4))) unsigned u32x4_t;
+  const u32x4_t v = __builtin_nontemporal_load((const u32x4_t*)p);
+  return make_uint4(v[0], v[1], v[2], v[3]);
+}
 
 template <bool BF16>
 __device__ __forceinline__ float elem_to_f32(uint32_t bits16) {
@@ -74,30 +82,40 @@ __global__ __launch_bounds__(kWaves * 64) void decode_splitkv_kernel(DecodeArgs 
   __shared__ float s_m[kWaves][16];
   __shared__ float s_l[kWaves][16];
 
+  // Workgroup = (token range, hpw kv heads, batch).  With hpw = 4 each wave streams one kv head over the same
+  // token range, so the workgroup as a whole reads whole cache rows of an NHD cache ([B, L, Hkv, D]).
   const int split = blockIdx.x;
-  const int kvh = blockIdx.y / a.head_chunks;
+  const int hy = blockIdx.y / a.head_chunks;
   const int hc = blockIdx.y % a.head_chunks;
   const int b = blockIdx.z;
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r = lane & 15;
   const int g = lane >> 4;
+  const int wpg = kWaves / a.hpw;            // waves per kv head
+  const int hsub = wave / wpg;               // which kv head of the workgroup this wave serves
+  const int wsub = wave % wpg;               // its position among the waves of that head
+  const int kvh = hy * a.hpw + hsub;
 
   int Lb = a.seqlens ? a.seqlens[b] : a.L;
   Lb = min(max(Lb, 0), a.L);
-  const int t0 = split * a.chunk;
-  const int t1 = min(t0 + a.chunk, Lb);
+  // Tokens are dealt to the workgroups tile by tile (tile = 16 tokens): workgroup `split` takes tiles split,
+  // split + S, split + 2S, ...  At any moment all resident workgroups then read neighbouring tiles, i.e. the chip
+  // sweeps the cache front to back, which HBM serves much better than hundreds of separate streams.
+  const int t1 = Lb;
+  const int ntiles_all = (Lb + kTile - 1) / kTile;
+  const int ntiles = (ntiles_all - split + a.num_splits - 1) / a.num_splits;   // tiles of this workgroup (<= 0: none)
   const int h0 = hc * 16;                    // first head of this chunk inside the kv group
   const int nh = min(16, a.group - h0);      // heads handled here
-  const int hq0 = kvh * a.group + h0;        // absolute first q head
+  const int hq0 = kvh * a.group + h0;        // absolute first q head of this wave
 
-  if (t1 <= t0) {  // empty split: weight 0 in the merge
-    for (int i = threadIdx.x; i < nh * kD; i += blockDim.x) {
-      const int h = i / kD, d = i % kD;
-      a.part_o[(((int64_t)b * a.Hq + hq0 + h) * a.num_splits + split) * kD + d] = 0.f;
+  if (ntiles <= 0) {  // empty split: weight 0 in the merge
+    for (int i = threadIdx.x; i < a.hpw * nh * kD; i += blockDim.x) {
+      const int hs = i / (nh * kD), h = (i / kD) % nh, d = i % kD;
+      const int hq = (hy * a.hpw + hs) * a.group + h0 + h;
+      a.part_o[(((int64_t)b * a.Hq + hq) * a.num_splits + split) * kD + d] = 0.f;
+      if (d == 0) a.part_lse[((int64_t)b * a.Hq + hq) * a.num_splits + split] = -INFINITY;
     }
-    if (threadIdx.x < nh)
-      a.part_lse[((int64_t)b * a.Hq + hq0 + threadIdx.x) * a.num_splits + split] = -INFINITY;
     return;
   }
 
@@ -131,22 +149,21 @@ __global__ __launch_bounds__(kWaves * 64) void decode_splitkv_kernel(DecodeArgs 
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-  const int ntiles = (t1 - t0 + kTile - 1) / kTile;
-  for (int tile = wave; tile < ntiles; tile += kWaves) {
-    const int n0 = t0 + tile * kTile;
-    // loads are clamped to the last valid token so that nothing past the valid prefix is touched
-    uint4 kf[4], vf[4];
-    {
-      const int tk = min(n0 + r, t1 - 1);
-      const uint16_t* kp = kbase + (int64_t)tk * a.k_sn + 8 * g;
+  // loads are clamped to the last valid token so that nothing past the valid prefix is touched
+  auto load_tile = [&](int tile, uint4 (&kf)[4], uint4 (&vf)[4]) {
+    const int n0 = (split + tile * a.num_splits) * kTile;
+    const int tk = min(n0 + r, t1 - 1);
+    const uint16_t* kp = kbase + (int64_t)tk * a.k_sn + 8 * g;
 #pragma unroll
-      for (int kk = 0; kk < 4; ++kk) kf[kk] = *(const uint4*)(kp + 32 * kk);
+    for (int kk = 0; kk < 4; ++kk) kf[kk] = stream_load(kp + 32 * kk);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int tv = min(n0 + 4 * g + i, t1 - 1);
-        vf[i] = *(const uint4*)(vbase + (int64_t)tv * a.v_sn + 8 * r);
-      }
+    for (int i = 0; i < 4; ++i) {
+      const int tv = min(n0 + 4 * g + i, t1 - 1);
+      vf[i] = stream_load(vbase + (int64_t)tv * a.v_sn + 8 * r);
     }
+  };
+  auto compute_tile = [&](int tile, const uint4 (&kf)[4], const uint4 (&vf)[4]) {
+    const int n0 = (split + tile * a.num_splits) * kTile;
     f32x4_t s = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) s = mfma_qk<BF16>(kf[kk], qf[kk], s);
@@ -187,9 +204,23 @@ __global__ __launch_bounds__(kWaves * 64) void decode_splitkv_kernel(DecodeArgs 
       }
     }
     m = m_new;
+  };
+  // two register sets: the loads of the wave's next tile are in flight while it works on the current one
+  uint4 kA[4], vA[4], kB[4], vB[4];
+  int tile = wsub;
+  if (tile < ntiles) load_tile(tile, kA, vA);
+  while (tile < ntiles) {
+    const int t2 = tile + wpg;
+    if (t2 < ntiles) load_tile(t2, kB, vB);
+    compute_tile(tile, kA, vA);
+    if (t2 >= ntiles) break;
+    const int t3 = t2 + wpg;
+    if (t3 < ntiles) load_tile(t3, kA, vA);
+    compute_tile(t2, kB, vB);
+    tile = t3;
   }
 
-  // fold the 4 lane groups' shares of l, then merge the 4 waves through LDS
+  // fold the 4 lane groups' shares of l, then merge the waves that share a kv head through LDS
   l += __shfl_xor(l, 16);
   l += __shfl_xor(l, 32);
 #pragma unroll
@@ -201,19 +232,19 @@ __global__ __launch_bounds__(kWaves * 64) void decode_splitkv_kernel(DecodeArgs 
     s_l[wave][r] = l;
   }
   __syncthreads();
-  for (int idx = threadIdx.x; idx < nh * kD; idx += blockDim.x) {
-    const int h = idx / kD, d = idx % kD;
+  for (int idx = threadIdx.x; idx < a.hpw * nh * kD; idx += blockDim.x) {
+    const int hs = idx / (nh * kD), h = (idx / kD) % nh, d = idx % kD;
+    const int w0 = hs * wpg;
     float mm = -INFINITY;
-#pragma unroll
-    for (int w = 0; w < kWaves; ++w) mm = fmaxf(mm, s_m[w][h]);
+    for (int w = 0; w < wpg; ++w) mm = fmaxf(mm, s_m[w0 + w][h]);
     float lt = 0.f, o = 0.f;
-#pragma unroll
-    for (int w = 0; w < kWaves; ++w) {
-      const float sc = exp2f(s_m[w][h] - mm);  // 0 for a wave that saw no tile (m = -inf)
-      lt += s_l[w][h] * sc;
-      o += s_o[w][h][d] * sc;
+    for (int w = 0; w < wpg; ++w) {
+      const float sc = exp2f(s_m[w0 + w][h] - mm);  // 0 for a wave that saw no tile (m = -inf)
+      lt += s_l[w0 + w][h] * sc;
+      o += s_o[w0 + w][h][d] * sc;
     }
-    const int64_t row = ((int64_t)b * a.Hq + hq0 + h) * a.num_splits + split;
+    const int hq = (hy * a.hpw + hs) * a.group + h0 + h;
+    const int64_t row = ((int64_t)b * a.Hq + hq) * a.num_splits + split;
     a.part_o[row * kD + d] = o / lt;
     if (d == 0) a.part_lse[row] = mm + log2f(lt);
   }
@@ -228,31 +259,70 @@ struct CombineArgs {
   int32_t Hq, num_splits, out_dtype;  // 0 bf16, 1 f16, 2 f32
 };
 
-__global__ __launch_bounds__(kD) void decode_combine_kernel(CombineArgs a) {
-  const int h = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
-  const int64_t row0 = ((int64_t)b * a.Hq + h) * a.num_splits;
+constexpr int kCombineThreads = 1024;
+constexpr int kCombineGroups = kCombineThreads / kD;   // 8 groups of 128 threads, each sums every 8th split
+
+// One workgroup per (q head, batch): weights of all splits are formed in parallel in LDS, then 8 groups of 128
+// threads (one thread per output channel) each sum an eighth of the splits with independent, unrolled loads.
+__global__ __launch_bounds__(kCombineThreads) void decode_combine_kernel(CombineArgs a) {
+  extern __shared__ float s_w[];          // [num_splits] weights, then [8][128] partial outputs
+  __shared__ float s_red[kCombineThreads];
+  const int h = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
+  const int S = a.num_splits;
+  const int64_t row0 = ((int64_t)b * a.Hq + h) * S;
   float mx = -INFINITY;
-  for (int s = 0; s < a.num_splits; ++s) mx = fmaxf(mx, a.part_lse[row0 + s]);
-  float tot = 0.f, o = 0.f;
-  if (mx > -INFINITY) {
-    for (int s = 0; s < a.num_splits; ++s) {
-      const float w = exp2f(a.part_lse[row0 + s] - mx);
-      if (w > 0.f) {
-        tot += w;
-        o += w * a.part_o[(row0 + s) * kD + d];
-      }
+  for (int s = tid; s < S; s += kCombineThreads) mx = fmaxf(mx, a.part_lse[row0 + s]);
+  s_red[tid] = mx;
+  __syncthreads();
+  for (int d = kCombineThreads / 2; d > 0; d >>= 1) {
+    if (tid < d) s_red[tid] = fmaxf(s_red[tid], s_red[tid + d]);
+    __syncthreads();
+  }
+  mx = s_red[0];
+  __syncthreads();
+  float tot = 0.f;
+  for (int s = tid; s < S; s += kCombineThreads) {
+    const float w = (mx > -INFINITY) ? exp2f(a.part_lse[row0 + s] - mx) : 0.f;
+    s_w[s] = w;
+    tot += w;
+  }
+  s_red[tid] = tot;
+  __syncthreads();
+  for (int d = kCombineThreads / 2; d > 0; d >>= 1) {
+    if (tid < d) s_red[tid] += s_red[tid + d];
+    __syncthreads();
+  }
+  tot = s_red[0];
+  const int d = tid & (kD - 1), grp = tid >> 7;
+  const float* po = a.part_o + row0 * kD + d;
+  constexpr int G = kCombineGroups;
+  float o = 0.f;
+  int s = grp;
+  for (; s + 3 * G < S; s += 4 * G) {   // 4 independent loads in flight
+    const float w0 = s_w[s], w1 = s_w[s + G], w2 = s_w[s + 2 * G], w3 = s_w[s + 3 * G];
+    const float x0 = po[(int64_t)s * kD], x1 = po[(int64_t)(s + G) * kD], x2 = po[(int64_t)(s + 2 * G) * kD],
+                x3 = po[(int64_t)(s + 3 * G) * kD];
+    o += w0 * x0 + w1 * x1 + w2 * x2 + w3 * x3;   // an empty split has weight 0 and a zero partial
+  }
+  for (; s < S; s += G) o += s_w[s] * po[(int64_t)s * kD];
+  float* s_part = s_w + S;
+  s_part[grp * kD + d] = o;
+  __syncthreads();
+  if (grp == 0) {
+    o = 0.f;
+#pragma unroll
+    for (int q = 0; q < G; ++q) o += s_part[q * kD + d];
+    o = (tot > 0.f) ? o / tot : 0.f;
+    const int64_t off = (int64_t)b * a.o_sb + (int64_t)h * a.o_sh + d;
+    if (a.out_dtype == 0) {
+      ((uint16_t*)a.out)[off] = (uint16_t)f32_to_bf16_bits(o);
+    } else if (a.out_dtype == 1) {
+      ((_Float16*)a.out)[off] = (_Float16)o;
+    } else {
+      ((float*)a.out)[off] = o;
     }
-    o /= tot;
+    if (a.lse && d == 0) a.lse[(int64_t)b * a.Hq + h] = (tot > 0.f) ? mx + log2f(tot) : -INFINITY;
   }
-  const int64_t off = (int64_t)b * a.o_sb + (int64_t)h * a.o_sh + d;
-  if (a.out_dtype == 0) {
-    ((uint16_t*)a.out)[off] = (uint16_t)f32_to_bf16_bits(o);
-  } else if (a.out_dtype == 1) {
-    ((_Float16*)a.out)[off] = (_Float16)o;
-  } else {
-    ((float*)a.out)[off] = o;
-  }
-  if (a.lse && d == 0) a.lse[(int64_t)b * a.Hq + h] = (mx > -INFINITY) ? mx + log2f(tot) : -INFINITY;
 }
 
 }  // namespace
@@ -262,10 +332,13 @@ using namespace sq;
 
 extern "C" int32_t sq_decode_num_splits(int64_t batch, int64_t num_kv_heads, int64_t max_len) {
   if (batch <= 0 || num_kv_heads <= 0 || max_len <= 0) return 1;
-  // about 4 workgroups per CU over 256 CUs, at least 256 tokens (4 waves x 4 tiles) per workgroup
-  const int64_t target_blocks = 1024;
-  int64_t s = (target_blocks + batch * num_kv_heads - 1) / (batch * num_kv_heads);
-  const int64_t max_s = (max_len + 255) / 256;
+  // two workgroups per CU over 256 CUs, all resident at once (a second round of workgroups would leave a tail);
+  // at least 256 tokens (4 waves x 4 tiles) per workgroup
+  const int64_t target_blocks = 512;
+  const int64_t hpw = (num_kv_heads % 4 == 0) ? 4 : ((num_kv_heads % 2 == 0) ? 2 : 1);
+  const int64_t groups = batch * (num_kv_heads / hpw);
+  int64_t s = (target_blocks + groups - 1) / groups;
+  const int64_t max_s = (max_len * hpw + 255) / 256;   // at least 4 tiles of 16 tokens per wave
   if (s > max_s) s = max_s;
   if (s < 1) s = 1;
   if (s > 4096) s = 4096;
@@ -358,6 +431,7 @@ extern "C" int sq_decode_fwd(const DLTensor* q, const DLTensor* kcache, const DL
   a.L = (int32_t)L;
   a.group = (int32_t)group;
   a.head_chunks = (int32_t)((group + 15) / 16);
+  a.hpw = (Hkv % 4 == 0) ? 4 : ((Hkv % 2 == 0) ? 2 : 1);
   a.num_splits = S;
   a.chunk = (int32_t)chunk;
   a.p_quant = params->p_quant;
@@ -369,7 +443,7 @@ extern "C" int sq_decode_fwd(const DLTensor* q, const DLTensor* kcache, const DL
   int cur = -1;
   SQ_HIP(hipGetDevice(&cur));
   SQ_REQUIRE(cur == dev, SQ_EDEVICE, "sq_decode_fwd: tensors live on device %d but the current device is %d", dev, cur);
-  const dim3 grid((unsigned)S, (unsigned)(Hkv * a.head_chunks), (unsigned)B);
+  const dim3 grid((unsigned)S, (unsigned)(Hkv / a.hpw * a.head_chunks), (unsigned)B);
   if (dt == DType::BF16) {
     hipLaunchKernelGGL(decode_splitkv_kernel<true>, grid, dim3(kWaves * 64), 0, st, a);
   } else {
@@ -386,7 +460,7 @@ extern "C" int sq_decode_fwd(const DLTensor* q, const DLTensor* kcache, const DL
   c.Hq = (int32_t)Hq;
   c.num_splits = S;
   c.out_dtype = odt == DType::BF16 ? 0 : (odt == DType::F16 ? 1 : 2);
-  hipLaunchKernelGGL(decode_combine_kernel, dim3((unsigned)Hq, (unsigned)B), dim3(kD), 0, st, c);
+  hipLaunchKernelGGL(decode_combine_kernel, dim3((unsigned)Hq, (unsigned)B), dim3(kCombineThreads), (size_t)(S + kCombineGroups * kD) * sizeof(float), st, c);
   SQ_HIP(hipGetLastError());
   return SQ_OK;
 }
