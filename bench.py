@@ -22,6 +22,9 @@ sys.path.insert(0, ROOT)
 METRIC = "prefill attn TFLOP/s @128K + decode HBM GB/s @1M, Qwen2.5-7B GQA 28/4 heads"
 PEAK_MFMA_BF16_TFLOPS = 2500.0   # MI355X dense bf16/fp16 MFMA
 PEAK_HBM_GBS = 8000.0            # MI355X HBM3E
+# L2<->fabric bytes of one prefill_kernel launch at seq 131072, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a
+# 1 GiB copy (x2.000 / x1.000): 16.26 GB fetched + 0.94 GB written (profiles/prefill_kernel_128k.md)
+PREFILL_TRAFFIC_BYTES_128K = 17.2e9
 
 
 def log(*a):
@@ -63,7 +66,7 @@ def time_prefill(torch, N, steps, warmup, p_quant):
     return ms, flops
 
 
-def time_decode(torch, B, L, iters=20, warmup=5):
+def time_decode(torch, B, L, iters=10, warmup=5, rounds=7):
     from longcontext_sqattn_paddle_amd.sqattn.attn_triton_decode import DecodePlan
 
     dev = torch.device("cuda:0")
@@ -83,15 +86,47 @@ def time_decode(torch, B, L, iters=20, warmup=5):
     for i in range(warmup):
         plans[i % nset].run()
     torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record(stream)
-    for i in range(iters):
-        plans[i % nset].run()
-    e1.record(stream)
-    torch.cuda.synchronize()
-    us = e0.elapsed_time(e1) / iters * 1e3
+    samples = []
+    for _ in range(rounds):   # median over rounds of `iters` back-to-back calls (HIP events on the launch stream)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for i in range(iters):
+            plans[i % nset].run()
+        e1.record(stream)
+        torch.cuda.synchronize()
+        samples.append(e0.elapsed_time(e1) / iters * 1e3)
+    us = sorted(samples)[len(samples) // 2]
     nbytes = 2048.0 * total   # K+V bf16, 4 kv heads x 128, read once for all 7 q-heads of a group
     return us, nbytes
+
+
+def time_kmeans(torch, iters=10):
+    """One Lloyd iteration (assign + counting sort + exact cluster sums + centroid update) at the benchmark's
+    clustering shape: 4 kv heads x 131072 tokens x 128, 1024 centroids."""
+    from longcontext_sqattn_paddle_amd import workloads
+    from longcontext_sqattn_paddle_amd.cache_hub.kmeans import _triton_k_means_train, _workspace
+
+    dev = torch.device("cuda:0")
+    G, N, C, D = 4, 131072, 1024, 128
+    key, _ = workloads.kmeans_inputs(G, N, D, seed=4)
+    key = key.to(dev)
+    idx0 = (torch.arange(C, dtype=torch.float32) * (N / C) + N / C / 2).to(torch.int64).to(dev)
+    cent = key.index_select(1, idx0).contiguous()
+    ws = _workspace(G, N, C, dev)
+    idx = torch.empty(G, N, dtype=torch.int32, device=dev)
+    for _ in range(2):
+        _triton_k_means_train(key, cent, max_idx=idx, workspace=ws)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        _triton_k_means_train(key, cent, max_idx=idx, workspace=ws)
+    e1.record()
+    torch.cuda.synchronize()
+    us = e0.elapsed_time(e1) / iters * 1e3
+    flops = 2.0 * N * C * D * G
+    nbytes = G * (N * D * 2 * 2 + N * 4 * 3 + C * D * 2 * 2)   # K read by assign and by the cluster sums, idx/order, centroids
+    return us, flops, nbytes
 
 
 def main():
@@ -100,7 +135,12 @@ def main():
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--seq-len", type=int, default=131072)
-    ap.add_argument("--p-quant", type=int, default=1, help="0 none, 1 e4m3 static 448 (reference), 2 e4m3 block absmax")
+    ap.add_argument("--p-quant", type=int, default=3,
+                    help="0 none, 1 e4m3 static 448 exactly as the reference rounds it, 2 e4m3 block absmax, "
+                         "3 e4m3 static 448 with the scale folded into the exponent (default)")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="run one 1 GiB device-to-device copy first: a kernel of known traffic for scaling FETCH_SIZE/WRITE_SIZE")
+    ap.add_argument("--no-kmeans", action="store_true")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode", action="store_true")
     args = ap.parse_args()
@@ -114,6 +154,13 @@ def main():
         print("bench.py needs an MI355X (torch.cuda.is_available() is False)", file=sys.stderr)
         sys.exit(3)
     N = args.seq_len
+    if args.calibration_copy:
+        src = torch.ones(1 << 29, dtype=torch.bfloat16, device="cuda:0")   # 1 GiB read + 1 GiB written
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+        torch.cuda.empty_cache()
     ms, flops = time_prefill(torch, N, args.steps, args.warmup, args.p_quant)
     tflops = flops / ms / 1e9
     log(f"[bench] prefill N={N}: {ms:.2f} ms/step, {tflops:.1f} TFLOP/s")
@@ -143,7 +190,7 @@ def main():
             "peak": PEAK_MFMA_BF16_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(tflops / PEAK_MFMA_BF16_TFLOPS, 4),
-            "traffic": None,
+            "traffic": PREFILL_TRAFFIC_BYTES_128K if N == 131072 else None,
         },
     }
     if not args.no_decode:
@@ -156,6 +203,13 @@ def main():
             log(f"[bench] decode {name}: {us:.1f} us, {gbs:.0f} GB/s")
             torch.cuda.empty_cache()
         result["decode"] = dec
+    if not args.no_kmeans:
+        us, kflops, kbytes = time_kmeans(torch)
+        result["kmeans"] = {"us_per_iteration": round(us, 1), "TFLOP_per_s": round(kflops / us / 1e6, 1),
+                            "frac_of_bf16_mfma_peak": round(kflops / us / 1e6 / PEAK_MFMA_BF16_TFLOPS, 4),
+                            "GB_per_s": round(kbytes / us / 1e3, 1), "frac_of_hbm_peak": round(kbytes / us / 1e3 / PEAK_HBM_GBS, 4),
+                            "shape": "4 heads x 131072 tokens x 128, 1024 centroids, one Lloyd iteration"}
+        log(f"[bench] kmeans iteration: {us:.0f} us")
     if not args.no_cpu_baseline:
         from oracle.cpu_baseline import time_cpu_baseline   # the checker's CPU path, timed as the baseline only
 
