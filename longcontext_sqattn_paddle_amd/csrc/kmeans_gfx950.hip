@@ -15,8 +15,6 @@ namespace {
 
 constexpr int kD = 128;
 constexpr int kCB = 64;            // centroids per LDS stage
-constexpr int kCStride = 272;      // bytes per centroid row in LDS (256 + 16 pad)
-constexpr int kStage = kCB * kCStride;
 constexpr int kTileTok = 256;      // tokens per workgroup in assign / sort kernels
 constexpr int kMaxC = 8192;
 
@@ -30,105 +28,112 @@ struct AssignArgs {
   const uint16_t* data;  // [G,N,128] bf16
   const uint16_t* cent;  // [G,C,128] bf16
   int32_t* idx;          // [G,N]
-  int32_t* cnt;          // [G,C] (pre-zeroed)
-  int64_t d_sg, d_sn, c_sg, c_sc, i_sg, n_sg;
+  int64_t d_sg, d_sn, c_sg, c_sc, i_sg;
   int32_t N, C;
 };
 
-__global__ __launch_bounds__(256, 2) void kmeans_assign_kernel(AssignArgs a) {
-  __shared__ __attribute__((aligned(16))) char smem[2 * kStage];
-  const int g_id = blockIdx.y;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int c32 = lane & 31, g = lane >> 5;
-  const int tok0 = blockIdx.x * kTileTok + wave * 64;
+constexpr int kAssignWaves = 8;   // x 32 tokens: 2 waves per SIMD, one wave's arg-max epilogue overlaps the other's MFMAs
 
-  // token fragments (B operand of S^T = Cent . Data^T): lane (column = token c32 of block bm, k-group g)
+// Workgroup = 256 tokens of one group.  Centroids stream through LDS in blocks of 64 (global_load_lds, unpadded
+// rows, 16-byte chunks XOR-swizzled by row so that the MFMA operand reads are conflict free); the scores of
+// block k+1 are issued on the matrix pipe before the arg-max epilogue of block k runs on the vector ALU.
+__global__ __launch_bounds__(kAssignWaves * 64) void kmeans_assign_kernel(AssignArgs a) {
+  __shared__ __attribute__((aligned(16))) char smem[2 * kCB * 256];
+  typedef __attribute__((address_space(3))) void* lds_ptr_t;
+  const int g_id = blockIdx.y;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int c32 = lane & 31, g = lane >> 5;
+  const int tok0 = blockIdx.x * kTileTok + wave * 32;
+
+  // token fragments (B operand of S^T = Cent . Data^T): lane (column = token c32, k-group g)
   const uint16_t* db = a.data + (int64_t)g_id * a.d_sg;
-  uint4 tf[2][8];
-#pragma unroll
-  for (int bm = 0; bm < 2; ++bm) {
-    const int n = min(tok0 + 32 * bm + c32, a.N - 1);
+  uint4 tf[8];
+  {
+    const int n = min(tok0 + c32, a.N - 1);
     const uint16_t* rp = db + (int64_t)n * a.d_sn + 8 * g;
 #pragma unroll
-    for (int kk = 0; kk < 8; ++kk) tf[bm][kk] = *(const uint4*)(rp + 16 * kk);
+    for (int kk = 0; kk < 8; ++kk) tf[kk] = *(const uint4*)(rp + 16 * kk);
   }
-  float best[2] = {-INFINITY, -INFINITY};
-  int bidx[2] = {0, 0};
-
   const uint16_t* cb = a.cent + (int64_t)g_id * a.c_sg;
-  uint4 creg[4];
-  auto gload = [&](int chunk) {
+  auto stage = [&](int chunk, int st) {
+    char* buf = smem + st * (kCB * 256);
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      const int ch = c * 256 + tid;
-      const int row = min(chunk * kCB + (ch >> 4), a.C - 1);
-      creg[c] = *(const uint4*)(cb + (int64_t)row * a.c_sc + 8 * (ch & 15));
+    for (int c = 0; c < 2; ++c) {
+      const int q = wave * 2 + c;                      // 1 KB = 4 centroid rows per wave instruction
+      const int row = 4 * q + (lane >> 4);
+      const int ch = (lane & 15) ^ (row & 15);
+      const int crow = min(chunk * kCB + row, a.C - 1);
+      __builtin_amdgcn_global_load_lds((const void*)(cb + (int64_t)crow * a.c_sc + 8 * ch), (lds_ptr_t)(buf + q * 1024), 16, 0, 0);
     }
   };
-  auto lstore = [&](int stage) {
-    char* buf = smem + stage * kStage;
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      const int ch = c * 256 + tid;
-      *(uint4*)(buf + (ch >> 4) * kCStride + (ch & 15) * 16) = creg[c];
-    }
-  };
-  const int nchunks = (a.C + kCB - 1) / kCB;
-  gload(0);
-  lstore(0);
-  __syncthreads();
-  for (int chunk = 0; chunk < nchunks; ++chunk) {
-    const bool have_next = chunk + 1 < nchunks;
-    if (have_next) gload(chunk + 1);
-    const char* buf = smem + (chunk & 1) * kStage;
-    f32x16_t S[2][2];
+  const int ksw = c32 & 15;
+  auto scores = [&](const char* buf, f32x16_t (&S)[2]) {
 #pragma unroll
     for (int bn = 0; bn < 2; ++bn)
 #pragma unroll
-      for (int bm = 0; bm < 2; ++bm)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) S[bn][bm][i] = 0.f;
+      for (int i = 0; i < 16; ++i) S[bn][i] = 0.f;
 #pragma unroll
     for (int kk = 0; kk < 8; ++kk) {
-      const uint4 a0 = *(const uint4*)(buf + c32 * kCStride + (16 * kk + 8 * g) * 2);
-      const uint4 a1 = *(const uint4*)(buf + (32 + c32) * kCStride + (16 * kk + 8 * g) * 2);
-      S[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a0), __builtin_bit_cast(bf16x8_t, tf[0][kk]), S[0][0], 0, 0, 0);
-      S[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a0), __builtin_bit_cast(bf16x8_t, tf[1][kk]), S[0][1], 0, 0, 0);
-      S[1][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a1), __builtin_bit_cast(bf16x8_t, tf[0][kk]), S[1][0], 0, 0, 0);
-      S[1][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a1), __builtin_bit_cast(bf16x8_t, tf[1][kk]), S[1][1], 0, 0, 0);
+      const uint4 a0 = *(const uint4*)(buf + c32 * 256 + (((2 * kk + g) ^ ksw) << 4));
+      const uint4 a1 = *(const uint4*)(buf + (32 + c32) * 256 + (((2 * kk + g) ^ ksw) << 4));
+      S[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a0), __builtin_bit_cast(bf16x8_t, tf[kk]), S[0], 0, 0, 0);
+      S[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a1), __builtin_bit_cast(bf16x8_t, tf[kk]), S[1], 0, 0, 0);
     }
-    // running arg-max in ascending centroid order with strict '>' = lowest index on ties (kmeans.py:62-65)
-    const bool tail = (chunk + 1) * kCB > a.C;
+  };
+  // Running arg-max in ascending centroid order with strict '>' = lowest index on ties (kmeans.py:62-65).  The
+  // winner is tracked as (block, position inside the block): positions are inline constants, so an element
+  // costs a compare and two selects.  Rows past C (C % 64 == 32) are clamped copies of the last centroid; they
+  // come after it in this order and can never beat it strictly.
+  float best = -INFINITY;
+  int bloc = 0, bchunk = 0;
+  auto argmax = [&](int chunk, const f32x16_t (&S)[2]) {
+    const float before = best;
 #pragma unroll
-    for (int bm = 0; bm < 2; ++bm)
+    for (int bn = 0; bn < 2; ++bn)
 #pragma unroll
-      for (int bn = 0; bn < 2; ++bn)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int c = chunk * kCB + 32 * bn + 8 * (i >> 2) + 4 * g + (i & 3);
-          float s = S[bn][bm][i];
-          if (tail && c >= a.C) s = -INFINITY;
-          if (s > best[bm]) {
-            best[bm] = s;
-            bidx[bm] = c;
-          }
-        }
-    if (have_next) lstore((chunk + 1) & 1);
-    __syncthreads();
+      for (int i = 0; i < 16; ++i) {
+        const float s = S[bn][i];
+        const bool gt = s > best;
+        bloc = gt ? (32 * bn + 8 * (i >> 2) + (i & 3)) : bloc;
+        best = gt ? s : best;
+      }
+    bchunk = (best > before) ? chunk : bchunk;
+  };
+  const int nchunks = (a.C + kCB - 1) / kCB;
+  stage(0, 0);
+  if (nchunks > 1) stage(1, 1);
+  __builtin_amdgcn_s_waitcnt(0);
+  __syncthreads();
+  f32x16_t Sa[2], Sb[2];
+  scores(smem, Sa);
+  __syncthreads();                                             // every wave has read block 0 out of LDS
+  auto step = [&](int chunk, f32x16_t (&Scur)[2], f32x16_t (&Snxt)[2]) {
+    // LDS holds block chunk+1; block `chunk` was read by every wave before the last barrier, so its buffer is free
+    if (chunk + 2 < nchunks) stage(chunk + 2, chunk & 1);
+    // unconditional, so that these MFMAs share a straight-line block with the arg-max below; after the last block
+    // they run once more on stale data and the result is dropped
+    scores(smem + ((chunk + 1) & 1) * (kCB * 256), Snxt);
+    argmax(chunk, Scur);
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();                                           // block chunk+2 has landed, block chunk+1 has been read
+  };
+  for (int chunk = 0; chunk < nchunks; chunk += 2) {
+    step(chunk, Sa, Sb);
+    if (chunk + 1 >= nchunks) break;
+    step(chunk + 1, Sb, Sa);
   }
-#pragma unroll
-  for (int bm = 0; bm < 2; ++bm) {
-    const float ob = __shfl_xor(best[bm], 32);
-    const int oi = __shfl_xor(bidx[bm], 32);
-    if (ob > best[bm] || (ob == best[bm] && oi < bidx[bm])) {
-      best[bm] = ob;
-      bidx[bm] = oi;
+  {
+    int bidx = bchunk * kCB + 4 * g + bloc;
+    const float ob = __shfl_xor(best, 32);
+    const int oi = __shfl_xor(bidx, 32);
+    if (ob > best || (ob == best && oi < bidx)) {
+      best = ob;
+      bidx = oi;
     }
-    const int n = tok0 + 32 * bm + c32;
-    if (g == 0 && n < a.N) {
-      a.idx[(int64_t)g_id * a.i_sg + n] = bidx[bm];
-      atomicAdd(a.cnt + (int64_t)g_id * a.n_sg + bidx[bm], 1);
-    }
+    const int n = tok0 + c32;
+    // cluster sizes come out of the counting sort that follows (per-tile histograms), not out of global atomics
+    if (g == 0 && n < a.N) a.idx[(int64_t)g_id * a.i_sg + n] = bidx;
   }
 }
 
@@ -158,17 +163,34 @@ __global__ __launch_bounds__(kTileTok) void sort_hist_kernel(SortArgs a) {
   for (int c = threadIdx.x; c < a.C; c += blockDim.x) out[c] = hist[c];
 }
 
+// Exclusive prefix over tiles of every cluster's per-tile count.  Workgroup = 32 clusters x 8 tile segments:
+// each thread sums its segment, the 8 segment sums are scanned through LDS, then each thread rewrites its segment.
 __global__ __launch_bounds__(256) void sort_scan_tiles_kernel(SortArgs a) {
-  const int c = blockIdx.x * blockDim.x + threadIdx.x, g = blockIdx.y;
-  if (c >= a.C) return;
+  __shared__ int32_t seg_sum[8][32];
+  const int cl = threadIdx.x & 31, seg = threadIdx.x >> 5;
+  const int c = blockIdx.x * 32 + cl, g = blockIdx.y;
+  const int per = (a.nT + 7) / 8;
+  const int tb = seg * per, te = min(tb + per, a.nT);
   int32_t* h = a.tile_hist + (int64_t)g * a.nT * a.C + c;
-  int run = 0;
-  for (int t = 0; t < a.nT; ++t) {
+  int sum = 0;
+  if (c < a.C)
+    for (int t = tb; t < te; ++t) sum += h[(int64_t)t * a.C];
+  seg_sum[seg][cl] = sum;
+  __syncthreads();
+  int run = 0, total = 0;
+#pragma unroll
+  for (int q = 0; q < 8; ++q) {
+    const int v = seg_sum[q][cl];
+    if (q < seg) run += v;
+    total += v;
+  }
+  if (c >= a.C) return;
+  for (int t = tb; t < te; ++t) {
     const int v = h[(int64_t)t * a.C];
     h[(int64_t)t * a.C] = run;
     run += v;
   }
-  a.total[(int64_t)g * a.C + c] = run;
+  if (seg == 0) a.total[(int64_t)g * a.C + c] = total;
 }
 
 __global__ __launch_bounds__(1024) void sort_scan_clusters_kernel(SortArgs a) {
@@ -413,7 +435,7 @@ int run_sort(const DLTensor* idx, char* wsp, const WsLayout& w, int32_t* dst, in
   s.M = M;
   s.use_off = use_off;
   hipLaunchKernelGGL(sort_hist_kernel, dim3(w.nT, (unsigned)G), dim3(kTileTok), (size_t)C * 4, st, s);
-  hipLaunchKernelGGL(sort_scan_tiles_kernel, dim3((C + 255) / 256, (unsigned)G), dim3(256), 0, st, s);
+  hipLaunchKernelGGL(sort_scan_tiles_kernel, dim3((C + 31) / 32, (unsigned)G), dim3(256), 0, st, s);
   if (use_off) hipLaunchKernelGGL(sort_scan_clusters_kernel, dim3((unsigned)G), dim3(1024), 0, st, s);
   hipLaunchKernelGGL(sort_scatter_kernel, dim3(w.nT, (unsigned)G), dim3(kTileTok), 0, st, s);
   SQ_HIP(hipGetLastError());
@@ -467,24 +489,21 @@ extern "C" int sq_kmeans_train(const DLTensor* data, DLTensor* centroids, DLTens
   hipStream_t st = (hipStream_t)stream;
   char* wsp = data_of(workspace);
 
-  hipLaunchKernelGGL(fill_i32_kernel, dim3(64), dim3(256), 0, st, (int32_t*)data_of(cnt), G * C, 0);
   AssignArgs a;
   a.data = (const uint16_t*)data_of(data);
   a.cent = (const uint16_t*)data_of(centroids);
   a.idx = (int32_t*)data_of(idx);
-  a.cnt = (int32_t*)data_of(cnt);
   a.d_sg = stride_of(data, 0);
   a.d_sn = stride_of(data, 1);
   a.c_sg = stride_of(centroids, 0);
   a.c_sc = stride_of(centroids, 1);
   a.i_sg = stride_of(idx, 0);
-  a.n_sg = stride_of(cnt, 0);
   a.N = (int)N;
   a.C = (int)C;
-  hipLaunchKernelGGL(kmeans_assign_kernel, dim3((unsigned)((N + kTileTok - 1) / kTileTok), (unsigned)G), dim3(256), 0, st, a);
+  hipLaunchKernelGGL(kmeans_assign_kernel, dim3((unsigned)((N + kTileTok - 1) / kTileTok), (unsigned)G), dim3(kAssignWaves * 64), 0, st, a);
   SQ_HIP(hipGetLastError());
   int32_t* order = (int32_t*)(wsp + w.off_bytes + w.hist_bytes);
-  if ((rc = run_sort(idx, wsp, w, order, N, 0, 0, true, nullptr, (int)C, st))) return rc;
+  if ((rc = run_sort(idx, wsp, w, order, N, 0, 0, true, (int32_t*)data_of(cnt), (int)C, st))) return rc;   // cnt = cluster sizes
   SumArgs s;
   s.src = a.data;
   s.order = order;
