@@ -21,6 +21,9 @@ sys.path.insert(0, ROOT)
 
 METRIC = "prefill attn TFLOP/s @128K + decode HBM GB/s @1M, Qwen2.5-7B GQA 28/4 heads"
 PEAK_MFMA_BF16_TFLOPS = 2500.0   # MI355X dense bf16/fp16 MFMA
+PEAK_MFMA_FP8_TFLOPS = 5000.0    # MI355X dense fp8 MFMA
+# Q.K^T (half of the FLOPs) runs on the bf16 pipe, P.V (the other half) on the fp8 pipe in the default mode
+PEAK_MFMA_BLEND_TFLOPS = 1.0 / (0.5 / PEAK_MFMA_BF16_TFLOPS + 0.5 / PEAK_MFMA_FP8_TFLOPS)
 PEAK_HBM_GBS = 8000.0            # MI355X HBM3E
 # L2<->fabric bytes of one prefill_kernel launch at seq 131072, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a
 # 1 GiB copy (x2.000 / x1.000): 16.26 GB fetched + 0.94 GB written (profiles/prefill_kernel_128k.md)
@@ -135,9 +138,11 @@ def main():
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--seq-len", type=int, default=131072)
-    ap.add_argument("--p-quant", type=int, default=3,
+    ap.add_argument("--p-quant", type=int, default=4,
                     help="0 none, 1 e4m3 static 448 exactly as the reference rounds it, 2 e4m3 block absmax, "
-                         "3 e4m3 static 448 with the scale folded into the exponent (default)")
+                         "3 e4m3 static 448 with the scale folded into the exponent, "
+                         "4 (default) = 3 plus e4m3 V so that P.V runs on the fp8 matrix pipe")
+    ap.add_argument("--variants", action="store_true", help="also time P modes 1 and 3 (fp16 P.V) and report them")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="run one 1 GiB device-to-device copy first: a kernel of known traffic for scaling FETCH_SIZE/WRITE_SIZE")
     ap.add_argument("--no-kmeans", action="store_true")
@@ -164,6 +169,10 @@ def main():
     ms, flops = time_prefill(torch, N, args.steps, args.warmup, args.p_quant)
     tflops = flops / ms / 1e9
     log(f"[bench] prefill N={N}: {ms:.2f} ms/step, {tflops:.1f} TFLOP/s")
+    if args.p_quant == 4:
+        peak, peak_note = PEAK_MFMA_BLEND_TFLOPS, "harmonic blend: Q.K^T on bf16 MFMA (2.5 PFLOP/s), P.V on fp8 MFMA (5.0 PFLOP/s)"
+    else:
+        peak, peak_note = PEAK_MFMA_BF16_TFLOPS, "both GEMMs on 16-bit MFMA"
 
     result = {
         "metric": METRIC,
@@ -180,19 +189,28 @@ def main():
         "data": "synthetic",
         "config": {
             "workload": f"prefill attention, batch 1, 28 q heads / 4 kv heads, head_dim 128, seq {N}, causal, "
-                        f"bf16 N(0,1)/sqrt(128) with 2% K outlier channels x8, P quant mode {args.p_quant} (e4m3), fp32 accumulate",
+                        f"bf16 N(0,1)/sqrt(128) with 2% K outlier channels x8, P quant mode {args.p_quant} "
+                        f"({'e4m3 P and e4m3 V, fp8 MFMA P.V' if args.p_quant == 4 else 'e4m3 P, fp16 MFMA P.V' if args.p_quant else 'no P quantisation'}), fp32 accumulate",
             "flops_per_step": flops,
         },
         "roofline": {
             "bound": "mfma",
             "kernel": "prefill_kernel",
             "achieved": round(tflops, 2),
-            "peak": PEAK_MFMA_BF16_TFLOPS,
+            "peak": round(peak, 1),
+            "peak_note": peak_note,
             "unit": "TFLOP/s",
-            "frac": round(tflops / PEAK_MFMA_BF16_TFLOPS, 4),
+            "frac": round(tflops / peak, 4),
+            "frac_of_bf16_peak": round(tflops / PEAK_MFMA_BF16_TFLOPS, 4),
             "traffic": PREFILL_TRAFFIC_BYTES_128K if N == 131072 else None,
         },
     }
+    if args.variants:
+        result["variants"] = {}
+        for mode, name in ((3, "e4m3_P_fp16_PV"), (1, "e4m3_P_reference_rounding_fp16_PV")):
+            vms, _ = time_prefill(torch, N, args.steps, args.warmup, mode)
+            result["variants"][name] = {"p_quant": mode, "ms_per_step": round(vms, 3), "TFLOP_per_s": round(flops / vms / 1e9, 1)}
+            log(f"[bench] prefill variant {name}: {vms:.2f} ms")
     if not args.no_decode:
         dec = {}
         for name, B, L in (("1M_b1", 1, 1048576), ("128K_b1", 1, 131072), ("128K_b8", 8, 131072)):

@@ -51,9 +51,12 @@ enum {
   SQ_P_NONE = 0,         /* p.to(fp16)                               attn_triton.py:83           */
   SQ_P_E4M3_STATIC = 1,  /* fp16(fp16(e4m3(p*448))/448)              attn_triton.py:81-82        */
   SQ_P_E4M3_BLOCK = 2,   /* per (64 rows x 64 keys) absmax scale a: e4m3(p*448/a)*a/448 (no ref.) */
-  SQ_P_E4M3_STATIC_FAST = 3 /* same e4m3 grid as STATIC with the factor 448 folded into the exponent  */
+  SQ_P_E4M3_STATIC_FAST = 3, /* same e4m3 grid as STATIC with the factor 448 folded into the exponent  */
                          /* of p and the 1/448 cancelled against the denominator: skips the       */
                          /* reference's fp16 rounding of p/448 (relative 2^-11), prefill only      */
+  SQ_P_E4M3_FP8_PV = 4   /* e4m3 P as in STATIC_FAST *and* e4m3 V (one scale per batch, kv head and   */
+                         /* channel, from a pre-pass): P.V runs on the fp8 matrix pipe.  No reference */
+                         /* counterpart (it keeps V in fp16, attn_triton.py:83); prefill only         */
 };
 
 enum { SQ_WINDOW_NONE = 0, SQ_WINDOW_SIZES = 1 };

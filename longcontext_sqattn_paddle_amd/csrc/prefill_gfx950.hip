@@ -43,7 +43,9 @@ struct PrefillArgs {
   const void* k;
   const void* q4;   // operands of the 4-bit window range (null: same as q/k)
   const void* k4;
-  const _Float16* vt;  // [B, Hkv, nT, 128, 64] fp16 transposed, permuted V tiles
+  const _Float16* vt;  // [B, Hkv, nT, 128, 64] fp16 transposed, permuted V tiles (MODE 0..3)
+  const uint8_t* vt8;  // [B, Hkv, nT, 128, 64] e4m3 transposed, permuted V tiles (MODE 4)
+  const float* v_inv_scale;  // [B, Hkv, 128] absmax/448 per channel (MODE 4)
   void* out;
   float* lse;
   int64_t q_sb, q_sh, q_sn;
@@ -60,6 +62,9 @@ struct PrefillArgs {
 struct PrepArgs {
   const void* v;
   _Float16* vt;
+  uint8_t* vt8;          // e4m3 tiles (MODE 4)
+  uint32_t* vmax_bits;   // [B, Hkv, 128] running |v| maximum as fp32 bit patterns (MODE 4)
+  float* v_inv_scale;    // [B, Hkv, 128]
   int64_t v_sb, v_sh, v_sn;
   int32_t Nk, nT, Hkv, is_bf16;
 };
@@ -92,6 +97,90 @@ __global__ __launch_bounds__(256) void prefill_prep_v_kernel(PrepArgs a) {
   for (int e = 0; e < 8; ++e) {
     f16x4_t val = {h[0][e], h[1][e], h[2][e], h[3][e]};
     *(f16x4_t*)(tile + (8 * o + e) * kBN + pos) = val;
+  }
+}
+
+// ---- fp8 P.V path (MODE 4): V is quantised to e4m3 with one scale per (batch, kv head, channel).
+// (1) per-channel |v| maximum over all keys: every workgroup reduces one 64-key tile and merges with an integer
+// atomic max (non-negative floats order like their bit patterns).
+__global__ void prefill_fill_u32_kernel(uint32_t* p, int n) {
+  for (int i = threadIdx.x; i < n; i += blockDim.x) p[i] = 0u;
+}
+
+__global__ __launch_bounds__(256) void prefill_vabsmax_kernel(PrepArgs a) {
+  __shared__ float red[16][kD];
+  const int j = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+  const int o = threadIdx.x & 15, tq = threadIdx.x >> 4;
+  const uint16_t* vb = (const uint16_t*)a.v + (int64_t)b * a.v_sb + (int64_t)kvh * a.v_sh;
+  float mx[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int n = j * kBN + 4 * tq + i;
+    if (n < a.Nk) {
+      const uint4 raw = *(const uint4*)(vb + (int64_t)n * a.v_sn + 8 * o);
+      const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const uint32_t bits = (e & 1) ? (w[e >> 1] >> 16) : (w[e >> 1] & 0xffffu);
+        const float x = a.is_bf16 ? bf16_bits_to_f32(bits) : (float)__builtin_bit_cast(_Float16, (uint16_t)bits);
+        mx[e] = fmaxf(mx[e], fabsf(x));
+      }
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) red[tq][8 * o + e] = mx[e];
+  __syncthreads();
+  if (threadIdx.x < kD) {
+    float m = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) m = fmaxf(m, red[r][threadIdx.x]);
+    atomicMax(a.vmax_bits + ((int64_t)b * a.Hkv + kvh) * kD + threadIdx.x, __float_as_uint(m));
+  }
+}
+
+// (2) e4m3 tiles, transposed and permuted for v_mfma_f32_32x32x64_f8f6f4: key u of a tile sits at byte
+// 32 g + 16 bn + 4 (w >> 3) + (w & 3) of its channel row, with bn = u >> 5, w = u & 31, g = (w >> 2) & 1 -- the order
+// in which a lane of the S^T accumulator holds its 32 keys.
+__global__ __launch_bounds__(256) void prefill_prep_v8_kernel(PrepArgs a) {
+  const int j = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+  const int o = threadIdx.x & 15;    // channel octet
+  const int tq = threadIdx.x >> 4;   // key quad
+  const uint16_t* vb = (const uint16_t*)a.v + (int64_t)b * a.v_sb + (int64_t)kvh * a.v_sh;
+  const int64_t ch0 = ((int64_t)b * a.Hkv + kvh) * kD + 8 * o;
+  float sc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    // power-of-two scale 2^floor(log2(448/amax)): bf16/fp16 values times it are exact in fp32, so the e4m3
+    // conversion only ever sees exact values (v_cvt_pk_fp8_f32 mis-rounds inputs that lie within an fp32 ulp or
+    // two of a tie, which arbitrary scales hit systematically for 8-bit-mantissa inputs); fp8 is a floating
+    // format, so a power-of-two scale costs no precision
+    const float amax = __uint_as_float(a.vmax_bits[ch0 + e]);
+    int ex = 1;
+    if (amax > 0.f) (void)frexpf(448.f / amax, &ex);   // 448/amax = f * 2^ex, f in [0.5, 1)
+    sc[e] = ldexpf(1.f, ex - 1);
+    if (j == 0 && tq == 0) a.v_inv_scale[ch0 + e] = ldexpf(1.f, 1 - ex);
+  }
+  float x[4][8];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int n = j * kBN + 4 * tq + i;
+    uint4 raw = make_uint4(0, 0, 0, 0);
+    if (n < a.Nk) raw = *(const uint4*)(vb + (int64_t)n * a.v_sn + 8 * o);
+    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const uint32_t bits = (e & 1) ? (w[e >> 1] >> 16) : (w[e >> 1] & 0xffffu);
+      const float v = a.is_bf16 ? bf16_bits_to_f32(bits) : (float)__builtin_bit_cast(_Float16, (uint16_t)bits);
+      x[i][e] = fminf(fmaxf(v * sc[e], -448.f), 448.f);
+    }
+  }
+  uint8_t* tile = a.vt8 + (((int64_t)b * a.Hkv + kvh) * a.nT + j) * (int64_t)(kD * kBN);
+  const int pos = 32 * (tq & 1) + 16 * (tq >> 3) + 4 * ((tq >> 1) & 3);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    int pk = __builtin_amdgcn_cvt_pk_fp8_f32(x[0][e], x[1][e], 0, false);
+    pk = __builtin_amdgcn_cvt_pk_fp8_f32(x[2][e], x[3][e], pk, true);
+    *(int*)(tile + (8 * o + e) * kBN + pos) = pk;
   }
 }
 
@@ -324,7 +413,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
   // Online-softmax state of this lane's query row.  The score accumulators are *initialised* with
   // cinit = kC - m_run (kC = log2(448) in MODE 3, else 0), so the MFMA chain delivers S - m_run + kC and, as
   // long as the running maximum does not move, p (or 448 p) is a bare exp2 of the accumulator.
-  constexpr float kC = (MODE == 3) ? kLog2_448 : 0.f;
+  constexpr float kC = (MODE >= 3) ? kLog2_448 : 0.f;
   float m_run = 0.f;       // reference point of the exponent; the first visited tile replaces it by the row maximum
   float l_run = 0.f;       // this lane's share of the denominator (times 448 in MODE 3)
   bool first = true;       // wave-uniform: no tile visited yet
@@ -355,6 +444,15 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
   };
   auto stage_v = [&](int j, int stage) {
     char* vbuf = vbase_lds + stage * kVTileBytes;
+    if constexpr (MODE == 4) {
+      // e4m3 tile: 128 rows x 64 bytes = 8 KB, one wave instruction per wave; 16-byte chunk c of row d -> slot
+      // c ^ ((d >> 2) & 3), which spreads the 16 rows a quarter-wave reads over all 16 bank groups
+      const uint8_t* vsrc8 = a.vt8 + (((int64_t)b * a.Hkv + kvh) * a.nT + j) * (int64_t)(kD * kBN);
+      const int vr = 16 * wave + (lane >> 2);
+      const int vc = (lane & 3) ^ ((vr >> 2) & 3);
+      __builtin_amdgcn_global_load_lds((const void*)(vsrc8 + vr * kBN + 16 * vc), (lds_ptr_t)(vbuf + wave * 1024), 16, 0, 0);
+      return;
+    }
     const _Float16* vsrc = vt_base + (int64_t)j * (kD * kBN);
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
@@ -459,11 +557,34 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
       sc = 448.f / amax;   // amax > 0: every visited tile has an unmasked key in every row
       inv = amax / 448.f;
     }
+    if constexpr (MODE == 4) {
+      // P^T as the e4m3 B operand of one K=64 fp8 MFMA per 32 output channels: byte 16 bn + i of this lane's
+      // 32 bytes is the probability in S[bn][i]; the V^T tiles were permuted to the same key order
+      typedef __attribute__((ext_vector_type(8))) int i32x8_t;
+      i32x8_t P8;
+#pragma unroll
+      for (int bn = 0; bn < 2; ++bn)
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+          int pk = __builtin_amdgcn_cvt_pk_fp8_f32(S[bn][4 * q4], S[bn][4 * q4 + 1], (bn | q4) ? P8[0] : 0, false);
+          P8[4 * bn + q4] = __builtin_amdgcn_cvt_pk_fp8_f32(S[bn][4 * q4 + 2], S[bn][4 * q4 + 3], pk, true);
+        }
+      const int vsw4 = (c32 >> 2) & 3;
+#pragma unroll
+      for (int bd = 0; bd < 4; ++bd) {
+        const char* rowp = vbuf + (32 * bd + c32) * 64;
+        const uint4 lo = *(const uint4*)(rowp + (((2 * g) ^ vsw4) << 4));
+        const uint4 hi = *(const uint4*)(rowp + (((2 * g + 1) ^ vsw4) << 4));
+        const i32x8_t av = {(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+        O[bd] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, P8, O[bd], 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
+      }
+      return;
+    }
     uint4 P[2][2];  // [bn][t]
 #pragma unroll
     for (int bn = 0; bn < 2; ++bn)
 #pragma unroll
-      for (int t = 0; t < 2; ++t) P[bn][t] = quant_pack8<MODE>(S[bn], t, sc, inv);
+      for (int t = 0; t < 2; ++t) P[bn][t] = quant_pack8<(MODE == 4 ? 3 : MODE)>(S[bn], t, sc, inv);
     // O^T[d, row] += V^T[d, key] . P^T[key, row]
 #pragma unroll
     for (int bd = 0; bd < 4; ++bd)
@@ -550,6 +671,13 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
       float v[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) v[e] = O[bd][4 * i4 + e] / l;
+      if constexpr (MODE == 4) {  // undo the per-channel V scale
+        const float4 isc = *(const float4*)(a.v_inv_scale + ((int64_t)b * a.Hkv + kvh) * kD + d);
+        v[0] *= isc.x;
+        v[1] *= isc.y;
+        v[2] *= isc.z;
+        v[3] *= isc.w;
+      }
       if (a.out_dtype == 0) {
         uint2 w = make_uint2(f32_to_bf16_bits(v[0]) | (f32_to_bf16_bits(v[1]) << 16),
                              f32_to_bf16_bits(v[2]) | (f32_to_bf16_bits(v[3]) << 16));
@@ -562,7 +690,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
       }
     }
   if (a.lse && g == 0) {
-    const float lt = (MODE == 3) ? l * (1.0f / 448.0f) : l;
+    const float lt = (MODE >= 3) ? l * (1.0f / 448.0f) : l;
     a.lse[((int64_t)b * a.Hq + head) * a.Nq + row] = log2f(lt) + m_run;
   }
 }
@@ -585,7 +713,7 @@ extern "C" int sq_prefill_fwd(const DLTensor* q, const DLTensor* k, const DLTens
   SQ_REQUIRE(p, SQ_EINVAL, "sq_prefill_fwd: params is null");
   SQ_REQUIRE(q && k && v && out, SQ_EINVAL, "sq_prefill_fwd: q, k, v and out must be non-null");
   SQ_REQUIRE(p->layout == SQ_LAYOUT_HND || p->layout == SQ_LAYOUT_NHD, SQ_EINVAL, "tensor_layout %d not supported", p->layout);
-  SQ_REQUIRE(p->p_quant >= SQ_P_NONE && p->p_quant <= SQ_P_E4M3_STATIC_FAST, SQ_EINVAL, "sq_prefill_fwd: p_quant %d not supported", p->p_quant);
+  SQ_REQUIRE(p->p_quant >= SQ_P_NONE && p->p_quant <= SQ_P_E4M3_FP8_PV, SQ_EINVAL, "sq_prefill_fwd: p_quant %d not supported", p->p_quant);
   SQ_REQUIRE((q4 == nullptr) == (k4 == nullptr), SQ_EINVAL, "sq_prefill_fwd: q4 and k4 must be given together");
   int rc;
   const int dev = q->device.device_id;
@@ -653,6 +781,8 @@ extern "C" int sq_prefill_fwd(const DLTensor* q, const DLTensor* k, const DLTens
     SQ_REQUIRE(p->window_mode == SQ_WINDOW_NONE, SQ_EINVAL, "sq_prefill_fwd: window_mode %d not supported", p->window_mode);
     SQ_REQUIRE(!q4, SQ_EINVAL, "sq_prefill_fwd: q4/k4 only apply to window mode");
   }
+  SQ_REQUIRE(!(p->p_quant == SQ_P_E4M3_FP8_PV && q4), SQ_EUNSUPPORTED,
+             "sq_prefill_fwd: the fp8 P.V mode does not take separate 4-bit operands");
   const size_t need = sq_prefill_workspace_bytes(B, Hkv, Nk, D);
   SQ_REQUIRE(workspace && on_gpu(workspace) && workspace->device.device_id == dev, SQ_EWORKSPACE,
              "sq_prefill_fwd: workspace missing or not on the device");
@@ -666,9 +796,16 @@ extern "C" int sq_prefill_fwd(const DLTensor* q, const DLTensor* k, const DLTens
   SQ_REQUIRE(cur == dev, SQ_EDEVICE, "sq_prefill_fwd: tensors live on device %d but the current device is %d", dev, cur);
 
   const int nT = (int)((Nk + kBN - 1) / kBN);
+  const bool pv8 = p->p_quant == SQ_P_E4M3_FP8_PV;
+  char* wsp = data_of(workspace);
+  // workspace: fp16 tiles (modes 0-3), or e4m3 tiles (half the size) followed by the per-channel scale tables
+  const size_t tiles8 = ((size_t)B * Hkv * nT * (kD * kBN) + 255) / 256 * 256;
   PrepArgs pa;
   pa.v = data_of(v);
-  pa.vt = (_Float16*)data_of(workspace);
+  pa.vt = (_Float16*)wsp;
+  pa.vt8 = (uint8_t*)wsp;
+  pa.vmax_bits = (uint32_t*)(wsp + tiles8);
+  pa.v_inv_scale = (float*)(wsp + tiles8 + (size_t)B * Hkv * kD * 4);
   pa.v_sb = stride_of(v, 0);
   pa.v_sh = stride_of(v, hdim);
   pa.v_sn = stride_of(v, ndim);
@@ -676,7 +813,15 @@ extern "C" int sq_prefill_fwd(const DLTensor* q, const DLTensor* k, const DLTens
   pa.nT = nT;
   pa.Hkv = (int)Hkv;
   pa.is_bf16 = dt == DType::BF16;
-  hipLaunchKernelGGL(prefill_prep_v_kernel, dim3(nT, (unsigned)Hkv, (unsigned)B), dim3(256), 0, st, pa);
+  const dim3 pgrid(nT, (unsigned)Hkv, (unsigned)B);
+  if (pv8) {
+    SQ_REQUIRE(tiles8 + (size_t)B * Hkv * kD * 8 <= need, SQ_EWORKSPACE, "sq_prefill_fwd: workspace too small for the fp8 tiles");
+    hipLaunchKernelGGL(prefill_fill_u32_kernel, dim3(1), dim3(256), 0, st, pa.vmax_bits, (int)(B * Hkv * kD));
+    hipLaunchKernelGGL(prefill_vabsmax_kernel, pgrid, dim3(256), 0, st, pa);
+    hipLaunchKernelGGL(prefill_prep_v8_kernel, pgrid, dim3(256), 0, st, pa);
+  } else {
+    hipLaunchKernelGGL(prefill_prep_v_kernel, pgrid, dim3(256), 0, st, pa);
+  }
   SQ_HIP(hipGetLastError());
 
   PrefillArgs local;  // passed to the kernel by value (about 1.2 KB with the per-head windows)
@@ -686,6 +831,8 @@ extern "C" int sq_prefill_fwd(const DLTensor* q, const DLTensor* k, const DLTens
   local.q4 = q4 ? data_of(q4) : nullptr;
   local.k4 = k4 ? data_of(k4) : nullptr;
   local.vt = pa.vt;
+  local.vt8 = pa.vt8;
+  local.v_inv_scale = pa.v_inv_scale;
   local.out = data_of(out);
   local.lse = lse ? (float*)data_of(lse) : nullptr;
   local.q_sb = stride_of(q, 0);
@@ -752,6 +899,7 @@ extern "C" int sq_prefill_fwd(const DLTensor* q, const DLTensor* k, const DLTens
       case SQ_P_NONE: SQ_LAUNCH_PREFILL(BF, W, 0); break;        \
       case SQ_P_E4M3_STATIC: SQ_LAUNCH_PREFILL(BF, W, 1); break; \
       case SQ_P_E4M3_BLOCK: SQ_LAUNCH_PREFILL(BF, W, 2); break;  \
+      case SQ_P_E4M3_FP8_PV: SQ_LAUNCH_PREFILL(BF, 8, 4); break; \
       default: SQ_LAUNCH_PREFILL(BF, W, 3); break;               \
     }                                                           \
   } while (0)

@@ -21,7 +21,7 @@ LOG2E = 1.44269504  # the literal the reference uses (attn_triton.py:250)
 BLOCK_N = 64        # KV block of every reference prefill/decode kernel (attn_triton.py:253)
 MASK_ADD = -1000000.0  # additive causal mask (attn_triton.py:71)
 
-P_NONE, P_STATIC448, P_BLOCK_ABSMAX = 0, 1, 2
+P_NONE, P_STATIC448, P_BLOCK_ABSMAX, P_STATIC448_GRID = 0, 1, 2, 3
 
 
 # --------------------------------------------------------------------------- helpers
@@ -78,6 +78,7 @@ def _quant_p(p: torch.Tensor, mode: int, group_rows: int = 64) -> torch.Tensor:
     mode 1: `fp16( fp16(e4m3(p*448)) / 448 )`                     (attn_triton.py:81-82)
     mode 2: per (64-row group x 64-col block) absmax scale a: `e4m3(p*(448/a)) * (a/448)` then fp16
             (build-defined generalisation; a == 1 reproduces mode 1 up to the fp16 divide).
+    mode 3: `e4m3(p*448)/448` kept in fp32 (build-defined: P as the fp8 operand of an fp8 P.V product).
     Returns fp32 values that are exactly representable in fp16.
     """
     if mode == P_NONE:
@@ -85,6 +86,8 @@ def _quant_p(p: torch.Tensor, mode: int, group_rows: int = 64) -> torch.Tensor:
     if mode == P_STATIC448:
         p8 = (p * 448.0).to(torch.float8_e4m3fn)
         return (p8.to(torch.float16) / 448).float()
+    if mode == P_STATIC448_GRID:   # the e4m3 grid of mode 1 without the fp16 rounding of p/448 (fp8 operand of an fp8 MFMA)
+        return (p * 448.0).to(torch.float8_e4m3fn).float() / 448.0
     if mode == P_BLOCK_ABSMAX:
         out = torch.empty_like(p)
         for r0 in range(0, p.shape[0], group_rows):
@@ -165,6 +168,7 @@ def prefill_blockwise(
     q4=None, k4=None,
     out_dtype=torch.bfloat16,
     group_rows: int = 64,
+    v_quant: Optional[str] = None,
 ):
     """Blockwise online-softmax prefill exactly in the reference's order of operations.
 
@@ -174,6 +178,9 @@ def prefill_blockwise(
     `w8`/`w4` = per-head window sizes in tokens (None = full causal).  `q4`/`k4` are the 4-bit
     fake-quantised operands used in the 4-bit window (default: alias of q/k, which is what the
     relative wrapper passes, attn_triton_mix_relative.py:441-444).
+    `v_quant="e4m3_channel"` (build-defined, for the fp8 P.V product): V is replaced by
+    `e4m3(v * s_d) / s_d` with the power-of-two scale `s_d = 2^floor(log2(448 / max_n |v[b, kvh, n, d]|))` per
+    (batch, kv head, channel).
     Returns (out [B,Hq,Nq,D] out_dtype, lse2 [B,Hq,Nq] fp32).
     """
     B, Hq, Nq, D = q.shape
@@ -183,7 +190,15 @@ def prefill_blockwise(
     q4f = fold_scale(q4, D).float() if q4 is not None else qf
     kf = k.float()
     k4f = k4.float() if k4 is not None else kf
-    vf = v.to(torch.float16).float()
+    if v_quant is None:
+        vf = v.to(torch.float16).float()
+    elif v_quant == "e4m3_channel":
+        amax = v.float().abs().amax(dim=2, keepdim=True)
+        _, ex = torch.frexp(torch.where(amax > 0, 448.0 / amax, torch.ones_like(amax)))   # 448/amax = f * 2^ex
+        sv = torch.ldexp(torch.ones_like(amax), ex - 1)                                    # 2^floor(log2(448/amax))
+        vf = (v.float() * sv).clamp(-448.0, 448.0).to(torch.float8_e4m3fn).float() / sv
+    else:
+        raise ValueError(f"unknown v_quant {v_quant}")
     out = torch.zeros(B, Hq, Nq, D, dtype=torch.float32)
     lse = torch.zeros(B, Hq, Nq, dtype=torch.float32)
     assert q_offset % block_m == 0

@@ -23,7 +23,7 @@ def _cos(a, b):
     return float(a @ b / (a.norm() * b.norm()))
 
 
-def _check(out, ref, quantised):
+def _check(out, ref, quantised, q_tol=2e-3):
     out, ref = out.double().cpu(), ref.double()
     rms = float(ref.pow(2).mean().sqrt())
     d = (out - ref).abs()
@@ -31,7 +31,7 @@ def _check(out, ref, quantised):
         assert float(d.max()) <= 2e-3 * rms, (float(d.max()), rms)
     else:
         assert _cos(out, ref) >= 0.99999
-        assert float(torch.quantile(d.flatten()[:: max(1, d.numel() // 1000000)], 0.999)) <= 2e-3 * rms
+        assert float(torch.quantile(d.flatten()[:: max(1, d.numel() // 1000000)], 0.999)) <= q_tol * rms
         assert float(d.max()) <= 0.25 * rms, (float(d.max()), rms)
 
 
@@ -58,6 +58,29 @@ def test_causal_matches_oracle(B, Hq, Hkv, N, mode):
     assert torch.allclose(lse.cpu(), lse_ref, atol=2e-4)
     exact, _ = A.exact_attention(q, k, v)
     assert _cos(out.cpu(), exact) >= 0.999
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,N,layout", [(1, 4, 2, 512, "HND"), (2, 14, 2, 700, "NHD"), (1, 7, 1, 2048, "HND")])
+def test_fp8_pv_mode_matches_oracle(B, Hq, Hkv, N, layout):
+    """Mode 4 (no reference counterpart): e4m3 P *and* e4m3 V (per batch/kv-head/channel scale) on the fp8 MFMA."""
+    from longcontext_sqattn_paddle_amd.sqattn.attn_triton import attn_causal
+
+    print(f"case prefill fp8-pv B={B} Hq={Hq} Hkv={Hkv} N={N} {layout}", flush=True)
+    q, k, v = inputs.prefill_inputs(B, Hq, Hkv, N, 128, seed=200 + N) if N == 2048 else _rand(B, Hq, Hkv, N, 128, 200 + N)
+    ref, lse_ref = A.prefill_blockwise(q, k, v, p_quant=A.P_STATIC448_GRID, v_quant="e4m3_channel", out_dtype=torch.float32)
+    args = [t.to(DEV) for t in (q, k, v)]
+    if layout == "NHD":
+        args = [t.permute(0, 2, 1, 3).contiguous() for t in args]
+    out, lse = attn_causal(*args, layout, torch.float32, return_lse=True, p_quant=4)
+    torch.cuda.synchronize()
+    if layout == "NHD":
+        out = out.permute(0, 2, 1, 3)
+    # 99.9 % of elements within 5e-3 * rms here (2e-3 for the fp16 P.V modes): the fp8 matrix instruction sums its 64
+    # products with its own internal alignment, which shows on near-uniform rows of thousands of keys
+    _check(out, ref, True, q_tol=5e-3)
+    assert torch.allclose(lse.cpu(), lse_ref, atol=2e-4)
+    exact, _ = A.exact_attention(q, k, v)
+    assert _cos(out.cpu(), exact) >= 0.999   # thin margin by construction: e4m3 on both operands (about 0.9995)
 
 
 def test_nhd_layout_bf16_out_and_gqa_7():
