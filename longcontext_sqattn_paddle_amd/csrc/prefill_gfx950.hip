@@ -428,8 +428,8 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
   typedef __attribute__((address_space(3))) void* lds_ptr_t;
   auto tile_uses4 = [&](int j) { return distinct4 && j >= wr.r4_lo && j < wr.r4_hi; };
   const int64_t k_head_off = (int64_t)b * a.k_sb + (int64_t)kvh * a.k_sh;
-  char* const kbase_lds = smem;                     // 2 x 16 KB
-  char* const vbase_lds = smem + 2 * kKTileBytes;   // 2 x 16 KB
+  char* const kbase_lds = smem;                     // 4 x 16 KB
+  char* const vbase_lds = smem + 4 * kKTileBytes;   // 4 x 16 KB (8 KB used per buffer in the fp8 mode)
   auto stage_k = [&](int j, int stage) {
     char* kbuf = kbase_lds + stage * kKTileBytes;
     const uint16_t* kb = (const uint16_t*)(tile_uses4(j) ? a.k4 : a.k) + k_head_off;
@@ -599,15 +599,23 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
 
   // ---- main loop, software pipelined inside each wave: in step `it` the wave issues the Q.K^T MFMAs of tile
   // t[it+1] and, while the matrix pipe works on them, runs the softmax of tile t[it] on the vector ALU, then the
-  // P.V MFMAs of tile t[it].  LDS therefore holds K(t[it+1]) and V^T(t[it]) while K(t[it+2]) and V^T(t[it+1])
-  // stream in.
-  int j = (segA_hi > 0) ? 0 : segB_lo;         // t[it]
-  int j1 = next_tile(j);                       // t[it+1]
-  if (j < segB_hi) {
-    stage_k(j, 0);
-    stage_v(j, 0);
-    if (j1 < segB_hi) stage_k(j1, 1);
+  // P.V MFMAs of tile t[it].  K and V^T live in rings of 4 LDS buffers and the workgroup synchronises once per
+  // TWO tiles: at the start of a pair (it even) every wave starts the copies of K(t[it+3]), K(t[it+4]),
+  // V^T(t[it+2]), V^T(t[it+3]) into the buffers the previous pair finished with, and between the barriers the
+  // waves drift apart by up to a tile, which lets one wave's matrix phase overlap another's vector phase.
+  int tq[5];                                   // t[it] .. t[it+4]
+  tq[0] = (segA_hi > 0) ? 0 : segB_lo;
+#pragma unroll
+  for (int u = 1; u < 5; ++u) tq[u] = next_tile(tq[u - 1]);
+  if (tq[0] < segB_hi) {
+    stage_k(tq[0], 0);
+    stage_v(tq[0], 0);
   }
+  if (tq[1] < segB_hi) {
+    stage_k(tq[1], 1);
+    stage_v(tq[1], 1);
+  }
+  if (tq[2] < segB_hi) stage_k(tq[2], 2);
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
   auto switch_q = [&](int jt) {
@@ -622,22 +630,27 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
     }
   };
   f32x16_t Sa[2], Sb[2];
-  bool vis_cur = wave_active && j < segB_hi && wr.visits(j);
+  bool vis_cur = wave_active && tq[0] < segB_hi && wr.visits(tq[0]);
   if (vis_cur) {
-    switch_q(j);
+    switch_q(tq[0]);
     qk_tile(kbase_lds, Sa);
   }
+  __syncthreads();   // ring buffer 0 is about to be refilled: every wave has read K(t[0]) out of it
   auto step = [&](int it, f32x16_t (&Scur)[2], f32x16_t (&Snxt)[2]) {
-    const int j2 = next_tile(j1);
-    if (j2 < segB_hi) stage_k(j2, it & 1);             // K(t[it]) in that buffer was consumed in the previous step
-    if (j1 < segB_hi) stage_v(j1, (it + 1) & 1);       // so was V^T(t[it-1])
+    const int j = tq[0], j1 = tq[1];
+    if ((it & 1) == 0) {   // start of a pair: refill the four buffers the previous pair released
+      if (tq[3] < segB_hi) stage_k(tq[3], (it + 3) & 3);
+      if (tq[4] < segB_hi) stage_k(tq[4], it & 3);
+      if (tq[2] < segB_hi) stage_v(tq[2], (it + 2) & 3);
+      if (tq[3] < segB_hi) stage_v(tq[3], (it + 3) & 3);
+    }
     const bool vis_nxt = wave_active && j1 < segB_hi && wr.visits(j1);
-    const char* knext = kbase_lds + ((it + 1) & 1) * kKTileBytes;
+    const char* knext = kbase_lds + ((it + 1) & 3) * kKTileBytes;
     if (vis_nxt) switch_q(j1);
     if (vis_cur) {
       // Q.K^T of the next tile is computed even if this wave will not use it (the buffer then holds an older
       // tile or nothing meaningful; the result is dropped): the common path stays free of branches
-      softmax_pv(j, it, vbase_lds + (it & 1) * kVTileBytes, j >= wr.diag_lo, Scur, knext, Snxt);
+      softmax_pv(j, it, vbase_lds + (it & 3) * kVTileBytes, j >= wr.diag_lo, Scur, knext, Snxt);
     } else {
       if (vis_nxt) qk_tile(knext, Snxt);
       if constexpr (MODE == 2) {
@@ -645,15 +658,19 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
         __syncthreads();                            // every wave passes one such barrier per tile
       }
     }
-    __builtin_amdgcn_s_waitcnt(0);   // this wave's share of the staged tiles has landed in LDS
-    __syncthreads();
+    if (it & 1) {          // end of a pair
+      __builtin_amdgcn_s_waitcnt(0);   // this wave's share of the tiles staged at the start of the pair has landed
+      __syncthreads();
+    }
     vis_cur = vis_nxt;
-    j = j1;
-    j1 = j2;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) tq[u] = tq[u + 1];
+    tq[4] = next_tile(tq[3]);
   };
-  for (int it = 0; j < segB_hi; it += 2) {
+  // both steps of a pair always run (the second one idles when the tile list has an odd length), so that every
+  // wave passes the same barriers
+  for (int it = 0; tq[0] < segB_hi; it += 2) {
     step(it, Sa, Sb);
-    if (j >= segB_hi) break;
     step(it + 1, Sb, Sa);
   }
 
@@ -885,7 +902,7 @@ extern "C" int sq_prefill_fwd(const DLTensor* q, const DLTensor* k, const DLTens
     local.sched_xpp = 1;
     blocks = (unsigned)pairs * (unsigned)items;
   }
-  const size_t smem = 2 * (size_t)kStageBytes;
+  const size_t smem = 4 * (size_t)kStageBytes;   // rings of 4 K tiles and 4 V^T tiles
   const bool bf = dt == DType::BF16;
 #define SQ_LAUNCH_PREFILL(BF, W, M)                                                                              \
   do {                                                                                                           \
