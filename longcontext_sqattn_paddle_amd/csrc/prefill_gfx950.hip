@@ -273,6 +273,13 @@ __device__ __forceinline__ float max3(float a, float b, float c) {
   return r;
 }
 
+// max3 above is opaque to the compiler's hazard logic, which therefore does not separate it from a matrix
+// instruction that has just written its inputs.  Where a max3 chain directly follows such instructions, this
+// supplies the wait states by hand (the longest requirement, after a 16-pass MFMA, is below 32).
+__device__ __forceinline__ void mfma_settle(f32x16_t& x, f32x16_t& y) {
+  asm volatile("s_nop 15\n\ts_nop 15" : "+v"(x), "+v"(y));
+}
+
 // exchange with the lane 32 away (the other half of the keys of the same query row)
 __device__ __forceinline__ float xor32_max(float v) {
   const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
@@ -284,6 +291,34 @@ __device__ __forceinline__ float xor32_sum(float v) {
 }
 
 constexpr float kLog2_448 = 8.807354922057604f;  // log2(448)
+
+// ---- hand-scheduled LDS reads.  The compiler cannot tell that a ds_read never touches the buffers that
+// global_load_lds copies are still filling, so it would stall every tile on vmcnt(0); reads issued through
+// these helpers are invisible to that logic, and the data dependence is carried by lds_wait instead.
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
+template <int OFF>
+__device__ __forceinline__ u32x4_t lds_read128(uint32_t addr) {
+  u32x4_t r;
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF));
+  return r;
+}
+// wait until at most N LDS reads issued after the one that produced x (and y) are outstanding; LDS reads
+// return in order, so x (and y) have landed afterwards
+template <int N>
+__device__ __forceinline__ void lds_wait(u32x4_t& x) {
+  asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(x) : "n"(N));
+}
+template <int N>
+__device__ __forceinline__ void lds_wait(u32x4_t& x, u32x4_t& y) {
+  asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(x), "+v"(y) : "n"(N));
+}
+template <int I, int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for<I + 1, N>(f);
+  }
+}
 
 // Quantise 8 probabilities (one k-step of the P.V MFMA) and pack them as fp16 B-operand registers.
 //   MODE 0  p.to(fp16)
@@ -462,13 +497,33 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
       __builtin_amdgcn_global_load_lds((const void*)(vsrc + vr * kBN + 8 * vc), (lds_ptr_t)(vbuf + q * 1024), 16, 0, 0);
     }
   };
-  auto next_tile = [&](int j) {
-    int n = j + 1;
-    if (n >= segA_hi && n < segB_lo) n = segB_lo;
-    return n;
+  // staging of full K tiles of the unquantised operand: uniform tile base + per-lane 32-bit offset, no per-lane
+  // 64-bit arithmetic in the loop
+  uint32_t kvoff[CH];
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    const int q = wave * CH + c;
+    const int kr = 4 * q + (lane >> 4);
+    const int kc = (lane & 15) ^ (kr & 15);
+    kvoff[c] = (uint32_t)(kr * (int)a.k_sn + 8 * kc) * 2u;
+  }
+  const char* const k_bytes = (const char*)a.k + k_head_off * 2;
+  const uint32_t k_tile_bytes = (uint32_t)(kBN * a.k_sn * 2);
+  auto stage_k_full = [&](int j, int stage) {
+    const char* base = k_bytes + (uint64_t)(uint32_t)j * k_tile_bytes;
+    char* kbuf = kbase_lds + stage * kKTileBytes;
+#pragma unroll
+    for (int c = 0; c < CH; ++c)
+      __builtin_amdgcn_global_load_lds((const void*)(base + kvoff[c]), (lds_ptr_t)(kbuf + (wave * CH + c) * 1024), 16, 0, 0);
   };
 
   const int ksw = c32 & 15;          // swizzle of this lane's K rows (c32 and c32 + 32 share it)
+  const uint32_t smem_addr = (uint32_t)(uintptr_t)(lds_ptr_t)smem;
+  uint32_t kx[8];                    // byte offset of k-step kk's chunk inside this lane's K rows
+#pragma unroll
+  for (int kk = 0; kk < 8; ++kk) kx[kk] = c32 * kKStride + (((2 * kk + g) ^ ksw) << 4);
+  typedef __attribute__((ext_vector_type(8))) int i32x8_t;
+  i32x8_t P8 = {0, 0, 0, 0, 0, 0, 0, 0};   // MODE 4: e4m3 probabilities of the current tile (registers reused tile after tile)
   const int vsw = (c32 >> 1) & 7;    // swizzle of this lane's V^T rows (32 bd + c32)
 
   // S^T = K . Q~^T + Cinit for one tile: 16 MFMAs that nothing below depends on until the next step
@@ -488,6 +543,22 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
     }
   };
 
+  // MODE 4: maximum over this lane's 32 scores of a tile, as four independent chains
+  auto lane_max = [&](const f32x16_t (&S)[2]) {
+    float c[4];
+#pragma unroll
+    for (int h = 0; h < 4; ++h) {
+      const f32x16_t& s = S[h >> 1];
+      const int o = 8 * (h & 1);
+      c[h] = max3(s[o], s[o + 1], s[o + 2]);
+      c[h] = max3(c[h], s[o + 3], s[o + 4]);
+      c[h] = max3(c[h], s[o + 5], s[o + 6]);
+      c[h] = max3(c[h], s[o + 7], s[o + 7]);
+    }
+    return max3(max3(c[0], c[1], c[2]), c[3], c[3]);
+  };
+  float tmax_lane = 0.f;   // MODE 4: lane_max of the tile whose scores the next step consumes (computed one step ahead)
+
   // softmax update + P.V for the tile whose scores are in S.  Once the running maximum of this tile is settled,
   // the Q.K^T MFMAs of the following tile (K in knext, result in Snext) are issued in the same straight-line
   // block as the exponentials, conversions and P.V MFMAs, so that the matrix pipe and the vector ALU of this
@@ -506,10 +577,16 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
           if (32 * bn + 8 * (i >> 2) + (i & 3) > rel) S[bn][i] = -INFINITY;
     }
     // row maximum of S - m_run + kC; the row's other 32 keys live in lane^32
-    float tmax = max3(S[0][0], S[1][0], S[0][1]);
+    float tmax;
+    if constexpr (MODE == 4) {
+      if (masked) tmax_lane = lane_max(S);
+      tmax = tmax_lane;   // came out of the previous step's P.V phase
+    } else {
+      tmax = max3(S[0][0], S[1][0], S[0][1]);
 #pragma unroll
-    for (int i = 1; i < 15; ++i) tmax = max3(tmax, S[1][i], S[0][i + 1]);
-    tmax = max3(tmax, S[1][15], S[1][15]);
+      for (int i = 1; i < 15; ++i) tmax = max3(tmax, S[1][i], S[0][i + 1]);
+      tmax = max3(tmax, S[1][15], S[1][15]);
+    }
     tmax = xor32_max(tmax);
     if (first || __any(tmax > kC)) {
       // some row's maximum moved by d (on the first tile: from the arbitrary reference 0 to the row maximum):
@@ -529,6 +606,79 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) Cinit[i] = c;
       first = false;
+    }
+    if constexpr (MODE == 4) {
+      __builtin_amdgcn_s_setprio(0);
+      // Hand-scheduled tile step.  16 slots of {Q.K^T MFMA of the next tile, one LDS prefetch, two exponentials
+      // and one e4m3 pack of the current tile}, then 4 slots of {fp8 P.V MFMA, two LDS prefetches, 8 additions of
+      // the row sum}.  K fragments are read 4 slots ahead of the MFMA that consumes them.
+      // P^T is the e4m3 B operand of one K=64 MFMA per 32 output channels: byte 16 bn + i of this lane's
+      // 32 bytes is the probability in S[bn][i]; the V^T tiles were permuted to the same key order.
+      const uint32_t kaddr = smem_addr + ((it + 1) & 3) * kKTileBytes;
+      const uint32_t vlo_addr = smem_addr + 4 * kKTileBytes + (it & 3) * kVTileBytes + c32 * 64 + (((2 * g) ^ ((c32 >> 2) & 3)) << 4);
+      const uint32_t vhi_addr = vlo_addr ^ 16;
+      u32x4_t kf[16], vlo[4], vhi[4];
+      auto kread = [&](auto I) {
+        constexpr int i = decltype(I)::value;
+        kf[i] = lds_read128<(i & 1) * 32 * kKStride>(kaddr + kx[i >> 1]);
+      };
+      static_for<0, 4>(kread);
+      static_for<0, 16>([&](auto I) {
+        constexpr int i = decltype(I)::value;
+        constexpr int bn = i & 1, kk = i >> 1;
+        lds_wait<3>(kf[i]);
+        const uint4 ka = make_uint4(kf[i][0], kf[i][1], kf[i][2], kf[i][3]);
+        if constexpr (kk == 0) Snext[bn] = mfma_qk32<BF16>(ka, qf[0], Cinit);
+        else Snext[bn] = mfma_qk32<BF16>(ka, qf[kk], Snext[bn]);
+        if constexpr (i + 4 < 16) kread(std::integral_constant<int, i + 4>{});
+        else if constexpr (i == 12) vlo[0] = lds_read128<0>(vlo_addr);
+        else if constexpr (i == 13) vhi[0] = lds_read128<0>(vhi_addr);
+        else if constexpr (i == 14) vlo[1] = lds_read128<2048>(vlo_addr);
+        else vhi[1] = lds_read128<2048>(vhi_addr);
+        constexpr int sb = i >> 3, e = 2 * (i & 7), r = 4 * sb + ((i & 7) >> 1);
+        const float p0 = __builtin_amdgcn_exp2f(S[sb][e]), p1 = __builtin_amdgcn_exp2f(S[sb][e + 1]);
+        S[sb][e] = p0;
+        S[sb][e + 1] = p1;
+        P8[r] = __builtin_amdgcn_cvt_pk_fp8_f32(p0, p1, P8[r], (i & 1) != 0);
+        __builtin_amdgcn_sched_barrier(0);
+      });
+      // P.V slots: the vector ALU is nearly idle under the four K=64 MFMAs, so the row sum of this tile and the
+      // lane maximum of the next tile's scores are computed here
+      float ps[2] = {0.f, 0.f}, cm[4];
+      static_for<0, 4>([&](auto I) {
+        constexpr int bd = decltype(I)::value;
+        lds_wait<(bd < 3 ? 2 : 0)>(vlo[bd], vhi[bd]);
+        const i32x8_t av = {(int)vlo[bd][0], (int)vlo[bd][1], (int)vlo[bd][2], (int)vlo[bd][3],
+                            (int)vhi[bd][0], (int)vhi[bd][1], (int)vhi[bd][2], (int)vhi[bd][3]};
+        O[bd] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, P8, O[bd], 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
+        if constexpr (bd + 2 < 4) {
+          vlo[bd + 2] = lds_read128<(bd + 2) * 2048>(vlo_addr);
+          vhi[bd + 2] = lds_read128<(bd + 2) * 2048>(vhi_addr);
+        }
+        if constexpr (bd < 2) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            ps[0] += S[bd][e];
+            ps[1] += S[bd][8 + e];
+          }
+        } else {
+          const f32x16_t& sn = Snext[bd - 2];
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            const int o = 8 * h;
+            float c = max3(sn[o], sn[o + 1], sn[o + 2]);
+            c = max3(c, sn[o + 3], sn[o + 4]);
+            c = max3(c, sn[o + 5], sn[o + 6]);
+            cm[2 * (bd - 2) + h] = max3(c, sn[o + 7], sn[o + 7]);
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      });
+      tmax_lane = max3(max3(cm[0], cm[1], cm[2]), cm[3], cm[3]);
+      const float psum = ps[0] + ps[1];
+      l_run += psum;
+      __builtin_amdgcn_s_setprio(3);
+      return;
     }
     qk_tile(knext, Snext);   // scores of the next tile, relative to the maximum just settled
     float psum = 0.f;
@@ -557,29 +707,6 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
       sc = 448.f / amax;   // amax > 0: every visited tile has an unmasked key in every row
       inv = amax / 448.f;
     }
-    if constexpr (MODE == 4) {
-      // P^T as the e4m3 B operand of one K=64 fp8 MFMA per 32 output channels: byte 16 bn + i of this lane's
-      // 32 bytes is the probability in S[bn][i]; the V^T tiles were permuted to the same key order
-      typedef __attribute__((ext_vector_type(8))) int i32x8_t;
-      i32x8_t P8;
-#pragma unroll
-      for (int bn = 0; bn < 2; ++bn)
-#pragma unroll
-        for (int q4 = 0; q4 < 4; ++q4) {
-          int pk = __builtin_amdgcn_cvt_pk_fp8_f32(S[bn][4 * q4], S[bn][4 * q4 + 1], (bn | q4) ? P8[0] : 0, false);
-          P8[4 * bn + q4] = __builtin_amdgcn_cvt_pk_fp8_f32(S[bn][4 * q4 + 2], S[bn][4 * q4 + 3], pk, true);
-        }
-      const int vsw4 = (c32 >> 2) & 3;
-#pragma unroll
-      for (int bd = 0; bd < 4; ++bd) {
-        const char* rowp = vbuf + (32 * bd + c32) * 64;
-        const uint4 lo = *(const uint4*)(rowp + (((2 * g) ^ vsw4) << 4));
-        const uint4 hi = *(const uint4*)(rowp + (((2 * g + 1) ^ vsw4) << 4));
-        const i32x8_t av = {(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
-        O[bd] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, P8, O[bd], 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
-      }
-      return;
-    }
     uint4 P[2][2];  // [bn][t]
 #pragma unroll
     for (int bn = 0; bn < 2; ++bn)
@@ -603,19 +730,29 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
   // TWO tiles: at the start of a pair (it even) every wave starts the copies of K(t[it+3]), K(t[it+4]),
   // V^T(t[it+2]), V^T(t[it+3]) into the buffers the previous pair finished with, and between the barriers the
   // waves drift apart by up to a tile, which lets one wave's matrix phase overlap another's vector phase.
-  int tq[5];                                   // t[it] .. t[it+4]
-  tq[0] = (segA_hi > 0) ? 0 : segB_lo;
-#pragma unroll
-  for (int u = 1; u < 5; ++u) tq[u] = next_tile(tq[u - 1]);
-  if (tq[0] < segB_hi) {
-    stage_k(tq[0], 0);
-    stage_v(tq[0], 0);
+  // The schedule is addressed by a flat step index t = 0 .. nTot-1: the sink tiles [0, nA) first, then the tiles
+  // [segB_lo, segB_hi).  The ring buffer of step t is t & 3.
+  const int nA = segA_hi, shiftB = segB_lo - segA_hi;
+  const int nTot = max(nA + segB_hi - segB_lo, 0);
+  auto tile_of = [&](int t) { return t < nA ? t : t + shiftB; };
+  // steps whose K tile is complete (only the very last tile of the sequence can be partial)
+  const int nFull = (nTot > 0 && (tile_of(nTot - 1) + 1) * kBN > a.Nk) ? nTot - 1 : nTot;
+  // this wave's tiles in step space: [0, fa) (sink) and [fb, fe] (window up to its diagonal tile); from step fm
+  // on the causal mask applies.  A wave without rows visits nothing.
+  const int fa = wave_active ? wr.sink_hi : 0;
+  const int fb = wave_active ? wr.win_lo - shiftB : (1 << 30);
+  const int fe = wr.diag_hi - shiftB, fm = wr.diag_lo - shiftB;
+  auto visits_step = [&](int t) { return t < fa || (t >= fb && t <= fe); };
+
+  if (0 < nTot) {
+    stage_k(tile_of(0), 0);
+    stage_v(tile_of(0), 0);
   }
-  if (tq[1] < segB_hi) {
-    stage_k(tq[1], 1);
-    stage_v(tq[1], 1);
+  if (1 < nTot) {
+    stage_k(tile_of(1), 1);
+    stage_v(tile_of(1), 1);
   }
-  if (tq[2] < segB_hi) stage_k(tq[2], 2);
+  if (2 < nTot) stage_k(tile_of(2), 2);
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
   auto switch_q = [&](int jt) {
@@ -630,48 +767,69 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
     }
   };
   f32x16_t Sa[2], Sb[2];
-  bool vis_cur = wave_active && tq[0] < segB_hi && wr.visits(tq[0]);
+  bool vis_cur = nTot > 0 && visits_step(0);
   if (vis_cur) {
-    switch_q(tq[0]);
+    switch_q(tile_of(0));
     qk_tile(kbase_lds, Sa);
-  }
-  __syncthreads();   // ring buffer 0 is about to be refilled: every wave has read K(t[0]) out of it
-  auto step = [&](int it, f32x16_t (&Scur)[2], f32x16_t (&Snxt)[2]) {
-    const int j = tq[0], j1 = tq[1];
-    if ((it & 1) == 0) {   // start of a pair: refill the four buffers the previous pair released
-      if (tq[3] < segB_hi) stage_k(tq[3], (it + 3) & 3);
-      if (tq[4] < segB_hi) stage_k(tq[4], it & 3);
-      if (tq[2] < segB_hi) stage_v(tq[2], (it + 2) & 3);
-      if (tq[3] < segB_hi) stage_v(tq[3], (it + 3) & 3);
+    if constexpr (MODE == 4) {
+      mfma_settle(Sa[0], Sa[1]);
+      tmax_lane = lane_max(Sa);
     }
-    const bool vis_nxt = wave_active && j1 < segB_hi && wr.visits(j1);
-    const char* knext = kbase_lds + ((it + 1) & 3) * kKTileBytes;
-    if (vis_nxt) switch_q(j1);
+  }
+  __syncthreads();   // ring buffer 0 is about to be refilled: every wave has read K(step 0) out of it
+  auto step = [&](int t, f32x16_t (&Scur)[2], f32x16_t (&Snxt)[2]) {
+    if ((t & 1) == 0) {   // start of a pair: refill the four buffers the previous pair released
+      if (t + 4 < nFull) {
+        const int j2 = tile_of(t + 2), j3 = tile_of(t + 3), j4 = tile_of(t + 4);
+        if constexpr (WAVES == 8) {
+          stage_k_full(j3, (t + 3) & 3);
+          stage_k_full(j4, t & 3);
+        } else {
+          stage_k(j3, (t + 3) & 3);
+          stage_k(j4, t & 3);
+        }
+        stage_v(j2, (t + 2) & 3);
+        stage_v(j3, (t + 3) & 3);
+      } else {
+        if (t + 3 < nTot) stage_k(tile_of(t + 3), (t + 3) & 3);
+        if (t + 4 < nTot) stage_k(tile_of(t + 4), t & 3);
+        if (t + 2 < nTot) stage_v(tile_of(t + 2), (t + 2) & 3);
+        if (t + 3 < nTot) stage_v(tile_of(t + 3), (t + 3) & 3);
+      }
+    }
+    const bool vis_nxt = visits_step(t + 1);
+    const char* knext = kbase_lds + ((t + 1) & 3) * kKTileBytes;
+    if constexpr (WAVES < 8) {
+      if (vis_nxt) switch_q(tile_of(t + 1));
+    }
     if (vis_cur) {
       // Q.K^T of the next tile is computed even if this wave will not use it (the buffer then holds an older
       // tile or nothing meaningful; the result is dropped): the common path stays free of branches
-      softmax_pv(j, it, vbase_lds + (it & 3) * kVTileBytes, j >= wr.diag_lo, Scur, knext, Snxt);
+      softmax_pv(tile_of(t), t, vbase_lds + (t & 3) * kVTileBytes, t >= fm, Scur, knext, Snxt);
     } else {
-      if (vis_nxt) qk_tile(knext, Snxt);
+      if (vis_nxt) {
+        qk_tile(knext, Snxt);
+        if constexpr (MODE == 4) {
+          mfma_settle(Snxt[0], Snxt[1]);
+          tmax_lane = lane_max(Snxt);
+        }
+      }
       if constexpr (MODE == 2) {
-        if (lane == 0) s_amax[it & 1][wave] = 0.f;  // a wave that skips the tile contributes nothing to the block maximum
+        if (lane == 0) s_amax[t & 1][wave] = 0.f;  // a wave that skips the tile contributes nothing to the block maximum
         __syncthreads();                            // every wave passes one such barrier per tile
       }
     }
-    if (it & 1) {          // end of a pair
+    if (t & 1) {          // end of a pair
       __builtin_amdgcn_s_waitcnt(0);   // this wave's share of the tiles staged at the start of the pair has landed
       __syncthreads();
     }
     vis_cur = vis_nxt;
-#pragma unroll
-    for (int u = 0; u < 4; ++u) tq[u] = tq[u + 1];
-    tq[4] = next_tile(tq[3]);
   };
-  // both steps of a pair always run (the second one idles when the tile list has an odd length), so that every
-  // wave passes the same barriers
-  for (int it = 0; tq[0] < segB_hi; it += 2) {
-    step(it, Sa, Sb);
-    step(it + 1, Sb, Sa);
+  // both steps of a pair always run (the second one idles when the number of steps is odd), so that every wave
+  // passes the same barriers
+  for (int t = 0; t < nTot; t += 2) {
+    step(t, Sa, Sb);
+    step(t + 1, Sb, Sa);
   }
 
   // ---- epilogue: out = acc / l (attn_triton.py:208-209), lse2 = log2(l) + m (:210-213)
