@@ -290,6 +290,9 @@ __device__ __forceinline__ float xor32_sum(float v) {
   return __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
 }
 
+#ifndef SQ_LDS_DEPTH
+#define SQ_LDS_DEPTH 4
+#endif
 constexpr float kLog2_448 = 8.807354922057604f;  // log2(448)
 
 // ---- hand-scheduled LDS reads.  The compiler cannot tell that a ds_read never touches the buffers that
@@ -368,7 +371,8 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
   constexpr int CH = (kBN * kD * 2 / 16) / NT;  // 16-byte chunks per thread and tile operand
   constexpr int ROWS = 32;                      // query rows per wave
   extern __shared__ __attribute__((aligned(16))) char smem[];
-  __shared__ float s_amax[2][WAVES];            // MODE 2: tile maxima of the two waves of a 64-row group
+  // MODE 2: tile maxima of the two waves of a 64-row group, behind the tile rings (which start at LDS address 0)
+  float (*s_amax)[WAVES] = (float (*)[WAVES])(smem + 4 * kStageBytes);
 
   // ---- schedule: blockIdx -> (pair = (b, kvh), item = (q block descending, head in group))
   int pair, item;
@@ -519,9 +523,10 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
 
   const int ksw = c32 & 15;          // swizzle of this lane's K rows (c32 and c32 + 32 share it)
   const uint32_t smem_addr = (uint32_t)(uintptr_t)(lds_ptr_t)smem;
-  uint32_t kx[8];                    // byte offset of k-step kk's chunk inside this lane's K rows
-#pragma unroll
-  for (int kk = 0; kk < 8; ++kk) kx[kk] = c32 * kKStride + (((2 * kk + g) ^ ksw) << 4);
+  // byte offset of k-step kk's chunk inside this lane's K rows: c32 * 256 + (((2 kk + g) ^ ksw) << 4) =
+  // kx0 ^ (kk << 5), and the same holds after adding a ring buffer's base (a multiple of 256; the rings start at
+  // LDS address 0)
+  const uint32_t kx0 = c32 * kKStride + ((g ^ ksw) << 4);
   typedef __attribute__((ext_vector_type(8))) int i32x8_t;
   i32x8_t P8 = {0, 0, 0, 0, 0, 0, 0, 0};   // MODE 4: e4m3 probabilities of the current tile (registers reused tile after tile)
   const int vsw = (c32 >> 1) & 7;    // swizzle of this lane's V^T rows (32 bd + c32)
@@ -557,13 +562,26 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
     }
     return max3(max3(c[0], c[1], c[2]), c[3], c[3]);
   };
-  float tmax_lane = 0.f;   // MODE 4: lane_max of the tile whose scores the next step consumes (computed one step ahead)
+  // MODE 4: row maximum (relative to the running reference) of the tile whose scores the next step consumes, and
+  // whether any row's maximum moved; both computed one step ahead, under the P.V MFMAs
+  float tmax_row = 0.f;
+  bool moved = false;
 
   // softmax update + P.V for the tile whose scores are in S.  Once the running maximum of this tile is settled,
   // the Q.K^T MFMAs of the following tile (K in knext, result in Snext) are issued in the same straight-line
   // block as the exponentials, conversions and P.V MFMAs, so that the matrix pipe and the vector ALU of this
   // wave work side by side.
   auto softmax_pv = [&](int j, int it, const char* vbuf, bool masked, f32x16_t (&S)[2], const char* knext, f32x16_t (&Snext)[2]) {
+    // MODE 4: the first K fragments of the next tile are requested before anything else, so that their LDS
+    // latency passes under the row-maximum bookkeeping
+    const uint32_t klane = smem_addr + (((it + 1) & 3) * kKTileBytes) + kx0;
+    u32x4_t kf[16];
+    constexpr int kDepth = SQ_LDS_DEPTH;   // K fragments are requested this many MFMA slots ahead (even, 2..8)
+    auto kread = [&](auto I) {
+      constexpr int i = decltype(I)::value;
+      kf[i] = lds_read128<(i & 1) * 32 * kKStride>(klane ^ ((i >> 1) << 5));
+    };
+    if constexpr (MODE == 4) static_for<0, kDepth>(kread);
     if (masked) {  // causal mask inside the query block's own tiles (attn_triton.py:69-71)
       // One tile in thousands takes this branch.  The laundered copy of g keeps the branch a branch and stops
       // the compiler from hoisting 32 per-lane column constants out of the loop into precious registers.
@@ -578,17 +596,23 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
     }
     // row maximum of S - m_run + kC; the row's other 32 keys live in lane^32
     float tmax;
+    bool slow;
     if constexpr (MODE == 4) {
-      if (masked) tmax_lane = lane_max(S);
-      tmax = tmax_lane;   // came out of the previous step's P.V phase
+      if (masked) {
+        tmax_row = xor32_max(lane_max(S));
+        moved = __any(tmax_row > kC);
+      }
+      tmax = tmax_row;   // came out of the previous step's P.V phase
+      slow = first || moved;
     } else {
       tmax = max3(S[0][0], S[1][0], S[0][1]);
 #pragma unroll
       for (int i = 1; i < 15; ++i) tmax = max3(tmax, S[1][i], S[0][i + 1]);
       tmax = max3(tmax, S[1][15], S[1][15]);
+      tmax = xor32_max(tmax);
+      slow = first || __any(tmax > kC);
     }
-    tmax = xor32_max(tmax);
-    if (first || __any(tmax > kC)) {
+    if (slow) {
       // some row's maximum moved by d (on the first tile: from the arbitrary reference 0 to the row maximum):
       // shift the scores, rescale the accumulators, re-centre the accumulator initialiser
       asm volatile("; new row maximum" ::: "memory");
@@ -614,27 +638,23 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
       // the row sum}.  K fragments are read 4 slots ahead of the MFMA that consumes them.
       // P^T is the e4m3 B operand of one K=64 MFMA per 32 output channels: byte 16 bn + i of this lane's
       // 32 bytes is the probability in S[bn][i]; the V^T tiles were permuted to the same key order.
-      const uint32_t kaddr = smem_addr + ((it + 1) & 3) * kKTileBytes;
       const uint32_t vlo_addr = smem_addr + 4 * kKTileBytes + (it & 3) * kVTileBytes + c32 * 64 + (((2 * g) ^ ((c32 >> 2) & 3)) << 4);
       const uint32_t vhi_addr = vlo_addr ^ 16;
-      u32x4_t kf[16], vlo[4], vhi[4];
-      auto kread = [&](auto I) {
-        constexpr int i = decltype(I)::value;
-        kf[i] = lds_read128<(i & 1) * 32 * kKStride>(kaddr + kx[i >> 1]);
-      };
-      static_for<0, 4>(kread);
+      u32x4_t vlo[4], vhi[4];
       static_for<0, 16>([&](auto I) {
         constexpr int i = decltype(I)::value;
         constexpr int bn = i & 1, kk = i >> 1;
-        lds_wait<3>(kf[i]);
+        lds_wait<kDepth - 1>(kf[i]);
         const uint4 ka = make_uint4(kf[i][0], kf[i][1], kf[i][2], kf[i][3]);
         if constexpr (kk == 0) Snext[bn] = mfma_qk32<BF16>(ka, qf[0], Cinit);
         else Snext[bn] = mfma_qk32<BF16>(ka, qf[kk], Snext[bn]);
-        if constexpr (i + 4 < 16) kread(std::integral_constant<int, i + 4>{});
-        else if constexpr (i == 12) vlo[0] = lds_read128<0>(vlo_addr);
-        else if constexpr (i == 13) vhi[0] = lds_read128<0>(vhi_addr);
-        else if constexpr (i == 14) vlo[1] = lds_read128<2048>(vlo_addr);
-        else vhi[1] = lds_read128<2048>(vhi_addr);
+        if constexpr (i + kDepth < 16) {
+          kread(std::integral_constant<int, i + kDepth>{});
+        } else {  // the K fragments are all requested: start on the V^T fragments, in the order the P.V slots use them
+          constexpr int r = i + kDepth - 16;
+          if constexpr (r & 1) vhi[r >> 1] = lds_read128<(r >> 1) * 2048>(vhi_addr);
+          else vlo[r >> 1] = lds_read128<(r >> 1) * 2048>(vlo_addr);
+        }
         constexpr int sb = i >> 3, e = 2 * (i & 7), r = 4 * sb + ((i & 7) >> 1);
         const float p0 = __builtin_amdgcn_exp2f(S[sb][e]), p1 = __builtin_amdgcn_exp2f(S[sb][e + 1]);
         S[sb][e] = p0;
@@ -647,13 +667,15 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
       float ps[2] = {0.f, 0.f}, cm[4];
       static_for<0, 4>([&](auto I) {
         constexpr int bd = decltype(I)::value;
-        lds_wait<(bd < 3 ? 2 : 0)>(vlo[bd], vhi[bd]);
+        // requests issued so far: kDepth in the Q.K slots, two more per earlier P.V slot
+        constexpr int issued = (kDepth + 2 * bd < 8) ? kDepth + 2 * bd : 8;
+        lds_wait<issued - 2 * bd - 2>(vlo[bd], vhi[bd]);
         const i32x8_t av = {(int)vlo[bd][0], (int)vlo[bd][1], (int)vlo[bd][2], (int)vlo[bd][3],
                             (int)vhi[bd][0], (int)vhi[bd][1], (int)vhi[bd][2], (int)vhi[bd][3]};
         O[bd] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, P8, O[bd], 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
-        if constexpr (bd + 2 < 4) {
-          vlo[bd + 2] = lds_read128<(bd + 2) * 2048>(vlo_addr);
-          vhi[bd + 2] = lds_read128<(bd + 2) * 2048>(vhi_addr);
+        if constexpr (issued < 8) {
+          vlo[issued / 2] = lds_read128<(issued / 2) * 2048>(vlo_addr);
+          vhi[issued / 2] = lds_read128<(issued / 2) * 2048>(vhi_addr);
         }
         if constexpr (bd < 2) {
 #pragma unroll
@@ -674,7 +696,8 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
         }
         __builtin_amdgcn_sched_barrier(0);
       });
-      tmax_lane = max3(max3(cm[0], cm[1], cm[2]), cm[3], cm[3]);
+      tmax_row = xor32_max(max3(max3(cm[0], cm[1], cm[2]), cm[3], cm[3]));
+      moved = __any(tmax_row > kC);
       const float psum = ps[0] + ps[1];
       l_run += psum;
       __builtin_amdgcn_s_setprio(3);
@@ -773,7 +796,8 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
     qk_tile(kbase_lds, Sa);
     if constexpr (MODE == 4) {
       mfma_settle(Sa[0], Sa[1]);
-      tmax_lane = lane_max(Sa);
+      tmax_row = xor32_max(lane_max(Sa));
+      moved = __any(tmax_row > kC);
     }
   }
   __syncthreads();   // ring buffer 0 is about to be refilled: every wave has read K(step 0) out of it
@@ -811,7 +835,8 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
         qk_tile(knext, Snxt);
         if constexpr (MODE == 4) {
           mfma_settle(Snxt[0], Snxt[1]);
-          tmax_lane = lane_max(Snxt);
+          tmax_row = xor32_max(lane_max(Snxt));
+          moved = __any(tmax_row > kC);
         }
       }
       if constexpr (MODE == 2) {
@@ -1060,7 +1085,7 @@ extern "C" int sq_prefill_fwd(const DLTensor* q, const DLTensor* k, const DLTens
     local.sched_xpp = 1;
     blocks = (unsigned)pairs * (unsigned)items;
   }
-  const size_t smem = 4 * (size_t)kStageBytes;   // rings of 4 K tiles and 4 V^T tiles
+  const size_t smem = 4 * (size_t)kStageBytes + 64;   // rings of 4 K tiles and 4 V^T tiles, MODE 2's block maxima
   const bool bf = dt == DType::BF16;
 #define SQ_LAUNCH_PREFILL(BF, W, M)                                                                              \
   do {                                                                                                           \
