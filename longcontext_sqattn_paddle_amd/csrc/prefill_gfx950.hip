@@ -363,6 +363,29 @@ __device__ __forceinline__ uint4 quant_pack8(const f32x16_t& s, int t, float sc,
   return make_uint4(w[0], w[1], w[2], w[3]);
 }
 
+// Four probabilities -> two fp16 B-operand words, MODE as in quant_pack8 (0, 1 or 3)
+template <int MODE>
+__device__ __forceinline__ void quant_pack4(float p0, float p1, float p2, float p3, uint32_t& w0, uint32_t& w1) {
+  if constexpr (MODE == 0) {
+    w0 = pack_f16(p0, p1);
+    w1 = pack_f16(p2, p3);
+  } else if constexpr (MODE == 3) {
+    int pk = __builtin_amdgcn_cvt_pk_fp8_f32(p0, p1, 0, false);
+    pk = __builtin_amdgcn_cvt_pk_fp8_f32(p2, p3, pk, true);
+    w0 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(pk, 1.0f, false));
+    w1 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(pk, 1.0f, true));
+  } else {
+    int pk = __builtin_amdgcn_cvt_pk_fp8_f32(p0 * 448.f, p1 * 448.f, 0, false);
+    pk = __builtin_amdgcn_cvt_pk_fp8_f32(p2 * 448.f, p3 * 448.f, pk, true);
+    typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+    const f32x2_t lo = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(pk, 1.0f, false);
+    const f32x2_t hi = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(pk, 1.0f, true);
+    constexpr float inv = 1.0f / 448.0f;
+    w0 = pack_f16(lo[0] * inv, lo[1] * inv);
+    w1 = pack_f16(hi[0] * inv, hi[1] * inv);
+  }
+}
+
 // One workgroup = WAVES waves x 32 query rows of one q-head (2 waves per SIMD when WAVES == 8, so that one
 // wave's MFMA phase overlaps the other's softmax phase).  MODE as in quant_pack8.
 template <bool BF16, int WAVES, int MODE>
@@ -581,7 +604,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
       constexpr int i = decltype(I)::value;
       kf[i] = lds_read128<(i & 1) * 32 * kKStride>(klane ^ ((i >> 1) << 5));
     };
-    if constexpr (MODE == 4) static_for<0, kDepth>(kread);
+    if constexpr (MODE != 2) static_for<0, kDepth>(kread);
     if (masked) {  // causal mask inside the query block's own tiles (attn_triton.py:69-71)
       // One tile in thousands takes this branch.  The laundered copy of g keeps the branch a branch and stops
       // the compiler from hoisting 32 per-lane column constants out of the loop into precious registers.
@@ -597,7 +620,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
     // row maximum of S - m_run + kC; the row's other 32 keys live in lane^32
     float tmax;
     bool slow;
-    if constexpr (MODE == 4) {
+    if constexpr (MODE != 2) {
       if (masked) {
         tmax_row = xor32_max(lane_max(S));
         moved = __any(tmax_row > kC);
@@ -703,6 +726,80 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
       __builtin_amdgcn_s_setprio(3);
       return;
     }
+    if constexpr (MODE == 0 || MODE == 1 || MODE == 3) {
+      // Hand-scheduled tile step, fp16 P.V: 16 slots of {Q.K^T MFMA of the next tile, one LDS prefetch, two
+      // exponentials, and every other slot the conversion of four finished probabilities}, then 16 slots of
+      // {P.V MFMA, one LDS prefetch, two additions of the row sum, later two steps of the next tile's row maximum}.
+      // P.V slot s multiplies V^T rows 32 (s & 3) .. +31 with the keys of group m = s >> 2 (8 keys per lane), whose
+      // probabilities are the B operand words Pw[m][0..3].
+      __builtin_amdgcn_s_setprio(0);
+      const uint32_t vlane = smem_addr + 4 * kKTileBytes + (it & 3) * kVTileBytes + c32 * kVStride + ((g ^ vsw) << 4);
+      u32x4_t vf[16];
+      uint32_t Pw[4][4];
+      auto vread = [&](auto I) {
+        constexpr int sl = decltype(I)::value;
+        vf[sl] = lds_read128<(sl & 3) * 32 * kVStride>(vlane ^ ((sl >> 2) << 5));
+      };
+      auto pack_unit = [&](auto U) {   // probabilities 4u .. 4u+3 of the tile (in S order)
+        constexpr int u = decltype(U)::value;
+        const f32x16_t& sv = S[u >> 2];
+        constexpr int o = 4 * (u & 3);
+        quant_pack4<MODE>(sv[o], sv[o + 1], sv[o + 2], sv[o + 3], Pw[u >> 1][2 * (u & 1)], Pw[u >> 1][2 * (u & 1) + 1]);
+      };
+      static_for<0, 16>([&](auto I) {
+        constexpr int i = decltype(I)::value;
+        constexpr int bn = i & 1, kk = i >> 1;
+        lds_wait<kDepth - 1>(kf[i]);
+        const uint4 ka = make_uint4(kf[i][0], kf[i][1], kf[i][2], kf[i][3]);
+        if constexpr (kk == 0) Snext[bn] = mfma_qk32<BF16>(ka, qf[0], Cinit);
+        else Snext[bn] = mfma_qk32<BF16>(ka, qf[kk], Snext[bn]);
+        if constexpr (i + kDepth < 16) kread(std::integral_constant<int, i + kDepth>{});
+        else vread(std::integral_constant<int, i + kDepth - 16>{});
+        constexpr int sb = i >> 3, e = 2 * (i & 7);
+        S[sb][e] = __builtin_amdgcn_exp2f(S[sb][e]);
+        S[sb][e + 1] = __builtin_amdgcn_exp2f(S[sb][e + 1]);
+        if constexpr (i >= 2 && (i & 1) == 0) pack_unit(std::integral_constant<int, (i - 2) / 2>{});
+        __builtin_amdgcn_sched_barrier(0);
+      });
+      float ps[2] = {0.f, 0.f}, cm[4], tm = 0.f;
+      auto max_op = [&](auto K) {   // step k of the lane maximum over the next tile's scores (18 steps)
+        constexpr int k = decltype(K)::value;
+        if constexpr (k < 16) {
+          constexpr int h = k >> 2, j = k & 3, o = 8 * (h & 1);
+          const f32x16_t& sn = Snext[h >> 1];
+          if constexpr (j == 0) cm[h] = max3(sn[o], sn[o + 1], sn[o + 2]);
+          else if constexpr (j == 1) cm[h] = max3(cm[h], sn[o + 3], sn[o + 4]);
+          else if constexpr (j == 2) cm[h] = max3(cm[h], sn[o + 5], sn[o + 6]);
+          else cm[h] = max3(cm[h], sn[o + 7], sn[o + 7]);
+        } else if constexpr (k == 16) {
+          tm = max3(cm[0], cm[1], cm[2]);
+        } else {
+          tm = max3(tm, cm[3], cm[3]);
+        }
+      };
+      static_for<0, 16>([&](auto I) {
+        constexpr int sl = decltype(I)::value;
+        constexpr int m = sl >> 2, bd = sl & 3;
+        constexpr int issued = (kDepth + sl < 16) ? kDepth + sl : 16;   // V^T requests issued before this slot
+        lds_wait<issued - sl - 1>(vf[sl]);
+        const uint4 av = make_uint4(vf[sl][0], vf[sl][1], vf[sl][2], vf[sl][3]);
+        O[bd] = mfma_pv32(av, make_uint4(Pw[m][0], Pw[m][1], Pw[m][2], Pw[m][3]), O[bd]);
+        if constexpr (issued < 16) vread(std::integral_constant<int, issued>{});
+        if constexpr (sl == 0) pack_unit(std::integral_constant<int, 7>{});
+        ps[0] += S[sl >> 3][2 * (sl & 7)];
+        ps[1] += S[sl >> 3][2 * (sl & 7) + 1];
+        if constexpr (sl >= 7) {
+          max_op(std::integral_constant<int, 2 * (sl - 7)>{});
+          max_op(std::integral_constant<int, 2 * (sl - 7) + 1>{});
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      });
+      tmax_row = xor32_max(tm);
+      moved = __any(tmax_row > kC);
+      l_run += ps[0] + ps[1];
+      __builtin_amdgcn_s_setprio(3);
+      return;
+    }
     qk_tile(knext, Snext);   // scores of the next tile, relative to the maximum just settled
     float psum = 0.f;
 #pragma unroll
@@ -794,7 +891,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
   if (vis_cur) {
     switch_q(tile_of(0));
     qk_tile(kbase_lds, Sa);
-    if constexpr (MODE == 4) {
+    if constexpr (MODE != 2) {
       mfma_settle(Sa[0], Sa[1]);
       tmax_row = xor32_max(lane_max(Sa));
       moved = __any(tmax_row > kC);
@@ -833,7 +930,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
     } else {
       if (vis_nxt) {
         qk_tile(knext, Snxt);
-        if constexpr (MODE == 4) {
+        if constexpr (MODE != 2) {
           mfma_settle(Snxt[0], Snxt[1]);
           tmax_row = xor32_max(lane_max(Snxt));
           moved = __any(tmax_row > kC);
