@@ -7,15 +7,17 @@
 // All three run the same KV-block step (S = q~.k, running max, p = exp2(S-m), l += sum p, optional e4m3
 // round trip of p, acc += fp16(p).fp16(v)); they differ only in which 64-key blocks a query block visits.
 //
-// Design (CDNA4, 64-wide waves, 1 wave per SIMD, 512 registers per lane):
-//   * workgroup = WAVES waves x 64 query rows of one q-head; K and V^T tiles of 64 keys are staged once per
-//     workgroup in LDS (double buffered, padded rows) and shared by all its rows;
+// Design (CDNA4, 64-wide waves, 2 waves per SIMD, at most 256 registers per lane):
+//   * workgroup = WAVES (8) waves x 32 query rows of one q-head; K and V^T tiles of 64 keys are copied once per
+//     workgroup into rings of 4 LDS buffers by global_load_lds (unpadded, XOR-swizzled) and shared by all its rows;
+//     one workgroup barrier per two tiles;
 //   * S^T = K . Q~^T on v_mfma_f32_32x32x16 (bf16 or f16): K rows are the A operand straight out of LDS, Q~
 //     stays in registers as the B operand for the whole kernel.  The accumulator then holds, per lane,
 //     one query row and 32 of the 64 keys, so the row max needs one cross-lane exchange and the row sum none;
-//   * P^T in that accumulator layout *is* the B-operand layout of O^T += V^T . P^T (f16 MFMA), provided V^T is
-//     stored with the matching key permutation -- a one-off pre-pass writes V as fp16, transposed, permuted
-//     tiles into the workspace (O(N) work against the O(N^2) main loop);
+//   * P^T in that accumulator layout *is* the B-operand layout of O^T += V^T . P^T (f16 MFMA, or the K=64 fp8 MFMA
+//     when P and V are e4m3), provided V^T is stored with the matching key permutation -- a one-off pre-pass
+//     writes V as transposed, permuted tiles into the workspace (O(N) work against the O(N^2) main loop);
+//   * the tile step is laid out by hand in slots of one MFMA plus the vector and LDS work that runs beside it;
 //   * blockIdx -> (kv head, q head, q block) mapping keeps the q-heads of one KV head on the same XCD(s) so
 //     their K/V tiles are shared in that XCD's L2, and issues the longest (last) query blocks first.
 #include <type_traits>
