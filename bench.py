@@ -132,6 +132,33 @@ def time_kmeans(torch, iters=10):
     return us, flops, nbytes
 
 
+def time_prepass(torch, N, want4, iters=10):
+    """The plugin closure's operand pre-pass (key centring + int8/int4 per-token + int8 per-channel fake quantisation)
+    at the prefill benchmark shape, tensors in the plugin's NHD layout."""
+    from longcontext_sqattn_paddle_amd.sqattn.fake_quant import fused_int_prepass
+
+    dev = torch.device("cuda:0")
+    Hq, Hkv, D = 28, 4, 128
+    g = torch.Generator(device=dev).manual_seed(2)
+    q = torch.randn(1, N, Hq, D, device=dev, generator=g).bfloat16()
+    k = torch.randn(1, N, Hkv, D, device=dev, generator=g).bfloat16()
+    v = torch.randn(1, N, Hkv, D, device=dev, generator=g).bfloat16()
+    for _ in range(2):
+        outs = fused_int_prepass(q, k, v, want_4bit=want4)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        outs = fused_int_prepass(q, k, v, want_4bit=want4)
+    e1.record()
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(outs[0][0, -1].float()).all())
+    us = e0.elapsed_time(e1) / iters * 1e3
+    qb, kb = N * Hq * D * 2, N * Hkv * D * 2
+    nbytes = (qb + 2 * kb + kb) + (qb + kb + kb) + ((qb + kb) if want4 else 0)   # reads (K twice) + writes
+    return us, float(nbytes)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -148,6 +175,7 @@ def main():
     ap.add_argument("--no-kmeans", action="store_true")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode", action="store_true")
+    ap.add_argument("--no-prepass", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -221,6 +249,15 @@ def main():
             log(f"[bench] decode {name}: {us:.1f} us, {gbs:.0f} GB/s")
             torch.cuda.empty_cache()
         result["decode"] = dec
+    if not args.no_prepass:
+        pre = {}
+        for name, want4 in (("int8", False), ("int8_int4", True)):
+            us, nbytes = time_prepass(torch, N, want4)
+            pre[name] = {"us_per_call": round(us, 1), "GB_per_s": round(nbytes / us / 1e3, 1),
+                         "frac_of_hbm_peak": round(nbytes / us / 1e3 / PEAK_HBM_GBS, 4), "bytes": nbytes}
+            log(f"[bench] plugin pre-pass {name}: {us:.0f} us, {nbytes / us / 1e3:.0f} GB/s")
+            torch.cuda.empty_cache()
+        result["plugin_prepass"] = pre
     if not args.no_kmeans:
         us, kflops, kbytes = time_kmeans(torch)
         result["kmeans"] = {"us_per_iteration": round(us, 1), "TFLOP_per_s": round(kflops / us / 1e6, 1),

@@ -18,6 +18,8 @@
  *   sq_reverse_index          cache_hub/kmeans.py:233-262
  *   sq_index_add              cache_hub/kmeans.py:307-329
  *   sq_topk_select            no reference counterpart (defined by this build's benchmark configuration)
+ *   sq_fake_quant_prepass     sqattn/attn_replacer.py:334-365 (GQA expand, key centring and the five fake-quant
+ *                             passes of mp_triton_wrapper's closure), sqattn/fake_quant.py:24-58, 98-125
  */
 #ifndef SQATTN_H_
 #define SQATTN_H_
@@ -141,6 +143,23 @@ int sq_index_add(const DLTensor* value, const DLTensor* idx, DLTensor* out, DLTe
 int sq_topk_select(const DLTensor* query, const DLTensor* centroids, const DLTensor* clusters,
                    const DLTensor* cluster_size, DLTensor* out, DLTensor* workspace, int32_t num_kv_groups,
                    void* stream);
+
+/* Bytes of scratch sq_fake_quant_prepass needs (partial column sums of the key, its mean). */
+size_t sq_fake_quant_prepass_workspace_bytes(int64_t batch, int64_t num_kv_heads, int64_t num_tokens);
+
+/*
+ * Operand pre-pass of the plugin closure for the integer quantiser types, fused and without expanding the kv
+ * heads: key_c = key - mean over tokens (mean = dtype(float(exact sum / N)), subtraction rounded to the tensor
+ * dtype); q8/q4 = IntegerQuantizer(8|4, True, "per_token").fake_quant_tensor(query); k8/k4 the same of key_c;
+ * v8 = IntegerQuantizer(8, True, "per_channel").fake_quant_tensor(value), whose scale is per (token, channel)
+ * over batch and heads as in the reference (range over dims 0 and 1 of [B,H,N,D]).  q4 and k4 may both be null.
+ * query/q8/q4 [B,N,Hq,128] and key/value/k8/k4/v8 [B,N,Hkv,128] for SQ_LAYOUT_NHD ([B,H,N,128] for
+ * SQ_LAYOUT_HND), bf16 or fp16, all of one dtype; any strides with a contiguous last dimension and 16-byte
+ * aligned rows.  Outputs are bit-identical to the formulas evaluated in fp32 on the host.
+ */
+int sq_fake_quant_prepass(const DLTensor* query, const DLTensor* key, const DLTensor* value, DLTensor* q8,
+                          DLTensor* q4, DLTensor* k8, DLTensor* k4, DLTensor* v8, DLTensor* workspace,
+                          int32_t layout, void* stream);
 
 #ifdef __cplusplus
 }

@@ -80,6 +80,8 @@ SYMBOLS = {
     "sq_reverse_index": (ctypes.c_int, [_P, _P, _P, _P, ctypes.c_void_p]),
     "sq_index_add": (ctypes.c_int, [_P, _P, _P, _P, ctypes.c_void_p]),
     "sq_topk_select": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, ctypes.c_int32, ctypes.c_void_p]),
+    "sq_fake_quant_prepass_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int64] * 3),
+    "sq_fake_quant_prepass": (ctypes.c_int, [_P] * 9 + [ctypes.c_int32, ctypes.c_void_p]),
 }
 
 _lib: Optional[ctypes.CDLL] = None

@@ -1,0 +1,303 @@
+// Fused operand pre-pass of the SQAttn plugin closure for gfx950 (MI355X).
+//
+// Replaces the tensor passes of the reference's `mp_triton_wrapper(...).attention_fn`
+// (sqattn/attn_replacer.py:334-365) for the integer quantiser types:
+//   :334-337  repeat_kv + permute           -> not materialised: the attention kernel reads the kv heads in place
+//   :338-339  key -= key.mean(token axis)   -> column sums (two deterministic stages, fp64) + subtraction in the
+//                                              tensor dtype
+//   :361-365  five fake-quant passes        -> IntegerQuantizer(8|4, True, "per_token") on query and centred key
+//                                              (sqattn/fake_quant.py:33-35, 47-52, 114-125), and
+//                                              IntegerQuantizer(8, True, "per_channel") on value, whose range is
+//                                              taken over dims (0, 1) of the [B, H, N, D] tensor (:30-32), i.e. one
+//                                              scale per (token, channel) shared by batch and heads
+// Every output element is computed with the same fp32 operations as the reference's formula (division by the
+// scale, round half away from zero as sign(x) * floor(|x| + 0.5), clamp, multiplication by the scale, cast to
+// the tensor dtype), so the results are bit-identical to a CPU restatement.
+//
+// HBM-bound streaming work: every input element is read once (K twice: sums, then quantisation) and every
+// output element written once; rows of 128 channels are handled by 16 lanes x 16 bytes.
+#include "common.hpp"
+
+namespace sq {
+namespace {
+
+constexpr int kPD = 128;          // channels per row (head_dim)
+constexpr int kSumBlocks = 512;   // partial-sum workgroups of the key mean (upper bound)
+
+struct View {   // [B, N, H, 128] addressed by element strides (either memory layout)
+  char* p;
+  int64_t sb, sn, sh;
+};
+
+struct PrepassArgs {
+  View q, k, v, q8, q4, k8, k4, v8;
+  double* part;     // [nblk, B*Hkv*128]
+  uint16_t* mean;   // [B*Hkv*128] bits of the key mean in the tensor dtype
+  int32_t B, N, Hq, Hkv, is_bf16, nblk, tok_per_blk, want4;
+};
+
+template <bool BF16>
+__device__ __forceinline__ float ld(uint32_t bits16) {
+  if constexpr (BF16) return bf16_bits_to_f32(bits16);
+  return (float)__builtin_bit_cast(_Float16, (uint16_t)bits16);
+}
+template <bool BF16>
+__device__ __forceinline__ uint32_t st(float x) {
+  if constexpr (BF16) return f32_to_bf16_bits(x);
+  return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)x);
+}
+template <bool BF16>
+__device__ __forceinline__ void unpack8(const uint4& r, float (&x)[8]) {
+  const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    x[2 * i] = ld<BF16>(w[i] & 0xffffu);
+    x[2 * i + 1] = ld<BF16>(w[i] >> 16);
+  }
+}
+template <bool BF16>
+__device__ __forceinline__ uint4 pack8(const float (&x)[8]) {
+  uint32_t w[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) w[i] = st<BF16>(x[2 * i]) | (st<BF16>(x[2 * i + 1]) << 16);
+  return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+// paddle.round / the reference's rounding: half away from zero, evaluated in fp32 exactly like
+// sign(x) * floor(abs(x) + 0.5)
+__device__ __forceinline__ float round_half_away(float t) { return copysignf(floorf(fabsf(t) + 0.5f), t); }
+
+// quant-dequant of one value: clamp(round(x / scale), qmin, qmax) * scale   (fake_quant.py:114-125, zero point 0)
+__device__ __forceinline__ float qdq(float x, float scale, float qmin, float qmax) {
+  const float q = fminf(fmaxf(round_half_away(x / scale), qmin), qmax);
+  return q * scale;
+}
+
+// ---- key mean, stage 1: workgroup b sums tokens [b*tok_per_blk, ...) of every (batch, kv head, channel) in fp64.
+// With few columns (Qwen2.5-7B: 4 kv heads x 16 groups of 8 channels = 64) the 256 threads split the tokens of the
+// workgroup between them and combine through LDS in a fixed order.
+template <bool BF16>
+__global__ __launch_bounds__(256) void prepass_ksum_kernel(PrepassArgs a) {
+  __shared__ double red[256][8];
+  const int ncol8 = a.B * a.Hkv * (kPD / 8);   // column groups of 8 channels
+  const int n0 = blockIdx.x * a.tok_per_blk, n1 = min(n0 + a.tok_per_blk, a.N);
+  const int TL = ncol8 < 256 ? 256 / ncol8 : 1;   // token lanes per column group
+  for (int cg0 = 0; cg0 < ncol8; cg0 += 256) {
+    const int cg = cg0 + (TL > 1 ? (int)threadIdx.x % ncol8 : (int)threadIdx.x);
+    const int tl = TL > 1 ? (int)threadIdx.x / ncol8 : 0;
+    const bool live = cg < ncol8 && tl < TL;
+    double s[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (live) {
+      const int c8 = cg % (kPD / 8), h = (cg / (kPD / 8)) % a.Hkv, b = cg / ((kPD / 8) * a.Hkv);
+      const uint16_t* base = (const uint16_t*)a.k.p + b * a.k.sb + h * a.k.sh + 8 * c8;
+      for (int n = n0 + tl; n < n1; n += TL) {
+        float x[8];
+        unpack8<BF16>(*(const uint4*)(base + (int64_t)n * a.k.sn), x);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) s[e] += (double)x[e];
+      }
+    }
+    if (TL > 1) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) red[threadIdx.x][e] = s[e];
+      __syncthreads();
+      if (live && tl == 0) {
+        for (int u = 1; u < TL; ++u)
+#pragma unroll
+          for (int e = 0; e < 8; ++e) s[e] += red[u * ncol8 + cg][e];
+      }
+      __syncthreads();
+    }
+    if (live && tl == 0) {
+      double* dst = a.part + (int64_t)blockIdx.x * (ncol8 * 8) + cg * 8;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) dst[e] = s[e];
+    }
+  }
+}
+
+// ---- key mean, stage 2: 16 lanes per column add the partial sums l, l+16, ... and combine in a fixed tree;
+// mean = dtype(float(sum / N))
+template <bool BF16>
+__global__ __launch_bounds__(256) void prepass_kmean_kernel(PrepassArgs a) {
+  const int ncol = a.B * a.Hkv * kPD;
+  const int c = (blockIdx.x * blockDim.x + threadIdx.x) >> 4, l = threadIdx.x & 15;
+  double s = 0;
+  if (c < ncol)
+    for (int b = l; b < a.nblk; b += 16) s += a.part[(int64_t)b * ncol + c];
+#pragma unroll
+  for (int sh = 8; sh >= 1; sh >>= 1) s += __shfl_xor(s, sh);
+  if (c >= ncol || l != 0) return;
+  // two roundings on purpose (fp64 -> fp32 -> tensor dtype), like a mean accumulated in fp32 and cast to the
+  // tensor dtype; the empty asm keeps the compiler from merging them into one fp64 -> fp16 conversion
+  float mf = (float)(s / (double)a.N);
+  asm volatile("" : "+v"(mf));
+  a.mean[c] = (uint16_t)st<BF16>(mf);
+}
+
+// ---- per-token 8-bit (and 4-bit) fake quantisation of the rows of q (CENTRE = false) or of k minus its mean
+template <bool BF16, bool CENTRE>
+__global__ __launch_bounds__(256) void prepass_rows_kernel(PrepassArgs a) {
+  const View& src = CENTRE ? a.k : a.q;
+  const View& d8 = CENTRE ? a.k8 : a.q8;
+  const View& d4 = CENTRE ? a.k4 : a.q4;
+  const int H = CENTRE ? a.Hkv : a.Hq;
+  const int64_t rows = (int64_t)a.B * a.N * H;
+  const int l16 = threadIdx.x & 15;
+  const int64_t row = (int64_t)blockIdx.x * (blockDim.x / 16) + (threadIdx.x >> 4);
+  if (row >= rows) return;   // whole 16-lane groups leave together; the shuffles below stay inside a group
+  const int h = (int)(row % H);
+  const int64_t n = (row / H) % a.N, b = row / ((int64_t)H * a.N);
+  float x[8];
+  unpack8<BF16>(*(const uint4*)((const uint16_t*)src.p + b * src.sb + n * src.sn + h * src.sh + 8 * l16), x);
+  if constexpr (CENTRE) {
+    float m[8];
+    unpack8<BF16>(*(const uint4*)(a.mean + ((int)b * H + h) * kPD + 8 * l16), m);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = ld<BF16>(st<BF16>(x[e] - m[e]));   // the subtraction rounds to the tensor dtype
+  }
+  float amax = 0.f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf(x[e]));
+#pragma unroll
+  for (int sh = 1; sh < 16; sh <<= 1) amax = fmaxf(amax, __shfl_xor(amax, sh));
+  amax = fmaxf(amax, 1e-5f);
+  {
+    const float scale = amax / 127.f;
+    float y[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) y[e] = qdq(x[e], scale, -128.f, 127.f);
+    *(uint4*)((uint16_t*)d8.p + b * d8.sb + n * d8.sn + h * d8.sh + 8 * l16) = pack8<BF16>(y);
+  }
+  if (a.want4) {
+    const float scale = amax / 7.f;
+    float y[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) y[e] = qdq(x[e], scale, -8.f, 7.f);
+    *(uint4*)((uint16_t*)d4.p + b * d4.sb + n * d4.sn + h * d4.sh + 8 * l16) = pack8<BF16>(y);
+  }
+}
+
+// ---- value: one 8-bit scale per (token, channel) over batch and heads
+template <bool BF16>
+__global__ __launch_bounds__(256) void prepass_v_kernel(PrepassArgs a) {
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;   // (token, group of 8 channels)
+  if (t >= (int64_t)a.N * (kPD / 8)) return;
+  const int c8 = (int)(t % (kPD / 8));
+  const int64_t n = t / (kPD / 8);
+  const uint16_t* base = (const uint16_t*)a.v.p + n * a.v.sn + 8 * c8;
+  float amax[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  for (int b = 0; b < a.B; ++b)
+    for (int h = 0; h < a.Hkv; ++h) {
+      float x[8];
+      unpack8<BF16>(*(const uint4*)(base + b * a.v.sb + h * a.v.sh), x);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) amax[e] = fmaxf(amax[e], fabsf(x[e]));
+    }
+  float scale[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) scale[e] = fmaxf(amax[e], 1e-5f) / 127.f;
+  uint16_t* obase = (uint16_t*)a.v8.p + n * a.v8.sn + 8 * c8;
+  for (int b = 0; b < a.B; ++b)
+    for (int h = 0; h < a.Hkv; ++h) {
+      float x[8], y[8];
+      unpack8<BF16>(*(const uint4*)(base + b * a.v.sb + h * a.v.sh), x);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) y[e] = qdq(x[e], scale[e], -128.f, 127.f);
+      *(uint4*)(obase + b * a.v8.sb + h * a.v8.sh) = pack8<BF16>(y);
+    }
+}
+
+int make_view(const DLTensor* t, const char* name, int layout, int dev, DType dt, int64_t B, int64_t N, int64_t H, View* out) {
+  int rc;
+  if ((rc = check_tensor(t, name, 4, dev))) return rc;
+  SQ_REQUIRE(dtype_of(t) == dt, SQ_EDTYPE, "sq_fake_quant_prepass: %s must have the dtype of query", name);
+  const int nd = layout == SQ_LAYOUT_HND ? 2 : 1, hd = layout == SQ_LAYOUT_HND ? 1 : 2;
+  SQ_REQUIRE(t->shape[0] == B && t->shape[nd] == N && t->shape[hd] == H && t->shape[3] == kPD, SQ_ESHAPE,
+             "sq_fake_quant_prepass: %s has the wrong shape", name);
+  for (int d = 0; d < 3; ++d)
+    SQ_REQUIRE(stride_of(t, d) % 8 == 0 || t->shape[d] == 1, SQ_ESHAPE, "sq_fake_quant_prepass: rows of %s are not 16-byte aligned", name);
+  out->p = data_of(t);
+  out->sb = stride_of(t, 0);
+  out->sn = stride_of(t, nd);
+  out->sh = stride_of(t, hd);
+  return SQ_OK;
+}
+
+int tokens_per_block(int64_t N) { return (int)((N + kSumBlocks - 1) / kSumBlocks); }
+
+}  // namespace
+}  // namespace sq
+
+using namespace sq;
+
+extern "C" size_t sq_fake_quant_prepass_workspace_bytes(int64_t batch, int64_t num_kv_heads, int64_t num_tokens) {
+  if (batch <= 0 || num_kv_heads <= 0 || num_tokens <= 0) return 0;
+  const int tpb = tokens_per_block(num_tokens);
+  const int64_t nblk = (num_tokens + tpb - 1) / tpb;
+  const size_t cols = (size_t)batch * num_kv_heads * kPD;
+  return (size_t)nblk * cols * sizeof(double) + ((cols * 2 + 255) & ~(size_t)255);
+}
+
+extern "C" int sq_fake_quant_prepass(const DLTensor* query, const DLTensor* key, const DLTensor* value, DLTensor* q8,
+                                     DLTensor* q4, DLTensor* k8, DLTensor* k4, DLTensor* v8, DLTensor* workspace,
+                                     int32_t layout, void* stream) {
+  SQ_REQUIRE(query && key && value && q8 && k8 && v8, SQ_EINVAL, "sq_fake_quant_prepass: null tensor argument");
+  SQ_REQUIRE((q4 == nullptr) == (k4 == nullptr), SQ_EINVAL, "sq_fake_quant_prepass: q4 and k4 must be given together");
+  SQ_REQUIRE(layout == SQ_LAYOUT_HND || layout == SQ_LAYOUT_NHD, SQ_EINVAL, "Unknown tensor layout: %d", (int)layout);
+  int rc;
+  if ((rc = check_tensor(query, "query", 4, query->device.device_id))) return rc;
+  const int dev = query->device.device_id;
+  const DType dt = dtype_of(query);
+  SQ_REQUIRE(dt == DType::BF16 || dt == DType::F16, SQ_EDTYPE, "sq_fake_quant_prepass: query must be bf16 or fp16");
+  const int nd = layout == SQ_LAYOUT_HND ? 2 : 1, hd = layout == SQ_LAYOUT_HND ? 1 : 2;
+  SQ_REQUIRE(query->shape[3] == kPD, SQ_EUNSUPPORTED, "sq_fake_quant_prepass: head_dim must be %d (pad smaller heads with zeros)", kPD);
+  if ((rc = check_tensor(key, "key", 4, dev))) return rc;
+  const int64_t B = query->shape[0], N = query->shape[nd], Hq = query->shape[hd], Hkv = key->shape[hd];
+  SQ_REQUIRE(B > 0 && N > 0 && Hq > 0 && Hkv > 0, SQ_ESHAPE, "sq_fake_quant_prepass: empty tensor");
+  SQ_REQUIRE(B * N * Hq < (int64_t)1 << 40 && B * Hkv * kPD < (int64_t)1 << 24, SQ_EUNSUPPORTED, "sq_fake_quant_prepass: tensor too large");
+  PrepassArgs a;
+  memset(&a, 0, sizeof(a));
+  if ((rc = make_view(query, "query", layout, dev, dt, B, N, Hq, &a.q)) || (rc = make_view(key, "key", layout, dev, dt, B, N, Hkv, &a.k)) ||
+      (rc = make_view(value, "value", layout, dev, dt, B, N, Hkv, &a.v)) || (rc = make_view(q8, "q8", layout, dev, dt, B, N, Hq, &a.q8)) ||
+      (rc = make_view(k8, "k8", layout, dev, dt, B, N, Hkv, &a.k8)) || (rc = make_view(v8, "v8", layout, dev, dt, B, N, Hkv, &a.v8)))
+    return rc;
+  if (q4 && ((rc = make_view(q4, "q4", layout, dev, dt, B, N, Hq, &a.q4)) || (rc = make_view(k4, "k4", layout, dev, dt, B, N, Hkv, &a.k4))))
+    return rc;
+  const size_t need = sq_fake_quant_prepass_workspace_bytes(B, Hkv, N);
+  SQ_REQUIRE(workspace && on_gpu(workspace) && workspace->device.device_id == dev, SQ_EWORKSPACE,
+             "sq_fake_quant_prepass: workspace missing or not on the device");
+  SQ_REQUIRE((size_t)numel_of(workspace) * (workspace->dtype.bits / 8) >= need && is_compact(workspace), SQ_EWORKSPACE,
+             "sq_fake_quant_prepass: workspace too small: need %zu bytes", need);
+  SQ_REQUIRE(((uintptr_t)data_of(workspace) & 255) == 0, SQ_EWORKSPACE, "sq_fake_quant_prepass: workspace not 256-byte aligned");
+  int cur = -1;
+  SQ_HIP(hipGetDevice(&cur));
+  SQ_REQUIRE(cur == dev, SQ_EDEVICE, "sq_fake_quant_prepass: tensors live on device %d but the current device is %d", dev, cur);
+
+  a.B = (int)B;
+  a.N = (int)N;
+  a.Hq = (int)Hq;
+  a.Hkv = (int)Hkv;
+  a.is_bf16 = dt == DType::BF16;
+  a.tok_per_blk = tokens_per_block(N);
+  a.nblk = (int)((N + a.tok_per_blk - 1) / a.tok_per_blk);
+  a.want4 = q4 != nullptr;
+  const size_t cols = (size_t)B * Hkv * kPD;
+  a.part = (double*)data_of(workspace);
+  a.mean = (uint16_t*)(data_of(workspace) + (size_t)a.nblk * cols * sizeof(double));
+  hipStream_t s = (hipStream_t)stream;
+  const int64_t qrows = B * N * Hq, krows = B * N * Hkv, vthreads = N * (kPD / 8);
+#define SQ_PREPASS_LAUNCH(BF)                                                                                  \
+  do {                                                                                                         \
+    hipLaunchKernelGGL(prepass_ksum_kernel<BF>, dim3(a.nblk), dim3(256), 0, s, a);                             \
+    hipLaunchKernelGGL(prepass_kmean_kernel<BF>, dim3((unsigned)((cols * 16 + 255) / 256)), dim3(256), 0, s, a);    \
+    hipLaunchKernelGGL((prepass_rows_kernel<BF, false>), dim3((unsigned)((qrows + 15) / 16)), dim3(256), 0, s, a); \
+    hipLaunchKernelGGL((prepass_rows_kernel<BF, true>), dim3((unsigned)((krows + 15) / 16)), dim3(256), 0, s, a);  \
+    hipLaunchKernelGGL(prepass_v_kernel<BF>, dim3((unsigned)((vthreads + 255) / 256)), dim3(256), 0, s, a);    \
+  } while (0)
+  if (a.is_bf16) SQ_PREPASS_LAUNCH(true);
+  else SQ_PREPASS_LAUNCH(false);
+#undef SQ_PREPASS_LAUNCH
+  SQ_HIP(hipGetLastError());
+  return SQ_OK;
+}

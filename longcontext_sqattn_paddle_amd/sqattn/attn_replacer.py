@@ -21,7 +21,7 @@ import torch
 from .attn_triton_decode import attn_decode
 from .attn_triton_mix_bad import attn_hierarchical_window
 from .attn_triton_mix_relative import attn_hierarchical_relative_window
-from .fake_quant import FloatQuantizer, IntegerQuantizer
+from .fake_quant import FloatQuantizer, IntegerQuantizer, fused_int_prepass
 from .sdpa_attention import sdpa_attention_forward
 
 
@@ -101,42 +101,53 @@ def mp_triton_wrapper(layer_idx, bit8_window_sizes=0, bit4_window_sizes=0, sink_
     bit8_window_sizes, bit4_window_sizes = _normalise_windows(bit8_window_sizes, bit4_window_sizes)
 
     def attention_fn(module, query, key, value, attention_mask, dropout=0.0, scaling=1.0, sliding_window=None, **kwargs):
-        # query [B,N,Hq,D], key/value [B,N,Hkv,D]  ->  HND views without expanding the kv heads
-        if hasattr(module, "num_key_value_groups"):
-            key = key.permute(0, 2, 1, 3)
-            value = value.permute(0, 2, 1, 3)
-            query = query.permute(0, 2, 1, 3)
-        bit8_qk, bit4_qk, bit8_v = _quantizers(args)
-        seq_len = query.shape[2]
+        # query [B,N,Hq,D], key/value [B,N,Hkv,D]; the kv heads are never expanded (the kernels take GQA as is)
+        nhd = hasattr(module, "num_key_value_groups")
+        layout = "NHD" if nhd else "HND"
+        seq_dim = 1 if nhd else 2
+        seq_len = query.shape[seq_dim]
         if seq_len == 1:
-            q_nhd = query.permute(0, 2, 1, 3)
-            out = attn_decode(q_nhd, key.permute(0, 2, 1, 3), value.permute(0, 2, 1, 3), "NHD", torch.bfloat16)
+            if not nhd:
+                query, key, value = (t.permute(0, 2, 1, 3) for t in (query, key, value))
+            out = attn_decode(query, key, value, "NHD", torch.bfloat16)
             b, n, h, d = out.shape
             return out.reshape(b, n, h * d)
-        key = key - key.mean(dim=2, keepdim=True)
-        q_bit8 = bit8_qk.fake_quant_tensor(query)
-        k_bit8 = bit8_qk.fake_quant_tensor(key)
-        v_bit8 = bit8_v.fake_quant_tensor(value)
         p_quant = kwargs.get("p_quant", None)
-        if args.use_relative_distance:
-            # the relative launch aliases the 4-bit operands to the 8-bit ones (attn_triton_mix_relative.py:441-444),
-            # so the two 4-bit passes of the reference (:362,364) would be dead work and are skipped
-            del query, key, value
+        relative = bool(args.use_relative_distance)
+        if args.qk_qtype == "int" and args.v_qtype == "int" and query.size(-1) == 128:
+            # one fused HIP pre-pass instead of the reference's tensor passes (:338-365).  The relative launch
+            # aliases the 4-bit operands to the 8-bit ones (attn_triton_mix_relative.py:441-444), so they are
+            # only produced for the absolute variant.
+            q_bit8, q_bit4, k_bit8, k_bit4, v_bit8 = fused_int_prepass(query, key, value, want_4bit=not relative,
+                                                                       tensor_layout=layout)
+        else:
+            bit8_qk, bit4_qk, bit8_v = _quantizers(args)
+            if nhd:   # the quantisers' "per_channel" range is over dims (0, 1) of [B,H,N,D]: quantise HND views
+                query, key, value = (t.permute(0, 2, 1, 3) for t in (query, key, value))
+            key = key - key.mean(dim=2, keepdim=True)
+            q_bit8 = bit8_qk.fake_quant_tensor(query)
+            k_bit8 = bit8_qk.fake_quant_tensor(key)
+            v_bit8 = bit8_v.fake_quant_tensor(value)
+            q_bit4 = k_bit4 = None
+            if not relative:
+                q_bit4 = bit4_qk.fake_quant_tensor(query)
+                k_bit4 = bit4_qk.fake_quant_tensor(key)
+            layout = "HND"
+        del query, key, value
+        if relative:
             attn_output = attn_hierarchical_relative_window(
                 q_bit8, k_bit8, q_bit8, k_bit8, v_bit8, int8_window_ratios=bit8_window_sizes,
-                int4_window_ratios=bit4_window_sizes, sink_size=sink_window_size, tensor_layout="HND",
+                int4_window_ratios=bit4_window_sizes, sink_size=sink_window_size, tensor_layout=layout,
                 output_dtype=torch.bfloat16, p_quant=p_quant)
         else:
-            q_bit4 = bit4_qk.fake_quant_tensor(query)
-            k_bit4 = bit4_qk.fake_quant_tensor(key)
-            del query, key, value
             attn_output = attn_hierarchical_window(
                 q_bit8, k_bit8, q_bit4, k_bit4, v_bit8, int8_window_sizes=bit8_window_sizes,
-                int4_window_sizes=bit4_window_sizes, sink_size=sink_window_size, tensor_layout="HND",
+                int4_window_sizes=bit4_window_sizes, sink_size=sink_window_size, tensor_layout=layout,
                 output_dtype=torch.bfloat16, p_quant=p_quant)
-        attn_output = attn_output.transpose(1, 2).contiguous()
+        if layout == "HND":
+            attn_output = attn_output.transpose(1, 2).contiguous()
         bs, seq_len, head, head_dim = attn_output.shape
-        return attn_output.view(bs, seq_len, head * head_dim)
+        return attn_output.reshape(bs, seq_len, head * head_dim)
 
     return attention_fn
 

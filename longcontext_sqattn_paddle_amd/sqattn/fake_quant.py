@@ -138,3 +138,33 @@ class FloatQuantizer(BaseQuantizer):
     def quant(self, tensor, scales, zeros, qmax, qmin):
         scaled = torch.minimum(torch.maximum(tensor / scales + zeros, qmin), qmax)
         return float_quantize(scaled.float(), self.e_bits, self.m_bits, rounding="nearest")
+
+
+def fused_int_prepass(query, key, value, want_4bit=True, tensor_layout="NHD"):
+    """The operand pre-pass of `mp_triton_wrapper`'s closure (attn_replacer.py:334-365) for the integer quantiser
+    types, as one call into the HIP library: key centring, per-token 8-bit (and 4-bit) fake quantisation of
+    query and centred key, per-channel 8-bit fake quantisation of value -- without expanding the kv heads.
+
+    query [B,N,Hq,D], key/value [B,N,Hkv,D] for "NHD" ([B,H,N,D] for "HND"), bf16 or fp16, D == 128.
+    Returns (q8, q4, k8, k4, v8) in the layout of the inputs; q4 and k4 are None unless `want_4bit`.
+    """
+    from .. import _native as N
+    from ._common import require_gpu
+
+    if tensor_layout not in N.LAYOUT:
+        raise ValueError(f"tensor_layout {tensor_layout} not supported")
+    require_gpu(query, key, value)
+    assert query.stride(-1) == 1 and key.stride(-1) == 1 and value.stride(-1) == 1, "Last dim of qkv must be contiguous."
+    if query.size(-1) != 128:
+        raise ValueError(f"Unsupported head_dim for the fused pre-pass: {query.size(-1)}")
+    hdim, ndim = (1, 2) if tensor_layout == "HND" else (2, 1)
+    B, Hkv, Nk = key.size(0), key.size(hdim), key.size(ndim)
+    lib = N.lib()
+    q8, k8, v8 = torch.empty_like(query), torch.empty_like(key), torch.empty_like(value)
+    q4 = torch.empty_like(query) if want_4bit else None
+    k4 = torch.empty_like(key) if want_4bit else None
+    need = lib.sq_fake_quant_prepass_workspace_bytes(B, Hkv, Nk)
+    ws = torch.empty((need + 7) // 8, dtype=torch.float64, device=query.device)
+    b = [N.dl(t) for t in (query, key, value, q8, q4, k8, k4, v8, ws)]
+    N.check(lib.sq_fake_quant_prepass(*[N.ptr(x) for x in b], N.LAYOUT[tensor_layout], N.current_stream(query.device)))
+    return q8, q4, k8, k4, v8

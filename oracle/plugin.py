@@ -33,6 +33,27 @@ def _v_quant(x, qtype: str):
     raise ValueError(f"Invalid quantization type: {qtype}")
 
 
+def key_mean_exact(key_hnd: torch.Tensor) -> torch.Tensor:
+    """Token mean of an HND key tensor as the fused pre-pass defines it: the exact sum (fp64; exact for 16-bit
+    inputs of ordinary range), divided by N, rounded to fp32 and then to the tensor dtype.  `Tensor.mean` of the
+    reference (attn_replacer.py:338-339) accumulates in an implementation-defined order and can differ from it by
+    one unit in the last place of the 16-bit result at near-ties."""
+    n = key_hnd.shape[2]
+    return (key_hnd.double().sum(dim=2, keepdim=True) / n).float().to(key_hnd.dtype)
+
+
+def int_prepass(query, key, value, want_4bit=True):
+    """CPU restatement of the operand pre-pass for the integer quantisers (attn_replacer.py:334-365) without the
+    GQA expansion (which repeats heads and changes no value): inputs NHD `[B,N,H,D]`, outputs NHD
+    `(q8, q4, k8, k4, v8)`; q4/k4 None unless `want_4bit`."""
+    q, k, v = (t.permute(0, 2, 1, 3) for t in (query, key, value))   # HND views, as the reference quantises them
+    kc = k - key_mean_exact(k)
+    outs = [FQ.int_fake_quant(q, 8, True, "per_token"), FQ.int_fake_quant(q, 4, True, "per_token") if want_4bit else None,
+            FQ.int_fake_quant(kc, 8, True, "per_token"), FQ.int_fake_quant(kc, 4, True, "per_token") if want_4bit else None,
+            FQ.int_fake_quant(v, 8, True, "per_channel")]
+    return tuple(None if t is None else t.permute(0, 2, 1, 3).contiguous() for t in outs)
+
+
 def plugin_attention(query, key, value, *, num_kv_groups, bit8, bit4, sink, relative,
                      qk_qtype="int", v_qtype="int", p_quant=A.P_NONE):
     """query [B,N,Hq,D], key/value [B,N,Hkv,D] (bf16) -> [B,N,Hq*D] bf16.
@@ -47,7 +68,7 @@ def plugin_attention(query, key, value, *, num_kv_groups, bit8, bit4, sink, rela
     k = repeat_kv(key, num_kv_groups)
     v = repeat_kv(value, num_kv_groups)
     q = query.permute(0, 2, 1, 3)
-    k = k - k.mean(dim=2, keepdim=True)
+    k = k - (key_mean_exact(k) if qk_qtype == "int" and v_qtype == "int" else k.mean(dim=2, keepdim=True))
     q8, q4 = _qk_quant(q, qk_qtype, 8), _qk_quant(q, qk_qtype, 4)
     k8, k4 = _qk_quant(k, qk_qtype, 8), _qk_quant(k, qk_qtype, 4)
     v8 = _v_quant(v, v_qtype)
