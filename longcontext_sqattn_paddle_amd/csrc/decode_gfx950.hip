@@ -119,27 +119,6 @@ __global__ __launch_bounds__(kWaves * 64) void decode_splitkv_kernel(DecodeArgs 
     return;
   }
 
-  // Q~ fragments (B operand): lane (col head r, k-group g) holds q~[r][32kk+8g .. +7]
-  uint4 qf[4];
-  {
-    const uint16_t* qp = (const uint16_t*)a.q + (int64_t)b * a.q_sb + (int64_t)(hq0 + r) * a.q_sh;
-#pragma unroll
-    for (int kk = 0; kk < 4; ++kk) {
-      uint32_t w[4] = {0, 0, 0, 0};
-      if (r < nh) {
-        const uint4 raw = *(const uint4*)(qp + 32 * kk + 8 * g);
-        const uint32_t in[4] = {raw.x, raw.y, raw.z, raw.w};
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const float lo = elem_to_f32<BF16>(in[j] & 0xffffu) * a.sm;
-          const float hi = elem_to_f32<BF16>(in[j] >> 16) * a.sm;
-          w[j] = f32_to_elem<BF16>(lo) | (f32_to_elem<BF16>(hi) << 16);
-        }
-      }
-      qf[kk] = make_uint4(w[0], w[1], w[2], w[3]);
-    }
-  }
-
   const uint16_t* kbase = (const uint16_t*)a.k + (int64_t)b * a.k_sb + (int64_t)kvh * a.k_sh;
   const uint16_t* vbase = (const uint16_t*)a.v + (int64_t)b * a.v_sb + (int64_t)kvh * a.v_sh;
 
@@ -162,6 +141,37 @@ __global__ __launch_bounds__(kWaves * 64) void decode_splitkv_kernel(DecodeArgs 
       vf[i] = stream_load(vbase + (int64_t)tv * a.v_sn + 8 * r);
     }
   };
+  // four register sets: the loads of the wave's next three tiles are in flight while it works on the current one
+  // (a workgroup of a 128K-token cache only has 16 tiles).  The first loads are issued before the query is
+  // fetched and scaled, so that the two latencies overlap.
+  constexpr int kSets = 4;
+  uint4 kR[kSets][4], vR[kSets][4];
+  int tile = wsub;
+#pragma unroll
+  for (int u = 0; u < kSets - 1; ++u)
+    if (tile + u * wpg < ntiles) load_tile(tile + u * wpg, kR[u], vR[u]);
+
+  // Q~ fragments (B operand): lane (col head r, k-group g) holds q~[r][32kk+8g .. +7]
+  uint4 qf[4];
+  {
+    const uint16_t* qp = (const uint16_t*)a.q + (int64_t)b * a.q_sb + (int64_t)(hq0 + r) * a.q_sh;
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      uint32_t w[4] = {0, 0, 0, 0};
+      if (r < nh) {
+        const uint4 raw = *(const uint4*)(qp + 32 * kk + 8 * g);
+        const uint32_t in[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float lo = elem_to_f32<BF16>(in[j] & 0xffffu) * a.sm;
+          const float hi = elem_to_f32<BF16>(in[j] >> 16) * a.sm;
+          w[j] = f32_to_elem<BF16>(lo) | (f32_to_elem<BF16>(hi) << 16);
+        }
+      }
+      qf[kk] = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+  }
+
   auto compute_tile = [&](int tile, const uint4 (&kf)[4], const uint4 (&vf)[4]) {
     const int n0 = (split + tile * a.num_splits) * kTile;
     f32x4_t s = {0.f, 0.f, 0.f, 0.f};
@@ -205,19 +215,15 @@ __global__ __launch_bounds__(kWaves * 64) void decode_splitkv_kernel(DecodeArgs 
     }
     m = m_new;
   };
-  // two register sets: the loads of the wave's next tile are in flight while it works on the current one
-  uint4 kA[4], vA[4], kB[4], vB[4];
-  int tile = wsub;
-  if (tile < ntiles) load_tile(tile, kA, vA);
   while (tile < ntiles) {
-    const int t2 = tile + wpg;
-    if (t2 < ntiles) load_tile(t2, kB, vB);
-    compute_tile(tile, kA, vA);
-    if (t2 >= ntiles) break;
-    const int t3 = t2 + wpg;
-    if (t3 < ntiles) load_tile(t3, kA, vA);
-    compute_tile(t2, kB, vB);
-    tile = t3;
+#pragma unroll
+    for (int u = 0; u < kSets; ++u) {
+      const int tn = tile + (kSets - 1) * wpg;
+      if (tn < ntiles) load_tile(tn, kR[(u + kSets - 1) % kSets], vR[(u + kSets - 1) % kSets]);
+      compute_tile(tile, kR[u], vR[u]);
+      tile += wpg;
+      if (tile >= ntiles) break;
+    }
   }
 
   // fold the 4 lane groups' shares of l, then merge the waves that share a kv head through LDS
@@ -232,8 +238,9 @@ __global__ __launch_bounds__(kWaves * 64) void decode_splitkv_kernel(DecodeArgs 
     s_l[wave][r] = l;
   }
   __syncthreads();
-  for (int idx = threadIdx.x; idx < a.hpw * nh * kD; idx += blockDim.x) {
-    const int hs = idx / (nh * kD), h = (idx / kD) % nh, d = idx % kD;
+  for (int hs = 0; hs < a.hpw; ++hs)
+  for (int idx = threadIdx.x; idx < nh * kD; idx += blockDim.x) {
+    const int h = idx >> 7, d = idx & (kD - 1);
     const int w0 = hs * wpg;
     float mm = -INFINITY;
     for (int w = 0; w < wpg; ++w) mm = fmaxf(mm, s_m[w0 + w][h]);
@@ -260,12 +267,13 @@ struct CombineArgs {
 };
 
 constexpr int kCombineThreads = 1024;
-constexpr int kCombineGroups = kCombineThreads / kD;   // 8 groups of 128 threads, each sums every 8th split
+constexpr int kCombineChunk = 32;                       // output channels per workgroup
+constexpr int kCombineGroups = kCombineThreads / kCombineChunk;   // 32 groups of 32 threads, each sums every 32nd split
 
 // One workgroup per (q head, batch): weights of all splits are formed in parallel in LDS, then 8 groups of 128
 // threads (one thread per output channel) each sum an eighth of the splits with independent, unrolled loads.
 __global__ __launch_bounds__(kCombineThreads) void decode_combine_kernel(CombineArgs a) {
-  extern __shared__ float s_w[];          // [num_splits] weights, then [8][128] partial outputs
+  extern __shared__ float s_w[];          // [num_splits] weights, then [32][32] partial outputs
   __shared__ float s_red[kCombineThreads];
   const int h = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
   const int S = a.num_splits;
@@ -293,7 +301,8 @@ __global__ __launch_bounds__(kCombineThreads) void decode_combine_kernel(Combine
     __syncthreads();
   }
   tot = s_red[0];
-  const int d = tid & (kD - 1), grp = tid >> 7;
+  const int dl = tid & (kCombineChunk - 1), grp = tid / kCombineChunk;
+  const int d = blockIdx.z * kCombineChunk + dl;
   const float* po = a.part_o + row0 * kD + d;
   constexpr int G = kCombineGroups;
   float o = 0.f;
@@ -306,12 +315,12 @@ __global__ __launch_bounds__(kCombineThreads) void decode_combine_kernel(Combine
   }
   for (; s < S; s += G) o += s_w[s] * po[(int64_t)s * kD];
   float* s_part = s_w + S;
-  s_part[grp * kD + d] = o;
+  s_part[grp * kCombineChunk + dl] = o;
   __syncthreads();
   if (grp == 0) {
     o = 0.f;
 #pragma unroll
-    for (int q = 0; q < G; ++q) o += s_part[q * kD + d];
+    for (int q = 0; q < G; ++q) o += s_part[q * kCombineChunk + dl];
     o = (tot > 0.f) ? o / tot : 0.f;
     const int64_t off = (int64_t)b * a.o_sb + (int64_t)h * a.o_sh + d;
     if (a.out_dtype == 0) {
@@ -460,7 +469,8 @@ extern "C" int sq_decode_fwd(const DLTensor* q, const DLTensor* kcache, const DL
   c.Hq = (int32_t)Hq;
   c.num_splits = S;
   c.out_dtype = odt == DType::BF16 ? 0 : (odt == DType::F16 ? 1 : 2);
-  hipLaunchKernelGGL(decode_combine_kernel, dim3((unsigned)Hq, (unsigned)B), dim3(kCombineThreads), (size_t)(S + kCombineGroups * kD) * sizeof(float), st, c);
+  hipLaunchKernelGGL(decode_combine_kernel, dim3((unsigned)Hq, (unsigned)B, kD / kCombineChunk), dim3(kCombineThreads),
+                     (size_t)(S + kCombineGroups * kCombineChunk) * sizeof(float), st, c);
   SQ_HIP(hipGetLastError());
   return SQ_OK;
 }
