@@ -295,6 +295,12 @@ __device__ __forceinline__ float xor32_sum(float v) {
 #ifndef SQ_LDS_DEPTH
 #define SQ_LDS_DEPTH 4
 #endif
+#ifndef SQ_LDS_DEPTH_F16
+#define SQ_LDS_DEPTH_F16 2
+#endif
+#ifndef SQ_STATIC_RING
+#define SQ_STATIC_RING 1
+#endif
 constexpr float kLog2_448 = 8.807354922057604f;  // log2(448)
 
 // ---- hand-scheduled LDS reads.  The compiler cannot tell that a ds_read never touches the buffers that
@@ -514,7 +520,9 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
       const uint8_t* vsrc8 = a.vt8 + (((int64_t)b * a.Hkv + kvh) * a.nT + j) * (int64_t)(kD * kBN);
       const int vr = 16 * wave + (lane >> 2);
       const int vc = (lane & 3) ^ ((vr >> 2) & 3);
-      __builtin_amdgcn_global_load_lds((const void*)(vsrc8 + vr * kBN + 16 * vc), (lds_ptr_t)(vbuf + wave * 1024), 16, 0, 0);
+      uint32_t off = (uint32_t)(vr * kBN + 16 * vc);
+      asm volatile("" : "+v"(off));   // 32-bit per-lane offset next to the uniform 64-bit tile base
+      __builtin_amdgcn_global_load_lds((const void*)(vsrc8 + off), (lds_ptr_t)(vbuf + wave * 1024), 16, 0, 0);
       return;
     }
     const _Float16* vsrc = vt_base + (int64_t)j * (kD * kBN);
@@ -542,8 +550,11 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
     const char* base = k_bytes + (uint64_t)(uint32_t)j * k_tile_bytes;
     char* kbuf = kbase_lds + stage * kKTileBytes;
 #pragma unroll
-    for (int c = 0; c < CH; ++c)
-      __builtin_amdgcn_global_load_lds((const void*)(base + kvoff[c]), (lds_ptr_t)(kbuf + (wave * CH + c) * 1024), 16, 0, 0);
+    for (int c = 0; c < CH; ++c) {
+      uint32_t off = kvoff[c];
+      asm volatile("" : "+v"(off));   // stays a 32-bit per-lane offset next to the uniform 64-bit tile base
+      __builtin_amdgcn_global_load_lds((const void*)(base + off), (lds_ptr_t)(kbuf + (wave * CH + c) * 1024), 16, 0, 0);
+    }
   };
 
   const int ksw = c32 & 15;          // swizzle of this lane's K rows (c32 and c32 + 32 share it)
@@ -552,6 +563,18 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
   // kx0 ^ (kk << 5), and the same holds after adding a ring buffer's base (a multiple of 256; the rings start at
   // LDS address 0)
   const uint32_t kx0 = c32 * kKStride + ((g ^ ksw) << 4);
+  // MODE 4 with the main loop unrolled over the four ring buffers: the LDS address of every fragment is a
+  // per-lane constant plus an immediate offset, so the tile step spends no vector instruction on addresses
+  constexpr bool kStaticRing = SQ_STATIC_RING && MODE != 2;
+  uint32_t kxr[8];
+#pragma unroll
+  for (int kk = 0; kk < 8; ++kk) kxr[kk] = smem_addr + (kx0 ^ (kk << 5));
+  const uint32_t v8lo_base = smem_addr + 4 * kKTileBytes + c32 * 64 + (((2 * g) ^ ((c32 >> 2) & 3)) << 4);
+  const uint32_t v8hi_base = v8lo_base ^ 16;
+  uint32_t vxr[4];   // fp16 V^T fragments: key group m of this lane's rows
+#pragma unroll
+  for (int m = 0; m < 4; ++m)
+    vxr[m] = smem_addr + 4 * kKTileBytes + ((c32 * kVStride + ((g ^ ((c32 >> 1) & 7)) << 4)) ^ (m << 5));
   typedef __attribute__((ext_vector_type(8))) int i32x8_t;
   i32x8_t P8 = {0, 0, 0, 0, 0, 0, 0, 0};   // MODE 4: e4m3 probabilities of the current tile (registers reused tile after tile)
   const int vsw = (c32 >> 1) & 7;    // swizzle of this lane's V^T rows (32 bd + c32)
@@ -596,15 +619,18 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
   // the Q.K^T MFMAs of the following tile (K in knext, result in Snext) are issued in the same straight-line
   // block as the exponentials, conversions and P.V MFMAs, so that the matrix pipe and the vector ALU of this
   // wave work side by side.
-  auto softmax_pv = [&](int j, int it, const char* vbuf, bool masked, f32x16_t (&S)[2], const char* knext, f32x16_t (&Snext)[2]) {
+  auto softmax_pv = [&](auto rg, int j, int it, const char* vbuf, bool masked, f32x16_t (&S)[2], const char* knext, f32x16_t (&Snext)[2]) {
+    constexpr int R = decltype(rg)::value;   // it & 3, known at compile time
     // MODE 4: the first K fragments of the next tile are requested before anything else, so that their LDS
     // latency passes under the row-maximum bookkeeping
     const uint32_t klane = smem_addr + (((it + 1) & 3) * kKTileBytes) + kx0;
     u32x4_t kf[16];
-    constexpr int kDepth = SQ_LDS_DEPTH;   // K fragments are requested this many MFMA slots ahead (even, 2..8)
+    // K fragments are requested this many MFMA slots ahead (even, 2..8); the fp16 P.V modes have fewer registers to spare
+    constexpr int kDepth = (MODE == 4) ? SQ_LDS_DEPTH : SQ_LDS_DEPTH_F16;
     auto kread = [&](auto I) {
       constexpr int i = decltype(I)::value;
-      kf[i] = lds_read128<(i & 1) * 32 * kKStride>(klane ^ ((i >> 1) << 5));
+      if constexpr (kStaticRing) kf[i] = lds_read128<((R + 1) & 3) * kKTileBytes + (i & 1) * 32 * kKStride>(kxr[i >> 1]);
+      else kf[i] = lds_read128<(i & 1) * 32 * kKStride>(klane ^ ((i >> 1) << 5));
     };
     if constexpr (MODE != 2) static_for<0, kDepth>(kread);
     if (masked) {  // causal mask inside the query block's own tiles (attn_triton.py:69-71)
@@ -663,8 +689,9 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
       // the row sum}.  K fragments are read 4 slots ahead of the MFMA that consumes them.
       // P^T is the e4m3 B operand of one K=64 MFMA per 32 output channels: byte 16 bn + i of this lane's
       // 32 bytes is the probability in S[bn][i]; the V^T tiles were permuted to the same key order.
-      const uint32_t vlo_addr = smem_addr + 4 * kKTileBytes + (it & 3) * kVTileBytes + c32 * 64 + (((2 * g) ^ ((c32 >> 2) & 3)) << 4);
-      const uint32_t vhi_addr = vlo_addr ^ 16;
+      constexpr int kVoff = kStaticRing ? R * kVTileBytes : 0;
+      const uint32_t vlo_addr = kStaticRing ? v8lo_base : v8lo_base + (it & 3) * kVTileBytes;
+      const uint32_t vhi_addr = kStaticRing ? v8hi_base : v8hi_base + (it & 3) * kVTileBytes;
       u32x4_t vlo[4], vhi[4];
       static_for<0, 16>([&](auto I) {
         constexpr int i = decltype(I)::value;
@@ -677,8 +704,8 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
           kread(std::integral_constant<int, i + kDepth>{});
         } else {  // the K fragments are all requested: start on the V^T fragments, in the order the P.V slots use them
           constexpr int r = i + kDepth - 16;
-          if constexpr (r & 1) vhi[r >> 1] = lds_read128<(r >> 1) * 2048>(vhi_addr);
-          else vlo[r >> 1] = lds_read128<(r >> 1) * 2048>(vlo_addr);
+          if constexpr (r & 1) vhi[r >> 1] = lds_read128<kVoff + (r >> 1) * 2048>(vhi_addr);
+          else vlo[r >> 1] = lds_read128<kVoff + (r >> 1) * 2048>(vlo_addr);
         }
         constexpr int sb = i >> 3, e = 2 * (i & 7), r = 4 * sb + ((i & 7) >> 1);
         const float p0 = __builtin_amdgcn_exp2f(S[sb][e]), p1 = __builtin_amdgcn_exp2f(S[sb][e + 1]);
@@ -699,8 +726,8 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
                             (int)vhi[bd][0], (int)vhi[bd][1], (int)vhi[bd][2], (int)vhi[bd][3]};
         O[bd] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, P8, O[bd], 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
         if constexpr (issued < 8) {
-          vlo[issued / 2] = lds_read128<(issued / 2) * 2048>(vlo_addr);
-          vhi[issued / 2] = lds_read128<(issued / 2) * 2048>(vhi_addr);
+          vlo[issued / 2] = lds_read128<kVoff + (issued / 2) * 2048>(vlo_addr);
+          vhi[issued / 2] = lds_read128<kVoff + (issued / 2) * 2048>(vhi_addr);
         }
         if constexpr (bd < 2) {
 #pragma unroll
@@ -740,7 +767,8 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
       uint32_t Pw[4][4];
       auto vread = [&](auto I) {
         constexpr int sl = decltype(I)::value;
-        vf[sl] = lds_read128<(sl & 3) * 32 * kVStride>(vlane ^ ((sl >> 2) << 5));
+        if constexpr (kStaticRing) vf[sl] = lds_read128<R * kVTileBytes + (sl & 3) * 32 * kVStride>(vxr[sl >> 2]);
+        else vf[sl] = lds_read128<(sl & 3) * 32 * kVStride>(vlane ^ ((sl >> 2) << 5));
       };
       auto pack_unit = [&](auto U) {   // probabilities 4u .. 4u+3 of the tile (in S order)
         constexpr int u = decltype(U)::value;
@@ -900,7 +928,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
     }
   }
   __syncthreads();   // ring buffer 0 is about to be refilled: every wave has read K(step 0) out of it
-  auto step = [&](int t, f32x16_t (&Scur)[2], f32x16_t (&Snxt)[2]) {
+  auto step = [&](auto rg, int t, f32x16_t (&Scur)[2], f32x16_t (&Snxt)[2]) {   // rg = t & 3
     if ((t & 1) == 0) {   // start of a pair: refill the four buffers the previous pair released
       if (t + 4 < nFull) {
         const int j2 = tile_of(t + 2), j3 = tile_of(t + 3), j4 = tile_of(t + 4);
@@ -928,7 +956,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
     if (vis_cur) {
       // Q.K^T of the next tile is computed even if this wave will not use it (the buffer then holds an older
       // tile or nothing meaningful; the result is dropped): the common path stays free of branches
-      softmax_pv(tile_of(t), t, vbase_lds + (t & 3) * kVTileBytes, t >= fm, Scur, knext, Snxt);
+      softmax_pv(rg, tile_of(t), t, vbase_lds + (t & 3) * kVTileBytes, t >= fm, Scur, knext, Snxt);
     } else {
       if (vis_nxt) {
         qk_tile(knext, Snxt);
@@ -951,9 +979,11 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
   };
   // both steps of a pair always run (the second one idles when the number of steps is odd), so that every wave
   // passes the same barriers
-  for (int t = 0; t < nTot; t += 2) {
-    step(t, Sa, Sb);
-    step(t + 1, Sb, Sa);
+  for (int t = 0; t < nTot; t += 4) {   // unrolled over the four ring buffers (steps past the end idle)
+    step(std::integral_constant<int, 0>{}, t, Sa, Sb);
+    step(std::integral_constant<int, 1>{}, t + 1, Sb, Sa);
+    step(std::integral_constant<int, 2>{}, t + 2, Sa, Sb);
+    step(std::integral_constant<int, 3>{}, t + 3, Sb, Sa);
   }
 
   // ---- epilogue: out = acc / l (attn_triton.py:208-209), lse2 = log2(l) + m (:210-213)
