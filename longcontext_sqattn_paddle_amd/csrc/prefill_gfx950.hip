@@ -693,58 +693,63 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
       const uint32_t vlo_addr = kStaticRing ? v8lo_base : v8lo_base + (it & 3) * kVTileBytes;
       const uint32_t vhi_addr = kStaticRing ? v8hi_base : v8hi_base + (it & 3) * kVTileBytes;
       u32x4_t vlo[4], vhi[4];
+      // Order inside a slot: the wait for the K fragment, the two exponentials, then the MFMA, then the next LDS
+      // request and the pack.  An MFMA placed directly behind an inline-asm statement (the wait or the request)
+      // would get a hazard s_nop from the compiler, 20 per tile.
       static_for<0, 16>([&](auto I) {
         constexpr int i = decltype(I)::value;
         constexpr int bn = i & 1, kk = i >> 1;
         lds_wait<kDepth - 1>(kf[i]);
-        const uint4 ka = make_uint4(kf[i][0], kf[i][1], kf[i][2], kf[i][3]);
-        if constexpr (kk == 0) Snext[bn] = mfma_qk32<BF16>(ka, qf[0], Cinit);
-        else Snext[bn] = mfma_qk32<BF16>(ka, qf[kk], Snext[bn]);
-        if constexpr (i + kDepth < 16) {
-          kread(std::integral_constant<int, i + kDepth>{});
-        } else {  // the K fragments are all requested: start on the V^T fragments, in the order the P.V slots use them
-          constexpr int r = i + kDepth - 16;
-          if constexpr (r & 1) vhi[r >> 1] = lds_read128<kVoff + (r >> 1) * 2048>(vhi_addr);
-          else vlo[r >> 1] = lds_read128<kVoff + (r >> 1) * 2048>(vlo_addr);
-        }
+        __builtin_amdgcn_sched_barrier(0);
         constexpr int sb = i >> 3, e = 2 * (i & 7), r = 4 * sb + ((i & 7) >> 1);
         const float p0 = __builtin_amdgcn_exp2f(S[sb][e]), p1 = __builtin_amdgcn_exp2f(S[sb][e + 1]);
         S[sb][e] = p0;
         S[sb][e + 1] = p1;
+        __builtin_amdgcn_sched_barrier(0);
+        const uint4 ka = make_uint4(kf[i][0], kf[i][1], kf[i][2], kf[i][3]);
+        if constexpr (kk == 0) Snext[bn] = mfma_qk32<BF16>(ka, qf[0], Cinit);
+        else Snext[bn] = mfma_qk32<BF16>(ka, qf[kk], Snext[bn]);
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (i + kDepth < 16) {
+          kread(std::integral_constant<int, i + kDepth>{});
+        } else {  // the K fragments are all requested: start on the V^T fragments, in the order the P.V slots use them
+          constexpr int rr = i + kDepth - 16;
+          if constexpr (rr & 1) vhi[rr >> 1] = lds_read128<kVoff + (rr >> 1) * 2048>(vhi_addr);
+          else vlo[rr >> 1] = lds_read128<kVoff + (rr >> 1) * 2048>(vlo_addr);
+        }
         P8[r] = __builtin_amdgcn_cvt_pk_fp8_f32(p0, p1, P8[r], (i & 1) != 0);
         __builtin_amdgcn_sched_barrier(0);
       });
       // P.V slots: the vector ALU is nearly idle under the four K=64 MFMAs, so the row sum of this tile and the
-      // lane maximum of the next tile's scores are computed here
+      // lane maximum of the next tile's scores are computed here (additions before the MFMA, max3 behind it)
       float ps[2] = {0.f, 0.f}, cm[4];
       static_for<0, 4>([&](auto I) {
         constexpr int bd = decltype(I)::value;
         // requests issued so far: kDepth in the Q.K slots, two more per earlier P.V slot
         constexpr int issued = (kDepth + 2 * bd < 8) ? kDepth + 2 * bd : 8;
         lds_wait<issued - 2 * bd - 2>(vlo[bd], vhi[bd]);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          ps[0] += S[bd >> 1][8 * (bd & 1) + e];
+          ps[1] += S[bd >> 1][8 * (bd & 1) + 4 + e];
+        }
+        __builtin_amdgcn_sched_barrier(0);
         const i32x8_t av = {(int)vlo[bd][0], (int)vlo[bd][1], (int)vlo[bd][2], (int)vlo[bd][3],
                             (int)vhi[bd][0], (int)vhi[bd][1], (int)vhi[bd][2], (int)vhi[bd][3]};
         O[bd] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, P8, O[bd], 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
+        __builtin_amdgcn_sched_barrier(0);
         if constexpr (issued < 8) {
           vlo[issued / 2] = lds_read128<kVoff + (issued / 2) * 2048>(vlo_addr);
           vhi[issued / 2] = lds_read128<kVoff + (issued / 2) * 2048>(vhi_addr);
         }
-        if constexpr (bd < 2) {
-#pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            ps[0] += S[bd][e];
-            ps[1] += S[bd][8 + e];
-          }
-        } else {
-          const f32x16_t& sn = Snext[bd - 2];
-#pragma unroll
-          for (int h = 0; h < 2; ++h) {
-            const int o = 8 * h;
-            float c = max3(sn[o], sn[o + 1], sn[o + 2]);
-            c = max3(c, sn[o + 3], sn[o + 4]);
-            c = max3(c, sn[o + 5], sn[o + 6]);
-            cm[2 * (bd - 2) + h] = max3(c, sn[o + 7], sn[o + 7]);
-          }
+        {   // a quarter of the next tile's scores: Snext[bd >> 1][8 (bd & 1) .. +7]; both halves are complete by now
+          const f32x16_t& sn = Snext[bd >> 1];
+          constexpr int o = 8 * (bd & 1);
+          float c = max3(sn[o], sn[o + 1], sn[o + 2]);
+          c = max3(c, sn[o + 3], sn[o + 4]);
+          c = max3(c, sn[o + 5], sn[o + 6]);
+          cm[bd] = max3(c, sn[o + 7], sn[o + 7]);
         }
         __builtin_amdgcn_sched_barrier(0);
       });
