@@ -6,6 +6,8 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <type_traits>
+
 #include "sqattn.h"
 
 namespace sq {
@@ -102,6 +104,34 @@ __device__ __forceinline__ float e4m3_roundtrip(float x) {
 }
 
 __device__ __forceinline__ float wave_xor_max(float v, int mask) { return fmaxf(v, __shfl_xor(v, mask)); }
+
+// ---- hand-scheduled LDS reads.  The compiler cannot tell that a ds_read never touches the buffers that
+// global_load_lds copies are still filling, so it would stall every tile on vmcnt(0); reads issued through
+// these helpers are invisible to that logic, and the data dependence is carried by lds_wait instead.
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
+template <int OFF>
+__device__ __forceinline__ u32x4_t lds_read128(uint32_t addr) {
+  u32x4_t r;
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF));
+  return r;
+}
+// wait until at most N LDS reads issued after the one that produced x (and y) are outstanding; LDS reads
+// return in order, so x (and y) have landed afterwards
+template <int N>
+__device__ __forceinline__ void lds_wait(u32x4_t& x) {
+  asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(x) : "n"(N));
+}
+template <int N>
+__device__ __forceinline__ void lds_wait(u32x4_t& x, u32x4_t& y) {
+  asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(x), "+v"(y) : "n"(N));
+}
+template <int I, int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for<I + 1, N>(f);
+  }
+}
 #endif
 
 }  // namespace sq

@@ -303,34 +303,6 @@ __device__ __forceinline__ float xor32_sum(float v) {
 #endif
 constexpr float kLog2_448 = 8.807354922057604f;  // log2(448)
 
-// ---- hand-scheduled LDS reads.  The compiler cannot tell that a ds_read never touches the buffers that
-// global_load_lds copies are still filling, so it would stall every tile on vmcnt(0); reads issued through
-// these helpers are invisible to that logic, and the data dependence is carried by lds_wait instead.
-typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
-template <int OFF>
-__device__ __forceinline__ u32x4_t lds_read128(uint32_t addr) {
-  u32x4_t r;
-  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF));
-  return r;
-}
-// wait until at most N LDS reads issued after the one that produced x (and y) are outstanding; LDS reads
-// return in order, so x (and y) have landed afterwards
-template <int N>
-__device__ __forceinline__ void lds_wait(u32x4_t& x) {
-  asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(x) : "n"(N));
-}
-template <int N>
-__device__ __forceinline__ void lds_wait(u32x4_t& x, u32x4_t& y) {
-  asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(x), "+v"(y) : "n"(N));
-}
-template <int I, int N, class F>
-__device__ __forceinline__ void static_for(F&& f) {
-  if constexpr (I < N) {
-    f(std::integral_constant<int, I>{});
-    static_for<I + 1, N>(f);
-  }
-}
-
 // Quantise 8 probabilities (one k-step of the P.V MFMA) and pack them as fp16 B-operand registers.
 //   MODE 0  p.to(fp16)
 //   MODE 1  fp16(e4m3(p*448)/448)   reference static scale (attn_triton.py:81-82): sc = 448, inv = 1/448
