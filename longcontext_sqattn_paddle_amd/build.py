@@ -20,13 +20,30 @@ HIPCC_FLAGS = [
 
 
 def build(verbose: bool = True, extra_flags=()) -> str:
-    """Compile every HIP source into one shared library; returns its path. Always recompiles."""
+    """Compile every HIP source (in parallel, one object each) and link them into one shared library; returns its
+    path.  Always recompiles."""
+    import tempfile
+
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    srcs = [os.path.join(CSRC, s) for s in SOURCES if os.path.exists(os.path.join(CSRC, s))]
-    cmd = [hipcc, *HIPCC_FLAGS, *extra_flags, "-I", INCLUDE, "-I", CSRC, *srcs, "-o", LIB_PATH]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    subprocess.run(cmd, check=True)
+    srcs = [s for s in SOURCES if os.path.exists(os.path.join(CSRC, s))]
+    compile_flags = [f for f in HIPCC_FLAGS if f != "-shared"]
+    with tempfile.TemporaryDirectory(prefix="sqattn_build_") as tmp:
+        jobs = []
+        for s in srcs:
+            obj = os.path.join(tmp, s.replace(".hip", ".o"))
+            cmd = [hipcc, *compile_flags, *extra_flags, "-I", INCLUDE, "-I", CSRC, "-c", os.path.join(CSRC, s), "-o", obj]
+            if verbose:
+                print(" ".join(cmd), flush=True)
+            jobs.append((cmd, obj, subprocess.Popen(cmd)))
+        objs = []
+        for cmd, obj, proc in jobs:
+            if proc.wait() != 0:
+                raise subprocess.CalledProcessError(proc.returncode, cmd)
+            objs.append(obj)
+        link = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", LIB_PATH]
+        if verbose:
+            print(" ".join(link), flush=True)
+        subprocess.run(link, check=True)
     return LIB_PATH
 
 
