@@ -26,8 +26,13 @@ PEAK_MFMA_FP8_TFLOPS = 5000.0    # MI355X dense fp8 MFMA
 PEAK_MFMA_BLEND_TFLOPS = 1.0 / (0.5 / PEAK_MFMA_BF16_TFLOPS + 0.5 / PEAK_MFMA_FP8_TFLOPS)
 PEAK_HBM_GBS = 8000.0            # MI355X HBM3E
 # L2<->fabric bytes of one prefill_kernel launch at seq 131072, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a
-# 1 GiB copy (x2.000 / x1.000): 12.49 GB fetched + 1.00 GB written in P mode 4 (profiles/prefill_kernel_128k.md)
+# 1 GiB copy (x2.000 / x1.000): 12.49 GB fetched + 1.00 GB written in P mode 4; mode 5 moves the same tiles (profiles/prefill_kernel_128k.md)
 PREFILL_TRAFFIC_BYTES_128K = 13.5e9
+P_MODE_NOTE = {
+    0: "no P quantisation",
+    4: "e4m3 P with the static scale 448 and e4m3 V, fp8 MFMA P.V",
+    5: "e4m3 P with a power-of-two block scale per query row and 64-key tile and e4m3 V, block-scaled fp8 MFMA P.V",
+}
 
 
 def log(*a):
@@ -165,10 +170,11 @@ def main():
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--seq-len", type=int, default=131072)
-    ap.add_argument("--p-quant", type=int, default=4,
+    ap.add_argument("--p-quant", type=int, default=5,
                     help="0 none, 1 e4m3 static 448 exactly as the reference rounds it, 2 e4m3 block absmax, "
                          "3 e4m3 static 448 with the scale folded into the exponent, "
-                         "4 (default) = 3 plus e4m3 V so that P.V runs on the fp8 matrix pipe")
+                         "4 = 3 plus e4m3 V so that P.V runs on the fp8 matrix pipe, "
+                         "5 (default) = 4 with one power-of-two block scale per query row and 64-key tile on P")
     ap.add_argument("--variants", action="store_true", help="also time P modes 1 and 3 (fp16 P.V) and report them")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="run one 1 GiB device-to-device copy first: a kernel of known traffic for scaling FETCH_SIZE/WRITE_SIZE")
@@ -197,7 +203,7 @@ def main():
     ms, flops = time_prefill(torch, N, args.steps, args.warmup, args.p_quant)
     tflops = flops / ms / 1e9
     log(f"[bench] prefill N={N}: {ms:.2f} ms/step, {tflops:.1f} TFLOP/s")
-    if args.p_quant == 4:
+    if args.p_quant >= 4:
         peak, peak_note = PEAK_MFMA_BLEND_TFLOPS, "harmonic blend: Q.K^T on bf16 MFMA (2.5 PFLOP/s), P.V on fp8 MFMA (5.0 PFLOP/s)"
     else:
         peak, peak_note = PEAK_MFMA_BF16_TFLOPS, "both GEMMs on 16-bit MFMA"
@@ -218,7 +224,7 @@ def main():
         "config": {
             "workload": f"prefill attention, batch 1, 28 q heads / 4 kv heads, head_dim 128, seq {N}, causal, "
                         f"bf16 N(0,1)/sqrt(128) with 2% K outlier channels x8, P quant mode {args.p_quant} "
-                        f"({'e4m3 P and e4m3 V, fp8 MFMA P.V' if args.p_quant == 4 else 'e4m3 P, fp16 MFMA P.V' if args.p_quant else 'no P quantisation'}), fp32 accumulate",
+                        f"({P_MODE_NOTE.get(args.p_quant, 'e4m3 P, fp16 MFMA P.V')}), fp32 accumulate",
             "flops_per_step": flops,
         },
         "roofline": {
@@ -230,12 +236,12 @@ def main():
             "unit": "TFLOP/s",
             "frac": round(tflops / peak, 4),
             "frac_of_bf16_peak": round(tflops / PEAK_MFMA_BF16_TFLOPS, 4),
-            "traffic": PREFILL_TRAFFIC_BYTES_128K if (N == 131072 and args.p_quant == 4) else None,
+            "traffic": PREFILL_TRAFFIC_BYTES_128K if (N == 131072 and args.p_quant >= 4) else None,
         },
     }
     if args.variants:
         result["variants"] = {}
-        for mode, name in ((3, "e4m3_P_fp16_PV"), (1, "e4m3_P_reference_rounding_fp16_PV")):
+        for mode, name in ((4, "e4m3_P_static_scale_fp8_PV"), (3, "e4m3_P_fp16_PV"), (1, "e4m3_P_reference_rounding_fp16_PV")):
             vms, _ = time_prefill(torch, N, args.steps, args.warmup, mode)
             result["variants"][name] = {"p_quant": mode, "ms_per_step": round(vms, 3), "TFLOP_per_s": round(flops / vms / 1e9, 1)}
             log(f"[bench] prefill variant {name}: {vms:.2f} ms")

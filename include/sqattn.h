@@ -56,9 +56,12 @@ enum {
   SQ_P_E4M3_STATIC_FAST = 3, /* same e4m3 grid as STATIC with the factor 448 folded into the exponent  */
                          /* of p and the 1/448 cancelled against the denominator: skips the       */
                          /* reference's fp16 rounding of p/448 (relative 2^-11), prefill only      */
-  SQ_P_E4M3_FP8_PV = 4   /* e4m3 P as in STATIC_FAST *and* e4m3 V (one scale per batch, kv head and   */
+  SQ_P_E4M3_FP8_PV = 4,  /* e4m3 P as in STATIC_FAST *and* e4m3 V (one scale per batch, kv head and   */
                          /* channel, from a pre-pass): P.V runs on the fp8 matrix pipe.  No reference */
                          /* counterpart (it keeps V in fp16, attn_triton.py:83); prefill only         */
+  SQ_P_E4M3_MX_FP8_PV = 5 /* as FP8_PV with a block scale on P: one power of two per query row and     */
+                         /* 64-key tile, 2^k with k = floor(-log2(largest p of the row in the tile)),  */
+                         /* carried in the scale operand of the block-scaled fp8 MFMA; prefill only   */
 };
 
 enum { SQ_WINDOW_NONE = 0, SQ_WINDOW_SIZES = 1 };

@@ -16,7 +16,7 @@ LIB_PATH = os.path.join(_PKG_DIR, "libsqattn_hip.so")
 
 SQ_OK, SQ_EINVAL, SQ_ESHAPE, SQ_EDEVICE, SQ_EDTYPE, SQ_EUNSUPPORTED, SQ_EHIP, SQ_EWORKSPACE = 0, -1, -2, -3, -4, -5, -6, -7
 LAYOUT = {"HND": 0, "NHD": 1}
-P_NONE, P_E4M3_STATIC, P_E4M3_BLOCK, P_E4M3_STATIC_FAST, P_E4M3_FP8_PV = 0, 1, 2, 3, 4
+P_NONE, P_E4M3_STATIC, P_E4M3_BLOCK, P_E4M3_STATIC_FAST, P_E4M3_FP8_PV, P_E4M3_MX_FP8_PV = 0, 1, 2, 3, 4, 5
 WINDOW_NONE, WINDOW_SIZES = 0, 1
 
 

@@ -486,7 +486,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
   };
   auto stage_v = [&](int j, int stage) {
     char* vbuf = vbase_lds + stage * kVTileBytes;
-    if constexpr (MODE == 4) {
+    if constexpr (MODE >= 4) {
       // e4m3 tile: 128 rows x 64 bytes = 8 KB, one wave instruction per wave; 16-byte chunk c of row d -> slot
       // c ^ ((d >> 2) & 3), which spreads the 16 rows a quarter-wave reads over all 16 bank groups
       const uint8_t* vsrc8 = a.vt8 + (((int64_t)b * a.Hkv + kvh) * a.nT + j) * (int64_t)(kD * kBN);
@@ -549,6 +549,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
     vxr[m] = smem_addr + 4 * kKTileBytes + ((c32 * kVStride + ((g ^ ((c32 >> 1) & 7)) << 4)) ^ (m << 5));
   typedef __attribute__((ext_vector_type(8))) int i32x8_t;
   i32x8_t P8 = {0, 0, 0, 0, 0, 0, 0, 0};   // MODE 4: e4m3 probabilities of the current tile (registers reused tile after tile)
+  int P8w[8] = {0, 0, 0, 0, 0, 0, 0, 0};   // MODE 5: the same as eight scalars
   const int vsw = (c32 >> 1) & 7;    // swizzle of this lane's V^T rows (32 bd + c32)
 
   // S^T = K . Q~^T + Cinit for one tile: 16 MFMAs that nothing below depends on until the next step
@@ -586,6 +587,11 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
   // whether any row's maximum moved; both computed one step ahead, under the P.V MFMAs
   float tmax_row = 0.f;
   bool moved = false;
+  // MODE 5: block scale of a row's 64 probabilities in a tile, 2^k with k = floor(log2 448 - t) in [0, 60] for the
+  // row maximum t of the scores (which carry log2 448); kept as the E8M0 exponent 127 - k = ceil(t + 127 - log2 448)
+  // of 2^-k.  Computed one step ahead like tmax_row, again after a shift of the reference.
+  auto block_exp = [](float t) { return (int)__builtin_ceilf(__builtin_amdgcn_fmed3f(t + (127.f - kC), 67.f, 127.f)); };
+  int e_row = 127;
 
   // softmax update + P.V for the tile whose scores are in S.  Once the running maximum of this tile is settled,
   // the Q.K^T MFMAs of the following tile (K in knext, result in Snext) are issued in the same straight-line
@@ -598,7 +604,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
     const uint32_t klane = smem_addr + (((it + 1) & 3) * kKTileBytes) + kx0;
     u32x4_t kf[16];
     // K fragments are requested this many MFMA slots ahead (even, 2..8); the fp16 P.V modes have fewer registers to spare
-    constexpr int kDepth = (MODE == 4) ? SQ_LDS_DEPTH : SQ_LDS_DEPTH_F16;
+    constexpr int kDepth = (MODE >= 4) ? SQ_LDS_DEPTH : SQ_LDS_DEPTH_F16;
     auto kread = [&](auto I) {
       constexpr int i = decltype(I)::value;
       if constexpr (kStaticRing) kf[i] = lds_read128<((R + 1) & 3) * kKTileBytes + (i & 1) * 32 * kKStride>(kxr[i >> 1]);
@@ -624,6 +630,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
       if (masked) {
         tmax_row = xor32_max(lane_max(S));
         moved = __any(tmax_row > kC);
+        if constexpr (MODE == 5) e_row = block_exp(tmax_row);
       }
       tmax = tmax_row;   // came out of the previous step's P.V phase
       slow = first || moved;
@@ -643,6 +650,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
       const float alpha = first ? 0.f : __builtin_amdgcn_exp2f(-d);
       m_run += d;
       l_run *= alpha;
+      if constexpr (MODE == 5) e_row = block_exp(tmax - d);
 #pragma unroll
       for (int bn = 0; bn < 2; ++bn)
 #pragma unroll
@@ -654,7 +662,11 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
       for (int i = 0; i < 16; ++i) Cinit[i] = c;
       first = false;
     }
-    if constexpr (MODE == 4) {
+    if constexpr (MODE >= 4) {
+      // MODE 5: the pack divides by 2^-k, the MFMA multiplies this lane's 32 values by 2^-k again (E8M0 scale in
+      // byte 0 of the operand).  MODE 4: k = 0.
+      const int mfma_scale_b = (MODE == 5) ? e_row : 0x7f7f7f7f;
+      const float pack_scale = __int_as_float(mfma_scale_b << 23);
       __builtin_amdgcn_s_setprio(0);
       // Hand-scheduled tile step.  16 slots of {Q.K^T MFMA of the next tile, one LDS prefetch, two exponentials
       // and one e4m3 pack of the current tile}, then 4 slots of {fp8 P.V MFMA, two LDS prefetches, 8 additions of
@@ -689,7 +701,16 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
           if constexpr (rr & 1) vhi[rr >> 1] = lds_read128<kVoff + (rr >> 1) * 2048>(vhi_addr);
           else vlo[rr >> 1] = lds_read128<kVoff + (rr >> 1) * 2048>(vlo_addr);
         }
-        P8[r] = __builtin_amdgcn_cvt_pk_fp8_f32(p0, p1, P8[r], (i & 1) != 0);
+        if constexpr (MODE == 5) {
+          typedef __attribute__((ext_vector_type(2))) short i16x2_t;
+          // The half of the word that is not written comes from the first operand.  With the words kept as elements
+          // of a vector, every element's old value came out as element 0's (a wrong fold of the element extraction
+          // with the cast to two shorts), hence eight scalars here.
+          P8w[r] = __builtin_bit_cast(int, __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(__builtin_bit_cast(i16x2_t, P8w[r]), p0, p1,
+                                                                                  pack_scale, (i & 1) != 0));
+        } else {
+          P8[r] = __builtin_amdgcn_cvt_pk_fp8_f32(p0, p1, P8[r], (i & 1) != 0);
+        }
         __builtin_amdgcn_sched_barrier(0);
       });
       // P.V slots: the vector ALU is nearly idle under the four K=64 MFMAs, so the row sum of this tile and the
@@ -709,26 +730,39 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
         __builtin_amdgcn_sched_barrier(0);
         const i32x8_t av = {(int)vlo[bd][0], (int)vlo[bd][1], (int)vlo[bd][2], (int)vlo[bd][3],
                             (int)vhi[bd][0], (int)vhi[bd][1], (int)vhi[bd][2], (int)vhi[bd][3]};
-        O[bd] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, P8, O[bd], 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
+        if constexpr (MODE == 5) {
+          const i32x8_t pb = {P8w[0], P8w[1], P8w[2], P8w[3], P8w[4], P8w[5], P8w[6], P8w[7]};
+          O[bd] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, pb, O[bd], 0, 0, 0, 0x7f7f7f7f, 0, mfma_scale_b);
+        } else {
+          O[bd] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, P8, O[bd], 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
+        }
         __builtin_amdgcn_sched_barrier(0);
         if constexpr (issued < 8) {
           vlo[issued / 2] = lds_read128<kVoff + (issued / 2) * 2048>(vlo_addr);
           vhi[issued / 2] = lds_read128<kVoff + (issued / 2) * 2048>(vhi_addr);
         }
-        {   // a quarter of the next tile's scores: Snext[bd >> 1][8 (bd & 1) .. +7]; both halves are complete by now
+        if constexpr (bd < 3) {
+          // a quarter of the next tile's scores: Snext[bd >> 1][8 (bd & 1) .. +7]; both halves are complete by now.
+          // The fourth quarter is spread over the first three slots, so that only the final reduction is left
+          // behind the last MFMA.
           const f32x16_t& sn = Snext[bd >> 1];
           constexpr int o = 8 * (bd & 1);
           float c = max3(sn[o], sn[o + 1], sn[o + 2]);
           c = max3(c, sn[o + 3], sn[o + 4]);
           c = max3(c, sn[o + 5], sn[o + 6]);
           cm[bd] = max3(c, sn[o + 7], sn[o + 7]);
+          const f32x16_t& s3 = Snext[1];
+          if constexpr (bd == 0) cm[3] = max3(s3[8], s3[9], s3[10]);
+          if constexpr (bd == 1) cm[3] = max3(cm[3], s3[11], s3[12]);
+          if constexpr (bd == 2) cm[3] = max3(max3(cm[3], s3[13], s3[14]), s3[15], s3[15]);
         }
         __builtin_amdgcn_sched_barrier(0);
       });
+      // (placing this reduction in the third slot as well, ahead of the last MFMA, measured 0.8 % slower)
       tmax_row = xor32_max(max3(max3(cm[0], cm[1], cm[2]), cm[3], cm[3]));
+      l_run += ps[0] + ps[1];
       moved = __any(tmax_row > kC);
-      const float psum = ps[0] + ps[1];
-      l_run += psum;
+      if constexpr (MODE == 5) e_row = block_exp(tmax_row);
       __builtin_amdgcn_s_setprio(3);
       return;
     }
@@ -838,7 +872,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
 #pragma unroll
     for (int bn = 0; bn < 2; ++bn)
 #pragma unroll
-      for (int t = 0; t < 2; ++t) P[bn][t] = quant_pack8<(MODE == 4 ? 3 : MODE)>(S[bn], t, sc, inv);
+      for (int t = 0; t < 2; ++t) P[bn][t] = quant_pack8<(MODE >= 4 ? 3 : MODE)>(S[bn], t, sc, inv);
     // O^T[d, row] += V^T[d, key] . P^T[key, row]
 #pragma unroll
     for (int bd = 0; bd < 4; ++bd)
@@ -902,6 +936,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
       mfma_settle(Sa[0], Sa[1]);
       tmax_row = xor32_max(lane_max(Sa));
       moved = __any(tmax_row > kC);
+      if constexpr (MODE == 5) e_row = block_exp(tmax_row);
     }
   }
   __syncthreads();   // ring buffer 0 is about to be refilled: every wave has read K(step 0) out of it
@@ -941,6 +976,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
           mfma_settle(Snxt[0], Snxt[1]);
           tmax_row = xor32_max(lane_max(Snxt));
           moved = __any(tmax_row > kC);
+          if constexpr (MODE == 5) e_row = block_exp(tmax_row);
         }
       }
       if constexpr (MODE == 2) {
@@ -977,7 +1013,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
       float v[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) v[e] = O[bd][4 * i4 + e] / l;
-      if constexpr (MODE == 4) {  // undo the per-channel V scale
+      if constexpr (MODE >= 4) {  // undo the per-channel V scale
         const float4 isc = *(const float4*)(a.v_inv_scale + ((int64_t)b * a.Hkv + kvh) * kD + d);
         v[0] *= isc.x;
         v[1] *= isc.y;
@@ -1019,7 +1055,7 @@ extern "C" int sq_prefill_fwd(const DLTensor* q, const DLTensor* k, const DLTens
   SQ_REQUIRE(p, SQ_EINVAL, "sq_prefill_fwd: params is null");
   SQ_REQUIRE(q && k && v && out, SQ_EINVAL, "sq_prefill_fwd: q, k, v and out must be non-null");
   SQ_REQUIRE(p->layout == SQ_LAYOUT_HND || p->layout == SQ_LAYOUT_NHD, SQ_EINVAL, "tensor_layout %d not supported", p->layout);
-  SQ_REQUIRE(p->p_quant >= SQ_P_NONE && p->p_quant <= SQ_P_E4M3_FP8_PV, SQ_EINVAL, "sq_prefill_fwd: p_quant %d not supported", p->p_quant);
+  SQ_REQUIRE(p->p_quant >= SQ_P_NONE && p->p_quant <= SQ_P_E4M3_MX_FP8_PV, SQ_EINVAL, "sq_prefill_fwd: p_quant %d not supported", p->p_quant);
   SQ_REQUIRE((q4 == nullptr) == (k4 == nullptr), SQ_EINVAL, "sq_prefill_fwd: q4 and k4 must be given together");
   int rc;
   const int dev = q->device.device_id;
@@ -1087,7 +1123,7 @@ extern "C" int sq_prefill_fwd(const DLTensor* q, const DLTensor* k, const DLTens
     SQ_REQUIRE(p->window_mode == SQ_WINDOW_NONE, SQ_EINVAL, "sq_prefill_fwd: window_mode %d not supported", p->window_mode);
     SQ_REQUIRE(!q4, SQ_EINVAL, "sq_prefill_fwd: q4/k4 only apply to window mode");
   }
-  SQ_REQUIRE(!(p->p_quant == SQ_P_E4M3_FP8_PV && q4), SQ_EUNSUPPORTED,
+  SQ_REQUIRE(!(p->p_quant >= SQ_P_E4M3_FP8_PV && q4), SQ_EUNSUPPORTED,
              "sq_prefill_fwd: the fp8 P.V mode does not take separate 4-bit operands");
   const size_t need = sq_prefill_workspace_bytes(B, Hkv, Nk, D);
   SQ_REQUIRE(workspace && on_gpu(workspace) && workspace->device.device_id == dev, SQ_EWORKSPACE,
@@ -1102,7 +1138,7 @@ extern "C" int sq_prefill_fwd(const DLTensor* q, const DLTensor* k, const DLTens
   SQ_REQUIRE(cur == dev, SQ_EDEVICE, "sq_prefill_fwd: tensors live on device %d but the current device is %d", dev, cur);
 
   const int nT = (int)((Nk + kBN - 1) / kBN);
-  const bool pv8 = p->p_quant == SQ_P_E4M3_FP8_PV;
+  const bool pv8 = p->p_quant >= SQ_P_E4M3_FP8_PV;
   char* wsp = data_of(workspace);
   // workspace: fp16 tiles (modes 0-3), or e4m3 tiles (half the size) followed by the per-channel scale tables
   const size_t tiles8 = ((size_t)B * Hkv * nT * (kD * kBN) + 255) / 256 * 256;
@@ -1206,6 +1242,7 @@ extern "C" int sq_prefill_fwd(const DLTensor* q, const DLTensor* k, const DLTens
       case SQ_P_E4M3_STATIC: SQ_LAUNCH_PREFILL(BF, W, 1); break; \
       case SQ_P_E4M3_BLOCK: SQ_LAUNCH_PREFILL(BF, W, 2); break;  \
       case SQ_P_E4M3_FP8_PV: SQ_LAUNCH_PREFILL(BF, 8, 4); break; \
+      case SQ_P_E4M3_MX_FP8_PV: SQ_LAUNCH_PREFILL(BF, 8, 5); break; \
       default: SQ_LAUNCH_PREFILL(BF, W, 3); break;               \
     }                                                           \
   } while (0)

@@ -9,6 +9,10 @@ Followed reference code:
   * `_attn_decode_fwd`, `attn_unified`                     sqattn/attn_triton_decode.py:175-241, 244-361
   * `attn_fwd_inner` + relative wrapper                    sqattn/attn_triton_mix_relative.py:8-99, 309-483
   * `_attn_fwd_inner` + absolute wrapper                   sqattn/attn_triton_mix_bad.py:9-98, 285-426
+
+Parity unpinned (build-defined, no reference counterpart; pinned only by their definitions' invariants in
+tests/test_oracle_attention.py and by exact attention): P modes `P_BLOCK_ABSMAX`, `P_STATIC448_GRID`, `P_MX_ROW`
+and `v_quant="e4m3_channel"`.
 """
 from __future__ import annotations
 
@@ -22,6 +26,7 @@ BLOCK_N = 64        # KV block of every reference prefill/decode kernel (attn_tr
 MASK_ADD = -1000000.0  # additive causal mask (attn_triton.py:71)
 
 P_NONE, P_STATIC448, P_BLOCK_ABSMAX, P_STATIC448_GRID = 0, 1, 2, 3
+P_MX_ROW = 5   # e4m3 with one power-of-two scale per query row and 64-key tile (block-scaled fp8 MFMA operand)
 
 
 # --------------------------------------------------------------------------- helpers
@@ -79,6 +84,7 @@ def _quant_p(p: torch.Tensor, mode: int, group_rows: int = 64) -> torch.Tensor:
     mode 2: per (64-row group x 64-col block) absmax scale a: `e4m3(p*(448/a)) * (a/448)` then fp16
             (build-defined generalisation; a == 1 reproduces mode 1 up to the fp16 divide).
     mode 3: `e4m3(p*448)/448` kept in fp32 (build-defined: P as the fp8 operand of an fp8 P.V product).
+    mode 5: as mode 3 with a power-of-two scale per row of the tile (build-defined, see below).
     Returns fp32 values that are exactly representable in fp16.
     """
     if mode == P_NONE:
@@ -88,6 +94,14 @@ def _quant_p(p: torch.Tensor, mode: int, group_rows: int = 64) -> torch.Tensor:
         return (p8.to(torch.float16) / 448).float()
     if mode == P_STATIC448_GRID:   # the e4m3 grid of mode 1 without the fp16 rounding of p/448 (fp8 operand of an fp8 MFMA)
         return (p * 448.0).to(torch.float8_e4m3fn).float() / 448.0
+    if mode == P_MX_ROW:
+        # build-defined: scale 2^k per row of the tile with k = floor(-log2(row maximum)) in [0, 60], so that the
+        # row's largest scaled probability lies in (224, 448]; the dequantised value is e4m3(p*448*2^k) / (448*2^k)
+        a = p.max(dim=1, keepdim=True).values
+        k = torch.floor(-torch.log2(a)).clamp(0.0, 60.0)
+        k = torch.where(a > 0, k, torch.full_like(k, 60.0))
+        sc = torch.exp2(k) * 448.0
+        return (p * sc).to(torch.float8_e4m3fn).float() / sc
     if mode == P_BLOCK_ABSMAX:
         out = torch.empty_like(p)
         for r0 in range(0, p.shape[0], group_rows):

@@ -60,18 +60,21 @@ def test_causal_matches_oracle(B, Hq, Hkv, N, mode):
     assert _cos(out.cpu(), exact) >= 0.999
 
 
+@pytest.mark.parametrize("mode", [4, 5])
 @pytest.mark.parametrize("B,Hq,Hkv,N,layout", [(1, 4, 2, 512, "HND"), (2, 14, 2, 700, "NHD"), (1, 7, 1, 2048, "HND")])
-def test_fp8_pv_mode_matches_oracle(B, Hq, Hkv, N, layout):
-    """Mode 4 (no reference counterpart): e4m3 P *and* e4m3 V (per batch/kv-head/channel scale) on the fp8 MFMA."""
+def test_fp8_pv_mode_matches_oracle(B, Hq, Hkv, N, layout, mode):
+    """Modes 4 and 5 (no reference counterpart): e4m3 P *and* e4m3 V (per batch/kv-head/channel scale) on the fp8
+    MFMA; mode 5 adds one power-of-two scale per query row and 64-key tile to P."""
     from longcontext_sqattn_paddle_amd.sqattn.attn_triton import attn_causal
 
-    print(f"case prefill fp8-pv B={B} Hq={Hq} Hkv={Hkv} N={N} {layout}", flush=True)
+    print(f"case prefill fp8-pv mode={mode} B={B} Hq={Hq} Hkv={Hkv} N={N} {layout}", flush=True)
     q, k, v = inputs.prefill_inputs(B, Hq, Hkv, N, 128, seed=200 + N) if N == 2048 else _rand(B, Hq, Hkv, N, 128, 200 + N)
-    ref, lse_ref = A.prefill_blockwise(q, k, v, p_quant=A.P_STATIC448_GRID, v_quant="e4m3_channel", out_dtype=torch.float32)
+    ref, lse_ref = A.prefill_blockwise(q, k, v, p_quant=A.P_STATIC448_GRID if mode == 4 else A.P_MX_ROW, v_quant="e4m3_channel",
+                                       out_dtype=torch.float32)
     args = [t.to(DEV) for t in (q, k, v)]
     if layout == "NHD":
         args = [t.permute(0, 2, 1, 3).contiguous() for t in args]
-    out, lse = attn_causal(*args, layout, torch.float32, return_lse=True, p_quant=4)
+    out, lse = attn_causal(*args, layout, torch.float32, return_lse=True, p_quant=mode)
     torch.cuda.synchronize()
     if layout == "NHD":
         out = out.permute(0, 2, 1, 3)
@@ -81,6 +84,35 @@ def test_fp8_pv_mode_matches_oracle(B, Hq, Hkv, N, layout):
     assert torch.allclose(lse.cpu(), lse_ref, atol=2e-4)
     exact, _ = A.exact_attention(q, k, v)
     assert _cos(out.cpu(), exact) >= 0.999   # thin margin by construction: e4m3 on both operands (about 0.9995)
+
+
+def test_block_scaled_p_keeps_small_probabilities_the_static_scale_flushes():
+    """Attention sink: key 0 outscores every other key by about 2^17, so all later tiles hold probabilities near
+    2^-17 whose 448-fold lies in the subnormal range of e4m3 (steps of 2^-9) and partly rounds to zero under the
+    static scale (modes 3 and 4), although the 8192 of them together carry a few percent of the row.  The per-row
+    block scale of mode 5 moves each tile's row maximum to (224, 448], i.e. back to three mantissa bits."""
+    from longcontext_sqattn_paddle_amd.sqattn.attn_triton import attn_causal
+
+    N, D = 8192, 128
+    g = torch.Generator().manual_seed(77)
+    q = torch.randn(1, 4, N, D, generator=g) * 0.3
+    k = torch.randn(1, 2, N, D, generator=g) * 0.3
+    v = torch.randn(1, 2, N, D, generator=g)
+    q[..., 0] = 4.0
+    k[..., 0] *= 0.1
+    k[:, :, 0, :] = 0.0
+    k[:, :, 0, 0] = 17.0 / (4.0 * 1.44269504 / D ** 0.5)   # score of key 0 in log2 units: 17 above the rest
+    v[:, :, 0, :] = 0.0   # the sink carries no value, so the output is made of the small probabilities alone
+    q, k, v = q.to(torch.bfloat16), k.to(torch.bfloat16), v.to(torch.bfloat16)
+    exact, _ = A.exact_attention(q, k, v)
+    errs = {}
+    for mode in (3, 4, 5):
+        print(f"case prefill sink mode={mode}", flush=True)
+        out = attn_causal(q.to(DEV), k.to(DEV), v.to(DEV), "HND", torch.float32, p_quant=mode)
+        torch.cuda.synchronize()
+        errs[mode] = float((out.cpu().double()[:, :, N // 2:] - exact[:, :, N // 2:]).pow(2).mean().sqrt())
+    print("rms error vs exact attention, rows N/2..N:", errs, flush=True)
+    assert errs[5] <= 0.5 * errs[4]
 
 
 def test_nhd_layout_bf16_out_and_gqa_7():

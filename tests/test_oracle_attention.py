@@ -138,6 +138,35 @@ def test_fp8_error_levels_against_exact():
         assert torch.allclose(lse.double(), lse_ref, atol=5e-2)
 
 
+def test_block_scaled_p_quantiser_properties():
+    """`P_MX_ROW` (build-defined, no reference counterpart) pinned by what the definition fixes:
+    rows whose maximum lies in (1/2, 1] get scale 1 and equal the static-scale grid; multiplying a row by 2^-j
+    multiplies its result by exactly 2^-j (the scale absorbs it) until the clamp at 2^60; every element within 2^6
+    of its row maximum keeps three mantissa bits (relative error <= 2^-4); a zero row stays zero."""
+    g = torch.Generator().manual_seed(11)
+    p = torch.rand(16, 64, generator=g) * 0.9 + 1e-3
+    p[:, 5] = torch.linspace(0.5001, 1.0, 16)          # row maximum in (1/2, 1]
+    base = A._quant_p(p, A.P_MX_ROW)
+    assert torch.equal(base, A._quant_p(p, A.P_STATIC448_GRID))
+    for j in (1, 7, 16, 40, 59):
+        assert torch.equal(A._quant_p(p * 2.0 ** -j, A.P_MX_ROW), base * 2.0 ** -j), j
+    # the scale is 2^k with k = floor(-log2(max)): a maximum of exactly 2^-9 takes k = 9 and is kept exactly
+    one = torch.zeros(1, 64)
+    one[0, 0] = 2.0 ** -9
+    assert float(A._quant_p(one, A.P_MX_ROW)[0, 0]) == 2.0 ** -9
+    # beyond the clamp the scale stays 2^60 and small values fall off the grid as under any fixed scale
+    tiny = torch.full((1, 64), 2.0 ** -80)
+    assert float(A._quant_p(tiny, A.P_MX_ROW).abs().max()) == 0.0
+    # precision: elements down to 2^-6 of the row maximum are e4m3 normals
+    p2 = torch.rand(32, 64, generator=g) * 2.0 ** -14
+    p2[:, 0] = 2.0 ** -14
+    q2 = A._quant_p(p2, A.P_MX_ROW)
+    big = p2 >= 2.0 ** -20
+    assert float(((q2 - p2).abs() / p2)[big].max()) <= 2.0 ** -4
+    assert float(((A._quant_p(p2, A.P_STATIC448_GRID) - p2).abs() / p2)[big].max()) > 0.2   # what the static scale loses
+    assert torch.equal(A._quant_p(torch.zeros(2, 64), A.P_MX_ROW), torch.zeros(2, 64))
+
+
 def test_window_invariants_and_explicit_mask():
     N, D = 512, 64
     q, k, v = _rand(1, 2, 1, N, N, D, 5)
