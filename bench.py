@@ -26,8 +26,8 @@ PEAK_MFMA_FP8_TFLOPS = 5000.0    # MI355X dense fp8 MFMA
 PEAK_MFMA_BLEND_TFLOPS = 1.0 / (0.5 / PEAK_MFMA_BF16_TFLOPS + 0.5 / PEAK_MFMA_FP8_TFLOPS)
 PEAK_HBM_GBS = 8000.0            # MI355X HBM3E
 # L2<->fabric bytes of one prefill_kernel launch at seq 131072, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a
-# 1 GiB copy (x2.000 / x1.000): 12.49 GB fetched + 1.00 GB written in P mode 4; mode 5 moves the same tiles (profiles/prefill_kernel_128k.md)
-PREFILL_TRAFFIC_BYTES_128K = 13.5e9
+# 1 GiB copy (x2.000 / x1.000): 12.43 GB fetched + 0.94 GB written in P mode 5; mode 4 moves the same tiles (profiles/prefill_kernel_128k.md)
+PREFILL_TRAFFIC_BYTES_128K = 13.4e9
 P_MODE_NOTE = {
     0: "no P quantisation",
     4: "e4m3 P with the static scale 448 and e4m3 V, fp8 MFMA P.V",
