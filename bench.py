@@ -108,6 +108,61 @@ def time_decode(torch, B, L, iters=10, warmup=5, rounds=7):
     return us, nbytes
 
 
+def time_kv_cache(torch, N, iters=10):
+    """The KV cache's two row movements at the benchmark shape (4 kv heads x 128, bf16): the store of an N-token
+    prompt (K and V, each read once and written once) and the append of one token per sequence at batch 8."""
+    from longcontext_sqattn_paddle_amd import _native as Nn
+
+    dev = torch.device("cuda:0")
+    Hkv, D = 4, 128
+    g = torch.Generator(device=dev).manual_seed(5)
+    lib = Nn.lib()
+    st = Nn.current_stream(dev)
+    nset = 2   # alternate source/destination sets: the 256 MB Infinity Cache must not serve the re-read
+    sets = []
+    for _ in range(nset):
+        ks = torch.randn(1, N, Hkv, D, device=dev, generator=g).bfloat16()
+        vs = torch.randn(1, N, Hkv, D, device=dev, generator=g).bfloat16()
+        kc = torch.empty(1, N, Hkv, D, device=dev, dtype=torch.bfloat16)
+        vc = torch.empty(1, N, Hkv, D, device=dev, dtype=torch.bfloat16)
+        sets.append([Nn.dl(t) for t in (ks, vs, kc, vc)])
+    def store(i):
+        Nn.check(lib.sq_kv_cache_store(*[Nn.ptr(x) for x in sets[i % nset]], 0, 0, st))
+    for i in range(2):
+        store(i)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for i in range(iters):
+        store(i)
+    e1.record()
+    torch.cuda.synchronize()
+    store_us = e0.elapsed_time(e1) / iters * 1e3
+    assert torch.equal(sets[0][2].tensor[0, -1], sets[0][0].tensor[0, -1])
+    store_bytes = 2.0 * 2 * N * Hkv * D * 2   # K and V, read + written
+    B, L = 8, 131072
+    kc = torch.empty(B, L, Hkv, D, device=dev, dtype=torch.bfloat16)
+    vc = torch.empty(B, L, Hkv, D, device=dev, dtype=torch.bfloat16)
+    kn = torch.randn(B, 1, Hkv, D, device=dev, generator=g).bfloat16()
+    vn = torch.randn(B, 1, Hkv, D, device=dev, generator=g).bfloat16()
+    lens = torch.full((B,), 1000, device=dev, dtype=torch.int32)
+    att = torch.zeros(B, device=dev, dtype=torch.int32)
+    b = [Nn.dl(t) for t in (kn, vn, kc, vc, lens, att)]
+    ptrs = [Nn.ptr(x) for x in b]
+    for _ in range(5):
+        Nn.check(lib.sq_kv_cache_append(*ptrs, 1, st))
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(100):
+        Nn.check(lib.sq_kv_cache_append(*ptrs, 1, st))
+    e1.record()
+    torch.cuda.synchronize()
+    append_us = e0.elapsed_time(e1) / 100 * 1e3
+    assert int(lens[0].item()) == 1105 and torch.equal(kc[:, 1104], kn[:, 0])
+    return store_us, store_bytes, append_us
+
+
 def time_kmeans(torch, iters=10):
     """One Lloyd iteration (assign + counting sort + exact cluster sums + centroid update) at the benchmark's
     clustering shape: 4 kv heads x 131072 tokens x 128, 1024 centroids."""
@@ -182,6 +237,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode", action="store_true")
     ap.add_argument("--no-prepass", action="store_true")
+    ap.add_argument("--no-kv-cache", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -264,6 +320,13 @@ def main():
             log(f"[bench] plugin pre-pass {name}: {us:.0f} us, {nbytes / us / 1e3:.0f} GB/s")
             torch.cuda.empty_cache()
         result["plugin_prepass"] = pre
+    if not args.no_kv_cache:
+        sus, sbytes, aus = time_kv_cache(torch, N)
+        result["kv_cache"] = {"store_us": round(sus, 1), "store_GB_per_s": round(sbytes / sus / 1e3, 1),
+                              "store_frac_of_hbm_peak": round(sbytes / sus / 1e3 / PEAK_HBM_GBS, 4), "store_bytes": sbytes,
+                              "append_us_batch8": round(aus, 2)}
+        log(f"[bench] kv cache: store of {N} tokens {sus:.0f} us ({sbytes / sus / 1e3:.0f} GB/s), append (batch 8) {aus:.1f} us")
+        torch.cuda.empty_cache()
     if not args.no_kmeans:
         us, kflops, kbytes = time_kmeans(torch)
         result["kmeans"] = {"us_per_iteration": round(us, 1), "TFLOP_per_s": round(kflops / us / 1e6, 1),

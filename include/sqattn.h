@@ -18,6 +18,8 @@
  *   sq_reverse_index          cache_hub/kmeans.py:233-262
  *   sq_index_add              cache_hub/kmeans.py:307-329
  *   sq_topk_select            no reference counterpart (defined by this build's benchmark configuration)
+ *   sq_kv_cache_store         cache_hub/flash_attn_cache.py:153-232 (prefill_update_kv_cache: the two slice copies)
+ *   sq_kv_cache_append        cache_hub/flash_attn_cache.py:239-256 (decode_update_kv_cache)
  *   sq_fake_quant_prepass     sqattn/attn_replacer.py:334-365 (GQA expand, key centring and the five fake-quant
  *                             passes of mp_triton_wrapper's closure), sqattn/fake_quant.py:24-58, 98-125
  */
@@ -163,6 +165,29 @@ size_t sq_fake_quant_prepass_workspace_bytes(int64_t batch, int64_t num_kv_heads
 int sq_fake_quant_prepass(const DLTensor* query, const DLTensor* key, const DLTensor* value, DLTensor* q8,
                           DLTensor* q4, DLTensor* k8, DLTensor* k4, DLTensor* v8, DLTensor* workspace,
                           int32_t layout, void* stream);
+
+/*
+ * Prefill side of the KV cache (cache_hub/flash_attn_cache.py:153-232): rows [valid_start, T) of one sequence's
+ * key_states / value_states [1, T, Hkv, D] go to rows [0, T - valid_start) of sequence `batch_index` of
+ * key_cache / value_cache [B, max_length, Hkv, D] (the per-layer buffers of :60-81, contiguous).  bf16 or fp16,
+ * states and caches of one dtype; the states may be strided views with contiguous D and 16-byte aligned heads.
+ * T > max_length is an error as in the reference (:170-172), so is a batch of more than one sequence (:166-169).
+ */
+int sq_kv_cache_store(const DLTensor* key_states, const DLTensor* value_states, DLTensor* key_cache,
+                      DLTensor* value_cache, int32_t batch_index, int64_t valid_start, void* stream);
+
+/*
+ * Decode side of the KV cache (cache_hub/flash_attn_cache.py:239-256): for every sequence b the new token's
+ * key_states[b, 0] / value_states[b, 0] ([B, 1, Hkv, D]) are written to row valid_length[b] of the caches.
+ * valid_length is int32 [B] on the device and is read there, so the call needs no host synchronisation.
+ * attend_length (int32 [B], may be null) receives valid_length[b] + 1, the number of cached tokens the attention
+ * of this decode step covers (what sq_decode_fwd takes as seqlens).  advance != 0 also stores that value to
+ * valid_length: the reference advances the length once per step, after the last layer (:253-255).  A sequence
+ * whose cache is full (valid_length[b] == max_length) is left unchanged.
+ */
+int sq_kv_cache_append(const DLTensor* key_states, const DLTensor* value_states, DLTensor* key_cache,
+                       DLTensor* value_cache, DLTensor* valid_length, DLTensor* attend_length, int32_t advance,
+                       void* stream);
 
 #ifdef __cplusplus
 }
