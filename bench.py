@@ -108,6 +108,42 @@ def time_decode(torch, B, L, iters=10, warmup=5, rounds=7):
     return us, nbytes
 
 
+def time_decode_selected(torch, B, L, k, iters=20, rounds=5):
+    """Decode attention over k selected tokens per (sequence, kv head) of an L-token cache: the consumer of the
+    k-means top-k selection.  Ids are random and distinct per head, so every row is a separate 256-byte read."""
+    from longcontext_sqattn_paddle_amd import _native as Nn
+
+    dev = torch.device("cuda:0")
+    Hq, Hkv, D = 28, 4, 128
+    g = torch.Generator(device=dev).manual_seed(6)
+    q = torch.randn(B, 1, Hq, D, device=dev, generator=g).bfloat16()
+    kc = torch.randn(B, L, Hkv, D, device=dev, generator=g, dtype=torch.bfloat16)
+    vc = torch.randn(B, L, Hkv, D, device=dev, generator=g, dtype=torch.bfloat16)
+    ids = torch.stack([torch.randperm(L, device=dev, generator=g)[:k] for _ in range(B * Hkv)]).to(torch.int32)
+    lib = Nn.lib()
+    S = lib.sq_decode_num_splits(B, Hkv, k)
+    ws = torch.empty(lib.sq_decode_workspace_bytes(B, Hq, 128, S) // 4, dtype=torch.float32, device=dev)
+    out = torch.empty_like(q)
+    params = Nn.DecodeParams(Nn.LAYOUT["NHD"], Nn.P_NONE, S, 128)
+    b = [Nn.dl(t) for t in (q, kc, vc, ids, None, out, None, ws)]
+    ptrs = [Nn.ptr(x) for x in b]
+    st = Nn.current_stream(dev)
+    for _ in range(5):
+        Nn.check(lib.sq_decode_selected_fwd(*ptrs, params, st))
+    torch.cuda.synchronize()
+    samples = []
+    for _ in range(rounds):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(iters):
+            Nn.check(lib.sq_decode_selected_fwd(*ptrs, params, st))
+        e1.record()
+        torch.cuda.synchronize()
+        samples.append(e0.elapsed_time(e1) / iters * 1e3)
+    assert bool(torch.isfinite(out.float()).all()) and float(out.float().abs().sum()) > 0
+    return sorted(samples)[len(samples) // 2], 2.0 * B * Hkv * k * D * 2
+
+
 def time_kv_cache(torch, N, iters=10):
     """The KV cache's two row movements at the benchmark shape (4 kv heads x 128, bf16): the store of an N-token
     prompt (K and V, each read once and written once) and the append of one token per sequence at batch 8."""
@@ -311,6 +347,13 @@ def main():
             log(f"[bench] decode {name}: {us:.1f} us, {gbs:.0f} GB/s")
             torch.cuda.empty_cache()
         result["decode"] = dec
+        sel = {}
+        for name, B, L, k in (("4096_of_128K_b1", 1, 131072, 4096), ("4096_of_128K_b8", 8, 131072, 4096), ("65536_of_1M_b1", 1, 1048576, 65536)):
+            us, nbytes = time_decode_selected(torch, B, L, k)
+            sel[name] = {"us_per_call": round(us, 2), "GB_per_s": round(nbytes / us / 1e3, 1), "bytes": nbytes}
+            log(f"[bench] decode over selected tokens {name}: {us:.1f} us, {nbytes / us / 1e3:.0f} GB/s")
+            torch.cuda.empty_cache()
+        result["decode_selected"] = sel
     if not args.no_prepass:
         pre = {}
         for name, want4 in (("int8", False), ("int8_int4", True)):

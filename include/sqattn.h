@@ -14,6 +14,7 @@
  *                             sqattn/attn_triton_mix_relative.py:309-483 (launch :439-475),
  *                             sqattn/attn_triton_mix_bad.py:285-426 (launch :388-424)
  *   sq_decode_fwd             sqattn/attn_triton_decode.py:244-361 (decode launch :293-324)
+ *   sq_decode_selected_fwd    no reference counterpart: the same decode over the tokens sq_topk_select picked
  *   sq_kmeans_train           cache_hub/kmeans.py:127-196 (assign launch :147-173, update launch :175-193)
  *   sq_reverse_index          cache_hub/kmeans.py:233-262
  *   sq_index_add              cache_hub/kmeans.py:307-329
@@ -120,6 +121,18 @@ size_t sq_decode_workspace_bytes(int64_t batch, int64_t num_q_heads, int64_t hea
 int sq_decode_fwd(const DLTensor* q, const DLTensor* kcache, const DLTensor* vcache, const DLTensor* seqlens,
                   DLTensor* out, DLTensor* lse, DLTensor* workspace, const sq_decode_params* params,
                   void* stream);
+
+/*
+ * The same decode over a selection of the cache (no reference counterpart; it consumes what sq_topk_select
+ * emits): token_ids int32 [B * Hkv, k], row b * Hkv + kvh lists the cache rows the q heads of kv head kvh of
+ * sequence b attend to, in any order; entries that are negative (the missing tail of a selection) or not below
+ * the cache length are skipped.  seqlens (int32 [B], may be NULL = k) limits each sequence to a prefix of its
+ * lists.  A head with no valid entry gets a zero output and lse = -inf.  Workspace as for sq_decode_fwd with
+ * max_len = k.
+ */
+int sq_decode_selected_fwd(const DLTensor* q, const DLTensor* kcache, const DLTensor* vcache,
+                           const DLTensor* token_ids, const DLTensor* seqlens, DLTensor* out, DLTensor* lse,
+                           DLTensor* workspace, const sq_decode_params* params, void* stream);
 
 /* ---------------------------------------------------------------------------------------- k-means */
 size_t sq_kmeans_workspace_bytes(int64_t groups, int64_t num_tokens, int64_t num_centroids, int64_t dim);

@@ -30,12 +30,15 @@ struct DecodeArgs {
   const void* k;
   const void* v;
   const int32_t* seqlens;
+  const int32_t* ids;   // gather mode: [B * Hkv, L] cache rows to attend to per (sequence, kv head); negative = none
+  int64_t ids_sg;       // its row stride
   float* part_o;    // [B, Hq, S, D] normalised partial outputs
   float* part_lse;  // [B, Hq, S]    base-2 LSE of each partial (-inf = empty)
   int64_t q_sb, q_sh;
   int64_t k_sb, k_sh, k_sn;
   int64_t v_sb, v_sh, v_sn;
   int32_t B, Hq, Hkv, L, group, head_chunks, num_splits, chunk, p_quant;
+  int32_t cache_len;  // gather mode: rows per sequence in the cache (L is then the length of the id lists)
   int32_t hpw;  // kv heads per workgroup (1, 2 or 4): 4/hpw waves share one kv head and interleave its tiles
   float sm;  // log2e / sqrt(D_original), rounded to fp32
 };
@@ -76,7 +79,10 @@ __device__ __forceinline__ f32x4_t mfma_qk(const uint4& a, const uint4& b, f32x4
   }
 }
 
-template <bool BF16>
+// GATHER: token t of the stream is cache row ids[b * Hkv + kvh][t] instead of row t (attention over a selection of
+// the cache, e.g. the tokens of the best-scoring k-means clusters); entries that are negative or beyond the cache
+// are skipped.
+template <bool BF16, bool GATHER>
 __global__ __launch_bounds__(kWaves * 64) void decode_splitkv_kernel(DecodeArgs a) {
   __shared__ float s_o[kWaves][16][kOStride];
   __shared__ float s_m[kWaves][16];
@@ -128,16 +134,28 @@ __global__ __launch_bounds__(kWaves * 64) void decode_splitkv_kernel(DecodeArgs 
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-  // loads are clamped to the last valid token so that nothing past the valid prefix is touched
-  auto load_tile = [&](int tile, uint4 (&kf)[4], uint4 (&vf)[4]) {
+  // loads are clamped to the last valid token so that nothing past the valid prefix is touched; bit i of `valid`
+  // says whether token n0 + 4g + i (the one whose score this lane holds in s[i]) takes part
+  const int32_t* idp = GATHER ? a.ids + ((int64_t)b * a.Hkv + kvh) * a.ids_sg : nullptr;
+  auto load_tile = [&](int tile, uint4 (&kf)[4], uint4 (&vf)[4], int& valid) {
     const int n0 = (split + tile * a.num_splits) * kTile;
-    const int tk = min(n0 + r, t1 - 1);
+    int tk = min(n0 + r, t1 - 1);
+    if constexpr (GATHER) tk = min(max(idp[tk], 0), a.cache_len - 1);
     const uint16_t* kp = kbase + (int64_t)tk * a.k_sn + 8 * g;
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) kf[kk] = stream_load(kp + 32 * kk);
+    valid = 0;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int tv = min(n0 + 4 * g + i, t1 - 1);
+      const int pos = n0 + 4 * g + i;
+      int tv = min(pos, t1 - 1);
+      bool ok = pos < t1;
+      if constexpr (GATHER) {
+        const int id = idp[tv];
+        ok = ok && id >= 0 && id < a.cache_len;
+        tv = min(max(id, 0), a.cache_len - 1);
+      }
+      valid |= (int)ok << i;
       vf[i] = stream_load(vbase + (int64_t)tv * a.v_sn + 8 * r);
     }
   };
@@ -146,10 +164,11 @@ __global__ __launch_bounds__(kWaves * 64) void decode_splitkv_kernel(DecodeArgs 
   // fetched and scaled, so that the two latencies overlap.
   constexpr int kSets = 4;
   uint4 kR[kSets][4], vR[kSets][4];
+  int mR[kSets];
   int tile = wsub;
 #pragma unroll
   for (int u = 0; u < kSets - 1; ++u)
-    if (tile + u * wpg < ntiles) load_tile(tile + u * wpg, kR[u], vR[u]);
+    if (tile + u * wpg < ntiles) load_tile(tile + u * wpg, kR[u], vR[u], mR[u]);
 
   // Q~ fragments (B operand): lane (col head r, k-group g) holds q~[r][32kk+8g .. +7]
   uint4 qf[4];
@@ -172,8 +191,7 @@ __global__ __launch_bounds__(kWaves * 64) void decode_splitkv_kernel(DecodeArgs 
     }
   }
 
-  auto compute_tile = [&](int tile, const uint4 (&kf)[4], const uint4 (&vf)[4]) {
-    const int n0 = (split + tile * a.num_splits) * kTile;
+  auto compute_tile = [&](const uint4 (&kf)[4], const uint4 (&vf)[4], int valid) {
     f32x4_t s = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) s = mfma_qk<BF16>(kf[kk], qf[kk], s);
@@ -182,17 +200,19 @@ __global__ __launch_bounds__(kWaves * 64) void decode_splitkv_kernel(DecodeArgs 
     float tmax = -INFINITY;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      p[i] = (n0 + 4 * g + i < t1) ? s[i] : -INFINITY;
+      p[i] = ((valid >> i) & 1) ? s[i] : -INFINITY;
       tmax = fmaxf(tmax, p[i]);
     }
     tmax = wave_xor_max(tmax, 16);
     tmax = wave_xor_max(tmax, 32);
-    const float m_new = fmaxf(m, tmax);      // finite: the tile holds at least one valid token
-    const float alpha = exp2f(m - m_new);    // exp2(-inf) = 0 on the first tile
+    const float m_new = fmaxf(m, tmax);
+    // nothing valid so far (only a selection can produce such a tile): any finite reference keeps exp2 off inf - inf
+    const float m_ref = (m_new == -INFINITY) ? 0.f : m_new;
+    const float alpha = exp2f(m - m_ref);    // exp2(-inf) = 0 on the first tile
     float psum = 0.f;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      p[i] = exp2f(p[i] - m_new);
+      p[i] = exp2f(p[i] - m_ref);
       psum += p[i];
     }
     l = l * alpha + psum;
@@ -219,8 +239,8 @@ __global__ __launch_bounds__(kWaves * 64) void decode_splitkv_kernel(DecodeArgs 
 #pragma unroll
     for (int u = 0; u < kSets; ++u) {
       const int tn = tile + (kSets - 1) * wpg;
-      if (tn < ntiles) load_tile(tn, kR[(u + kSets - 1) % kSets], vR[(u + kSets - 1) % kSets]);
-      compute_tile(tile, kR[u], vR[u]);
+      if (tn < ntiles) load_tile(tn, kR[(u + kSets - 1) % kSets], vR[(u + kSets - 1) % kSets], mR[(u + kSets - 1) % kSets]);
+      compute_tile(kR[u], vR[u], mR[u]);
       tile += wpg;
       if (tile >= ntiles) break;
     }
@@ -246,14 +266,15 @@ __global__ __launch_bounds__(kWaves * 64) void decode_splitkv_kernel(DecodeArgs 
     for (int w = 0; w < wpg; ++w) mm = fmaxf(mm, s_m[w0 + w][h]);
     float lt = 0.f, o = 0.f;
     for (int w = 0; w < wpg; ++w) {
-      const float sc = exp2f(s_m[w0 + w][h] - mm);  // 0 for a wave that saw no tile (m = -inf)
+      // 0 for a wave that saw no valid token (m = -inf); when no wave did, the partial is empty
+      const float sc = (mm > -INFINITY) ? exp2f(s_m[w0 + w][h] - mm) : 0.f;
       lt += s_l[w0 + w][h] * sc;
       o += s_o[w0 + w][h][d] * sc;
     }
     const int hq = (hy * a.hpw + hs) * a.group + h0 + h;
     const int64_t row = ((int64_t)b * a.Hq + hq) * a.num_splits + split;
-    a.part_o[row * kD + d] = o / lt;
-    if (d == 0) a.part_lse[row] = mm + log2f(lt);
+    a.part_o[row * kD + d] = (lt > 0.f) ? o / lt : 0.f;
+    if (d == 0) a.part_lse[row] = (lt > 0.f) ? mm + log2f(lt) : -INFINITY;
   }
 }
 
@@ -360,9 +381,11 @@ extern "C" size_t sq_decode_workspace_bytes(int64_t batch, int64_t num_q_heads, 
   return (size_t)batch * num_q_heads * num_splits * (kD + 1) * sizeof(float);
 }
 
-extern "C" int sq_decode_fwd(const DLTensor* q, const DLTensor* kcache, const DLTensor* vcache, const DLTensor* seqlens,
-                             DLTensor* out, DLTensor* lse, DLTensor* workspace, const sq_decode_params* params,
-                             void* stream) {
+// Shared body of sq_decode_fwd (token_ids == null) and sq_decode_selected_fwd.  The messages keep the name of the
+// dense entry point for both.
+static int decode_impl(const DLTensor* q, const DLTensor* kcache, const DLTensor* vcache, const DLTensor* seqlens,
+                       const DLTensor* token_ids, DLTensor* out, DLTensor* lse, DLTensor* workspace,
+                       const sq_decode_params* params, void* stream) {
   SQ_REQUIRE(params, SQ_EINVAL, "sq_decode_fwd: params is null");
   SQ_REQUIRE(q && kcache && vcache && out, SQ_EINVAL, "sq_decode_fwd: q, kcache, vcache and out must be non-null");
   SQ_REQUIRE(params->layout == SQ_LAYOUT_HND || params->layout == SQ_LAYOUT_NHD, SQ_EINVAL,
@@ -383,16 +406,24 @@ extern "C" int sq_decode_fwd(const DLTensor* q, const DLTensor* kcache, const DL
   const bool hnd = params->layout == SQ_LAYOUT_HND;
   const int hdim = hnd ? 1 : 2, ndim = hnd ? 2 : 1;
   const int64_t B = q->shape[0], Hq = q->shape[hdim], Nq = q->shape[ndim], D = q->shape[3];
-  const int64_t Hkv = kcache->shape[hdim], L = kcache->shape[ndim];
+  const int64_t Hkv = kcache->shape[hdim], Lcache = kcache->shape[ndim];
+  int64_t L = Lcache;   // length of the token stream: the cache, or the id lists of a selection
+  if (token_ids) {
+    SQ_REQUIRE(on_gpu(token_ids) && token_ids->device.device_id == dev, SQ_EDEVICE, "sq_decode_selected_fwd: token_ids not on the same device");
+    SQ_REQUIRE(dtype_of(token_ids) == DType::I32 && token_ids->ndim == 2 && token_ids->shape[0] == B * Hkv && token_ids->shape[1] > 0 &&
+                   stride_of(token_ids, 1) == 1,
+               SQ_ESHAPE, "sq_decode_selected_fwd: token_ids must be int32 [B * Hkv = %lld, k] with contiguous rows", (long long)(B * Hkv));
+    L = token_ids->shape[1];
+  }
   SQ_REQUIRE(D == kD, SQ_EINVAL, "Unsupported head_dim: %lld (the kernels take 128; pad smaller heads with zeros)", (long long)D);
   SQ_REQUIRE(Nq == 1, SQ_ESHAPE, "sq_decode_fwd: query length must be 1, got %lld", (long long)Nq);
-  SQ_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && L > 0, SQ_ESHAPE, "sq_decode_fwd: empty tensor");
+  SQ_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && L > 0 && Lcache > 0, SQ_ESHAPE, "sq_decode_fwd: empty tensor");
   SQ_REQUIRE(Hq % Hkv == 0, SQ_ESHAPE, "sq_decode_fwd: Hq=%lld not a multiple of Hkv=%lld", (long long)Hq, (long long)Hkv);
   SQ_REQUIRE(kcache->shape[0] == B && kcache->shape[3] == D, SQ_ESHAPE, "sq_decode_fwd: kcache shape mismatch");
   for (int i = 0; i < 4; ++i)
     SQ_REQUIRE(vcache->shape[i] == kcache->shape[i], SQ_ESHAPE, "sq_decode_fwd: vcache shape differs from kcache");
   for (int i = 0; i < 4; ++i) SQ_REQUIRE(out->shape[i] == q->shape[i], SQ_ESHAPE, "sq_decode_fwd: out shape differs from q");
-  SQ_REQUIRE(L < (1ll << 31) - 65536, SQ_EUNSUPPORTED, "sq_decode_fwd: cache longer than 2^31 tokens");
+  SQ_REQUIRE(L < (1ll << 31) - 65536 && Lcache < (1ll << 31) - 65536, SQ_EUNSUPPORTED, "sq_decode_fwd: cache longer than 2^31 tokens");
   SQ_REQUIRE(stride_of(kcache, ndim) % 8 == 0 && stride_of(vcache, ndim) % 8 == 0 && stride_of(kcache, hdim) % 8 == 0 &&
                  stride_of(vcache, hdim) % 8 == 0 && stride_of(kcache, 0) % 8 == 0 && stride_of(vcache, 0) % 8 == 0 &&
                  stride_of(q, hdim) % 8 == 0 && stride_of(q, 0) % 8 == 0,
@@ -424,6 +455,9 @@ extern "C" int sq_decode_fwd(const DLTensor* q, const DLTensor* kcache, const DL
   a.k = data_of(kcache);
   a.v = data_of(vcache);
   a.seqlens = seqlens ? (const int32_t*)data_of(seqlens) : nullptr;
+  a.ids = token_ids ? (const int32_t*)data_of(token_ids) : nullptr;
+  a.ids_sg = token_ids ? stride_of(token_ids, 0) : 0;
+  a.cache_len = (int32_t)Lcache;
   a.part_o = (float*)data_of(workspace);
   a.part_lse = a.part_o + (size_t)B * Hq * S * kD;
   a.q_sb = stride_of(q, 0);
@@ -453,10 +487,12 @@ extern "C" int sq_decode_fwd(const DLTensor* q, const DLTensor* kcache, const DL
   SQ_HIP(hipGetDevice(&cur));
   SQ_REQUIRE(cur == dev, SQ_EDEVICE, "sq_decode_fwd: tensors live on device %d but the current device is %d", dev, cur);
   const dim3 grid((unsigned)S, (unsigned)(Hkv / a.hpw * a.head_chunks), (unsigned)B);
-  if (dt == DType::BF16) {
-    hipLaunchKernelGGL(decode_splitkv_kernel<true>, grid, dim3(kWaves * 64), 0, st, a);
+  if (token_ids) {
+    if (dt == DType::BF16) hipLaunchKernelGGL((decode_splitkv_kernel<true, true>), grid, dim3(kWaves * 64), 0, st, a);
+    else hipLaunchKernelGGL((decode_splitkv_kernel<false, true>), grid, dim3(kWaves * 64), 0, st, a);
   } else {
-    hipLaunchKernelGGL(decode_splitkv_kernel<false>, grid, dim3(kWaves * 64), 0, st, a);
+    if (dt == DType::BF16) hipLaunchKernelGGL((decode_splitkv_kernel<true, false>), grid, dim3(kWaves * 64), 0, st, a);
+    else hipLaunchKernelGGL((decode_splitkv_kernel<false, false>), grid, dim3(kWaves * 64), 0, st, a);
   }
   SQ_HIP(hipGetLastError());
   CombineArgs c;
@@ -473,4 +509,17 @@ extern "C" int sq_decode_fwd(const DLTensor* q, const DLTensor* kcache, const DL
                      (size_t)(S + kCombineGroups * kCombineChunk) * sizeof(float), st, c);
   SQ_HIP(hipGetLastError());
   return SQ_OK;
+}
+
+extern "C" int sq_decode_fwd(const DLTensor* q, const DLTensor* kcache, const DLTensor* vcache, const DLTensor* seqlens,
+                             DLTensor* out, DLTensor* lse, DLTensor* workspace, const sq_decode_params* params,
+                             void* stream) {
+  return decode_impl(q, kcache, vcache, seqlens, nullptr, out, lse, workspace, params, stream);
+}
+
+extern "C" int sq_decode_selected_fwd(const DLTensor* q, const DLTensor* kcache, const DLTensor* vcache,
+                                      const DLTensor* token_ids, const DLTensor* seqlens, DLTensor* out, DLTensor* lse,
+                                      DLTensor* workspace, const sq_decode_params* params, void* stream) {
+  SQ_REQUIRE(token_ids, SQ_EINVAL, "sq_decode_selected_fwd: token_ids is null");
+  return decode_impl(q, kcache, vcache, seqlens, token_ids, out, lse, workspace, params, stream);
 }

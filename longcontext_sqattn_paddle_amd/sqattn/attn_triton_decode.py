@@ -45,6 +45,33 @@ def attn_decode(q, k, v, tensor_layout="HND", output_dtype=torch.float16, return
     return (o, lse) if return_lse else o
 
 
+def attn_decode_selected(q, k, v, token_ids, tensor_layout="NHD", output_dtype=torch.float16, return_lse=False,
+                         is_P_fp8_quant=False, seqlens: Optional[torch.Tensor] = None, num_splits: int = 0,
+                         workspace: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None):
+    """Decode attention over a selection of the cache (no reference counterpart): `token_ids` int32 [B*Hkv, k]
+    lists, per sequence and kv head, the cache rows to attend to -- what `cache_hub.kmeans.topk_select` returns.
+    Negative entries (the missing tail of a selection) are skipped.  Other arguments as `attn_decode`."""
+    if tensor_layout not in N.LAYOUT:
+        raise ValueError(f"tensor_layout {tensor_layout} not supported")
+    require_gpu(q, k, v)
+    head_dim_og = q.size(-1)
+    q, k, v = pad_head_dim((q, k, v), head_dim_og)
+    hdim = 1 if tensor_layout == "HND" else 2
+    B, Hq, Hkv = q.size(0), q.size(hdim), k.size(hdim)
+    lib = N.lib()
+    S = num_splits if num_splits > 0 else lib.sq_decode_num_splits(B, Hkv, token_ids.size(1))
+    need = lib.sq_decode_workspace_bytes(B, Hq, 128, S)
+    if workspace is None:
+        workspace = torch.empty(need // 4, dtype=torch.float32, device=q.device)
+    o = out if out is not None else torch.empty(q.shape, dtype=output_dtype, device=q.device)
+    lse = torch.empty([B, Hq, 1], dtype=torch.float32, device=q.device) if return_lse else None
+    params = N.DecodeParams(N.LAYOUT[tensor_layout], N.P_E4M3_STATIC if is_P_fp8_quant else N.P_NONE, S, head_dim_og)
+    b = [N.dl(t) for t in (q, k, v, token_ids, seqlens, o, lse, workspace)]
+    N.check(lib.sq_decode_selected_fwd(*[N.ptr(x) for x in b], params, N.current_stream(q.device)))
+    o = o[..., :head_dim_og]
+    return (o, lse) if return_lse else o
+
+
 class DecodePlan:
     """A decode launch prepared once and replayed: every tensor (query, caches, seqlens, output, LSE,
     workspace) is borrowed up front, so `run()` is one C call that allocates nothing.  For serving loops

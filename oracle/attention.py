@@ -329,3 +329,27 @@ def combine_splits(outs, lses):
     lse = torch.log2(tot) + mx_safe
     o = (w[..., None] * outs).sum(dim=0) / tot[..., None]
     return o, lse
+
+
+def decode_selected_exact(q, k, v, token_ids, score_scale=None):
+    """Closed form of decode attention over a selection of the cache (build-defined; consumes the ids of
+    `kmeans.topk_select`): q [B,Hq,1,D], k/v [B,Hkv,L,D], token_ids int [B*Hkv, n].  Row b*Hkv+kvh lists the tokens
+    the q heads of kv head kvh attend to; negative or out-of-range entries are skipped.  Returns (out fp64
+    [B,Hq,1,D], lse2 fp64 [B,Hq,1]); a head without valid entries gets zeros and -inf.  Gathers the rows and calls
+    `exact_attention` (`score_scale` is passed on), so it is pinned by that function's checks."""
+    B, Hq, _, D = q.shape
+    Hkv, L = k.shape[1], k.shape[2]
+    g = Hq // Hkv
+    out = torch.zeros(B, Hq, 1, D, dtype=torch.float64)
+    lse = torch.full((B, Hq, 1), float("-inf"), dtype=torch.float64)
+    for b in range(B):
+        for h in range(Hkv):
+            ids = token_ids[b * Hkv + h].long()
+            ids = ids[(ids >= 0) & (ids < L)]
+            if ids.numel() == 0:
+                continue
+            o, l2 = exact_attention(q[b:b + 1, h * g:(h + 1) * g], k[b:b + 1, h:h + 1, ids], v[b:b + 1, h:h + 1, ids], causal=False,
+                                    score_scale=score_scale)
+            out[b, h * g:(h + 1) * g] = o[0]
+            lse[b, h * g:(h + 1) * g] = l2[0]
+    return out, lse

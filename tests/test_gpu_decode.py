@@ -96,3 +96,83 @@ def test_decode_argument_errors():
         attn_decode(q, k, k[:, :, :32])
     with pytest.raises(ValueError):
         attn_decode(q.float(), k.float(), k.float())
+
+
+def _selected(q, kc, vc, ids, layout, **kw):
+    from longcontext_sqattn_paddle_amd.sqattn.attn_triton_decode import attn_decode_selected
+
+    dev = torch.device("cuda:0")
+    res = attn_decode_selected(q.to(dev), kc.to(dev), vc.to(dev), ids.to(dev), layout, **kw)
+    torch.cuda.synchronize()
+    return res
+
+
+@pytest.mark.parametrize("layout", ["NHD", "HND"])
+@pytest.mark.parametrize("B,Hq,Hkv,L,n", [(1, 28, 4, 5000, 1000), (2, 28, 4, 3000, 333), (1, 8, 8, 777, 16), (2, 6, 2, 900, 2100)])
+def test_decode_over_selected_tokens_matches_closed_form(layout, B, Hq, Hkv, L, n):
+    """Attention over per-(sequence, kv head) lists of cache rows: random order, duplicates, a tail of -1 and one
+    head whose list is empty."""
+    print(f"case decode selected layout={layout} B={B} Hq={Hq} Hkv={Hkv} L={L} n={n}", flush=True)
+    q, kc, vc, _ = inputs.decode_inputs(B, Hq, Hkv, L, 128, seed=60 + B)
+    g = torch.Generator().manual_seed(n)
+    ids = torch.randint(0, L, (B * Hkv, n), generator=g, dtype=torch.int32)
+    ids[1, n // 2:] = -1                       # missing tail
+    ids[B * Hkv - 1, :] = -1                   # a head with nothing selected
+    ids[0, 0] = L + 5                          # beyond the cache: skipped as well
+    qh, kh, vh = _to_hnd(q, kc, vc)
+    ref, lse_ref = A.decode_selected_exact(A.fold_scale(qh, 128), kh, vh, ids, score_scale=math.log(2.0))
+    args = (q, kc, vc) if layout == "NHD" else (qh, kh, vh)
+    out, lse = _selected(*args, ids, layout, output_dtype=torch.float32, return_lse=True)
+    out = out.cpu()
+    out = out[:, 0] if layout == "NHD" else out[:, :, 0]
+    rms = float(ref.pow(2).mean().sqrt())
+    err = float((out.double() - ref[:, :, 0]).abs().max())
+    assert err <= 2e-4 * rms, f"max abs err {err} vs rms {rms}"
+    empty = lse_ref[:, :, 0] == float("-inf")
+    assert bool((lse.cpu()[:, :, 0][empty] == float("-inf")).all()) and bool((out[empty] == 0).all())
+    assert torch.allclose(lse.cpu()[:, :, 0][~empty].double(), lse_ref[:, :, 0][~empty], atol=2e-4)
+
+
+def test_selected_decode_with_all_tokens_equals_dense_decode():
+    """The identity list reproduces the dense kernel bit for bit (same tiles, same order)."""
+    print("case decode selected identity", flush=True)
+    B, Hq, Hkv, L = 2, 28, 4, 2048
+    q, kc, vc, _ = inputs.decode_inputs(B, Hq, Hkv, L, 128, seed=71)
+    ids = torch.arange(L, dtype=torch.int32).repeat(B * Hkv, 1)
+    dense = _run(q, kc, vc, None, "NHD", output_dtype=torch.float32)
+    sel = _selected(q, kc, vc, ids, "NHD", output_dtype=torch.float32)
+    assert torch.equal(dense, sel)
+
+
+def test_kmeans_topk_then_selected_decode():
+    """The retrieval pipeline end to end: cluster the keys, pick the tokens of the best-scoring clusters for a query,
+    attend over them; checked against the closed form over the same ids."""
+    from longcontext_sqattn_paddle_amd.cache_hub.kmeans import segment_k_means, topk_select
+
+    print("case kmeans -> topk -> selected decode", flush=True)
+    dev = torch.device("cuda:0")
+    B, Hq, Hkv, L, C, k = 1, 28, 4, 8192, 128, 1024
+    q, kc, vc, _ = inputs.decode_inputs(B, Hq, Hkv, L, 128, seed=72)
+    key = kc.permute(0, 2, 1, 3).reshape(B * Hkv, L, 128).contiguous().to(dev)
+    val = vc.permute(0, 2, 1, 3).reshape(B * Hkv, L, 128).contiguous().to(dev)
+    centroids, _, clusters, cluster_size = segment_k_means(key, val, C, num_iters=3)
+    ids = topk_select(q[:, 0].to(dev), centroids, clusters, cluster_size, k, Hq // Hkv)
+    torch.cuda.synchronize()
+    assert ids.shape == (B * Hkv, k) and int(ids.min()) >= 0 and int(ids.max()) < L
+    out = _selected(q, kc, vc, ids.cpu(), "NHD", output_dtype=torch.float32)
+    qh, kh, vh = _to_hnd(q, kc, vc)
+    ref, _ = A.decode_selected_exact(A.fold_scale(qh, 128), kh, vh, ids.cpu(), score_scale=math.log(2.0))
+    err = float((out.cpu()[:, 0].double() - ref[:, :, 0]).abs().max())
+    assert err <= 2e-4 * float(ref.pow(2).mean().sqrt())
+
+
+def test_selected_decode_argument_errors():
+    from longcontext_sqattn_paddle_amd.sqattn.attn_triton_decode import attn_decode_selected
+
+    dev = torch.device("cuda:0")
+    q = torch.zeros(1, 1, 8, 128, dtype=torch.bfloat16, device=dev)
+    kc = torch.zeros(1, 64, 2, 128, dtype=torch.bfloat16, device=dev)
+    with pytest.raises(AssertionError, match="token_ids"):
+        attn_decode_selected(q, kc, kc, torch.zeros(3, 8, dtype=torch.int32, device=dev), "NHD")
+    with pytest.raises(AssertionError, match="token_ids"):
+        attn_decode_selected(q, kc, kc, torch.zeros(2, 8, dtype=torch.int64, device=dev), "NHD")
