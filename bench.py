@@ -144,6 +144,49 @@ def time_decode_selected(torch, B, L, k, iters=20, rounds=5):
     return sorted(samples)[len(samples) // 2], 2.0 * B * Hkv * k * D * 2
 
 
+def time_layer_kernels(torch, N, iters=10):
+    """The element-wise passes around the attention call at Qwen2.5-7B's sizes (hidden 3584, intermediate 18944,
+    28/4 heads of 128): RMSNorm and RoPE over the N-token prompt, SiLU*mul over one 8192-token chunk of the MLP
+    (the reference's chunk, model_hub/LLM.py:72-81)."""
+    from longcontext_sqattn_paddle_amd.model_hub import utils as U
+
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(7)
+    out = {}
+
+    def timed(fn):
+        for _ in range(2):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(iters):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / iters * 1e3
+
+    x = torch.randn(N, 3584, device=dev, generator=g).bfloat16()
+    w = torch.ones(3584, device=dev, dtype=torch.bfloat16)
+    y = torch.empty_like(x)
+    us = timed(lambda: U.rmsnorm(x, w, 1e-6, out=y))
+    out["rmsnorm"] = (us, 2.0 * x.numel() * 2)
+    del x, y
+    h = torch.randn(8192, 2 * 18944, device=dev, generator=g).bfloat16()
+    o = torch.empty(8192, 18944, device=dev, dtype=torch.bfloat16)
+    us = timed(lambda: U.silu_and_mul(h, out=o))
+    out["silu_and_mul"] = (us, 1.5 * h.numel() * 2)
+    del h, o
+    q = torch.randn(N, 28 * 128, device=dev, generator=g).bfloat16()
+    k = torch.randn(N, 4 * 128, device=dev, generator=g).bfloat16()
+    table = U.yarn_cos_sin_cache(128, 1000000.0, 32768, N, dev)
+    pos = torch.arange(N, device=dev)[None]
+    us = timed(lambda: U.apply_rope_with_cos_sin_cache_inplace(pos, q, k, 128, table))
+    out["rope"] = (us, 2.0 * (q.numel() + k.numel()) * 2 + table.numel() * 4 + N * 8)
+    torch.cuda.empty_cache()
+    return out
+
+
 def time_kv_cache(torch, N, iters=10):
     """The KV cache's two row movements at the benchmark shape (4 kv heads x 128, bf16): the store of an N-token
     prompt (K and V, each read once and written once) and the append of one token per sequence at batch 8."""
@@ -274,6 +317,7 @@ def main():
     ap.add_argument("--no-decode", action="store_true")
     ap.add_argument("--no-prepass", action="store_true")
     ap.add_argument("--no-kv-cache", action="store_true")
+    ap.add_argument("--no-layer", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -370,6 +414,13 @@ def main():
                               "append_us_batch8": round(aus, 2)}
         log(f"[bench] kv cache: store of {N} tokens {sus:.0f} us ({sbytes / sus / 1e3:.0f} GB/s), append (batch 8) {aus:.1f} us")
         torch.cuda.empty_cache()
+    if not args.no_layer:
+        lay = {}
+        for name, (us, nbytes) in time_layer_kernels(torch, N).items():
+            lay[name] = {"us_per_call": round(us, 1), "GB_per_s": round(nbytes / us / 1e3, 1),
+                         "frac_of_hbm_peak": round(nbytes / us / 1e3 / PEAK_HBM_GBS, 4), "bytes": nbytes}
+            log(f"[bench] layer kernel {name}: {us:.0f} us, {nbytes / us / 1e3:.0f} GB/s")
+        result["layer_kernels"] = lay
     if not args.no_kmeans:
         us, kflops, kbytes = time_kmeans(torch)
         result["kmeans"] = {"us_per_iteration": round(us, 1), "TFLOP_per_s": round(kflops / us / 1e6, 1),

@@ -21,6 +21,9 @@
  *   sq_topk_select            no reference counterpart (defined by this build's benchmark configuration)
  *   sq_kv_cache_store         cache_hub/flash_attn_cache.py:153-232 (prefill_update_kv_cache: the two slice copies)
  *   sq_kv_cache_append        cache_hub/flash_attn_cache.py:239-256 (decode_update_kv_cache)
+ *   sq_rmsnorm                model_hub/utils.py:15-19 (rmsnorm; caller model_hub/qwen.py:345-350)
+ *   sq_silu_and_mul           model_hub/utils.py:4-13 (silu_and_mul; caller model_hub/qwen.py:319-326)
+ *   sq_rope                   model_hub/utils.py:21-106 (apply_rope_with_cos_sin_cache_inplace; caller qwen.py:352-367)
  *   sq_fake_quant_prepass     sqattn/attn_replacer.py:334-365 (GQA expand, key centring and the five fake-quant
  *                             passes of mp_triton_wrapper's closure), sqattn/fake_quant.py:24-58, 98-125
  */
@@ -201,6 +204,31 @@ int sq_kv_cache_store(const DLTensor* key_states, const DLTensor* value_states, 
 int sq_kv_cache_append(const DLTensor* key_states, const DLTensor* value_states, DLTensor* key_cache,
                        DLTensor* value_cache, DLTensor* valid_length, DLTensor* attend_length, int32_t advance,
                        void* stream);
+
+/*
+ * RMS normalisation of the rows of x [R, dim] (model_hub/utils.py:15-19): out = (x * rsqrt(mean(x^2) + epsilon))
+ * * weight, with the reference's operator sequence on 16-bit tensors -- square, mean (fp32 accumulation), + epsilon,
+ * rsqrt, x * r, * weight, each result rounded to the tensor dtype.  x, out [R, dim] (row strides free, 16-byte
+ * aligned rows), weight [dim]; bf16 or fp16, all of one dtype; dim a multiple of 8, at most 8192.
+ */
+int sq_rmsnorm(const DLTensor* x, const DLTensor* weight, DLTensor* out, float epsilon, void* stream);
+
+/*
+ * out = x2 * (x1 * sigmoid(x1)) for x = [x1 | x2] [R, 2 I] -> out [R, I] (model_hub/utils.py:4-13), the three tensor
+ * operators each rounded to the tensor dtype.  bf16 or fp16; I a multiple of 8.
+ */
+int sq_silu_and_mul(const DLTensor* x, DLTensor* out, void* stream);
+
+/*
+ * Rotary position embedding of query [T, Hq * head_dim] and key [T, Hkv * head_dim] (T = batch * seq_len tokens)
+ * with the rows position_ids[t] of cos_sin_cache, fp32 [max_position, head_dim] holding cos in the first half of a
+ * row and sin in the second (model_hub/utils.py:21-106): per head, out1 = x1 cos - x2 sin, out2 = x1 sin + x2 cos
+ * over the two halves, formed in fp32 and rounded once to the tensor dtype.  The outputs have the inputs' shape
+ * and may be the inputs themselves.  position_ids int32 or int64, T entries, each in [0, max_position) (the
+ * caller's responsibility; the kernel clamps).
+ */
+int sq_rope(const DLTensor* query, const DLTensor* key, DLTensor* query_out, DLTensor* key_out,
+            const DLTensor* position_ids, const DLTensor* cos_sin_cache, int32_t head_dim, void* stream);
 
 #ifdef __cplusplus
 }

@@ -83,6 +83,9 @@ SYMBOLS = {
     "sq_topk_select": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, ctypes.c_int32, ctypes.c_void_p]),
     "sq_fake_quant_prepass_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int64] * 3),
     "sq_fake_quant_prepass": (ctypes.c_int, [_P] * 9 + [ctypes.c_int32, ctypes.c_void_p]),
+    "sq_rmsnorm": (ctypes.c_int, [_P, _P, _P, ctypes.c_float, ctypes.c_void_p]),
+    "sq_silu_and_mul": (ctypes.c_int, [_P, _P, ctypes.c_void_p]),
+    "sq_rope": (ctypes.c_int, [_P] * 6 + [ctypes.c_int32, ctypes.c_void_p]),
     "sq_kv_cache_store": (ctypes.c_int, [_P] * 4 + [ctypes.c_int32, ctypes.c_int64, ctypes.c_void_p]),
     "sq_kv_cache_append": (ctypes.c_int, [_P] * 6 + [ctypes.c_int32, ctypes.c_void_p]),
 }

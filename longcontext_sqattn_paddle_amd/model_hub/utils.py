@@ -1,0 +1,100 @@
+"""The element-wise helpers of the reference's model_hub/utils.py on the gfx950 kernels (same names and arguments):
+`silu_and_mul` (:4-13), `rmsnorm` (:15-19), `apply_rope_with_cos_sin_cache_inplace` (:21-106), plus
+`yarn_cos_sin_cache`, the cos | sin table the reference builds in `model_hub/qwen.py:133-198, 227-228`.
+
+Each helper is one kernel launch and writes nothing but its result, where the reference launches one kernel per
+tensor operator (the rotary embedding alone peaks at 81 GB of temporaries at 1M tokens by the reference's own
+comments, :82-91).  There is no CPU path.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional
+
+import torch
+
+from .. import _native as N
+
+
+def _need_gpu(*ts):
+    for t in ts:
+        if not t.is_cuda:
+            raise RuntimeError(f"tensors must live on the MI355X (got {t.device}); there is no CPU path")
+
+
+def silu_and_mul(hidden_states: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """[..., 2*I] -> [..., I]: `x2 * (x1 * sigmoid(x1))` for the two halves of the last dimension (utils.py:4-13)."""
+    _need_gpu(hidden_states)
+    two = hidden_states.shape[-1]
+    x = hidden_states.reshape(-1, two)
+    if x.stride(-1) != 1:
+        x = x.contiguous()
+    if out is None:
+        out = torch.empty(*hidden_states.shape[:-1], two // 2, dtype=hidden_states.dtype, device=hidden_states.device)
+    b = [N.dl(x), N.dl(out.view(-1, two // 2))]
+    N.check(N.lib().sq_silu_and_mul(N.ptr(b[0]), N.ptr(b[1]), N.current_stream(x.device)))
+    return out
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, epsilon: float = 1e-6, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """`x * rsqrt(mean(x^2, -1) + epsilon) * weight` over the last dimension (utils.py:15-19)."""
+    _need_gpu(x, weight)
+    dim = x.shape[-1]
+    x2 = x.reshape(-1, dim)
+    if x2.stride(-1) != 1:
+        x2 = x2.contiguous()
+    if out is None:
+        out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    b = [N.dl(x2), N.dl(weight), N.dl(out.view(-1, dim))]
+    N.check(N.lib().sq_rmsnorm(N.ptr(b[0]), N.ptr(b[1]), N.ptr(b[2]), float(epsilon), N.current_stream(x.device)))
+    return out
+
+
+def apply_rope_with_cos_sin_cache_inplace(position_ids: torch.Tensor, query_states: torch.Tensor, key_states: torch.Tensor,
+                                          head_dim: int, cos_sin_cache: torch.Tensor, use_cache: bool = True):
+    """Rotary embedding (utils.py:21-106).  position_ids [batch, seq_len]; query_states [batch*seq_len, Hq*head_dim];
+    key_states [batch*seq_len, Hkv*head_dim]; cos_sin_cache fp32 [max_seq_len, head_dim] (cos | sin).
+    Returns `(q_out [batch, seq_len, Hq, head_dim], k_out [batch, seq_len, Hkv, head_dim])` like the reference; the
+    inputs are left as they were (the reference overwrites them with values it then discards, :87-90)."""
+    _need_gpu(query_states, key_states, position_ids, cos_sin_cache)
+    bsz, seq_len = position_ids.shape
+    q_out = torch.empty_like(query_states)
+    k_out = torch.empty_like(key_states)
+    pos = position_ids.reshape(-1)
+    if pos.dtype not in (torch.int32, torch.int64):
+        pos = pos.to(torch.int64)
+    b = [N.dl(t) for t in (query_states, key_states, q_out, k_out, pos.contiguous(), cos_sin_cache)]
+    N.check(N.lib().sq_rope(*[N.ptr(x) for x in b], int(head_dim), N.current_stream(query_states.device)))
+    return (q_out.view(bsz, seq_len, -1, head_dim), k_out.view(bsz, seq_len, -1, head_dim))
+
+
+def yarn_cos_sin_cache(head_dim: int, base: float, max_position_embeddings: int, max_length: int, device,
+                       yarn_factor: float = 4.0, inv_freq: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The fp32 [max_length, head_dim] cos | sin table of `model_hub/qwen.py:133-198, 227-228`.
+
+    Up to 32768 positions: plain rotary frequencies `base^(-2i/head_dim)` (or the checkpoint's `inv_freq`), scaling 1.
+    Beyond: YaRN with factor 4 -- dimensions that turn more than 32 times within the trained context keep their
+    frequency, those that turn less than once are divided by the factor, a linear ramp in between, and cos/sin are
+    multiplied by `0.1 ln(factor) + 1`.  Host-side set-up work (once per model), plain torch on the target device.
+    """
+    half = head_dim // 2
+    exponent = torch.arange(0, head_dim, 2, dtype=torch.float32, device=device) / head_dim
+    scaling = 1.0
+    if max_length > 32768:
+        def correction_dim(num_rotations):
+            return head_dim * math.log(max_position_embeddings / (num_rotations * 2 * math.pi)) / (2 * math.log(base))
+
+        low = max(math.floor(correction_dim(32)), 0)          # beta_fast
+        high = min(math.ceil(correction_dim(1)), head_dim - 1)  # beta_slow
+        hi = high + 0.001 if low == high else high
+        ramp = ((torch.arange(half, dtype=torch.float32, device=device) - low) / (hi - low)).clamp(0, 1)
+        keep = 1 - ramp
+        pos_freqs = base ** exponent
+        inv_freq = (1.0 / (yarn_factor * pos_freqs)) * (1 - keep) + (1.0 / pos_freqs) * keep
+        scaling = 0.1 * math.log(yarn_factor) + 1.0
+    elif inv_freq is None:
+        inv_freq = 1.0 / (base ** exponent)
+    inv_freq = inv_freq.to(device=device, dtype=torch.float32)
+    t = torch.arange(max_length, device=device, dtype=torch.float32)
+    freqs = torch.outer(t, inv_freq)
+    return torch.cat((freqs.cos() * scaling, freqs.sin() * scaling), dim=-1).contiguous()

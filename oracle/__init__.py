@@ -4,7 +4,7 @@ Everything in this package is a CPU restatement (torch-CPU / numpy) of the
 algorithms in the reference's `sqattn/attn_triton.py`, `sqattn/attn_triton_decode.py`,
 `sqattn/attn_triton_mix_relative.py`, `sqattn/attn_triton_mix_bad.py`,
 `sqattn/fake_quant.py`, `sqattn/attn_replacer.py`, `cache_hub/kmeans.py` and
-`cache_hub/flash_attn_cache.py`.
+`cache_hub/flash_attn_cache.py` and `model_hub/utils.py`.
 It exists to check the HIP kernels, never to serve a request: only `tests/`,
 `__graft_entry__.smoke()` and the `cpu_baseline` leg of `bench.py` import it.
 The product package (`longcontext_sqattn_paddle_amd`) must not import it and
@@ -25,6 +25,8 @@ ships no golden vectors for this path):
 * `kmeans.*`                       -- brute-force argmax, partition invariants, bincount identities.
 * `kv_cache.*`                     -- index arithmetic only: element-by-element loops on tiny inputs, untouched-row
                                       and concatenation invariants.
+* `layer.*`                        -- torch's own 16-bit CPU operators evaluating the reference's expressions, fp64
+                                      closed forms, rotation invariants (parity unpinned: Paddle's rounding points).
 * `kmeans.topk_select`             -- build-defined (the reference has no top-k code): parity unpinned
                                       by the reference, pinned by brute force only.
 """

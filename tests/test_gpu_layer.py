@@ -1,0 +1,126 @@
+"""Element-wise layer kernels (RMSNorm, SiLU*mul, RoPE) through the C ABI against oracle/layer.py.
+
+RoPE is bit-exact (separate fp32 products and sums, one rounding).  RMSNorm and SiLU*mul agree bit for bit except
+where an fp32 intermediate lies on a rounding boundary of a 16-bit operator result (the GPU's exp/accumulation order
+differ from the CPU's in the last fp32 bit): at most one 16-bit spacing, on a stated fraction of the elements."""
+import pytest
+import torch
+
+from oracle import layer as OL
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _mismatch(a, b):
+    a32, b32 = a.float().cpu(), b.float()
+    diff = (a32 - b32).abs()
+    spacing = torch.maximum(a32.abs(), b32.abs()).clamp_min(1e-30) * (2.0 ** -7 if b.dtype == torch.bfloat16 else 2.0 ** -10)
+    return float((diff > 0).float().mean()), float((diff / spacing).max())
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows,dim", [(300, 3584), (17, 4096), (5, 8192), (1000, 128), (3, 8)])
+def test_rmsnorm_matches_oracle(dtype, rows, dim):
+    from longcontext_sqattn_paddle_amd.model_hub.utils import rmsnorm
+
+    print(f"case rmsnorm {dtype} rows={rows} dim={dim}", flush=True)
+    g = torch.Generator().manual_seed(rows + dim)
+    x = (torch.randn(rows, dim, generator=g) * 1.3).to(dtype)
+    w = (1 + 0.2 * torch.randn(dim, generator=g)).to(dtype)
+    ref = OL.rmsnorm(x, w, 1e-6)
+    out = rmsnorm(x.to(DEV), w.to(DEV), 1e-6)
+    torch.cuda.synchronize()
+    frac, ulps = _mismatch(out, ref)
+    # a row whose fp32 sum of squares rounds to the neighbouring 16-bit variance shifts by one spacing as a whole
+    assert ulps <= 1.01 and frac <= 0.02, (frac, ulps)
+    if rows >= 100:
+        rows_equal = (out.cpu() == ref).all(dim=-1).float().mean()
+        assert float(rows_equal) >= 0.97
+
+
+def test_rmsnorm_3d_input_and_strided_rows():
+    from longcontext_sqattn_paddle_amd.model_hub.utils import rmsnorm
+
+    g = torch.Generator().manual_seed(4)
+    big = torch.randn(2, 40, 1024, generator=g).bfloat16()
+    w = torch.ones(512, dtype=torch.bfloat16)
+    x = big[..., :512]                                   # rows 1024 apart
+    ref = OL.rmsnorm(x, w)
+    out = rmsnorm(big.to(DEV)[..., :512], w.to(DEV))
+    torch.cuda.synchronize()
+    assert out.shape == x.shape
+    frac, ulps = _mismatch(out, ref)
+    assert ulps <= 1.01 and frac <= 0.02
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows,inter", [(64, 18944), (3, 8), (1000, 512)])
+def test_silu_and_mul_matches_oracle(dtype, rows, inter):
+    from longcontext_sqattn_paddle_amd.model_hub.utils import silu_and_mul
+
+    print(f"case silu_and_mul {dtype} rows={rows} I={inter}", flush=True)
+    g = torch.Generator().manual_seed(rows + inter)
+    h = (torch.randn(rows, 2 * inter, generator=g) * 3.0).to(dtype)
+    ref = OL.silu_and_mul(h)
+    out = silu_and_mul(h.to(DEV))
+    torch.cuda.synchronize()
+    assert out.shape == (rows, inter)
+    frac, ulps = _mismatch(out, ref)
+    assert ulps <= 1.01 and frac <= 2e-3, (frac, ulps)   # sigmoid within an fp32 ulp or two of a 16-bit boundary
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,S,Hq,Hkv,D,maxpos", [(1, 700, 28, 4, 128, 4096), (2, 33, 8, 8, 64, 50000), (1, 1, 4, 2, 128, 16)])
+def test_rope_is_bit_exact(dtype, B, S, Hq, Hkv, D, maxpos):
+    from longcontext_sqattn_paddle_amd.model_hub.utils import apply_rope_with_cos_sin_cache_inplace, yarn_cos_sin_cache
+
+    print(f"case rope {dtype} B={B} S={S} Hq={Hq} Hkv={Hkv} D={D} maxpos={maxpos}", flush=True)
+    g = torch.Generator().manual_seed(S + D)
+    q = torch.randn(B * S, Hq * D, generator=g).to(dtype)
+    k = torch.randn(B * S, Hkv * D, generator=g).to(dtype)
+    table = yarn_cos_sin_cache(D, 1000000.0, 32768, maxpos, "cpu")
+    pos = torch.randint(0, maxpos, (B, S), generator=g)
+    rq, rk = OL.rope(pos, q, k, D, table)
+    qd, kd = q.to(DEV), k.to(DEV)
+    oq, ok = apply_rope_with_cos_sin_cache_inplace(pos.to(DEV), qd, kd, D, table.to(DEV))
+    torch.cuda.synchronize()
+    assert oq.shape == (B, S, Hq, D) and ok.shape == (B, S, Hkv, D)
+    assert torch.equal(oq.cpu().view(B * S, -1), rq) and torch.equal(ok.cpu().view(B * S, -1), rk)
+    assert torch.equal(qd.cpu(), q) and torch.equal(kd.cpu(), k)              # inputs untouched
+    oq32, _ = apply_rope_with_cos_sin_cache_inplace(pos.to(DEV).to(torch.int32), qd, kd, D, table.to(DEV))
+    assert torch.equal(oq32, oq)
+
+
+def test_rope_feeds_the_kv_cache_layout():
+    """rope output [B, S, Hkv, D] is what `prefill_update_kv_cache` takes (model_hub/LLM.py:56-66)."""
+    from longcontext_sqattn_paddle_amd.cache_hub.flash_attn_cache import flash_attn_cache
+    from longcontext_sqattn_paddle_amd.model_hub.utils import apply_rope_with_cos_sin_cache_inplace, yarn_cos_sin_cache
+
+    S, Hq, Hkv, D = 96, 8, 2, 128
+    g = torch.Generator().manual_seed(8)
+    q = torch.randn(S, Hq * D, generator=g).bfloat16().to(DEV)
+    k = torch.randn(S, Hkv * D, generator=g).bfloat16().to(DEV)
+    v = torch.randn(1, S, Hkv, D, generator=g).bfloat16().to(DEV)
+    table = yarn_cos_sin_cache(D, 1000000.0, 32768, 256, DEV)
+    pos = torch.arange(S, device=DEV)[None]
+    _, ko = apply_rope_with_cos_sin_cache_inplace(pos, q, k, D, table)
+    cache = flash_attn_cache(0, 1, 1, 128, Hkv, Hq, D, torch.bfloat16, {"0": DEV}, 1, 7)
+    cache.prefill_update_kv_cache(None, ko, v, 0, 0)
+    cache.sync(0, 0)
+    torch.cuda.synchronize()
+    assert torch.equal(cache.key_cache[0][0, :S], ko[0])
+
+
+def test_layer_kernel_argument_errors():
+    from longcontext_sqattn_paddle_amd.model_hub.utils import rmsnorm, silu_and_mul
+
+    x = torch.zeros(4, 8200, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(ValueError, match="at most"):
+        rmsnorm(x, torch.ones(8200, dtype=torch.bfloat16, device=DEV))
+    with pytest.raises((ValueError, AssertionError)):
+        rmsnorm(x[:, :512], torch.ones(512, dtype=torch.float16, device=DEV))
+    with pytest.raises(ValueError, match="multiple of 16"):
+        silu_and_mul(torch.zeros(4, 24, dtype=torch.bfloat16, device=DEV))
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        silu_and_mul(torch.zeros(4, 32, dtype=torch.bfloat16))
