@@ -187,6 +187,74 @@ def time_layer_kernels(torch, N, iters=10):
     return out
 
 
+def time_model_layers(torch, N):
+    """Two decoder layers of Qwen2.5-7B's shapes (random weights) through the runtime mirror: prompt of N tokens
+    (embedding, 2 x layer_prefill, final norm, lm head), then decode steps against the N-token cache."""
+    from longcontext_sqattn_paddle_amd.model_hub.qwen import QwenConfig, QwenModel
+
+    dev = "cuda:0"
+    cfg = QwenConfig(num_hidden_layers=2)
+    model = QwenModel("Qwen2.5-7B-shaped", N + 16, torch.bfloat16, dev, "SDPA", config=cfg, seed=1)
+    ids = torch.randint(0, cfg.vocab_size, (1, N), device=dev, generator=torch.Generator(device=dev).manual_seed(2))
+    out = {}
+    for name, pq in (("exact_attention", None), ("fp8_pv_attention", 5)):
+        for layer in model.layers:
+            layer.p_quant = pq
+        ms = []
+        for _ in range(3):
+            model.batch_size, model.max_new_length = 1, 16
+            model.init_kv_cache(N, [0])
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            logits = model.prefill_forward(ids)
+            e1.record()
+            torch.cuda.synchronize()
+            ms.append(e0.elapsed_time(e1))
+        assert bool(torch.isfinite(logits).all())
+        out["prefill_ms_per_layer_" + name] = sorted(ms)[1] / cfg.num_hidden_layers
+    tok = logits.argmax(dim=-1)
+    for _ in range(3):
+        model.decode_forward(tok)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(8):
+        model.decode_forward(tok)
+    e1.record()
+    torch.cuda.synchronize()
+    out["decode_ms_per_layer"] = e0.elapsed_time(e1) / 8 / cfg.num_hidden_layers
+    del model
+    torch.cuda.empty_cache()
+    return out
+
+
+def time_e2e(torch, N, new_tokens=17, sqattn=False):
+    """The whole 28-layer decoder of Qwen2.5-7B's shapes (random weights) through `generate`: prefill of one N-token
+    prompt and greedy decoding, as the reference's latency logs measure them (model_hub/LLM.py:167-203).  With
+    `sqattn`, layers 1..26 run the quantised sink/window closure of `process_model` with relative windows 0.25 / 0.5
+    (the reference keeps exact attention in the first and last layer)."""
+    import types
+
+    from longcontext_sqattn_paddle_amd.model_hub.qwen import QwenConfig, QwenModel
+    from longcontext_sqattn_paddle_amd.sqattn.attn_replacer import process_model
+
+    dev = "cuda:0"
+    cfg = QwenConfig()
+    model = QwenModel("Qwen2.5-7B-shaped", N + new_tokens, torch.bfloat16, dev, "SQAttn" if sqattn else "FlashAttn", config=cfg, seed=1)
+    if sqattn:
+        ws = {i: {"bit8": 0.25, "bit4": 0.5, "sink": 256} for i in range(1, cfg.num_hidden_layers - 1)}
+        process_model(model, "SQAttn", ws, types.SimpleNamespace(qk_qtype="int", v_qtype="int", use_relative_distance=True))
+    ids = torch.randint(0, cfg.vocab_size, (1, N), device=dev, generator=torch.Generator(device=dev).manual_seed(2))
+    model.generate(model.attention_type, ids[:, :4096], None, 3, verbose=False)    # warm-up: library handles, GEMM heuristics
+    model.generate(model.attention_type, ids, None, new_tokens, verbose=False)
+    res = {"prefill_s": round(model.prefill_latency, 3), "decode_ms_per_step": round(model.decode_latency * 1e3, 3),
+           "tokens": N, "layers": cfg.num_hidden_layers, "attention": "SQAttn windows 0.25/0.5, sink 256" if sqattn else "exact causal"}
+    del model
+    torch.cuda.empty_cache()
+    return res
+
+
 def time_kv_cache(torch, N, iters=10):
     """The KV cache's two row movements at the benchmark shape (4 kv heads x 128, bf16): the store of an N-token
     prompt (K and V, each read once and written once) and the append of one token per sequence at batch 8."""
@@ -318,6 +386,9 @@ def main():
     ap.add_argument("--no-prepass", action="store_true")
     ap.add_argument("--no-kv-cache", action="store_true")
     ap.add_argument("--no-layer", action="store_true")
+    ap.add_argument("--no-model", action="store_true")
+    ap.add_argument("--e2e", action="store_true",
+                    help="also run the whole 28-layer Qwen2.5-7B-shaped decoder (random weights): prefill latency and decode ms/step")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -421,6 +492,15 @@ def main():
                          "frac_of_hbm_peak": round(nbytes / us / 1e3 / PEAK_HBM_GBS, 4), "bytes": nbytes}
             log(f"[bench] layer kernel {name}: {us:.0f} us, {nbytes / us / 1e3:.0f} GB/s")
         result["layer_kernels"] = lay
+    if not args.no_model:
+        ml = time_model_layers(torch, N)
+        result["model_layers"] = {k: round(v, 3) for k, v in ml.items()}
+        result["model_layers"]["note"] = ("Qwen2.5-7B-shaped decoder layers with random weights, batch 1: per-layer time of a "
+                                          f"{N}-token prefill (includes 1/2 of embedding + lm head) and of a decode step at that context")
+        log(f"[bench] model layers: {ml}")
+    if args.e2e:
+        result["e2e"] = [time_e2e(torch, N, sqattn=False), time_e2e(torch, N, sqattn=True)]
+        log(f"[bench] end to end: {result['e2e']}")
     if not args.no_kmeans:
         us, kflops, kbytes = time_kmeans(torch)
         result["kmeans"] = {"us_per_iteration": round(us, 1), "TFLOP_per_s": round(kflops / us / 1e6, 1),

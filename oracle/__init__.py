@@ -27,6 +27,7 @@ ships no golden vectors for this path):
                                       and concatenation invariants.
 * `layer.*`                        -- torch's own 16-bit CPU operators evaluating the reference's expressions, fp64
                                       closed forms, rotation invariants (parity unpinned: Paddle's rounding points).
+* `model.CpuDecoder`               -- assembled from the pieces above and torch's CPU `linear`; no arithmetic of its own.
 * `kmeans.topk_select`             -- build-defined (the reference has no top-k code): parity unpinned
                                       by the reference, pinned by brute force only.
 """

@@ -1,0 +1,75 @@
+"""The decoder runtime (model_hub.LLM / model_hub.qwen) end to end on a small random-weight model of the Qwen
+architecture, against the CPU restatement in oracle/model.py with teacher forcing.
+
+Tolerance: the GPU's GEMMs (hipBLASLt) and the CPU's accumulate in different orders and every layer rounds to bf16, so
+logits agree to a cosine of 0.999 and the greedy token agrees wherever the oracle's top-2 margin exceeds the
+observed logit error."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _small_model(max_length=512, layers=2):
+    from longcontext_sqattn_paddle_amd.model_hub.qwen import QwenConfig, QwenModel
+
+    cfg = QwenConfig(hidden_size=512, intermediate_size=1024, num_hidden_layers=layers, num_attention_heads=4,
+                     num_key_value_heads=2, vocab_size=1000, max_position_embeddings=32768)
+    return QwenModel("qwen-test-1B", max_length, torch.bfloat16, DEV, "SDPA", config=cfg, seed=3)
+
+
+def _cos(a, b):
+    return float(torch.nn.functional.cosine_similarity(a.flatten().double(), b.flatten().double(), dim=0))
+
+
+def test_generate_matches_cpu_restatement_with_teacher_forcing():
+    from oracle.model import CpuDecoder
+
+    print("case model generate vs oracle", flush=True)
+    model = _small_model()
+    g = torch.Generator().manual_seed(1)
+    ids = torch.randint(0, 1000, (1, 300), generator=g)
+    new = 4
+    out = model.generate("SDPA", ids.to(DEV), None, new, verbose=False)
+    assert len(out) == 1 and len(out[0]) == new
+    assert model.kv_cache.context == 300 + new - 1 and model.kv_cache.valid_length.cpu().tolist() == [300 + new - 1]
+    # replay on the GPU to get the logits of every step, and on the CPU with the same forced tokens
+    model2 = _small_model()
+    model2.batch_size, model2.max_new_length = 1, new
+    model2.init_kv_cache(300, [0])
+    ref = CpuDecoder(model2)
+    feed = ids
+    for step in range(new):
+        gl = (model2.prefill_forward(feed.to(DEV)) if step == 0 else model2.decode_forward(feed.to(DEV))).cpu()
+        rl = ref.forward(feed)
+        c = _cos(gl, rl)
+        err = float((gl - rl).abs().max())
+        top2 = torch.topk(rl.flatten(), 2).values
+        print(f"  step {step}: cosine {c:.6f}, max logit err {err:.4f}, oracle top-2 margin {float(top2[0] - top2[1]):.4f}", flush=True)
+        assert c >= 0.999, (step, c)
+        if float(top2[0] - top2[1]) > 2 * err:
+            assert int(gl.argmax()) == int(rl.argmax())
+        assert int(gl.argmax()) == out[0][step]        # the replay reproduces generate()
+        feed = torch.tensor([[out[0][step]]])
+
+
+def test_left_padded_batch_and_sqattn_plugin_layers():
+    """Two sequences with different amounts of left padding (valid_start from the attention mask, LLM.py:226-229),
+    and `process_model` swapping the quantised-window closure into the middle layers."""
+    import types
+
+    from longcontext_sqattn_paddle_amd.sqattn.attn_replacer import process_model
+
+    print("case model batch 2 with padding + SQAttn layers", flush=True)
+    model = _small_model(max_length=1024, layers=3)
+    g = torch.Generator().manual_seed(2)
+    ids = torch.randint(0, 1000, (2, 512), generator=g)
+    mask = torch.ones(2, 512, dtype=torch.int64)
+    mask[1, :128] = 0
+    args = types.SimpleNamespace(qk_qtype="int", v_qtype="int", use_relative_distance=True)
+    process_model(model, "SQAttn", {1: {"bit8": 0.5, "bit4": 1.0, "sink": 256}}, args)
+    out = model.generate("SQAttn", ids.to(DEV), mask.to(DEV), 3, verbose=False)
+    assert len(out) == 2 and all(len(o) == 3 for o in out)
+    assert model.kv_cache.valid_length.cpu().tolist() == [512 + 2, 384 + 2]
+    assert all(0 <= t < 1000 for o in out for t in o)
