@@ -241,15 +241,20 @@ def time_e2e(torch, N, new_tokens=17, sqattn=False):
 
     dev = "cuda:0"
     cfg = QwenConfig()
-    model = QwenModel("Qwen2.5-7B-shaped", N + new_tokens, torch.bfloat16, dev, "SQAttn" if sqattn else "FlashAttn", config=cfg, seed=1)
+    model = QwenModel("Qwen2.5-7B-shaped", N + new_tokens + 32, torch.bfloat16, dev, "SQAttn" if sqattn else "FlashAttn", config=cfg, seed=1)
     if sqattn:
         ws = {i: {"bit8": 0.25, "bit4": 0.5, "sink": 256} for i in range(1, cfg.num_hidden_layers - 1)}
         process_model(model, "SQAttn", ws, types.SimpleNamespace(qk_qtype="int", v_qtype="int", use_relative_distance=True))
     ids = torch.randint(0, cfg.vocab_size, (1, N), device=dev, generator=torch.Generator(device=dev).manual_seed(2))
     model.generate(model.attention_type, ids[:, :4096], None, 3, verbose=False)    # warm-up: library handles, GEMM heuristics
-    model.generate(model.attention_type, ids, None, new_tokens, verbose=False)
+    eager = model.generate(model.attention_type, ids, None, new_tokens, verbose=False)
     res = {"prefill_s": round(model.prefill_latency, 3), "decode_ms_per_step": round(model.decode_latency * 1e3, 3),
            "tokens": N, "layers": cfg.num_hidden_layers, "attention": "SQAttn windows 0.25/0.5, sink 256" if sqattn else "exact causal"}
+    if not sqattn:
+        # the same generation with the decode step replayed from a HIP graph: must produce the same tokens
+        graphed = model.generate(model.attention_type, ids, None, new_tokens + 32, verbose=False, use_graph=True)
+        assert graphed[0][:new_tokens] == eager[0], "graph-replayed decode diverged from the eager decode"
+        res["decode_ms_per_step_hip_graph"] = round(model.decode_latency * 1e3, 3)
     del model
     torch.cuda.empty_cache()
     return res

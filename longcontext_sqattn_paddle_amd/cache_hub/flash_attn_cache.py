@@ -113,13 +113,22 @@ class flash_attn_cache(KV_Cache):
         reference; `self.attend_length` (int32 [batch], on the device) holds how many of their rows are valid for
         this step's attention.  `valid_length` and `context` advance after the last layer.
         """
-        if max(self._host_valid) >= self.max_length:
-            raise IndexError(f"KV cache is full: a sequence already holds max_length = {self.max_length} tokens")
+        self.check_room()
         last = layer_idx == self.layer_num - 1
         b = [N.dl(t) for t in (key_states, value_states, self.key_cache[layer_idx], self.value_cache[layer_idx],
                                self.valid_length, self.attend_length)]
         N.check(self._lib.sq_kv_cache_append(*[N.ptr(x) for x in b], 1 if last else 0, N.current_stream(self.device)))
         if last:
-            self.context += 1
-            self._host_valid = [n + 1 for n in self._host_valid]
+            self.note_decode_step()
         return self.key_cache[layer_idx], self.value_cache[layer_idx]
+
+    def check_room(self) -> None:
+        if max(self._host_valid) >= self.max_length:
+            raise IndexError(f"KV cache is full: a sequence already holds max_length = {self.max_length} tokens")
+
+    def note_decode_step(self) -> None:
+        """Host-side bookkeeping of one finished decode step (`context`, the mirror of `valid_length`).  Called by
+        `decode_update_kv_cache` after the last layer; a caller that replays a captured decode step, where no Python
+        runs between the layers, calls `check_room()` before and this after every replay."""
+        self.context += 1
+        self._host_valid = [n + 1 for n in self._host_valid]

@@ -12,7 +12,8 @@ Differences, all deliberate:
     of 8192 // batch tokens, which bounds its 2 x intermediate-size activations;
   * decode attention covers `kv_cache.attend_length` tokens of each sequence, not the whole cache buffer;
   * a left-padded prompt (`valid_start > 0`) runs its attention over the valid tokens only, the padding rows get
-    zeros (the reference hands the kernels more queries than keys, which they reject).
+    zeros (the reference hands the kernels more queries than keys, which they reject);
+  * `generate(..., use_graph=True)` replays the decode step from a HIP graph (no reference counterpart).
 """
 from __future__ import annotations
 
@@ -114,7 +115,41 @@ class LLM:
         hidden_states = self.layernorm(hidden_states[:, -1:, :], self.norm_variance_epsilon, self.norm_weight)
         return self.lm(hidden_states)
 
-    def inference(self, inputs_ids, verbose: bool = True):
+    # ------------------------------------------------------------------ captured decode step (extension)
+    def capture_decode_step(self, first_token):
+        """Record one decode step (all layers, final norm, lm head) into a HIP graph and run it once.
+
+        Outside the attention kernel a decode step is a chain of small launches (five GEMMs, two norms, rotary,
+        cache append, residual adds per layer) whose launch cost exceeds their run time; replaying them as one graph
+        removes it.  Everything the step depends on lives on the device and is advanced by the graph itself: the
+        token buffer is written by the caller, the position by an in-graph increment, the cache lengths by the
+        append kernel.  The arg-max over the logits stays outside the graph.  Returns the logits of this step."""
+        dev = first_token.device
+        self._graph_token = first_token.clone()
+        self._graph_positions = torch.full((first_token.shape[0], 1), self.kv_cache.context, dtype=torch.int64, device=dev)
+        self.kv_cache.check_room()
+        torch.cuda.synchronize()
+        self._graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self._graph):
+            self._graph_logits = self.decode_forward(self._graph_token)   # host bookkeeping of this step runs here, once
+            self._graph_positions += 1
+        self._graph.replay()
+        return self._graph_logits
+
+    def replay_decode_step(self, token):
+        """Run the captured step for `token` [batch, 1]; returns its logits (a buffer reused by every replay)."""
+        self.kv_cache.check_room()
+        self._graph_token.copy_(token)
+        self._graph.replay()
+        self.kv_cache.note_decode_step()
+        return self._graph_logits
+
+    def release_decode_graph(self):
+        self._graph = None
+        self._graph_positions = None
+        self._graph_token = self._graph_logits = None
+
+    def inference(self, inputs_ids, verbose: bool = True, use_graph: bool = False):
         """LLM.py:167-203: greedy decoding; returns the generated ids as nested lists [batch][max_new_length]."""
         outputs_ids = []
         torch.cuda.synchronize()
@@ -128,19 +163,30 @@ class LLM:
         if verbose:
             print(f"Prefilling latency: {round(self.prefill_latency, 4)} s")
         if self.max_new_length > 1:
-            decode_start = time.time()
-            for _ in range(self.max_new_length - 1):
-                logits = self.decode_forward(inputs_ids=output_ids)
+            decode_start, timed_steps = time.time(), self.max_new_length - 1
+            for step in range(self.max_new_length - 1):
+                if not use_graph or step == 0:
+                    logits = self.decode_forward(inputs_ids=output_ids)    # the first step also warms the libraries up
+                elif step == 1:
+                    logits = self.capture_decode_step(output_ids)
+                else:
+                    logits = self.replay_decode_step(output_ids)
                 output_ids = logits.argmax(dim=-1)
                 outputs_ids.append(output_ids)
+                if use_graph and step == 1 and self.max_new_length > 3:
+                    torch.cuda.synchronize()      # steady state of the replays: leave the warm-up and capture steps out
+                    decode_start, timed_steps = time.time(), self.max_new_length - 3
             torch.cuda.synchronize()
-            self.decode_latency = (time.time() - decode_start) / (self.max_new_length - 1)
+            if use_graph:
+                self.release_decode_graph()
+            self.decode_latency = (time.time() - decode_start) / timed_steps
             if verbose:
                 print(f"Decoding latency: {round(self.decode_latency * 1000, 2)} ms/step, "
                       f"Throughput: {round(self.batch_size / self.decode_latency, 2)} tokens/s")
         return torch.cat(outputs_ids, dim=-1).tolist()
 
-    def generate(self, attention_type, inputs_ids, attention_masks, max_new_length, verbose: bool = True):
+    def generate(self, attention_type, inputs_ids, attention_masks, max_new_length, verbose: bool = True,
+                 use_graph: bool = False):
         """LLM.py:205-235.  attention_masks [batch, input_length] of 0/1 with the padding on the left, or None."""
         bs, input_length = inputs_ids.shape
         assert input_length + max_new_length <= self.max_length, (
@@ -154,4 +200,4 @@ class LLM:
         else:
             valid_start = (attention_masks.shape[1] - attention_masks.sum(dim=-1)).tolist()
         self.init_kv_cache(input_length, valid_start)
-        return self.inference(inputs_ids, verbose=verbose)
+        return self.inference(inputs_ids, verbose=verbose, use_graph=use_graph)

@@ -210,5 +210,8 @@ class QwenModel(LLM):
     def position_embedd(self, query_states, key_states):
         """qwen.py:369-379: every sequence of the batch sits at positions context .. context + seq_len."""
         bsz, seq_len, _ = key_states.shape
-        position_ids = self.position_ids[self.kv_cache.context:self.kv_cache.context + seq_len].unsqueeze(0).repeat(bsz, 1)
+        if getattr(self, "_graph_positions", None) is not None and seq_len == 1:
+            position_ids = self._graph_positions   # device-resident position of a captured decode step
+        else:
+            position_ids = self.position_ids[self.kv_cache.context:self.kv_cache.context + seq_len].unsqueeze(0).repeat(bsz, 1)
         return self.apply_rotary_pos_emb(query_states, key_states, position_ids)

@@ -73,3 +73,44 @@ def test_left_padded_batch_and_sqattn_plugin_layers():
     assert len(out) == 2 and all(len(o) == 3 for o in out)
     assert model.kv_cache.valid_length.cpu().tolist() == [512 + 2, 384 + 2]
     assert all(0 <= t < 1000 for o in out for t in o)
+
+
+def test_graph_replayed_decode_equals_eager_decode():
+    """The captured decode step is replayed many times, with eager work and synchronisations in between, and every
+    replay must give the tokens and logits of the eager loop."""
+    print("case model decode graph", flush=True)
+    g = torch.Generator().manual_seed(5)
+    ids = torch.randint(0, 1000, (2, 200), generator=g).to(DEV)
+    new = 12
+    eager_model = _small_model()
+    eager = eager_model.generate("SDPA", ids, None, new, verbose=False)
+    model = _small_model()
+    graphed = model.generate("SDPA", ids, None, new, verbose=False, use_graph=True)
+    assert graphed == eager
+    assert model.kv_cache.context == eager_model.kv_cache.context == 200 + new - 1
+    assert model.kv_cache.valid_length.cpu().tolist() == [200 + new - 1] * 2
+    for layer in range(2):
+        assert torch.equal(model.kv_cache.key_cache[layer][:, :200 + new - 1], eager_model.kv_cache.key_cache[layer][:, :200 + new - 1])
+    # step by step with unrelated eager work between the replays: logits bit-identical to the eager path
+    a, b = _small_model(), _small_model()
+    for m in (a, b):
+        m.batch_size, m.max_new_length = 2, new
+        m.init_kv_cache(200, [0, 0])
+    tok = a.prefill_forward(ids).argmax(dim=-1)
+    b.prefill_forward(ids)
+    la = a.decode_forward(tok)
+    lb = b.decode_forward(tok)
+    assert torch.equal(la, lb)
+    tok = la.argmax(dim=-1)
+    lb = b.capture_decode_step(tok).clone()
+    la = a.decode_forward(tok)
+    assert torch.equal(la, lb)
+    for _ in range(6):
+        tok = la.argmax(dim=-1)
+        junk = torch.randn(512, 512, device=DEV) @ torch.randn(512, 512, device=DEV)   # eager work between replays
+        torch.cuda.synchronize()
+        lb = b.replay_decode_step(tok).clone()
+        la = a.decode_forward(tok)
+        torch.cuda.synchronize()
+        assert torch.equal(la, lb) and bool(torch.isfinite(junk).all())
+    b.release_decode_graph()
