@@ -275,6 +275,26 @@ __device__ __forceinline__ float max3(float a, float b, float c) {
   return r;
 }
 
+// Chains of max3 as single asm statements: the compiler puts a wait-state nop behind every asm statement that a
+// vector instruction follows, so a chain written as separate statements carries one nop per link.
+__device__ __forceinline__ float max3_of8(float a0, float a1, float a2, float a3, float a4, float a5, float a6, float a7) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3\n\tv_max3_f32 %0, %0, %4, %5\n\tv_max3_f32 %0, %0, %6, %7\n\tv_max3_f32 %0, %0, %8, %8"
+      : "=&v"(r)
+      : "v"(a0), "v"(a1), "v"(a2), "v"(a3), "v"(a4), "v"(a5), "v"(a6), "v"(a7));
+  return r;
+}
+__device__ __forceinline__ float max3_of5(float a0, float a1, float a2, float a3, float a4) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3\n\tv_max3_f32 %0, %0, %4, %5" : "=&v"(r) : "v"(a0), "v"(a1), "v"(a2), "v"(a3), "v"(a4));
+  return r;
+}
+__device__ __forceinline__ float max3_of4(float a0, float a1, float a2, float a3) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3\n\tv_max3_f32 %0, %0, %4, %4" : "=&v"(r) : "v"(a0), "v"(a1), "v"(a2), "v"(a3));
+  return r;
+}
+
 // max3 above is opaque to the compiler's hazard logic, which therefore does not separate it from a matrix
 // instruction that has just written its inputs.  Where a max3 chain directly follows such instructions, this
 // supplies the wait states by hand (the longest requirement, after a 16-pass MFMA, is below 32).
@@ -747,19 +767,16 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
           // behind the last MFMA.
           const f32x16_t& sn = Snext[bd >> 1];
           constexpr int o = 8 * (bd & 1);
-          float c = max3(sn[o], sn[o + 1], sn[o + 2]);
-          c = max3(c, sn[o + 3], sn[o + 4]);
-          c = max3(c, sn[o + 5], sn[o + 6]);
-          cm[bd] = max3(c, sn[o + 7], sn[o + 7]);
+          cm[bd] = max3_of8(sn[o], sn[o + 1], sn[o + 2], sn[o + 3], sn[o + 4], sn[o + 5], sn[o + 6], sn[o + 7]);
           const f32x16_t& s3 = Snext[1];
           if constexpr (bd == 0) cm[3] = max3(s3[8], s3[9], s3[10]);
           if constexpr (bd == 1) cm[3] = max3(cm[3], s3[11], s3[12]);
-          if constexpr (bd == 2) cm[3] = max3(max3(cm[3], s3[13], s3[14]), s3[15], s3[15]);
+          if constexpr (bd == 2) cm[3] = max3_of4(cm[3], s3[13], s3[14], s3[15]);
         }
         __builtin_amdgcn_sched_barrier(0);
       });
       // (placing this reduction in the third slot as well, ahead of the last MFMA, measured 0.8 % slower)
-      tmax_row = xor32_max(max3(max3(cm[0], cm[1], cm[2]), cm[3], cm[3]));
+      tmax_row = xor32_max(max3_of4(cm[0], cm[1], cm[2], cm[3]));
       l_run += ps[0] + ps[1];
       moved = __any(tmax_row > kC);
       if constexpr (MODE == 5) e_row = block_exp(tmax_row);
@@ -803,19 +820,15 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
         __builtin_amdgcn_sched_barrier(0);
       });
       float ps[2] = {0.f, 0.f}, cm[4], tm = 0.f;
-      auto max_op = [&](auto K) {   // step k of the lane maximum over the next tile's scores (18 steps)
+      auto max_pair = [&](auto K) {   // two links of the lane maximum over the next tile's scores (9 pairs), one asm each
         constexpr int k = decltype(K)::value;
-        if constexpr (k < 16) {
-          constexpr int h = k >> 2, j = k & 3, o = 8 * (h & 1);
+        if constexpr (k < 8) {
+          constexpr int h = k >> 1, o = 8 * (h & 1);
           const f32x16_t& sn = Snext[h >> 1];
-          if constexpr (j == 0) cm[h] = max3(sn[o], sn[o + 1], sn[o + 2]);
-          else if constexpr (j == 1) cm[h] = max3(cm[h], sn[o + 3], sn[o + 4]);
-          else if constexpr (j == 2) cm[h] = max3(cm[h], sn[o + 5], sn[o + 6]);
-          else cm[h] = max3(cm[h], sn[o + 7], sn[o + 7]);
-        } else if constexpr (k == 16) {
-          tm = max3(cm[0], cm[1], cm[2]);
+          if constexpr ((k & 1) == 0) cm[h] = max3_of5(sn[o], sn[o + 1], sn[o + 2], sn[o + 3], sn[o + 4]);
+          else cm[h] = max3_of4(cm[h], sn[o + 5], sn[o + 6], sn[o + 7]);
         } else {
-          tm = max3(tm, cm[3], cm[3]);
+          tm = max3_of4(cm[0], cm[1], cm[2], cm[3]);
         }
       };
       static_for<0, 16>([&](auto I) {
@@ -829,10 +842,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
         if constexpr (sl == 0) pack_unit(std::integral_constant<int, 7>{});
         ps[0] += S[sl >> 3][2 * (sl & 7)];
         ps[1] += S[sl >> 3][2 * (sl & 7) + 1];
-        if constexpr (sl >= 7) {
-          max_op(std::integral_constant<int, 2 * (sl - 7)>{});
-          max_op(std::integral_constant<int, 2 * (sl - 7) + 1>{});
-        }
+        if constexpr (sl >= 7) max_pair(std::integral_constant<int, sl - 7>{});
         __builtin_amdgcn_sched_barrier(0);
       });
       tmax_row = xor32_max(tm);
