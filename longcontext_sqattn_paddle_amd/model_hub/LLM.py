@@ -85,6 +85,8 @@ class LLM:
         value_states = value_states.view(bsz, -1, self.num_key_value_heads, self.head_dim)
         key_states, value_states = self.kv_cache.decode_update_kv_cache(key_states, value_states, layer_idx)
         attn_out = layer.decode_attention(query_states, key_states, value_states, None)
+        if isinstance(attn_out, tuple):   # the slot `process_model(..., patch_decode=True)` binds returns a 1-tuple (LLM.py:105)
+            attn_out = attn_out[0]
         hidden_states = self.wo(attn_out, layer, bsz, seq_len, dim)
         hidden_states = residual + hidden_states
         residual = hidden_states

@@ -54,6 +54,9 @@ def process_model(model, method, window_sizes=None, args=None, patch_decode=Fals
 def decode_attention_fn(module, query_states, key_states, value_states, layer_idx=None, seqlens=None):
     """`layer.decode_attention(q [B,1,Hq,D], Kcache, Vcache [B,L,Hkv,D], None)[0]` slot (model_hub/LLM.py:105):
     returns a 1-tuple so that the caller's `[0]` picks the [B,1,Hq*D] output."""
+    cache = getattr(module, "kv_cache", None)
+    if seqlens is None and cache is not None:
+        seqlens = cache.attend_length   # this package's cache knows how many rows of the buffers are valid
     out = attn_decode(query_states, key_states, value_states, "NHD", query_states.dtype, seqlens=seqlens)
     b, n, h, d = out.shape
     return (out.reshape(b, n, h * d),)

@@ -68,7 +68,7 @@ def test_left_padded_batch_and_sqattn_plugin_layers():
     mask = torch.ones(2, 512, dtype=torch.int64)
     mask[1, :128] = 0
     args = types.SimpleNamespace(qk_qtype="int", v_qtype="int", use_relative_distance=True)
-    process_model(model, "SQAttn", {1: {"bit8": 0.5, "bit4": 1.0, "sink": 256}}, args)
+    process_model(model, "SQAttn", {1: {"bit8": 0.5, "bit4": 1.0, "sink": 256}}, args, patch_decode=True)
     out = model.generate("SQAttn", ids.to(DEV), mask.to(DEV), 3, verbose=False)
     assert len(out) == 2 and all(len(o) == 3 for o in out)
     assert model.kv_cache.valid_length.cpu().tolist() == [512 + 2, 384 + 2]
