@@ -176,3 +176,36 @@ def test_selected_decode_argument_errors():
         attn_decode_selected(q, kc, kc, torch.zeros(3, 8, dtype=torch.int32, device=dev), "NHD")
     with pytest.raises(AssertionError, match="token_ids"):
         attn_decode_selected(q, kc, kc, torch.zeros(2, 8, dtype=torch.int64, device=dev), "NHD")
+
+
+@pytest.mark.parametrize("B,L", [(1, 1048576), (8, 131072)])
+def test_full_size_decode_against_closed_form(B, L):
+    """The benchmark shapes (1M-token cache at batch 1; 128K-token cache at batch 8 with ragged lengths): every q head
+    against the closed form on the CPU."""
+    print(f"case decode full size B={B} L={L}", flush=True)
+    dev = torch.device("cuda:0")
+    Hq, Hkv, D = 28, 4, 128
+    g = torch.Generator(device=dev).manual_seed(9)
+    q = torch.randn(B, 1, Hq, D, device=dev, generator=g).bfloat16()
+    kc = (torch.randn(B, L, Hkv, D, device=dev, generator=g) * 0.5).bfloat16()
+    vc = torch.randn(B, L, Hkv, D, device=dev, generator=g).bfloat16()
+    lens = [L] if B == 1 else [int(x) for x in torch.randint((3 * L) // 4, L + 1, (B,), generator=torch.Generator().manual_seed(1))]
+    from longcontext_sqattn_paddle_amd.sqattn.attn_triton_decode import attn_decode
+
+    out, lse = attn_decode(q, kc, vc, "NHD", torch.float32, return_lse=True,
+                           seqlens=torch.tensor(lens, dtype=torch.int32, device=dev))
+    torch.cuda.synchronize()
+    qf = A.fold_scale(q.cpu().permute(0, 2, 1, 3), D).double()      # [B, Hq, 1, D], carries log2e / sqrt(D)
+    for b in range(B):
+        kb = kc[b, :lens[b]].cpu().double()
+        vb = vc[b, :lens[b]].cpu().double()
+        for kvh in range(Hkv):
+            s = torch.einsum("nd,hd->hn", kb[:, kvh], qf[b, kvh * 7:(kvh + 1) * 7, 0])
+            m = s.max(dim=1, keepdim=True).values
+            p = torch.exp2(s - m)
+            ref = (p @ vb[:, kvh]) / p.sum(dim=1, keepdim=True)
+            ref_lse = (m + torch.log2(p.sum(dim=1, keepdim=True)))[:, 0]
+            got = out[b, 0, kvh * 7:(kvh + 1) * 7].cpu().double()
+            rms = float(ref.pow(2).mean().sqrt())
+            assert float((got - ref).abs().max()) <= 2e-4 * rms + 1e-6
+            assert torch.allclose(lse[b, kvh * 7:(kvh + 1) * 7, 0].cpu().double(), ref_lse, atol=2e-4)

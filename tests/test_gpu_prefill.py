@@ -269,3 +269,41 @@ def test_prefill_argument_errors():
         attn_hierarchical_relative_window(q, k, q, k, k, 0.1, 0.1, 2.5)
     with pytest.raises(RuntimeError):     # no CPU path
         attn_causal(q.cpu(), k.cpu(), k.cpu())
+
+
+@pytest.mark.parametrize("mode", [0, 5])
+def test_full_size_128k_sampled_rows(mode):
+    """The benchmark shape (1 x 28/4 heads x 131072 x 128): rows sampled over the whole sequence (first row, tile and
+    block edges, middle, last) against exact attention of that row on the CPU, plus the base-2 LSE."""
+    from longcontext_sqattn_paddle_amd.sqattn.attn_triton import attn_causal
+
+    print(f"case prefill 128K sampled rows mode={mode}", flush=True)
+    N, Hq, Hkv, D = 131072, 28, 4, 128
+    g = torch.Generator(device=DEV).manual_seed(5)
+    q = (torch.randn(1, Hq, N, D, device=DEV, generator=g) * 0.7).bfloat16()
+    k = (torch.randn(1, Hkv, N, D, device=DEV, generator=g) * 0.7).bfloat16()
+    v = torch.randn(1, Hkv, N, D, device=DEV, generator=g).bfloat16()
+    out, lse = attn_causal(q, k, v, "HND", torch.float32, return_lse=True, p_quant=mode)
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(out).all())
+    kc, vc = k.cpu().double(), v.cpu().double()
+    rows = [0, 1, 63, 64, 255, 256, 4095, 65535, 65536, 100000, 131071]
+    worst = 0.0
+    for h in (0, 6, 7, 27):
+        kvh = h // (Hq // Hkv)
+        for i in rows:
+            qi = A.fold_scale(q[:, h:h + 1, i:i + 1].cpu(), D).double()[0, 0, 0]       # carries log2e / sqrt(D)
+            s = kc[0, kvh, :i + 1] @ qi
+            m = s.max()
+            p = torch.exp2(s - m)
+            ref = (p[:, None] * vc[0, kvh, :i + 1]).sum(0) / p.sum()
+            ref_lse = float(m + torch.log2(p.sum()))
+            got = out[0, h, i].cpu().double()
+            err = float((got - ref).abs().max())
+            scale = float(ref.abs().max()) + 1e-3
+            worst = max(worst, err / scale)
+            # exact mode: fp16 P and V.  Mode 5: e4m3 P (block-scaled) and e4m3 V, whose elements sit within half a
+            # spacing (2^-4 relative) of the true value: a row with one key reproduces a quantised V row
+            assert err <= (4e-3 if mode == 0 else 7e-2) * scale, (h, i, err, scale)
+            assert abs(float(lse[0, h, i]) - ref_lse) <= 2e-3, (h, i, float(lse[0, h, i]), ref_lse)
+    print(f"  worst relative row error {worst:.2e}", flush=True)
