@@ -476,6 +476,13 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
   // cinit = kC - m_run (kC = log2(448) in MODE 3, else 0), so the MFMA chain delivers S - m_run + kC and, as
   // long as the running maximum does not move, p (or 448 p) is a bare exp2 of the accumulator.
   constexpr float kC = (MODE >= 3) ? kLog2_448 : 0.f;
+  // Lazy re-centring (MODE 5): a row maximum may rise up to kLazy (in log2 units) above the reference before the
+  // accumulators are rescaled; the block scale absorbs any power of two (its exponent then exceeds 127), while the
+  // fp32 accumulators and the denominator carry the common factor until the division at the end.  A row is shifted
+  // only when its own maximum passes the limit, so its arithmetic does not depend on the other rows of the wave.
+  // The other modes keep the reference's rounding points (fp16 P, static e4m3 scale) and re-centre at once.
+  constexpr float kLazy = (MODE == 5) ? 16.f : 0.f;
+  constexpr float kMove = kC + kLazy;
   float m_run = 0.f;       // reference point of the exponent; the first visited tile replaces it by the row maximum
   float l_run = 0.f;       // this lane's share of the denominator (times 448 in MODE 3)
   bool first = true;       // wave-uniform: no tile visited yet
@@ -610,7 +617,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
   // MODE 5: block scale of a row's 64 probabilities in a tile, 2^k with k = floor(log2 448 - t) in [0, 60] for the
   // row maximum t of the scores (which carry log2 448); kept as the E8M0 exponent 127 - k = ceil(t + 127 - log2 448)
   // of 2^-k.  Computed one step ahead like tmax_row, again after a shift of the reference.
-  auto block_exp = [](float t) { return (int)__builtin_ceilf(__builtin_amdgcn_fmed3f(t + (127.f - kC), 67.f, 127.f)); };
+  auto block_exp = [](float t) { return (int)__builtin_ceilf(__builtin_amdgcn_fmed3f(t + (127.f - kC), 67.f, 127.f + kLazy)); };
   int e_row = 127;
 
   // softmax update + P.V for the tile whose scores are in S.  Once the running maximum of this tile is settled,
@@ -649,7 +656,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
     if constexpr (MODE != 2) {
       if (masked) {
         tmax_row = xor32_max(lane_max(S));
-        moved = __any(tmax_row > kC);
+        moved = __any(tmax_row > kMove);
         if constexpr (MODE == 5) e_row = block_exp(tmax_row);
       }
       tmax = tmax_row;   // came out of the previous step's P.V phase
@@ -660,13 +667,13 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
       for (int i = 1; i < 15; ++i) tmax = max3(tmax, S[1][i], S[0][i + 1]);
       tmax = max3(tmax, S[1][15], S[1][15]);
       tmax = xor32_max(tmax);
-      slow = first || __any(tmax > kC);
+      slow = first || __any(tmax > kMove);
     }
     if (slow) {
       // some row's maximum moved by d (on the first tile: from the arbitrary reference 0 to the row maximum):
       // shift the scores, rescale the accumulators, re-centre the accumulator initialiser
       asm volatile("; new row maximum" ::: "memory");
-      const float d = first ? (tmax - kC) : fmaxf(tmax - kC, 0.f);
+      const float d = first ? (tmax - kC) : ((tmax > kMove) ? tmax - kC : 0.f);
       const float alpha = first ? 0.f : __builtin_amdgcn_exp2f(-d);
       m_run += d;
       l_run *= alpha;
@@ -778,7 +785,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
       // (placing this reduction in the third slot as well, ahead of the last MFMA, measured 0.8 % slower)
       tmax_row = xor32_max(max3_of4(cm[0], cm[1], cm[2], cm[3]));
       l_run += ps[0] + ps[1];
-      moved = __any(tmax_row > kC);
+      moved = __any(tmax_row > kMove);
       if constexpr (MODE == 5) e_row = block_exp(tmax_row);
       __builtin_amdgcn_s_setprio(3);
       return;
@@ -846,7 +853,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
         __builtin_amdgcn_sched_barrier(0);
       });
       tmax_row = xor32_max(tm);
-      moved = __any(tmax_row > kC);
+      moved = __any(tmax_row > kMove);
       l_run += ps[0] + ps[1];
       __builtin_amdgcn_s_setprio(3);
       return;
@@ -945,7 +952,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
     if constexpr (MODE != 2) {
       mfma_settle(Sa[0], Sa[1]);
       tmax_row = xor32_max(lane_max(Sa));
-      moved = __any(tmax_row > kC);
+      moved = __any(tmax_row > kMove);
       if constexpr (MODE == 5) e_row = block_exp(tmax_row);
     }
   }
@@ -985,7 +992,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
         if constexpr (MODE != 2) {
           mfma_settle(Snxt[0], Snxt[1]);
           tmax_row = xor32_max(lane_max(Snxt));
-          moved = __any(tmax_row > kC);
+          moved = __any(tmax_row > kMove);
           if constexpr (MODE == 5) e_row = block_exp(tmax_row);
         }
       }

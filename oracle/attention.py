@@ -27,6 +27,7 @@ MASK_ADD = -1000000.0  # additive causal mask (attn_triton.py:71)
 
 P_NONE, P_STATIC448, P_BLOCK_ABSMAX, P_STATIC448_GRID = 0, 1, 2, 3
 P_MX_ROW = 5   # e4m3 with one power-of-two scale per query row and 64-key tile (block-scaled fp8 MFMA operand)
+MX_LAZY = 16.0  # P_MX_ROW: a row's reference point follows its maximum only once the maximum leads by more than this (log2)
 
 
 # --------------------------------------------------------------------------- helpers
@@ -95,10 +96,11 @@ def _quant_p(p: torch.Tensor, mode: int, group_rows: int = 64) -> torch.Tensor:
     if mode == P_STATIC448_GRID:   # the e4m3 grid of mode 1 without the fp16 rounding of p/448 (fp8 operand of an fp8 MFMA)
         return (p * 448.0).to(torch.float8_e4m3fn).float() / 448.0
     if mode == P_MX_ROW:
-        # build-defined: scale 2^k per row of the tile with k = floor(-log2(row maximum)) in [0, 60], so that the
-        # row's largest scaled probability lies in (224, 448]; the dequantised value is e4m3(p*448*2^k) / (448*2^k)
+        # build-defined: scale 2^k per row of the tile with k = floor(-log2(row maximum)) in [-MX_LAZY, 60], so that the
+        # row's largest scaled probability lies in (224, 448]; the dequantised value is e4m3(p*448*2^k) / (448*2^k).
+        # (p is taken relative to a reference that may trail the row maximum by up to MX_LAZY, see _RowState.update.)
         a = p.max(dim=1, keepdim=True).values
-        k = torch.floor(-torch.log2(a)).clamp(0.0, 60.0)
+        k = torch.floor(-torch.log2(a)).clamp(-MX_LAZY, 60.0)
         k = torch.where(a > 0, k, torch.full_like(k, 60.0))
         sc = torch.exp2(k) * 448.0
         return (p * sc).to(torch.float8_e4m3fn).float() / sc
@@ -130,6 +132,13 @@ class _RowState:
         """One KV-block step (attn_triton.py:72-84). `s` fp32 [rows, cols], `vblk` fp32 [cols, D]
         holding fp16-representable values."""
         m_new = torch.maximum(self.m, s.max(dim=1).values)
+        if p_quant == P_MX_ROW:
+            # build-defined: the reference point m is not the running maximum itself.  It is set by the first block and
+            # afterwards replaced by a row's block maximum only when that exceeds it by more than MX_LAZY; until then
+            # p = 2^(s - m) may exceed 1 (the block scale of _quant_p absorbs the factor) and l, acc carry the same factor,
+            # which cancels in finish().  Mathematically the same softmax; the e4m3 grid points differ.
+            keep = (self.m > float("-inf")) & ~(m_new - self.m > MX_LAZY)
+            m_new = torch.where(keep, self.m, m_new)
         p = torch.exp2(s - m_new[:, None])
         alpha = torch.exp2(self.m - m_new)
         self.l = self.l * alpha + p.sum(dim=1)

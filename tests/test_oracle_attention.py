@@ -167,6 +167,32 @@ def test_block_scaled_p_quantiser_properties():
     assert torch.equal(A._quant_p(torch.zeros(2, 64), A.P_MX_ROW), torch.zeros(2, 64))
 
 
+def test_block_scaled_p_reference_point_is_lazy_but_the_softmax_is_not():
+    """`P_MX_ROW` keeps a row's reference point until the row maximum leads it by more than `MX_LAZY`.  What that must
+    not change: the log-sum-exp (no quantised quantity enters it) and the output up to e4m3 noise, also when the
+    maxima rise block after block by more than the limit in total and, for some rows, in one step."""
+    N, D = 512, 64
+    g = torch.Generator().manual_seed(21)
+    q = torch.randn(1, 2, N, D, generator=g)
+    k = torch.randn(1, 1, N, D, generator=g)
+    v = torch.randn(1, 1, N, D, generator=g)
+    # scores grow with the key index: about +6 (log2) per 64-key block, and +40 at key 320 for every later row
+    ramp = torch.arange(N, dtype=torch.float32) / 64.0 * 6.0
+    ramp[320:] += 40.0
+    q[..., 0] = 1.0
+    k[0, 0, :, 0] = ramp * (D ** 0.5 / 1.44269504)
+    q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
+    exact, lse_exact = A.exact_attention(q, k, v)
+    out, lse = A.prefill_blockwise(q, k, v, p_quant=A.P_MX_ROW, out_dtype=torch.float32)
+    eager, lse_eager = A.prefill_blockwise(q, k, v, p_quant=A.P_STATIC448_GRID, out_dtype=torch.float32)
+    # (the blockwise path rounds the pre-scaled q to 16 bits like the reference, hence the loose bound against exact)
+    assert torch.allclose(lse, lse_exact.float(), atol=1e-2, rtol=5e-3)
+    assert torch.allclose(lse, lse_eager, atol=2e-4, rtol=1e-6)
+    cos = lambda a, b: float((a.double() * b.double()).sum() / (a.double().norm() * b.double().norm()))
+    assert cos(out, exact) >= 0.9995
+    assert cos(out, exact) >= cos(eager, exact) - 1e-4   # no worse than the static scale with its eager reference
+
+
 def test_window_invariants_and_explicit_mask():
     N, D = 512, 64
     q, k, v = _rand(1, 2, 1, N, N, D, 5)
