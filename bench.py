@@ -326,6 +326,32 @@ def time_kv_cache(torch, N, iters=10):
     return store_us, store_bytes, append_us
 
 
+def time_calibration(torch, N, iters=3):
+    """The window search's histogram kernel at the benchmark's head shape (28 q heads / 4 kv heads / 128) on an
+    N-token sample, both binning rules the calibration drivers use.  Work: Q.K^T over the causal half twice (once for
+    the row normalisers, once for the probabilities) = 4 N^2 D Hq / 2 FLOP, i.e. what the prefill kernel does."""
+    from longcontext_sqattn_paddle_amd.sqattn.window_search import ABSOLUTE, RELATIVE_SINK, attention_histograms
+
+    dev = torch.device("cuda:0")
+    Hq, Hkv, D = 28, 4, 128
+    g = torch.Generator(device=dev).manual_seed(6)
+    q = (torch.randn(1, N, Hq, D, device=dev, generator=g) * 1.5).bfloat16()
+    k = torch.randn(1, N, Hkv, D, device=dev, generator=g).bfloat16()
+    out = {}
+    for name, kind, bins, sink in (("absolute", ABSOLUTE, N, 0), ("relative_sink", RELATIVE_SINK, 200, 256)):
+        hist = torch.zeros(1, Hq, bins, dtype=torch.float64, device=dev)
+        attention_histograms(q, k, kind, bins, sink, out=hist)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(iters):
+            attention_histograms(q, k, kind, bins, sink, out=hist)
+        e1.record()
+        torch.cuda.synchronize()
+        out[name] = e0.elapsed_time(e1) / iters
+    return out, 4.0 * N * N * D * Hq / 2
+
+
 def time_kmeans(torch, iters=10):
     """One Lloyd iteration (assign + counting sort + exact cluster sums + centroid update) at the benchmark's
     clustering shape: 4 kv heads x 131072 tokens x 128, 1024 centroids."""
@@ -403,6 +429,7 @@ def main():
     ap.add_argument("--no-kv-cache", action="store_true")
     ap.add_argument("--no-layer", action="store_true")
     ap.add_argument("--no-model", action="store_true")
+    ap.add_argument("--no-calibration", action="store_true")
     ap.add_argument("--e2e", action="store_true",
                     help="also run the whole 28-layer Qwen2.5-7B-shaped decoder (random weights): prefill latency and decode ms/step")
     args = ap.parse_args()
@@ -514,6 +541,14 @@ def main():
         result["model_layers"]["note"] = ("Qwen2.5-7B-shaped decoder layers with random weights, batch 1: per-layer time of a "
                                           f"{N}-token prefill (includes 1/2 of embedding + lm head) and of a decode step at that context")
         log(f"[bench] model layers: {ml}")
+    if not args.no_calibration:
+        n_cal = 32768
+        cal, cflops = time_calibration(torch, n_cal)
+        result["calibration"] = {name: {"ms_per_call": round(ms, 3), "TFLOP_per_s": round(cflops / ms / 1e9, 1)} for name, ms in cal.items()}
+        result["calibration"]["shape"] = (f"one {n_cal}-token sample, 28 q heads / 4 kv heads / 128: energy histograms of all heads from "
+                                          f"Q and K; the dense attention map the reference reduces would hold {28 * n_cal * n_cal * 2 / 1e9:.0f} GB")
+        log(f"[bench] calibration histograms: {cal}")
+        torch.cuda.empty_cache()
     if args.e2e:
         result["e2e"] = [time_e2e(torch, N, sqattn=False), time_e2e(torch, N, sqattn=True)]
         log(f"[bench] end to end: {result['e2e']}")

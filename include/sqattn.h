@@ -230,6 +230,32 @@ int sq_silu_and_mul(const DLTensor* x, DLTensor* out, void* stream);
 int sq_rope(const DLTensor* query, const DLTensor* key, DLTensor* query_out, DLTensor* key_out,
             const DLTensor* position_ids, const DLTensor* cos_sin_cache, int32_t head_dim, void* stream);
 
+/*
+ * Calibration histograms of the window search, straight from Q and K: for every (batch, query head) the causal
+ * attention probabilities p[i, j] = softmax_j(softmax_scale * q_i . k_j) are added, weighted, into hist[b, h, bin].
+ * Replaces the reference's dense attention map [Hq, N, N] (sqattn/attn_replacer.py:253-278, stored as
+ * `current_attention`, model_hub/qwen.py:38-41) and the index-tensor + bincount reductions over it:
+ *   SQ_HIST_ABSOLUTE       bin = i - j,                         weight p * (i - j); distances >= bins are dropped,
+ *                          keys j < sink excluded   (sqattn/window_search.py:20-48 with sink = 0, :283-321)
+ *   SQ_HIST_RELATIVE       bin = floor(bins * (i - j) / max(i, 1)), weight p * (i - j); sink must be 0   (:51-87)
+ *   SQ_HIST_RELATIVE_SINK  keys j < sink excluded, rows i <= sink go to bin 0, otherwise
+ *                          bin = floor(bins * (i - j) / max(i - sink, 1)); weight p * (bins * rel + 1)   (:244-280)
+ * Bins are clamped to [0, bins - 1] and formed with the reference's fp32 operator sequence.  q [B, Hq, N, 128] and
+ * k [B, Hkv, N, 128] (views with any strides, contiguous last dimension, 16-byte aligned rows; Hq a multiple of Hkv),
+ * bf16 or fp16.  hist float64 [B, Hq, bins], contiguous; the call ADDS to it (clear it before the first sample,
+ * keep it across samples as the reference sums its per-sample histograms, window_search.py:158-159).  The relative
+ * kinds take at most 8192 bins.  Probabilities are formed in fp32 from the 16-bit inputs (the reference rounds the
+ * map itself to the model dtype).
+ */
+enum { SQ_HIST_ABSOLUTE = 0, SQ_HIST_RELATIVE = 1, SQ_HIST_RELATIVE_SINK = 2 };
+typedef struct sq_histogram_params {
+  int32_t kind;         /* SQ_HIST_*                                                        */
+  int32_t bins;         /* max_len (absolute) or num_bins (relative)                        */
+  int32_t sink;         /* sink_len: leading keys left out of the histogram                 */
+  float softmax_scale;  /* 1/sqrt(head_dim before padding) (attn_replacer.py:260)            */
+} sq_histogram_params;
+int sq_attention_histogram(const DLTensor* q, const DLTensor* k, DLTensor* hist, const sq_histogram_params* p, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -64,6 +64,17 @@ class DecodeParams(ctypes.Structure):
     ]
 
 
+class HistogramParams(ctypes.Structure):
+    _fields_ = [
+        ("kind", ctypes.c_int32),
+        ("bins", ctypes.c_int32),
+        ("sink", ctypes.c_int32),
+        ("softmax_scale", ctypes.c_float),
+    ]
+
+
+HIST_ABSOLUTE, HIST_RELATIVE, HIST_RELATIVE_SINK = 0, 1, 2
+
 _P = ctypes.POINTER(DLTensor)
 
 # every symbol include/sqattn.h declares: name -> (restype, argtypes)
@@ -88,6 +99,7 @@ SYMBOLS = {
     "sq_rope": (ctypes.c_int, [_P] * 6 + [ctypes.c_int32, ctypes.c_void_p]),
     "sq_kv_cache_store": (ctypes.c_int, [_P] * 4 + [ctypes.c_int32, ctypes.c_int64, ctypes.c_void_p]),
     "sq_kv_cache_append": (ctypes.c_int, [_P] * 6 + [ctypes.c_int32, ctypes.c_void_p]),
+    "sq_attention_histogram": (ctypes.c_int, [_P, _P, _P, ctypes.POINTER(HistogramParams), ctypes.c_void_p]),
 }
 
 _lib: Optional[ctypes.CDLL] = None

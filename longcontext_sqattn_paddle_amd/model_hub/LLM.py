@@ -41,7 +41,7 @@ class LLM:
     def layer_prefill(self, layer_idx, start_bdx, hidden_states):
         """LLM.py:40-86.  hidden_states [bsz, seq_len, hidden] is updated in place and returned."""
         if self.capture_layer_inps is not None:
-            self.capture_layer_inps.append(hidden_states.detach())
+            self.capture_layer_inps.append(hidden_states.detach().clone())   # the layers below update hidden_states in place
         bsz, seq_len, dim = hidden_states.shape
         layer = self.layers[layer_idx]
         normed = self.layernorm(hidden_states, layer.input_layernorm_variance_epsilon, layer.input_layernorm_weight)

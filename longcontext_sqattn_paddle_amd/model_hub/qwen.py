@@ -52,12 +52,17 @@ class QwenLayer:
         self.max_length = max_length
         self.kv_cache = None   # set by QwenModel.init_kv_cache: decode attention needs the per-sequence lengths
         self.p_quant = None    # extension: a P mode of the prefill kernel (e.g. 5 = fp8 P.V); None = exact attention
+        self.calibration = None   # a sqattn.window_search.CalibrationCapture while the window search runs on this layer
 
     def prefill_attention(self, query_states, key_states, value_states, layer_idx=None):
         """qwen.py:37-46: exact causal attention over [B, N, H, D] tensors (SDPA / flash attention in the reference;
         `process_model` replaces this slot by the quantised-window closure for the SQAttn layers)."""
         if self.attention_type not in ("SQAttn", "SDPA", "FlashAttn"):
             raise ValueError(f"Unsupported attention type: {self.attention_type}")
+        if self.calibration is not None:
+            # the reference stores the dense map here, and only for layer_idx 0 / last although its runtime always
+            # passes None (qwen.py:38-41, LLM.py:67); the capture reduces Q and K to the histograms directly
+            self.calibration.record(query_states, key_states)
         return attn_causal(query_states, key_states, value_states, "NHD", query_states.dtype, p_quant=self.p_quant)
 
     def decode_attention(self, query_states, key_states, value_states, layer_idx=None):
