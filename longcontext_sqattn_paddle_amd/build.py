@@ -19,6 +19,11 @@ HIPCC_FLAGS = [
 ]
 
 
+# Per-source flags.  The k-means assign kernel reads its MFMA results with the vector ALU right away (arg-max): the MFMAs
+# are kept in their VGPR form there, otherwise every score passes through a v_accvgpr_read first.
+SOURCE_FLAGS = {"kmeans_gfx950.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
+
+
 def build(verbose: bool = True, extra_flags=()) -> str:
     """Compile every HIP source (in parallel, one object each) and link them into one shared library; returns its
     path.  Always recompiles."""
@@ -31,7 +36,7 @@ def build(verbose: bool = True, extra_flags=()) -> str:
         jobs = []
         for s in srcs:
             obj = os.path.join(tmp, s.replace(".hip", ".o"))
-            cmd = [hipcc, *compile_flags, *extra_flags, "-I", INCLUDE, "-I", CSRC, "-c", os.path.join(CSRC, s), "-o", obj]
+            cmd = [hipcc, *compile_flags, *SOURCE_FLAGS.get(s, []), *extra_flags, "-I", INCLUDE, "-I", CSRC, "-c", os.path.join(CSRC, s), "-o", obj]
             if verbose:
                 print(" ".join(cmd), flush=True)
             jobs.append((cmd, obj, subprocess.Popen(cmd)))

@@ -32,106 +32,170 @@ struct AssignArgs {
   int32_t N, C;
 };
 
-constexpr int kAssignWaves = 8;   // x 32 tokens: 2 waves per SIMD, one wave's arg-max epilogue overlaps the other's MFMAs
+constexpr int kAssignWaves = 4;   // x 64 tokens; two workgroups per CU put two waves on every SIMD
 
-// Workgroup = 256 tokens of one group.  Centroids stream through LDS in blocks of 64 (global_load_lds, unpadded
-// rows, 16-byte chunks XOR-swizzled by row so that the MFMA operand reads are conflict free); the scores of
-// block k+1 are issued on the matrix pipe before the arg-max epilogue of block k runs on the vector ALU.
-__global__ __launch_bounds__(kAssignWaves * 64) void kmeans_assign_kernel(AssignArgs a) {
+// Workgroup = 256 tokens of one group, 64 per wave (two 32-token operand sets in registers): every centroid fragment
+// read from LDS feeds two MFMAs, which halves the LDS traffic per MFMA -- with 32 tokens per wave the fragment reads
+// of the four SIMDs add up to the LDS's whole 128 bytes per cycle.  Centroids stream through LDS in blocks of 64
+// (global_load_lds, unpadded rows, 16-byte chunks XOR-swizzled by row so that the MFMA operand reads are conflict
+// free); the scores of block k+1 are issued on the matrix pipe before the arg-max epilogue of block k runs on the
+// vector ALU.
+__global__ __launch_bounds__(kAssignWaves * 64, 1) void kmeans_assign_kernel(AssignArgs a) {
   __shared__ __attribute__((aligned(16))) char smem[2 * kCB * 256];
   typedef __attribute__((address_space(3))) void* lds_ptr_t;
   const int g_id = blockIdx.y;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c32 = lane & 31, g = lane >> 5;
-  const int tok0 = blockIdx.x * kTileTok + wave * 32;
+  const int tok0 = blockIdx.x * kTileTok + wave * 64;
 
-  // token fragments (B operand of S^T = Cent . Data^T): lane (column = token c32, k-group g)
+  // token fragments (B operand of S^T = Cent . Data^T): lane (column = token 32 tb + c32, k-group g)
   const uint16_t* db = a.data + (int64_t)g_id * a.d_sg;
-  uint4 tf[8];
-  {
-    const int n = min(tok0 + c32, a.N - 1);
+  uint4 tf[2][8];
+#pragma unroll
+  for (int tb = 0; tb < 2; ++tb) {
+    const int n = min(tok0 + 32 * tb + c32, a.N - 1);
     const uint16_t* rp = db + (int64_t)n * a.d_sn + 8 * g;
 #pragma unroll
-    for (int kk = 0; kk < 8; ++kk) tf[kk] = *(const uint4*)(rp + 16 * kk);
+    for (int kk = 0; kk < 8; ++kk) tf[tb][kk] = *(const uint4*)(rp + 16 * kk);
   }
   const uint16_t* cb = a.cent + (int64_t)g_id * a.c_sg;
+  // per-lane source of the wave's four 1 KB copies of a block (4 centroid rows each), as a byte offset from the block's
+  // first row; rows past C are clamped to the last centroid, which only a block that runs past C has to do
+  int64_t src_off[4];
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    const int row = 4 * (wave * 4 + c) + (lane >> 4);
+    src_off[c] = ((int64_t)row * a.c_sc + 8 * ((lane & 15) ^ (row & 15))) * 2;
+  }
   auto stage = [&](int chunk, int st) {
     char* buf = smem + st * (kCB * 256);
+    const char* blk = (const char*)cb + (int64_t)chunk * kCB * a.c_sc * 2;
+    if ((chunk + 1) * kCB <= a.C) {
 #pragma unroll
-    for (int c = 0; c < 2; ++c) {
-      const int q = wave * 2 + c;                      // 1 KB = 4 centroid rows per wave instruction
-      const int row = 4 * q + (lane >> 4);
-      const int ch = (lane & 15) ^ (row & 15);
-      const int crow = min(chunk * kCB + row, a.C - 1);
-      __builtin_amdgcn_global_load_lds((const void*)(cb + (int64_t)crow * a.c_sc + 8 * ch), (lds_ptr_t)(buf + q * 1024), 16, 0, 0);
+      for (int c = 0; c < 4; ++c)
+        __builtin_amdgcn_global_load_lds((const void*)(blk + src_off[c]), (lds_ptr_t)(buf + (wave * 4 + c) * 1024), 16, 0, 0);
+    } else {
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const int q = wave * 4 + c;
+        const int row = 4 * q + (lane >> 4);
+        const int ch = (lane & 15) ^ (row & 15);
+        const int crow = min(chunk * kCB + row, a.C - 1);
+        __builtin_amdgcn_global_load_lds((const void*)(cb + (int64_t)crow * a.c_sc + 8 * ch), (lds_ptr_t)(buf + q * 1024), 16, 0, 0);
+      }
     }
   };
   const int ksw = c32 & 15;
-  auto scores = [&](const char* buf, f32x16_t (&S)[2]) {
-#pragma unroll
-    for (int bn = 0; bn < 2; ++bn)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) S[bn][i] = 0.f;
-#pragma unroll
-    for (int kk = 0; kk < 8; ++kk) {
-      const uint4 a0 = *(const uint4*)(buf + c32 * 256 + (((2 * kk + g) ^ ksw) << 4));
-      const uint4 a1 = *(const uint4*)(buf + (32 + c32) * 256 + (((2 * kk + g) ^ ksw) << 4));
-      S[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a0), __builtin_bit_cast(bf16x8_t, tf[kk]), S[0], 0, 0, 0);
-      S[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a1), __builtin_bit_cast(bf16x8_t, tf[kk]), S[1], 0, 0, 0);
-    }
+  auto frag = [&](const char* buf, int half, int kk) {
+    return __builtin_bit_cast(bf16x8_t, *(const uint4*)(buf + (32 * half + c32) * 256 + (((2 * kk + g) ^ ksw) << 4)));
   };
-  // Running arg-max in ascending centroid order with strict '>' = lowest index on ties (kmeans.py:62-65).  The
-  // winner is tracked as (block, position inside the block): positions are inline constants, so an element
-  // costs a compare and two selects.  Rows past C (C % 64 == 32) are clamped copies of the last centroid; they
-  // come after it in this order and can never beat it strictly.
-  float best = -INFINITY;
-  int bloc = 0, bchunk = 0;
-  auto argmax = [&](int chunk, const f32x16_t (&S)[2]) {
-    const float before = best;
+  // Running arg-max in ascending centroid order with strict '>' = lowest index on ties (kmeans.py:62-65), four scores
+  // at a time: the group's maximum (v_max3 + v_max) is compared with the running best; a group that wins leaves its
+  // id and its first three scores behind, from which the position inside the group follows at the end (the first score
+  // equal to the best; if none of the three, the fourth).  Eight vector instructions per four scores instead of
+  // twelve.  Rows past C (C % 64 == 32) are clamped copies of the last centroid; they come after it in this order and
+  // can never beat it strictly.
+  float best[2] = {-INFINITY, -INFINITY};
+  float keep0[2] = {0.f, 0.f}, keep1[2] = {0.f, 0.f}, keep2[2] = {0.f, 0.f};
+  int bgrp[2] = {0, 0}, bhalf[2] = {0, 0};
+  // S[tb][h]: scores of token set tb against centroid half h (32 centroids) of the current block.  A block is
+  // computed in two phases of 16 MFMAs, half 0 then half 1, each as two accumulator chains (tb = 0, 1) over the eight
+  // 16-wide slices of the dimension.  Underneath the MFMAs of one phase runs the arg-max over the results of the
+  // previous phase, as one hand-ordered instruction stream: an MFMA occupies the matrix pipe for 32 cycles, half a
+  // group's arg-max (four vector instructions) issues behind it.  The accumulators are not double-buffered; with
+  // the MFMAs in their VGPR form (build flag) the arg-max reads them without copies out of the accumulation registers.
+  f32x16_t S[2][2];
 #pragma unroll
-    for (int bn = 0; bn < 2; ++bn)
+  for (int tb = 0; tb < 2; ++tb)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const float s = S[bn][i];
-        const bool gt = s > best;
-        bloc = gt ? (32 * bn + 8 * (i >> 2) + (i & 3)) : bloc;
-        best = gt ? s : best;
-      }
-    bchunk = (best > before) ? chunk : bchunk;
+    for (int i = 0; i < 16; ++i) S[tb][1][i] = -INFINITY;   // "previous phase" of the very first one
+  auto group_max = [](const f32x16_t& P, int q) {
+    // (fmaxf would quiet each operand first, one more instruction per score; the scores are never signalling NaNs)
+    float m;
+    asm("v_max3_f32 %0, %1, %2, %3\n\tv_max_f32 %0, %0, %4" : "=&v"(m) : "v"(P[4 * q]), "v"(P[4 * q + 1]), "v"(P[4 * q + 2]), "v"(P[4 * q + 3]));
+    return m;
+  };
+  auto group_take = [&](const f32x16_t& P, int tb, int q, float m, bool gt) {
+    best[tb] = gt ? m : best[tb];
+    bgrp[tb] = gt ? q : bgrp[tb];
+    keep0[tb] = gt ? P[4 * q] : keep0[tb];
+    keep1[tb] = gt ? P[4 * q + 1] : keep1[tb];
+    keep2[tb] = gt ? P[4 * q + 2] : keep2[tb];
+  };
+  auto phase = [&](auto H, const char* buf, int half_id) {
+    constexpr int h = decltype(H)::value;   // centroid half computed now; the arg-max runs over half 1 - h
+    const float before0 = best[0], before1 = best[1];
+    bf16x8_t af = frag(buf, h, 0);
+    float m = 0.f;
+    bool gt = false;
+    static_for<0, 8>([&](auto KK) {
+      constexpr int kk = decltype(KK)::value;
+      bf16x8_t nf = af;
+      if constexpr (kk < 7) nf = frag(buf, h, kk + 1);
+      static_for<0, 2>([&](auto TB) {
+        constexpr int tb = decltype(TB)::value;
+        const bf16x8_t t = __builtin_bit_cast(bf16x8_t, tf[tb][kk]);
+        if constexpr (kk == 0) {
+          const f32x16_t zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+          S[tb][h] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, t, zero, 0, 0, 0);
+        } else {
+          S[tb][h] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, t, S[tb][h], 0, 0, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // group kk of the previous phase's 8 groups (token set kk >> 2, scores 4 (kk & 3) .. + 3): its maximum under
+        // the first MFMA of the pair, the selects under the second
+        constexpr int ctb = kk >> 2, q = kk & 3;
+        if constexpr (tb == 0) {
+          m = group_max(S[ctb][1 - h], q);
+          gt = m > best[ctb];
+        } else {
+          group_take(S[ctb][1 - h], ctb, q, m, gt);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      });
+      af = nf;
+    });
+    // the scores just examined belong to the half before this one
+    bhalf[0] = (best[0] > before0) ? half_id - 1 : bhalf[0];
+    bhalf[1] = (best[1] > before1) ? half_id - 1 : bhalf[1];
   };
   const int nchunks = (a.C + kCB - 1) / kCB;
   stage(0, 0);
-  if (nchunks > 1) stage(1, 1);
-  __builtin_amdgcn_s_waitcnt(0);
-  __syncthreads();
-  f32x16_t Sa[2], Sb[2];
-  scores(smem, Sa);
-  __syncthreads();                                             // every wave has read block 0 out of LDS
-  auto step = [&](int chunk, f32x16_t (&Scur)[2], f32x16_t (&Snxt)[2]) {
-    // LDS holds block chunk+1; block `chunk` was read by every wave before the last barrier, so its buffer is free
-    if (chunk + 2 < nchunks) stage(chunk + 2, chunk & 1);
-    // unconditional, so that these MFMAs share a straight-line block with the arg-max below; after the last block
-    // they run once more on stale data and the result is dropped
-    scores(smem + ((chunk + 1) & 1) * (kCB * 256), Snxt);
-    argmax(chunk, Scur);
+  for (int chunk = 0; chunk < nchunks; ++chunk) {
     __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();                                           // block chunk+2 has landed, block chunk+1 has been read
-  };
-  for (int chunk = 0; chunk < nchunks; chunk += 2) {
-    step(chunk, Sa, Sb);
-    if (chunk + 1 >= nchunks) break;
-    step(chunk + 1, Sb, Sa);
+    // block `chunk` has landed for every wave, and every wave has finished reading block chunk - 1, whose buffer the
+    // next block may now overwrite; it has this block's 32 MFMAs per wave to arrive
+    __syncthreads();
+    if (chunk + 1 < nchunks) stage(chunk + 1, (chunk + 1) & 1);
+    const char* buf = smem + (chunk & 1) * (kCB * 256);
+    phase(std::integral_constant<int, 0>{}, buf, 2 * chunk);
+    phase(std::integral_constant<int, 1>{}, buf, 2 * chunk + 1);
   }
-  {
-    int bidx = bchunk * kCB + 4 * g + bloc;
-    const float ob = __shfl_xor(best, 32);
+  {   // the last half block
+    const float before0 = best[0], before1 = best[1];
+#pragma unroll
+    for (int tb = 0; tb < 2; ++tb)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const float m = group_max(S[tb][1], q);
+        group_take(S[tb][1], tb, q, m, m > best[tb]);
+      }
+    bhalf[0] = (best[0] > before0) ? 2 * nchunks - 1 : bhalf[0];
+    bhalf[1] = (best[1] > before1) ? 2 * nchunks - 1 : bhalf[1];
+  }
+#pragma unroll
+  for (int tb = 0; tb < 2; ++tb) {
+    const int in_group = (keep0[tb] == best[tb]) ? 0 : (keep1[tb] == best[tb]) ? 1 : (keep2[tb] == best[tb]) ? 2 : 3;
+    int bidx = bhalf[tb] * 32 + 4 * g + 8 * bgrp[tb] + in_group;
+    float bv = best[tb];
+    const float ob = __shfl_xor(bv, 32);
     const int oi = __shfl_xor(bidx, 32);
-    if (ob > best || (ob == best && oi < bidx)) {
-      best = ob;
+    if (ob > bv || (ob == bv && oi < bidx)) {
+      bv = ob;
       bidx = oi;
     }
-    const int n = tok0 + c32;
+    const int n = tok0 + 32 * tb + c32;
     // cluster sizes come out of the counting sort that follows (per-tile histograms), not out of global atomics
     if (g == 0 && n < a.N) a.idx[(int64_t)g_id * a.i_sg + n] = bidx;
   }
@@ -163,13 +227,14 @@ __global__ __launch_bounds__(kTileTok) void sort_hist_kernel(SortArgs a) {
   for (int c = threadIdx.x; c < a.C; c += blockDim.x) out[c] = hist[c];
 }
 
-// Exclusive prefix over tiles of every cluster's per-tile count.  Workgroup = 32 clusters x 8 tile segments:
-// each thread sums its segment, the 8 segment sums are scanned through LDS, then each thread rewrites its segment.
-__global__ __launch_bounds__(256) void sort_scan_tiles_kernel(SortArgs a) {
-  __shared__ int32_t seg_sum[8][32];
+// Exclusive prefix over tiles of every cluster's per-tile count.  Workgroup = 32 clusters x 32 tile segments:
+// each thread sums its segment, the 32 segment sums are scanned through LDS, then each thread rewrites its segment.
+constexpr int kScanSegs = 32;
+__global__ __launch_bounds__(32 * kScanSegs) void sort_scan_tiles_kernel(SortArgs a) {
+  __shared__ int32_t seg_sum[kScanSegs][32];
   const int cl = threadIdx.x & 31, seg = threadIdx.x >> 5;
   const int c = blockIdx.x * 32 + cl, g = blockIdx.y;
-  const int per = (a.nT + 7) / 8;
+  const int per = (a.nT + kScanSegs - 1) / kScanSegs;
   const int tb = seg * per, te = min(tb + per, a.nT);
   int32_t* h = a.tile_hist + (int64_t)g * a.nT * a.C + c;
   int sum = 0;
@@ -179,7 +244,7 @@ __global__ __launch_bounds__(256) void sort_scan_tiles_kernel(SortArgs a) {
   __syncthreads();
   int run = 0, total = 0;
 #pragma unroll
-  for (int q = 0; q < 8; ++q) {
+  for (int q = 0; q < kScanSegs; ++q) {
     const int v = seg_sum[q][cl];
     if (q < seg) run += v;
     total += v;
@@ -435,7 +500,7 @@ int run_sort(const DLTensor* idx, char* wsp, const WsLayout& w, int32_t* dst, in
   s.M = M;
   s.use_off = use_off;
   hipLaunchKernelGGL(sort_hist_kernel, dim3(w.nT, (unsigned)G), dim3(kTileTok), (size_t)C * 4, st, s);
-  hipLaunchKernelGGL(sort_scan_tiles_kernel, dim3((C + 31) / 32, (unsigned)G), dim3(256), 0, st, s);
+  hipLaunchKernelGGL(sort_scan_tiles_kernel, dim3((C + 31) / 32, (unsigned)G), dim3(32 * kScanSegs), 0, st, s);
   if (use_off) hipLaunchKernelGGL(sort_scan_clusters_kernel, dim3((unsigned)G), dim3(1024), 0, st, s);
   hipLaunchKernelGGL(sort_scatter_kernel, dim3(w.nT, (unsigned)G), dim3(kTileTok), 0, st, s);
   SQ_HIP(hipGetLastError());
