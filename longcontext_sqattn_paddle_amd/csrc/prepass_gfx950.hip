@@ -73,6 +73,33 @@ __device__ __forceinline__ float qdq(float x, float scale, float qmin, float qma
   return q * scale;
 }
 
+// The same with the division spelled out.  A correctly rounded fp32 division is, on this hardware, a reciprocal
+// estimate refined once, a first quotient and two residual corrections, wrapped in a range pre-scaling and a fix-up
+// of special operands.  A row's elements share the divisor, so the refined reciprocal is formed once per row, and
+// the wrapping is not needed here: the divisor lies in [1e-5 / 127, 65504 / 7] and |x / scale| <= 128, far from the
+// exponent range where intermediates could overflow or lose bits; x = +-0 comes out as +-0.
+struct Divisor {
+  float d, rcp;
+};
+__device__ __forceinline__ Divisor make_divisor(float d) {
+#pragma clang fp contract(off)
+  const float y0 = __builtin_amdgcn_rcpf(d);
+  const float e = __builtin_fmaf(-d, y0, 1.0f);
+  return Divisor{d, __builtin_fmaf(e, y0, y0)};
+}
+__device__ __forceinline__ float divide(float n, const Divisor& s) {
+#pragma clang fp contract(off)
+  const float q0 = n * s.rcp;
+  const float r0 = __builtin_fmaf(-s.d, q0, n);
+  const float q1 = __builtin_fmaf(r0, s.rcp, q0);
+  const float r1 = __builtin_fmaf(-s.d, q1, n);
+  return __builtin_fmaf(r1, s.rcp, q1);
+}
+__device__ __forceinline__ float qdq(float x, const Divisor& s, float qmin, float qmax) {
+  const float q = fminf(fmaxf(round_half_away(divide(x, s)), qmin), qmax);
+  return q * s.d;
+}
+
 // ---- key mean, stage 1: workgroup b sums tokens [b*tok_per_blk, ...) of every (batch, kv head, channel) in fp64.
 // With few columns (Qwen2.5-7B: 4 kv heads x 16 groups of 8 channels = 64) the 256 threads split the tokens of the
 // workgroup between them and combine through LDS in a fixed order.
@@ -90,7 +117,22 @@ __global__ __launch_bounds__(256) void prepass_ksum_kernel(PrepassArgs a) {
     if (live) {
       const int c8 = cg % (kPD / 8), h = (cg / (kPD / 8)) % a.Hkv, b = cg / ((kPD / 8) * a.Hkv);
       const uint16_t* base = (const uint16_t*)a.k.p + b * a.k.sb + h * a.k.sh + 8 * c8;
-      for (int n = n0 + tl; n < n1; n += TL) {
+      // eight rows requested before the first is used: with one row in flight per lane the workgroups of this small
+      // grid keep too few bytes on the wire
+      int n = n0 + tl;
+      for (; n + 7 * TL < n1; n += 8 * TL) {
+        uint4 raw[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) raw[u] = *(const uint4*)(base + (int64_t)(n + u * TL) * a.k.sn);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          float x[8];
+          unpack8<BF16>(raw[u], x);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) s[e] += (double)x[e];
+        }
+      }
+      for (; n < n1; n += TL) {
         float x[8];
         unpack8<BF16>(*(const uint4*)(base + (int64_t)n * a.k.sn), x);
 #pragma unroll
@@ -144,37 +186,56 @@ __global__ __launch_bounds__(256) void prepass_rows_kernel(PrepassArgs a) {
   const int H = CENTRE ? a.Hkv : a.Hq;
   const int64_t rows = (int64_t)a.B * a.N * H;
   const int l16 = threadIdx.x & 15;
-  const int64_t row = (int64_t)blockIdx.x * (blockDim.x / 16) + (threadIdx.x >> 4);
-  if (row >= rows) return;   // whole 16-lane groups leave together; the shuffles below stay inside a group
-  const int h = (int)(row % H);
-  const int64_t n = (row / H) % a.N, b = row / ((int64_t)H * a.N);
-  float x[8];
-  unpack8<BF16>(*(const uint4*)((const uint16_t*)src.p + b * src.sb + n * src.sn + h * src.sh + 8 * l16), x);
-  if constexpr (CENTRE) {
-    float m[8];
-    unpack8<BF16>(*(const uint4*)(a.mean + ((int)b * H + h) * kPD + 8 * l16), m);
+  // two consecutive rows per 16-lane group, both loads issued before any arithmetic
+  constexpr int R = 2;
+  const int64_t row0 = ((int64_t)blockIdx.x * (blockDim.x / 16) + (threadIdx.x >> 4)) * R;
+  if (row0 >= rows) return;   // whole 16-lane groups leave together; the shuffles below stay inside a group
+  uint4 raw[R], mraw[R];
+  int64_t off8[R], off4[R];
+  bool live[R];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) x[e] = ld<BF16>(st<BF16>(x[e] - m[e]));   // the subtraction rounds to the tensor dtype
+  for (int u = 0; u < R; ++u) {
+    const int64_t row = row0 + u;
+    live[u] = row < rows;
+    const int64_t rr = live[u] ? row : row0;
+    const int h = (int)(rr % H);
+    const int64_t n = (rr / H) % a.N, b = rr / ((int64_t)H * a.N);
+    raw[u] = *(const uint4*)((const uint16_t*)src.p + b * src.sb + n * src.sn + h * src.sh + 8 * l16);
+    if constexpr (CENTRE) mraw[u] = *(const uint4*)(a.mean + ((int)b * H + h) * kPD + 8 * l16);
+    off8[u] = b * d8.sb + n * d8.sn + h * d8.sh + 8 * l16;
+    off4[u] = a.want4 ? b * d4.sb + n * d4.sn + h * d4.sh + 8 * l16 : 0;
   }
-  float amax = 0.f;
 #pragma unroll
-  for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf(x[e]));
+  for (int u = 0; u < R; ++u) {
+    float x[8];
+    unpack8<BF16>(raw[u], x);
+    if constexpr (CENTRE) {
+      float m[8];
+      unpack8<BF16>(mraw[u], m);
 #pragma unroll
-  for (int sh = 1; sh < 16; sh <<= 1) amax = fmaxf(amax, __shfl_xor(amax, sh));
-  amax = fmaxf(amax, 1e-5f);
-  {
-    const float scale = amax / 127.f;
-    float y[8];
+      for (int e = 0; e < 8; ++e) x[e] = ld<BF16>(st<BF16>(x[e] - m[e]));   // the subtraction rounds to the tensor dtype
+    }
+    float amax = 0.f;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) y[e] = qdq(x[e], scale, -128.f, 127.f);
-    *(uint4*)((uint16_t*)d8.p + b * d8.sb + n * d8.sn + h * d8.sh + 8 * l16) = pack8<BF16>(y);
-  }
-  if (a.want4) {
-    const float scale = amax / 7.f;
-    float y[8];
+    for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf(x[e]));
 #pragma unroll
-    for (int e = 0; e < 8; ++e) y[e] = qdq(x[e], scale, -8.f, 7.f);
-    *(uint4*)((uint16_t*)d4.p + b * d4.sb + n * d4.sn + h * d4.sh + 8 * l16) = pack8<BF16>(y);
+    for (int sh = 1; sh < 16; sh <<= 1) amax = fmaxf(amax, __shfl_xor(amax, sh));
+    amax = fmaxf(amax, 1e-5f);
+    if (!live[u]) continue;
+    {
+      const Divisor scale = make_divisor(amax / 127.f);
+      float y[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) y[e] = qdq(x[e], scale, -128.f, 127.f);
+      *(uint4*)((uint16_t*)d8.p + off8[u]) = pack8<BF16>(y);
+    }
+    if (a.want4) {
+      const Divisor scale = make_divisor(amax / 7.f);
+      float y[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) y[e] = qdq(x[e], scale, -8.f, 7.f);
+      *(uint4*)((uint16_t*)d4.p + off4[u]) = pack8<BF16>(y);
+    }
   }
 }
 
@@ -194,9 +255,9 @@ __global__ __launch_bounds__(256) void prepass_v_kernel(PrepassArgs a) {
 #pragma unroll
       for (int e = 0; e < 8; ++e) amax[e] = fmaxf(amax[e], fabsf(x[e]));
     }
-  float scale[8];
+  Divisor scale[8];
 #pragma unroll
-  for (int e = 0; e < 8; ++e) scale[e] = fmaxf(amax[e], 1e-5f) / 127.f;
+  for (int e = 0; e < 8; ++e) scale[e] = make_divisor(fmaxf(amax[e], 1e-5f) / 127.f);
   uint16_t* obase = (uint16_t*)a.v8.p + n * a.v8.sn + 8 * c8;
   for (int b = 0; b < a.B; ++b)
     for (int h = 0; h < a.Hkv; ++h) {
@@ -291,8 +352,8 @@ extern "C" int sq_fake_quant_prepass(const DLTensor* query, const DLTensor* key,
   do {                                                                                                         \
     hipLaunchKernelGGL(prepass_ksum_kernel<BF>, dim3(a.nblk), dim3(256), 0, s, a);                             \
     hipLaunchKernelGGL(prepass_kmean_kernel<BF>, dim3((unsigned)((cols * 16 + 255) / 256)), dim3(256), 0, s, a);    \
-    hipLaunchKernelGGL((prepass_rows_kernel<BF, false>), dim3((unsigned)((qrows + 15) / 16)), dim3(256), 0, s, a); \
-    hipLaunchKernelGGL((prepass_rows_kernel<BF, true>), dim3((unsigned)((krows + 15) / 16)), dim3(256), 0, s, a);  \
+    hipLaunchKernelGGL((prepass_rows_kernel<BF, false>), dim3((unsigned)((qrows + 31) / 32)), dim3(256), 0, s, a); \
+    hipLaunchKernelGGL((prepass_rows_kernel<BF, true>), dim3((unsigned)((krows + 31) / 32)), dim3(256), 0, s, a);  \
     hipLaunchKernelGGL(prepass_v_kernel<BF>, dim3((unsigned)((vthreads + 255) / 256)), dim3(256), 0, s, a);    \
   } while (0)
   if (a.is_bf16) SQ_PREPASS_LAUNCH(true);
