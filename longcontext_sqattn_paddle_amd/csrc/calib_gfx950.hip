@@ -129,7 +129,8 @@ __global__ __launch_bounds__(256) void attn_histogram_kernel(HistArgs a) {
 
   // ---- pass 2: probabilities into the LDS histogram
   const float nbf = (float)a.bins;
-  const float den = (KIND == 1) ? (float)(row > 1 ? row : 1) : fmaxf((float)row - (float)a.sink, 1.0f);
+  // one divisor per row: integers in [1, 2^24], quotients in [0, 2^24], so the shared-divisor division is exact IEEE
+  const Divisor den = make_divisor((KIND == 1) ? (float)(row > 1 ? row : 1) : fmaxf((float)row - (float)a.sink, 1.0f));
   __syncthreads();
   for (int t = tid; t < (KIND == 0 ? 256 : a.bins); t += 256) hl[t] = 0.f;
   double* hist = a.hist + ((int64_t)b * a.Hq + h) * a.bins;
@@ -194,12 +195,12 @@ __global__ __launch_bounds__(256) void attn_histogram_kernel(HistArgs a) {
           const float p = __builtin_amdgcn_exp2f(S[bn][e] * a.scale2 - mt) * inv_l;
           const int dist = row - key;
           if constexpr (KIND == 1) {
-            const float sc = ((float)dist / den) * nbf;
+            const float sc = divide((float)dist, den) * nbf;
             int bi = (int)__builtin_floorf(sc);
             bi = bi < a.bins - 1 ? bi : a.bins - 1;
             add_relative(bi, p * (float)dist);
           } else {
-            float sc = ((float)dist / den) * nbf;
+            float sc = divide((float)dist, den) * nbf;
             if (row <= a.sink) sc = 0.f;
             int bi = (int)__builtin_floorf(sc);
             bi = bi < a.bins - 1 ? bi : a.bins - 1;

@@ -105,6 +105,30 @@ __device__ __forceinline__ float e4m3_roundtrip(float x) {
 
 __device__ __forceinline__ float wave_xor_max(float v, int mask) { return fmaxf(v, __shfl_xor(v, mask)); }
 
+// ---- division by a divisor that many dividends share.  A correctly rounded fp32 division is, on this hardware, a
+// reciprocal estimate refined once, a first quotient and two residual corrections, wrapped in a range pre-scaling and
+// a fix-up of special operands (zero, infinite, denormal divisors; quotients near the ends of the exponent range).
+// Here the refined reciprocal is formed once per divisor and the wrapping is left out: the result equals n / d bit
+// for bit as long as d is a normal number well inside the exponent range, and so are the quotients (callers state
+// their ranges); n = +-0 gives +-0.
+struct Divisor {
+  float d, rcp;
+};
+__device__ __forceinline__ Divisor make_divisor(float d) {
+#pragma clang fp contract(off)
+  const float y0 = __builtin_amdgcn_rcpf(d);
+  const float e = __builtin_fmaf(-d, y0, 1.0f);
+  return Divisor{d, __builtin_fmaf(e, y0, y0)};
+}
+__device__ __forceinline__ float divide(float n, const Divisor& s) {
+#pragma clang fp contract(off)
+  const float q0 = n * s.rcp;
+  const float r0 = __builtin_fmaf(-s.d, q0, n);
+  const float q1 = __builtin_fmaf(r0, s.rcp, q0);
+  const float r1 = __builtin_fmaf(-s.d, q1, n);
+  return __builtin_fmaf(r1, s.rcp, q1);
+}
+
 // ---- hand-scheduled LDS reads.  The compiler cannot tell that a ds_read never touches the buffers that
 // global_load_lds copies are still filling, so it would stall every tile on vmcnt(0); reads issued through
 // these helpers are invisible to that logic, and the data dependence is carried by lds_wait instead.

@@ -73,28 +73,8 @@ __device__ __forceinline__ float qdq(float x, float scale, float qmin, float qma
   return q * scale;
 }
 
-// The same with the division spelled out.  A correctly rounded fp32 division is, on this hardware, a reciprocal
-// estimate refined once, a first quotient and two residual corrections, wrapped in a range pre-scaling and a fix-up
-// of special operands.  A row's elements share the divisor, so the refined reciprocal is formed once per row, and
-// the wrapping is not needed here: the divisor lies in [1e-5 / 127, 65504 / 7] and |x / scale| <= 128, far from the
-// exponent range where intermediates could overflow or lose bits; x = +-0 comes out as +-0.
-struct Divisor {
-  float d, rcp;
-};
-__device__ __forceinline__ Divisor make_divisor(float d) {
-#pragma clang fp contract(off)
-  const float y0 = __builtin_amdgcn_rcpf(d);
-  const float e = __builtin_fmaf(-d, y0, 1.0f);
-  return Divisor{d, __builtin_fmaf(e, y0, y0)};
-}
-__device__ __forceinline__ float divide(float n, const Divisor& s) {
-#pragma clang fp contract(off)
-  const float q0 = n * s.rcp;
-  const float r0 = __builtin_fmaf(-s.d, q0, n);
-  const float q1 = __builtin_fmaf(r0, s.rcp, q0);
-  const float r1 = __builtin_fmaf(-s.d, q1, n);
-  return __builtin_fmaf(r1, s.rcp, q1);
-}
+// The same with the shared-divisor division of common.hpp (bit-identical to x / scale for these operand ranges: the
+// divisor lies in [1e-5 / 127, 65504 / 7] and |x / scale| <= 128).
 __device__ __forceinline__ float qdq(float x, const Divisor& s, float qmin, float qmax) {
   const float q = fminf(fmaxf(round_half_away(divide(x, s)), qmin), qmax);
   return q * s.d;

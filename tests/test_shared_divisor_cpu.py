@@ -1,0 +1,84 @@
+"""The kernels divide many dividends by one divisor with a reciprocal that is refined once per divisor and two residual
+corrections per quotient (csrc/common.hpp: make_divisor / divide) and claim the result equals the correctly rounded
+fp32 quotient for their operand ranges.  Checked here in exact rational arithmetic, with the hardware's reciprocal
+estimate modelled as the correctly rounded reciprocal moved by -1, 0 or +1 units in the last place (v_rcp_f32 is
+specified to 1 ulp)."""
+from fractions import Fraction
+
+import numpy as np
+
+
+def _round_f32(x: Fraction) -> np.float32:
+    """round-to-nearest-even of an exact rational to fp32 (normal range)"""
+    if x == 0:
+        return np.float32(0.0)
+    sign = -1 if x < 0 else 1
+    x = abs(x)
+    e = x.numerator.bit_length() - x.denominator.bit_length()
+    if Fraction(2) ** e > x:
+        e -= 1
+    assert Fraction(2) ** e <= x < Fraction(2) ** (e + 1) and -126 <= e <= 127
+    scaled = x / Fraction(2) ** (e - 23)            # in [2^23, 2^24)
+    m, rem = divmod(scaled.numerator, scaled.denominator)
+    twice = 2 * rem
+    if twice > scaled.denominator or (twice == scaled.denominator and (m & 1)):
+        m += 1
+    return np.float32(sign * float(m) * 2.0 ** (e - 23))
+
+
+def _fma(a, b, c):
+    return _round_f32(Fraction(float(a)) * Fraction(float(b)) + Fraction(float(c)))
+
+
+def _divide(n, d, ulp_shift):
+    y0 = _round_f32(1 / Fraction(float(d)))
+    if ulp_shift:
+        y0 = np.nextafter(y0, np.float32(np.inf if ulp_shift > 0 else 0), dtype=np.float32)
+    e = _fma(-d, y0, np.float32(1))
+    y = _fma(e, y0, y0)
+    q0 = _round_f32(Fraction(float(n)) * Fraction(float(y)))
+    r0 = _fma(-d, q0, n)
+    q1 = _fma(r0, y, q0)
+    r1 = _fma(-d, q1, n)
+    return _fma(r1, y, q1)
+
+
+def _check(pairs):
+    for n, d in pairs:
+        want = _round_f32(Fraction(float(n)) / Fraction(float(d)))
+        for shift in (-1, 0, 1):
+            got = _divide(np.float32(n), np.float32(d), shift)
+            assert got == want and np.signbit(got) == np.signbit(want), (float(n), float(d), shift, float(got), float(want))
+
+
+def test_quantiser_ranges():
+    """pre-pass: x a bf16/fp16 value of a row, d = max(absmax, 1e-5) / 127 or / 7, |x / d| <= 127 (or 7)"""
+    rng = np.random.default_rng(1)
+    pairs = []
+    for _ in range(400):
+        amax = np.float32(10.0 ** rng.uniform(-5, 4.8))
+        for levels in (127.0, 7.0):
+            d = np.float32(amax / np.float32(levels))
+            xs = (rng.uniform(-1, 1, 3) * amax).astype(np.float32)
+            xs = (xs.view(np.uint32) & 0xFFFF0000).view(np.float32)        # bf16-representable
+            pairs += [(x, d) for x in xs]
+            # dividends next to the rounding boundaries k + 1/2 of the quantiser
+            k = rng.integers(0, int(levels))
+            pairs.append((np.float32((k + 0.5) * float(d)), d))
+    _check(pairs)
+
+
+def test_index_ranges():
+    """calibration: n = i - j and d = a row index, both integers in [0, 2^24] / [1, 2^24]"""
+    rng = np.random.default_rng(2)
+    pairs = [(np.float32(0), np.float32(1)), (np.float32(2 ** 24), np.float32(2 ** 24)), (np.float32(1), np.float32(2 ** 24))]
+    for _ in range(500):
+        d = int(rng.integers(1, 2 ** int(rng.integers(1, 25))))
+        n = int(rng.integers(0, d + 1))
+        pairs.append((np.float32(n), np.float32(d)))
+    # bins are floor(num_bins * n / d): quotients just around k / num_bins
+    for d in (199, 200, 3001, 65537, 131071):
+        for k in (1, 7, 99, 150):
+            n = (k * d) // 200
+            pairs += [(np.float32(n), np.float32(d)), (np.float32(n + 1), np.float32(d))]
+    _check(pairs)
