@@ -1,0 +1,112 @@
+"""The HIP kernels against the committed fixtures of tests/golden (inputs and oracle outputs frozen on disk), through
+the same entry points and with the same tolerances as the seeded parity tests."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def _load(name):
+    with np.load(os.path.join(GOLDEN, name), allow_pickle=False) as z:
+        return {k: z[k] for k in z.files}
+
+
+def _bf16(bits):
+    return torch.from_numpy(bits.view(np.int16).copy()).view(torch.bfloat16)
+
+
+def test_prefill_fixture():
+    from longcontext_sqattn_paddle_amd.sqattn.attn_triton import attn_causal
+
+    z = _load("prefill_small.npz")
+    q, k, v = (_bf16(z[n]).to(DEV) for n in ("q", "k", "v"))
+    for name, mode, quantised in (("none", 0, False), ("e4m3_static", 1, True)):
+        out, lse = attn_causal(q, k, v, "HND", torch.float32, return_lse=True, p_quant=mode)
+        torch.cuda.synchronize()
+        ref = torch.from_numpy(z[f"out_{name}"]).double()
+        d = (out.double().cpu() - ref).abs()
+        rms = float(ref.pow(2).mean().sqrt())
+        if not quantised:
+            assert float(d.max()) <= 2e-3 * rms
+        else:   # a probability within an ulp of an e4m3 boundary may land on the neighbouring grid value
+            assert float(d.flatten().kthvalue(int(0.999 * d.numel())).values) <= 2e-3 * rms and float(d.max()) <= 0.25 * rms
+        assert np.allclose(lse.cpu().numpy(), z[f"lse_{name}"], atol=2e-4)
+    # the fixture's windows were evaluated per 64-row query block (the relative entry point's block size); go through the
+    # kernel-level wrapper, which takes window sizes in tokens directly
+    from longcontext_sqattn_paddle_amd.sqattn._prefill import run_prefill
+
+    window = {"block_m": 64, "sink": 64, "w8": [64, 128, 64, 128], "w4": [128, 128, 192, 192]}
+    out, lse = run_prefill(q, k, v, tensor_layout="HND", output_dtype=torch.float32, return_lse=True, p_quant=0, window=window)
+    torch.cuda.synchronize()
+    ref = torch.from_numpy(z["out_window"]).double()
+    assert float((out.double().cpu() - ref).abs().max()) <= 2e-3 * float(ref.pow(2).mean().sqrt())
+    assert np.allclose(lse.cpu().numpy(), z["lse_window"], atol=2e-4)
+
+
+def test_decode_fixture():
+    from longcontext_sqattn_paddle_amd.sqattn.attn_triton_decode import attn_decode
+
+    z = _load("decode_small.npz")
+    q, k, v = (_bf16(z[n]).to(DEV) for n in ("q", "k", "v"))
+    lens = torch.from_numpy(z["lens"]).to(DEV)
+    out, lse = attn_decode(q, k, v, "HND", torch.float32, return_lse=True, seqlens=lens)
+    torch.cuda.synchronize()
+    ref = torch.from_numpy(z["out"]).double()
+    assert float((out.double().cpu().reshape(ref.shape) - ref).abs().max()) <= 2e-4 * float(ref.pow(2).mean().sqrt())
+    assert np.allclose(lse.cpu().numpy().reshape(z["lse"].shape), z["lse"], atol=2e-4)
+
+
+def test_prepass_fixture_bit_for_bit():
+    from longcontext_sqattn_paddle_amd.sqattn.fake_quant import fused_int_prepass
+
+    z = _load("prepass_small.npz")
+    q, k, v = (_bf16(z[n]).to(DEV) for n in ("q", "k", "v"))
+    outs = fused_int_prepass(q, k, v, want_4bit=True)
+    torch.cuda.synchronize()
+    for name, t in zip(("q8", "q4", "k8", "k4", "v8"), outs):
+        got = t.cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+        assert np.array_equal(got, z[name]), name
+
+
+def test_kmeans_fixture():
+    from longcontext_sqattn_paddle_amd.cache_hub.kmeans import segment_k_means
+
+    z = _load("kmeans_small.npz")
+    key, value = _bf16(z["key"]).to(DEV), _bf16(z["value"]).to(DEV)
+    cent, vsum, clusters, size = segment_k_means(key, value, 32, num_iters=4, num_segments=1)
+    torch.cuda.synchronize()
+    assert np.array_equal(size.cpu().numpy().astype(np.int32), z["cluster_size"])
+    m = z["clusters"].shape[2]
+    got = clusters.cpu().numpy().astype(np.int32)
+    assert got.shape[2] >= m or got.shape[2] == m
+    # same members per cluster (the kernel stores them in ascending token order, the oracle too)
+    for g in range(2):
+        for c in range(32):
+            n = int(z["cluster_size"][g, c])
+            assert np.array_equal(np.sort(got[g, c, :n]), np.sort(z["clusters"][g, c, :n])), (g, c)
+    cb = cent.cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+    assert np.mean(cb != z["centroids"]) <= 1e-3          # at most a unit in the last place on a few components
+    assert np.allclose(_bf16(cb).float().numpy(), _bf16(z["centroids"]).float().numpy(), rtol=2 ** -7, atol=1e-6)
+    vb = vsum.cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+    assert np.allclose(_bf16(vb).float().numpy(), _bf16(z["value_sum"]).float().numpy(), rtol=2 ** -7, atol=1e-3)
+
+
+def test_window_search_fixture():
+    from longcontext_sqattn_paddle_amd.sqattn import window_search as H
+
+    z = _load("window_search_small.npz")
+    q, k = _bf16(z["q"]).to(DEV), _bf16(z["k"]).to(DEV)
+    for name, kind, bins, sink in (("absolute", 0, 200, 0), ("absolute_sink", 0, 128, 32), ("relative", 1, 50, 0), ("relative_sink", 2, 40, 32)):
+        got = H.attention_histograms(q, k, kind, bins, sink)[0].cpu().numpy()
+        want = z[name]
+        tol = 1e-4 * np.abs(want) + 1e-6 * np.abs(want).sum(axis=-1, keepdims=True) + 1e-12
+        assert (np.abs(got - want) <= tol).all(), name
+        if name == "absolute":
+            assert [H.find_optimal_window(h, 0.9) for h in got] == list(z["window_absolute_0p9"])
+        if name == "relative_sink":
+            assert [H.find_optimal_relative_window(h, 0.9, 40) for h in got] == list(z["window_relative_0p9"])

@@ -38,6 +38,8 @@ def test_prepass_is_bit_exact(B, N, Hq, Hkv, dtype, want4):
             continue
         assert a.dtype == dtype and a.shape == b.shape
         assert torch.equal(a.cpu(), b), (name, float((a.cpu().float() - b.float()).abs().max()))
+        # ... and to the bit, which torch.equal does not see for the sign of zero
+        assert torch.equal(a.cpu().contiguous().view(torch.int16), b.contiguous().view(torch.int16)), name
 
 
 def test_prepass_hnd_views_and_strides():
