@@ -87,6 +87,9 @@ def test_rope_is_bit_exact(dtype, B, S, Hq, Hkv, D, maxpos):
     torch.cuda.synchronize()
     assert oq.shape == (B, S, Hq, D) and ok.shape == (B, S, Hkv, D)
     assert torch.equal(oq.cpu().view(B * S, -1), rq) and torch.equal(ok.cpu().view(B * S, -1), rk)
+    # to the bit (torch.equal takes -0.0 for +0.0)
+    assert torch.equal(oq.cpu().view(B * S, -1).contiguous().view(torch.int16), rq.contiguous().view(torch.int16))
+    assert torch.equal(ok.cpu().view(B * S, -1).contiguous().view(torch.int16), rk.contiguous().view(torch.int16))
     assert torch.equal(qd.cpu(), q) and torch.equal(kd.cpu(), k)              # inputs untouched
     oq32, _ = apply_rope_with_cos_sin_cache_inplace(pos.to(DEV).to(torch.int32), qd, kd, D, table.to(DEV))
     assert torch.equal(oq32, oq)
