@@ -38,8 +38,8 @@ constexpr int kAssignWaves = 4;   // x 64 tokens; two workgroups per CU put two 
 // read from LDS feeds two MFMAs, which halves the LDS traffic per MFMA -- with 32 tokens per wave the fragment reads
 // of the four SIMDs add up to the LDS's whole 128 bytes per cycle.  Centroids stream through LDS in blocks of 64
 // (global_load_lds, unpadded rows, 16-byte chunks XOR-swizzled by row so that the MFMA operand reads are conflict
-// free); the scores of block k+1 are issued on the matrix pipe before the arg-max epilogue of block k runs on the
-// vector ALU.
+// free), double buffered with one barrier per block; the arg-max over one half block's scores runs underneath the
+// MFMAs of the next half block (see `phase` below).
 __global__ __launch_bounds__(kAssignWaves * 64, 1) void kmeans_assign_kernel(AssignArgs a) {
   __shared__ __attribute__((aligned(16))) char smem[2 * kCB * 256];
   typedef __attribute__((address_space(3))) void* lds_ptr_t;

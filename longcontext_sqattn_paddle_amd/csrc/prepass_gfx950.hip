@@ -67,13 +67,8 @@ __device__ __forceinline__ uint4 pack8(const float (&x)[8]) {
 // sign(x) * floor(abs(x) + 0.5)
 __device__ __forceinline__ float round_half_away(float t) { return copysignf(floorf(fabsf(t) + 0.5f), t); }
 
-// quant-dequant of one value: clamp(round(x / scale), qmin, qmax) * scale   (fake_quant.py:114-125, zero point 0)
-__device__ __forceinline__ float qdq(float x, float scale, float qmin, float qmax) {
-  const float q = fminf(fmaxf(round_half_away(x / scale) + 0.0f, qmin), qmax);   // + zero point: -0.0 becomes +0.0
-  return q * scale;
-}
-
-// The same with the shared-divisor division of common.hpp (bit-identical to x / scale for these operand ranges: the
+// quant-dequant of one value: clamp(round(x / scale) + zero, qmin, qmax) * scale   (fake_quant.py:114-125, zero point 0),
+// with the shared-divisor division of common.hpp (bit-identical to x / scale for these operand ranges: the
 // divisor lies in [1e-5 / 127, 65504 / 7] and |x / scale| <= 128).
 // `round(x / scale) + zero` with the symmetric quantiser's zero point 0.0 (fake_quant.py:114-116): the addition is
 // kept because it turns a rounded -0.0 into +0.0, so a small negative x comes out as +0.0 like in the reference
