@@ -108,9 +108,11 @@ def time_decode(torch, B, L, iters=10, warmup=5, rounds=7):
     return us, nbytes
 
 
-def time_decode_selected(torch, B, L, k, iters=20, rounds=5):
+def time_decode_selected(torch, B, L, k, iters=20, rounds=5, run=1):
     """Decode attention over k selected tokens per (sequence, kv head) of an L-token cache: the consumer of the
-    k-means top-k selection.  Ids are random and distinct per head, so every row is a separate 256-byte read."""
+    k-means top-k selection.  With run == 1 the ids are random and distinct per head, so every row is a separate
+    256-byte read; with run > 1 they are runs of `run` neighbouring rows at random places, which is what a selection
+    of whole clusters reads from a cache kept in cluster order (sq_kv_cache_reorder)."""
     from longcontext_sqattn_paddle_amd import _native as Nn
 
     dev = torch.device("cuda:0")
@@ -119,7 +121,11 @@ def time_decode_selected(torch, B, L, k, iters=20, rounds=5):
     q = torch.randn(B, 1, Hq, D, device=dev, generator=g).bfloat16()
     kc = torch.randn(B, L, Hkv, D, device=dev, generator=g, dtype=torch.bfloat16)
     vc = torch.randn(B, L, Hkv, D, device=dev, generator=g, dtype=torch.bfloat16)
-    ids = torch.stack([torch.randperm(L, device=dev, generator=g)[:k] for _ in range(B * Hkv)]).to(torch.int32)
+    if run == 1:
+        ids = torch.stack([torch.randperm(L, device=dev, generator=g)[:k] for _ in range(B * Hkv)]).to(torch.int32)
+    else:
+        starts = torch.stack([torch.randperm(L // run, device=dev, generator=g)[:k // run] for _ in range(B * Hkv)]) * run
+        ids = (starts[:, :, None] + torch.arange(run, device=dev)).reshape(B * Hkv, k).to(torch.int32)
     lib = Nn.lib()
     S = lib.sq_decode_num_splits(B, Hkv, k)
     ws = torch.empty(lib.sq_decode_workspace_bytes(B, Hq, 128, S) // 4, dtype=torch.float32, device=dev)
@@ -506,8 +512,10 @@ def main():
             torch.cuda.empty_cache()
         result["decode"] = dec
         sel = {}
-        for name, B, L, k in (("4096_of_128K_b1", 1, 131072, 4096), ("4096_of_128K_b8", 8, 131072, 4096), ("65536_of_1M_b1", 1, 1048576, 65536)):
-            us, nbytes = time_decode_selected(torch, B, L, k)
+        for name, B, L, k, run in (("4096_of_128K_b1", 1, 131072, 4096, 1), ("4096_of_128K_b8", 8, 131072, 4096, 1),
+                                   ("65536_of_1M_b1", 1, 1048576, 65536, 1), ("65536_of_1M_b1_runs_of_64", 1, 1048576, 65536, 64),
+                                   ("4096_of_128K_b8_runs_of_64", 8, 131072, 4096, 64)):
+            us, nbytes = time_decode_selected(torch, B, L, k, run=run)
             sel[name] = {"us_per_call": round(us, 2), "GB_per_s": round(nbytes / us / 1e3, 1), "bytes": nbytes}
             log(f"[bench] decode over selected tokens {name}: {us:.1f} us, {nbytes / us / 1e3:.0f} GB/s")
             torch.cuda.empty_cache()

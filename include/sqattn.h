@@ -206,6 +206,18 @@ int sq_kv_cache_append(const DLTensor* key_states, const DLTensor* value_states,
                        void* stream);
 
 /*
+ * A copy of a layer's KV cache with each kv head's rows permuted (no counterpart in the reference, whose k-means code
+ * in cache_hub/kmeans.py has no consumer): key_out[b, p, h] = key_cache[b, order[b * Hkv + h][p], h], the same for
+ * value.  With `order` = the tokens of every head listed cluster by cluster (the order triton_reverse_index stores
+ * them in, cache_hub/kmeans.py:199-262), a selection of whole clusters becomes runs of neighbouring rows of the copy,
+ * and sq_decode_selected_fwd on the copy, with positions in place of token ids, reads them as such.
+ * key_cache / value_cache [B, L, Hkv, D], key_out / value_out [B, n, Hkv, D], all contiguous, one 16-bit dtype;
+ * order int32 [B * Hkv, n]; entries outside [0, L) give zero rows.
+ */
+int sq_kv_cache_reorder(const DLTensor* key_cache, const DLTensor* value_cache, const DLTensor* order, DLTensor* key_out,
+                        DLTensor* value_out, void* stream);
+
+/*
  * RMS normalisation of the rows of x [R, dim] (model_hub/utils.py:15-19): out = (x * rsqrt(mean(x^2) + epsilon))
  * * weight, with the reference's operator sequence on 16-bit tensors -- square, mean (fp32 accumulation), + epsilon,
  * rsqrt, x * r, * weight, each result rounded to the tensor dtype.  x, out [R, dim] (row strides free, 16-byte

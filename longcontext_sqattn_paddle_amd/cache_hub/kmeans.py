@@ -107,3 +107,37 @@ def topk_select(query, centroids, clusters, cluster_size, k: int, num_kv_groups:
     b = [N.dl(t) for t in (query, centroids, clusters, cluster_size, out, ws)]
     N.check(N.lib().sq_topk_select(*[N.ptr(x) for x in b], num_kv_groups, N.current_stream(query.device)))
     return out
+
+
+def cluster_order(clusters: torch.Tensor, cluster_size: torch.Tensor):
+    """From the reverse index (`clusters` int32 [G,C,M], `cluster_size` int32 [G,C]) the two tables of a cache kept in
+    cluster order (no reference counterpart): `order` int32 [G,n] lists every group's tokens cluster by cluster (n = the
+    largest group total; shorter groups are padded with -1), and `positions` int32 [G,C,M] holds, in the layout of
+    `clusters`, where each of those tokens sits in that list.  `topk_select(query, centroids, positions, cluster_size,
+    ...)` then yields rows of the reordered cache instead of token ids."""
+    G, C, M = clusters.shape
+    size = cluster_size.to(torch.int64)
+    offset = torch.cumsum(size, dim=1) - size                                   # [G,C] exclusive prefix
+    slot = torch.arange(M, device=clusters.device).view(1, 1, M)
+    used = slot < size.unsqueeze(-1)                                            # [G,C,M]
+    positions = torch.where(used, offset.unsqueeze(-1) + slot, torch.zeros_like(slot)).to(torch.int32)
+    n = int(size.sum(dim=1).max().item())
+    order = torch.full((G, n), -1, dtype=torch.int32, device=clusters.device)
+    rows = torch.arange(G, device=clusters.device).view(G, 1, 1).expand(G, C, M)
+    order[rows[used], positions[used].long()] = clusters[used]
+    return order, positions
+
+
+def reorder_cache(key_cache: torch.Tensor, value_cache: torch.Tensor, order: torch.Tensor):
+    """Copies of a layer's cache [B,L,Hkv,D] with each kv head's rows in the order `order` int32 [B*Hkv,n] gives
+    (`sq_kv_cache_reorder`): out[b, p, h] = cache[b, order[b*Hkv + h, p], h]; rows for -1 are zero."""
+    _require(key_cache, "key_cache")
+    _require(value_cache, "value_cache")
+    B, _, H, D = key_cache.shape
+    n = order.shape[1]
+    key_out = torch.empty((B, n, H, D), dtype=key_cache.dtype, device=key_cache.device)
+    value_out = torch.empty_like(key_out)
+    b = [N.dl(t) for t in (key_cache, value_cache, order, key_out, value_out)]
+    N.check(N.lib().sq_kv_cache_reorder(*[N.ptr(x) for x in b], N.current_stream(key_cache.device)))
+    return key_out, value_out
+

@@ -13,6 +13,9 @@
 //   * append: one workgroup per sequence copies the K row and the V row to position valid_length[b], then
 //     publishes attend_length[b] = position + 1 (what the attention of this step covers) and, when `advance` is
 //     set, valid_length[b] = position + 1.  No host synchronisation: the lengths never leave the device.
+//   * reorder (no reference counterpart): a copy of a layer's cache with every kv head's rows permuted, e.g. into the
+//     order of its k-means clusters, so that a selection of whole clusters reads runs of neighbouring rows instead
+//     of scattered ones.
 #include "common.hpp"
 
 namespace sq {
@@ -76,6 +79,35 @@ __global__ __launch_bounds__(128) void kv_append_kernel(AppendArgs a) {
     const int next = pos < a.max_length ? pos + 1 : pos;
     if (a.attend_length) a.attend_length[b] = next;
     if (a.advance) a.valid_length[b] = next;
+  }
+}
+
+struct ReorderArgs {
+  const char* k_src;
+  const char* v_src;
+  char* k_dst;
+  char* v_dst;
+  const int32_t* order;             // [B * heads, n]
+  int64_t n, src_len;               // rows per head in the copy, rows per sequence in the source
+  int32_t batch, heads, head_chunks;
+};
+
+// One 16-byte chunk per thread: chunk (b, p, h, cc) of the copy comes from row order[b * heads + h][p] of head h.
+// Writes are contiguous; reads are one 256-byte head row per 16 lanes.  Ids outside [0, src_len) give zero rows.
+__global__ __launch_bounds__(256) void kv_reorder_kernel(ReorderArgs a) {
+  const int64_t row_chunks = (int64_t)a.heads * a.head_chunks;
+  const int64_t per_tensor = (int64_t)a.batch * a.n * row_chunks;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < 2 * per_tensor; i += (int64_t)gridDim.x * blockDim.x) {
+    const bool is_v = i >= per_tensor;
+    const int64_t j = is_v ? i - per_tensor : i;
+    const int64_t row = j / row_chunks;                 // b * n + p
+    const int c = (int)(j - row * row_chunks);
+    const int h = c / a.head_chunks;
+    const int64_t b = row / a.n, p = row - b * a.n;
+    const int32_t id = a.order[(b * a.heads + h) * a.n + p];
+    u32x4_t w = {0u, 0u, 0u, 0u};
+    if (id >= 0 && id < a.src_len) w = __builtin_nontemporal_load((const u32x4_t*)((is_v ? a.v_src : a.k_src) + ((b * a.src_len + id) * row_chunks + c) * 16));
+    __builtin_nontemporal_store(w, (u32x4_t*)((is_v ? a.v_dst : a.k_dst) + j * 16));
   }
 }
 
@@ -194,6 +226,54 @@ extern "C" int sq_kv_cache_append(const DLTensor* key_states, const DLTensor* va
   a.head_chunks = (int)(D / 8);
   a.advance = advance;
   hipLaunchKernelGGL(kv_append_kernel, dim3((unsigned)B), dim3(128), 0, (hipStream_t)stream, a);
+  SQ_HIP(hipGetLastError());
+  return SQ_OK;
+}
+
+extern "C" int sq_kv_cache_reorder(const DLTensor* key_cache, const DLTensor* value_cache, const DLTensor* order, DLTensor* key_out,
+                                   DLTensor* value_out, void* stream) {
+  const char* fn = "sq_kv_cache_reorder";
+  SQ_REQUIRE(key_cache && value_cache && order && key_out && value_out, SQ_EINVAL, "%s: null tensor argument", fn);
+  int rc;
+  if ((rc = check_tensor(key_cache, "key_cache", 4, key_cache->device.device_id))) return rc;
+  const int dev = key_cache->device.device_id;
+  const DType dt = dtype_of(key_cache);
+  SQ_REQUIRE(dt == DType::BF16 || dt == DType::F16, SQ_EDTYPE, "%s: key_cache must be bf16 or fp16", fn);
+  const DLTensor* all[4] = {key_cache, value_cache, key_out, value_out};
+  const char* names[4] = {"key_cache", "value_cache", "key_out", "value_out"};
+  for (int i = 0; i < 4; ++i) {
+    if ((rc = check_tensor(all[i], names[i], 4, dev))) return rc;
+    SQ_REQUIRE(dtype_of(all[i]) == dt, SQ_EDTYPE, "%s: %s must have key_cache's dtype", fn, names[i]);
+    SQ_REQUIRE(is_compact(all[i]), SQ_ESHAPE, "%s: %s must be contiguous [B, rows, Hkv, D]", fn, names[i]);
+    SQ_REQUIRE(all[i]->shape[0] == key_cache->shape[0] && all[i]->shape[2] == key_cache->shape[2] && all[i]->shape[3] == key_cache->shape[3],
+               SQ_ESHAPE, "%s: %s differs from key_cache in batch, heads or head_dim", fn, names[i]);
+  }
+  const int64_t B = key_cache->shape[0], L = key_cache->shape[1], H = key_cache->shape[2], D = key_cache->shape[3], n = key_out->shape[1];
+  SQ_REQUIRE(value_cache->shape[1] == L && value_out->shape[1] == n, SQ_ESHAPE, "%s: key and value tensors differ in rows", fn);
+  SQ_REQUIRE(D % 8 == 0, SQ_EUNSUPPORTED, "%s: head_dim must be a multiple of 8", fn);
+  SQ_REQUIRE(on_gpu(order) && order->device.device_id == dev, SQ_EDEVICE, "%s: order must live on the cache's device", fn);
+  SQ_REQUIRE(dtype_of(order) == DType::I32 && order->ndim == 2 && order->shape[0] == B * H && order->shape[1] == n && is_compact(order), SQ_ESHAPE,
+             "%s: order must be contiguous int32 [%lld, %lld]", fn, (long long)(B * H), (long long)n);
+  SQ_REQUIRE(L < ((int64_t)1 << 31) && n < ((int64_t)1 << 31), SQ_EUNSUPPORTED, "%s: cache too large", fn);
+  int cur = -1;
+  SQ_HIP(hipGetDevice(&cur));
+  SQ_REQUIRE(cur == dev, SQ_EDEVICE, "%s: tensors live on device %d but the current device is %d", fn, dev, cur);
+  if (n == 0 || B == 0) return SQ_OK;
+  ReorderArgs a;
+  a.k_src = data_of(key_cache);
+  a.v_src = data_of(value_cache);
+  a.k_dst = data_of(key_out);
+  a.v_dst = data_of(value_out);
+  a.order = (const int32_t*)data_of(order);
+  a.n = n;
+  a.src_len = L;
+  a.batch = (int32_t)B;
+  a.heads = (int32_t)H;
+  a.head_chunks = (int32_t)(D / 8);
+  const int64_t chunks = 2 * B * n * H * (D / 8);
+  int64_t blocks = (chunks + 1023) / 1024;
+  if (blocks > 8192) blocks = 8192;
+  hipLaunchKernelGGL(kv_reorder_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, a);
   SQ_HIP(hipGetLastError());
   return SQ_OK;
 }

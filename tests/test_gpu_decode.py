@@ -166,6 +166,58 @@ def test_kmeans_topk_then_selected_decode():
     assert err <= 2e-4 * float(ref.pow(2).mean().sqrt())
 
 
+def test_cluster_ordered_cache_gives_the_same_attention_from_neighbouring_rows():
+    """A copy of the cache in cluster order (`sq_kv_cache_reorder`): the copy holds exactly the rows the order names
+    (checked row by row on the host), the positions table sends the selection to the same tokens, and the attention
+    over positions of the copy equals, bit for bit, the attention over token ids of the original (same rows, same
+    order).  The selected positions form runs: one run per selected cluster."""
+    from longcontext_sqattn_paddle_amd.cache_hub.kmeans import cluster_order, reorder_cache, segment_k_means, topk_select
+
+    print("case cluster-ordered cache", flush=True)
+    dev = torch.device("cuda:0")
+    B, Hq, Hkv, L, C, k = 2, 8, 2, 4096, 64, 700
+    q, kc, vc, _ = inputs.decode_inputs(B, Hq, Hkv, L, 128, seed=73)
+    key = kc.permute(0, 2, 1, 3).reshape(B * Hkv, L, 128).contiguous().to(dev)
+    val = vc.permute(0, 2, 1, 3).reshape(B * Hkv, L, 128).contiguous().to(dev)
+    centroids, _, clusters, cluster_size = segment_k_means(key, val, C, num_iters=3)
+    order, positions = cluster_order(clusters, cluster_size)
+    kg, vg = reorder_cache(kc.to(dev), vc.to(dev), order)
+    torch.cuda.synchronize()
+    G = B * Hkv
+    assert order.shape == (G, L) and kg.shape == (B, L, Hkv, 128)
+    o = order.cpu().long()
+    for g in range(G):
+        assert torch.equal(torch.sort(o[g]).values, torch.arange(L))          # a permutation of the head's tokens
+        b, h = divmod(g, Hkv)
+        assert torch.equal(kg[b, :, h].cpu().view(torch.int16), kc[b, o[g], h].contiguous().view(torch.int16))
+        assert torch.equal(vg[b, :, h].cpu().view(torch.int16), vc[b, o[g], h].contiguous().view(torch.int16))
+    # positions[g, c, j] is where clusters[g, c, j] went
+    cl, sz, pos = clusters.cpu().long(), cluster_size.cpu().long(), positions.cpu().long()
+    for g in range(G):
+        for c in (0, 17, C - 1):
+            n = int(sz[g, c])
+            assert torch.equal(o[g, pos[g, c, :n]], cl[g, c, :n])
+    qd = q[:, 0].to(dev)
+    ids = topk_select(qd, centroids, clusters, cluster_size, k, Hq // Hkv)
+    rows = topk_select(qd, centroids, positions, cluster_size, k, Hq // Hkv)
+    torch.cuda.synchronize()
+    assert torch.equal(torch.gather(o, 1, rows.cpu().long()), ids.cpu().long())
+    steps = (rows.cpu()[:, 1:] - rows.cpu()[:, :-1]) != 1
+    assert int(steps.sum(dim=1).max()) < C                                    # runs, at most one break per cluster
+    a = _selected(q, kc, vc, ids.cpu(), "NHD", output_dtype=torch.float32)
+    b_ = _selected(q, kg.cpu(), vg.cpu(), rows.cpu(), "NHD", output_dtype=torch.float32)
+    assert torch.equal(a, b_)
+    # ids outside the cache give zero rows; shapes are checked
+    bad = order.clone()
+    bad[0, 5] = -1
+    bad[1, 6] = L
+    kz, vz = reorder_cache(kc.to(dev), vc.to(dev), bad)
+    assert float(kz[0, 5, 0].abs().max()) == 0.0 and float(vz[0, 6, 1].abs().max()) == 0.0
+    assert torch.equal(kz[0, 5, 1], kg[0, 5, 1])                              # the other head of that row is untouched
+    with pytest.raises(AssertionError):
+        reorder_cache(kc.to(dev), vc.to(dev), order[:3])
+
+
 def test_selected_decode_argument_errors():
     from longcontext_sqattn_paddle_amd.sqattn.attn_triton_decode import attn_decode_selected
 
