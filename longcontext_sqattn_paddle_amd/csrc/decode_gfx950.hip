@@ -79,6 +79,16 @@ __device__ __forceinline__ f32x4_t mfma_qk(const uint4& a, const uint4& b, f32x4
   }
 }
 
+template <bool BF16>
+__device__ __forceinline__ f32x4_t mfma_pv16(const i32x2_t& a, const i32x2_t& b, f32x4_t c) {
+  typedef __attribute__((ext_vector_type(4))) short i16x4_t;
+  if constexpr (BF16) {
+    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(i16x4_t, a), __builtin_bit_cast(i16x4_t, b), c, 0, 0, 0);
+  } else {
+    return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(f16x4_t, a), __builtin_bit_cast(f16x4_t, b), c, 0, 0, 0);
+  }
+}
+
 // GATHER: token t of the stream is cache row ids[b * Hkv + kvh][t] instead of row t (attention over a selection of
 // the cache, e.g. the tokens of the best-scoring k-means clusters); entries that are negative or beyond the cache
 // are skipped.
@@ -224,14 +234,34 @@ __global__ __launch_bounds__(kWaves * 64) void decode_splitkv_kernel(DecodeArgs 
 #pragma unroll
       for (int e = 0; e < 8; ++e) acc[e] *= alpha;
     }
+    // P.V on the 16-bit matrix instruction with K = 16 tokens: V stays exact, and p goes in as the sum of two 16-bit
+    // numbers, p = hi + lo with hi = p rounded to the tensor dtype and lo = the rounded remainder (relative error
+    // 2^-16 for bf16, 2^-22 for fp16), both accumulated in fp32.  Operand layouts need no transposition: lane
+    // (r, g) holds V[token 4g + j][channel 8r + e] in vf[j] and p[token 4g + j][head r] in p[j], which is the A
+    // (16 channels 8m + e x 16 tokens) and the B (16 tokens x 16 heads) operand of one MFMA per e.  16 MFMAs of four
+    // passes per tile, where the fp32 instruction (one token quartet and one e at a time) took 32 of eight.
+    i32x2_t p_hi, p_lo;
+    {
+      float rem[4];
+      uint32_t hb[4], lb[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const uint32_t w[4] = {vf[i].x, vf[i].y, vf[i].z, vf[i].w};
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const uint32_t bits = (e & 1) ? (w[e >> 1] >> 16) : (w[e >> 1] & 0xffffu);
-        acc[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(elem_to_f32<BF16>(bits), p[i], acc[e], 0, 0, 0);
+      for (int i = 0; i < 4; ++i) {
+        hb[i] = f32_to_elem<BF16>(p[i]);
+        rem[i] = p[i] - elem_to_f32<BF16>(hb[i]);
+        lb[i] = f32_to_elem<BF16>(rem[i]);
       }
+      p_hi = i32x2_t{(int)(hb[0] | (hb[1] << 16)), (int)(hb[2] | (hb[3] << 16))};
+      p_lo = i32x2_t{(int)(lb[0] | (lb[1] << 16)), (int)(lb[2] | (lb[3] << 16))};
+    }
+    const uint32_t vw[4][4] = {{vf[0].x, vf[0].y, vf[0].z, vf[0].w}, {vf[1].x, vf[1].y, vf[1].z, vf[1].w},
+                               {vf[2].x, vf[2].y, vf[2].z, vf[2].w}, {vf[3].x, vf[3].y, vf[3].z, vf[3].w}};
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      // element e of the four tokens' rows: the low or the high halves of word e >> 1
+      const uint32_t sel = (e & 1) ? 0x07060302u : 0x05040100u;
+      const i32x2_t av = {(int)__builtin_amdgcn_perm(vw[1][e >> 1], vw[0][e >> 1], sel), (int)__builtin_amdgcn_perm(vw[3][e >> 1], vw[2][e >> 1], sel)};
+      acc[e] = mfma_pv16<BF16>(av, p_hi, acc[e]);
+      acc[e] = mfma_pv16<BF16>(av, p_lo, acc[e]);
     }
     m = m_new;
   };
