@@ -21,6 +21,9 @@
  *   sq_topk_select            no reference counterpart (defined by this build's benchmark configuration)
  *   sq_kv_cache_store         cache_hub/flash_attn_cache.py:153-232 (prefill_update_kv_cache: the two slice copies)
  *   sq_kv_cache_append        cache_hub/flash_attn_cache.py:239-256 (decode_update_kv_cache)
+ *   sq_kv_cache_reorder       no reference counterpart: a copy of a layer's cache in k-means cluster order
+ *   sq_attention_histogram    sqattn/attn_replacer.py:253-278 (cal_attn_weight) + sqattn/window_search.py:20-87, 244-321
+ *                             (the four histogram reductions over the dense map; capture slot model_hub/qwen.py:38-41)
  *   sq_rmsnorm                model_hub/utils.py:15-19 (rmsnorm; caller model_hub/qwen.py:345-350)
  *   sq_silu_and_mul           model_hub/utils.py:4-13 (silu_and_mul; caller model_hub/qwen.py:319-326)
  *   sq_rope                   model_hub/utils.py:21-106 (apply_rope_with_cos_sin_cache_inplace; caller qwen.py:352-367)

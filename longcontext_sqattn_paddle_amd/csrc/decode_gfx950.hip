@@ -218,11 +218,12 @@ __global__ __launch_bounds__(kWaves * 64) void decode_splitkv_kernel(DecodeArgs 
     const float m_new = fmaxf(m, tmax);
     // nothing valid so far (only a selection can produce such a tile): any finite reference keeps exp2 off inf - inf
     const float m_ref = (m_new == -INFINITY) ? 0.f : m_new;
-    const float alpha = exp2f(m - m_ref);    // exp2(-inf) = 0 on the first tile
+    // the bare v_exp_f32: arguments are <= 0, and results below the normal range may flush to zero
+    const float alpha = __builtin_amdgcn_exp2f(m - m_ref);    // exp2(-inf) = 0 on the first tile
     float psum = 0.f;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      p[i] = exp2f(p[i] - m_ref);
+      p[i] = __builtin_amdgcn_exp2f(p[i] - m_ref);
       psum += p[i];
     }
     l = l * alpha + psum;

@@ -4,7 +4,7 @@ Everything in this package is a CPU restatement (torch-CPU / numpy) of the
 algorithms in the reference's `sqattn/attn_triton.py`, `sqattn/attn_triton_decode.py`,
 `sqattn/attn_triton_mix_relative.py`, `sqattn/attn_triton_mix_bad.py`,
 `sqattn/fake_quant.py`, `sqattn/attn_replacer.py`, `cache_hub/kmeans.py` and
-`cache_hub/flash_attn_cache.py` and `model_hub/utils.py`.
+`cache_hub/flash_attn_cache.py`, `model_hub/utils.py` and `sqattn/window_search.py`.
 It exists to check the HIP kernels, never to serve a request: only `tests/`,
 `__graft_entry__.smoke()` and the `cpu_baseline` leg of `bench.py` import it.
 The product package (`longcontext_sqattn_paddle_amd`) must not import it and
@@ -28,6 +28,10 @@ ships no golden vectors for this path):
 * `layer.*`                        -- torch's own 16-bit CPU operators evaluating the reference's expressions, fp64
                                       closed forms, rotation invariants (parity unpinned: Paddle's rounding points).
 * `model.CpuDecoder`               -- assembled from the pieces above and torch's CPU `linear`; no arithmetic of its own.
+* `window_search.*`                -- dense float64 restatement of the calibration histograms and the window search:
+                                      element-by-element loops on tiny maps, closed forms (uniform rows, one
+                                      sub-diagonal, a sink column), conservation sums, known answers of the search
+                                      (parity unpinned where the reference rounds the map to 16 bits first).
 * `kmeans.topk_select`             -- build-defined (the reference has no top-k code): parity unpinned
                                       by the reference, pinned by brute force only.
 """
