@@ -177,7 +177,10 @@ __global__ __launch_bounds__(256) void prepass_rows_kernel(PrepassArgs a) {
     const int64_t rr = live[u] ? row : row0;
     const int h = (int)(rr % H);
     const int64_t n = (rr / H) % a.N, b = rr / ((int64_t)H * a.N);
-    raw[u] = *(const uint4*)((const uint16_t*)src.p + b * src.sb + n * src.sn + h * src.sh + 8 * l16);
+    {   // rows are read once and written once: non-temporal accesses keep them from displacing each other in L2
+      const u32x4_t w = __builtin_nontemporal_load((const u32x4_t*)((const uint16_t*)src.p + b * src.sb + n * src.sn + h * src.sh + 8 * l16));
+      raw[u] = make_uint4(w[0], w[1], w[2], w[3]);
+    }
     if constexpr (CENTRE) mraw[u] = *(const uint4*)(a.mean + ((int)b * H + h) * kPD + 8 * l16);
     off8[u] = b * d8.sb + n * d8.sn + h * d8.sh + 8 * l16;
     off4[u] = a.want4 ? b * d4.sb + n * d4.sn + h * d4.sh + 8 * l16 : 0;
@@ -204,14 +207,16 @@ __global__ __launch_bounds__(256) void prepass_rows_kernel(PrepassArgs a) {
       float y[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e) y[e] = qdq(x[e], scale, -128.f, 127.f);
-      *(uint4*)((uint16_t*)d8.p + off8[u]) = pack8<BF16>(y);
+      const uint4 o = pack8<BF16>(y);
+      __builtin_nontemporal_store(u32x4_t{o.x, o.y, o.z, o.w}, (u32x4_t*)((uint16_t*)d8.p + off8[u]));
     }
     if (a.want4) {
       const Divisor scale = make_divisor(amax / 7.f);
       float y[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e) y[e] = qdq(x[e], scale, -8.f, 7.f);
-      *(uint4*)((uint16_t*)d4.p + off4[u]) = pack8<BF16>(y);
+      const uint4 o = pack8<BF16>(y);
+      __builtin_nontemporal_store(u32x4_t{o.x, o.y, o.z, o.w}, (u32x4_t*)((uint16_t*)d4.p + off4[u]));
     }
   }
 }
