@@ -57,3 +57,20 @@ def test_sdpa_forward_shapes_on_cpu():
     ref = torch.nn.functional.scaled_dot_product_attention(q.permute(0, 2, 1, 3), k.permute(0, 2, 1, 3).repeat_interleave(2, 1),
                                                            k.permute(0, 2, 1, 3).repeat_interleave(2, 1), is_causal=True)
     assert torch.allclose(out, ref.transpose(1, 2).reshape(1, 10, 64), atol=1e-6)
+
+
+def test_calibration_host_logic_without_a_gpu():
+    """`compress_model` needs token samples (no dataset loading here); the calibration drivers refuse CPU tensors
+    loudly instead of falling back; the capture object only exists on a device."""
+    import pytest
+    import torch
+
+    from longcontext_sqattn_paddle_amd.sqattn import compress, window_search
+
+    with pytest.raises(ValueError):
+        compress.compress_model(model=None, tokenizer=None, device="cuda:0", args=None)
+    q = torch.zeros(1, 8, 2, 128, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError):
+        window_search.attention_histograms(q, q, window_search.ABSOLUTE, 8)
+    assert (window_search.ABSOLUTE, window_search.RELATIVE, window_search.RELATIVE_SINK) == (0, 1, 2)
+    assert compress.SINK_TOKENS == 256 and compress.MAX_SAMPLE_TOKENS == 5000
