@@ -98,12 +98,15 @@ def segment_k_means(key, value, num_centroids: int, num_iters: int = 10, num_seg
     return centroids, value_sum, clusters, cluster_size
 
 
-def topk_select(query, centroids, clusters, cluster_size, k: int, num_kv_groups: int):
-    """Centroid-scored token selection (no reference counterpart): query [B,Hq,D] -> token ids int32 [G,k]."""
+def topk_select(query, centroids, clusters, cluster_size, k: int, num_kv_groups: int, out=None, workspace=None):
+    """Centroid-scored token selection (no reference counterpart): query [B,Hq,D] -> token ids int32 [G,k].
+    `out` (int32 [G,k], contiguous) and `workspace` (`_workspace(G, 1, C, device)`) may be passed by a caller that
+    selects every step."""
     _require(query, "query")
     G, C, _ = centroids.shape
-    out = torch.empty((G, k), dtype=torch.int32, device=query.device)
-    ws = _workspace(G, 1, C, query.device)
+    if out is None:
+        out = torch.empty((G, k), dtype=torch.int32, device=query.device)
+    ws = workspace if workspace is not None else _workspace(G, 1, C, query.device)
     b = [N.dl(t) for t in (query, centroids, clusters, cluster_size, out, ws)]
     N.check(N.lib().sq_topk_select(*[N.ptr(x) for x in b], num_kv_groups, N.current_stream(query.device)))
     return out

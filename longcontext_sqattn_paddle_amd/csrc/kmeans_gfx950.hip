@@ -381,70 +381,129 @@ struct TopkArgs {
   int32_t C, M, k, Hkv, group;
 };
 
+// Cluster score = max over the kv head's q heads of <q_h, centroid>: one thread per centroid, the centroid row in
+// registers (sixteen 16-byte loads), the group's queries in LDS as fp32; every dot product is one fp32 FMA chain over
+// d = 0..127 in order.
 __global__ __launch_bounds__(256) void topk_score_kernel(TopkArgs a) {
+  __shared__ float qs[16][kD];
   const int g = blockIdx.y, b = g / a.Hkv, kvh = g % a.Hkv;
+  const int nh = a.group < 16 ? a.group : 16;
+  for (int i = threadIdx.x; i < nh * kD; i += blockDim.x) {
+    const int h = i / kD, d = i % kD;
+    qs[h][d] = bf16_bits_to_f32(a.query[(int64_t)b * a.q_sb + (int64_t)(kvh * a.group + h) * a.q_sh + d]);
+  }
+  __syncthreads();
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= a.C) return;
   const uint16_t* cp = a.cent + (int64_t)g * a.c_sg + (int64_t)c * a.c_sc;
   float best = -INFINITY;
-  for (int h = 0; h < a.group; ++h) {
-    const uint16_t* qp = a.query + (int64_t)b * a.q_sb + (int64_t)(kvh * a.group + h) * a.q_sh;
-    float s = 0.f;
-    for (int d = 0; d < kD; ++d) s += bf16_bits_to_f32(qp[d]) * bf16_bits_to_f32(cp[d]);
-    best = fmaxf(best, s);
+  if (a.group <= 16) {
+    float cf[kD];
+#pragma unroll
+    for (int j = 0; j < kD / 8; ++j) {
+      const uint4 w = *(const uint4*)(cp + 8 * j);
+      const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        cf[8 * j + 2 * e] = bf16_bits_to_f32(ww[e] & 0xffffu);
+        cf[8 * j + 2 * e + 1] = bf16_bits_to_f32(ww[e] >> 16);
+      }
+    }
+    for (int h = 0; h < nh; ++h) {
+      float sacc = 0.f;
+#pragma unroll
+      for (int d = 0; d < kD; ++d) sacc += qs[h][d] * cf[d];
+      best = fmaxf(best, sacc);
+    }
+  } else {   // more than 16 q heads per kv head: straight from memory
+    for (int h = 0; h < a.group; ++h) {
+      const uint16_t* qp = a.query + (int64_t)b * a.q_sb + (int64_t)(kvh * a.group + h) * a.q_sh;
+      float sacc = 0.f;
+      for (int d = 0; d < kD; ++d) sacc += bf16_bits_to_f32(qp[d]) * bf16_bits_to_f32(cp[d]);
+      best = fmaxf(best, sacc);
+    }
   }
   a.score[(int64_t)g * a.C + c] = best;
 }
 
-// rank clusters by (score desc, index asc), prefix-sum their sizes in rank order, copy token ids.
+// Order the clusters by (score descending, index ascending), prefix-sum their sizes in that order and emit the first k
+// token ids: one workgroup per group, everything in LDS.  The order comes from a bitonic sort of 64-bit keys
+// (score mapped to an unsigned integer of the same order in the high word, ~index in the low word; a counting rank
+// with C compares per cluster took 50 us at C = 1024).  Each output position finds its cluster by a binary search
+// over the prefix; positions past the total number of tokens get -1.
 __global__ __launch_bounds__(1024) void topk_emit_kernel(TopkArgs a) {
-  extern __shared__ int32_t sh[];          // [C] size in rank order, then exclusive prefix
+  extern __shared__ int32_t sh[];          // [P] 64-bit keys (P = C rounded up to a power of two), then [C + 1] prefix
+  int P = 1;
+  while (P < a.C) P <<= 1;
+  unsigned long long* key = (unsigned long long*)sh;
+  int32_t* pre = sh + 2 * P;
+  __shared__ int32_t part[1024];
   const int g = blockIdx.x, t = threadIdx.x;
-  const float* sc = a.score + (int64_t)g * a.C;
   const int32_t* size = a.size + (int64_t)g * a.C;
-  int32_t* start = a.start + (int64_t)g * a.C;
-  for (int c = t; c < a.C; c += blockDim.x) {
-    const float s = sc[c];
-    int rank = 0;
-    for (int u = 0; u < a.C; ++u) {
-      const float v = sc[u];
-      rank += (v > s) || (v == s && u < c);
+  for (int c = t; c < P; c += blockDim.x) {
+    unsigned long long kk = 0;             // padding sorts behind every cluster
+    if (c < a.C) {
+      const uint32_t bits = __float_as_uint(a.score[(int64_t)g * a.C + c] + 0.0f);    // -0.0 counts as +0.0
+      const uint32_t ord = (bits & 0x80000000u) ? ~bits : (bits | 0x80000000u);
+      kk = ((unsigned long long)ord << 32) | (0xffffffffu - (uint32_t)c);
     }
-    start[c] = rank;            // temporarily the rank
-    sh[rank] = size[c];
+    key[c] = kk;
   }
   __syncthreads();
-  if (t == 0) {                 // C <= 8192: a serial prefix is a few microseconds
-    int run = 0;
-    for (int r = 0; r < a.C; ++r) {
-      const int v = sh[r];
-      sh[r] = run;
-      run += v;
+  for (int len = 2; len <= P; len <<= 1)
+    for (int d = len >> 1; d > 0; d >>= 1) {
+      for (int i = t; i < P / 2; i += blockDim.x) {
+        const int lo = ((i & ~(d - 1)) << 1) | (i & (d - 1)), hi = lo | d;
+        const bool descending = (lo & len) == 0;
+        const unsigned long long x = key[lo], y = key[hi];
+        if ((x < y) == descending) {
+          key[lo] = y;
+          key[hi] = x;
+        }
+      }
+      __syncthreads();
+    }
+  auto by_rank = [&](int r) { return (int)(0xffffffffu - (uint32_t)key[r]); };
+  // exclusive prefix of the (clamped) sizes in rank order: per-thread runs of `per` ranks, a scan over the 1024 run sums
+  const int per = (a.C + 1023) / 1024;
+  int run = 0;
+  for (int i = 0; i < per; ++i) {
+    const int r = t * per + i;
+    if (r < a.C) run += min(size[by_rank(r)], a.M);
+  }
+  part[t] = run;
+  __syncthreads();
+  for (int d = 1; d < 1024; d <<= 1) {   // Hillis-Steele inclusive scan
+    const int v = (t >= d) ? part[t - d] : 0;
+    __syncthreads();
+    part[t] += v;
+    __syncthreads();
+  }
+  int acc = part[t] - run;
+  for (int i = 0; i < per; ++i) {
+    const int r = t * per + i;
+    if (r < a.C) {
+      pre[r] = acc;
+      acc += min(size[by_rank(r)], a.M);
     }
   }
+  if (t == 1023) pre[a.C] = part[1023];
   __syncthreads();
+  const int total = pre[a.C];
   int32_t* out = a.out + (int64_t)g * a.k;
-  for (int c = t; c < a.C; c += blockDim.x) {
-    const int st = sh[start[c]];
-    const int n = min(size[c], a.M);
-    const int32_t* src = a.clusters + (int64_t)g * a.cl_sg + (int64_t)c * a.cl_sc;
-    for (int i = 0; i < n && st + i < a.k; ++i) out[st + i] = src[i];
+  for (int p = t; p < a.k; p += blockDim.x) {
+    int32_t id = -1;
+    if (p < total) {
+      int lo = 0, hi = a.C;               // the rank r with pre[r] <= p < pre[r + 1]
+      while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (pre[mid] <= p) lo = mid;
+        else hi = mid;
+      }
+      id = a.clusters[(int64_t)g * a.cl_sg + (int64_t)by_rank(lo) * a.cl_sc + (p - pre[lo])];
+    }
+    out[p] = id;
   }
-}
-
-__global__ void topk_tail_kernel(TopkArgs a) {
-  // positions past the total number of tokens stay -1
-  const int g = blockIdx.y;
-  const int32_t* size = a.size + (int64_t)g * a.C;
-  __shared__ int tot;
-  if (threadIdx.x == 0) {
-    int s = 0;
-    for (int c = 0; c < a.C; ++c) s += min(size[c], a.M);
-    tot = s;
-  }
-  __syncthreads();
-  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < a.k; i += gridDim.x * blockDim.x)
-    if (i >= tot) a.out[(int64_t)g * a.k + i] = -1;
 }
 
 struct WsLayout {
@@ -681,8 +740,12 @@ extern "C" int sq_topk_select(const DLTensor* query, const DLTensor* centroids, 
   a.Hkv = (int)Hkv;
   a.group = num_kv_groups;
   hipLaunchKernelGGL(topk_score_kernel, dim3((unsigned)((C + 255) / 256), (unsigned)G), dim3(256), 0, st, a);
-  hipLaunchKernelGGL(topk_emit_kernel, dim3((unsigned)G), dim3(1024), (size_t)C * 4, st, a);
-  hipLaunchKernelGGL(topk_tail_kernel, dim3(8, (unsigned)G), dim3(256), 0, st, a);
+  int P = 1;
+  while (P < C) P <<= 1;
+  const size_t emit_lds = (size_t)(2 * P + C + 1) * 4;
+  if (emit_lds > 48 * 1024)   // beyond the default limit of dynamic LDS (C > 4096)
+    SQ_HIP(hipFuncSetAttribute((const void*)topk_emit_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)emit_lds));
+  hipLaunchKernelGGL(topk_emit_kernel, dim3((unsigned)G), dim3(1024), emit_lds, st, a);
   SQ_HIP(hipGetLastError());
   return SQ_OK;
 }

@@ -36,6 +36,26 @@ class LLM:
         self.dtype = dtype
         self.device_map = device_map
         self.capture_layer_inps = None
+        self.kv_selection = None   # see enable_kv_selection
+
+    def enable_kv_selection(self, num_centroids: int = 1024, topk: int = 4096, num_iters: int = 10, num_segments: int = 1):
+        """Extension (the reference's k-means code has no caller): after every prefill the prompt's keys are clustered
+        per layer, sequence and kv head, and the decode steps attend to the `topk` tokens of the best-scoring clusters
+        plus the generated tokens instead of the whole cache.  `disable_kv_selection()` returns to dense decoding."""
+        from ..cache_hub.kv_selection import KVSelection
+
+        self.kv_selection = KVSelection(num_centroids, topk, num_iters, num_segments)
+
+    def cluster_prompt(self):
+        """Cluster the keys the cache holds now (the prefilled prompt) and switch the decode slots to the selection."""
+        self.kv_selection.build(self.kv_cache, self.num_key_value_heads, self.num_key_value_groups)
+        for layer in self.layers:
+            layer.kv_selection = self.kv_selection
+
+    def disable_kv_selection(self):
+        self.kv_selection = None
+        for layer in getattr(self, "layers", []):
+            layer.kv_selection = None
 
     # ------------------------------------------------------------------ one layer
     def layer_prefill(self, layer_idx, start_bdx, hidden_states):
@@ -154,6 +174,8 @@ class LLM:
     def inference(self, inputs_ids, verbose: bool = True, use_graph: bool = False):
         """LLM.py:167-203: greedy decoding; returns the generated ids as nested lists [batch][max_new_length]."""
         outputs_ids = []
+        for layer in self.layers:
+            layer.kv_selection = None     # clusters of an earlier prompt
         torch.cuda.synchronize()
         prefill_start = time.time()
         logits = self.prefill_forward(inputs_ids=inputs_ids)
@@ -164,6 +186,13 @@ class LLM:
         self.prefill_latency = time.time() - prefill_start
         if verbose:
             print(f"Prefilling latency: {round(self.prefill_latency, 4)} s")
+        if self.kv_selection is not None and self.max_new_length > 1:
+            cluster_start = time.time()
+            self.cluster_prompt()
+            torch.cuda.synchronize()
+            self.cluster_latency = time.time() - cluster_start
+            if verbose:
+                print(f"Clustering latency: {round(self.cluster_latency, 4)} s")
         if self.max_new_length > 1:
             decode_start, timed_steps = time.time(), self.max_new_length - 1
             for step in range(self.max_new_length - 1):

@@ -53,6 +53,7 @@ class QwenLayer:
         self.kv_cache = None   # set by QwenModel.init_kv_cache: decode attention needs the per-sequence lengths
         self.p_quant = None    # extension: a P mode of the prefill kernel (e.g. 5 = fp8 P.V); None = exact attention
         self.calibration = None   # a sqattn.window_search.CalibrationCapture while the window search runs on this layer
+        self.kv_selection = None  # a cache_hub.kv_selection.KVSelection once the prompt's keys are clustered (extension)
 
     def prefill_attention(self, query_states, key_states, value_states, layer_idx=None):
         """qwen.py:37-46: exact causal attention over [B, N, H, D] tensors (SDPA / flash attention in the reference;
@@ -69,6 +70,11 @@ class QwenLayer:
         """qwen.py:48-54: one query token against the layer's cache buffers [B, max_length, Hkv, D]."""
         if self.attention_type not in ("SQAttn", "SDPA", "FlashAttn"):
             raise ValueError(f"Unsupported attention type: {self.attention_type}")
+        if self.kv_selection is not None:
+            # extension: attend to the tokens of the best-scoring k-means clusters and to the generated tokens only
+            if self.layer_idx == 0:
+                self.kv_selection.begin_step(self.kv_cache.attend_length)
+            return self.kv_selection.attend(self.layer_idx, query_states, key_states, value_states, self.num_key_value_groups)
         lens = self.kv_cache.attend_length if self.kv_cache is not None else None
         return attn_decode(query_states, key_states, value_states, "NHD", query_states.dtype, seqlens=lens)
 

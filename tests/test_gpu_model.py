@@ -114,3 +114,62 @@ def test_graph_replayed_decode_equals_eager_decode():
         torch.cuda.synchronize()
         assert torch.equal(la, lb) and bool(torch.isfinite(junk).all())
     b.release_decode_graph()
+
+
+def test_kmeans_kv_selection_in_the_decode_steps():
+    """Extension of the runtime: decode over the k-means selection.  (1) With a selection wide enough to hold every
+    cluster, the steps see the whole cache (in cluster order) plus the generated tokens, so their logits agree with
+    dense decoding.  (2) With a narrow selection, a layer's attention equals the oracle's closed form over exactly
+    the rows the selection lists: the top clusters' tokens and the generated tokens."""
+    import math
+
+    from oracle import attention as A
+
+    new = 6
+    g = torch.Generator().manual_seed(21)
+    prompt = torch.randint(0, 1000, (1, 640), generator=g).to(DEV)
+    forced = torch.randint(0, 1000, (new, 1, 1), generator=g).to(DEV)
+
+    def run(select, topk=0):
+        model = _small_model(640 + new + 2, layers=3)
+        if select:
+            model.enable_kv_selection(num_centroids=32, topk=topk, num_iters=3)
+        model.batch_size, model.input_length, model.max_new_length = 1, 640, new + 2
+        model.init_kv_cache(640, [0])
+        for layer in model.layers:
+            layer.kv_selection = None
+        model.prefill_forward(prompt)
+        if select:
+            model.cluster_prompt()
+        logits = []
+        for t in range(new):
+            logits.append(model.decode_forward(forced[t]).float().cpu())
+        return model, torch.stack(logits)
+
+    _, dense = run(False)
+    _, wide = run(True, topk=640)
+    assert _cos(dense, wide) >= 0.9995 and float((dense - wide).abs().max()) <= 0.05 * float(dense.abs().max())
+    model, narrow = run(True, topk=96)
+    assert bool(torch.isfinite(narrow).all()) and _cos(dense, narrow) < 0.99999      # the selection does change the result
+    # one layer's attention by hand: lists = 96 selected tokens + the generated ones so far
+    sel, cache, layer = model.kv_selection, model.kv_cache, model.layers[1]
+    q = torch.randn(1, 1, 4, 128, generator=g).to(torch.bfloat16).to(DEV)
+    sel.begin_step(cache.attend_length)
+    out = sel.attend(1, q, cache.key_cache[1], cache.value_cache[1], 2)
+    torch.cuda.synchronize()
+    n_list = int(sel.list_len[0])
+    assert n_list == 96 + int(cache.attend_length[0]) - 640
+    ids = sel.ids[:, :n_list].cpu()
+    assert int(ids[:, :96].max()) < 640 and torch.equal(ids[0, 96:], torch.arange(640, 640 + n_list - 96, dtype=torch.int32))
+    kc, vc = cache.key_cache[1].cpu(), cache.value_cache[1].cpu()
+    qh = q.cpu().permute(0, 2, 1, 3)
+    ref, _ = A.decode_selected_exact(A.fold_scale(qh, 128), kc.permute(0, 2, 1, 3), vc.permute(0, 2, 1, 3), ids, score_scale=math.log(2.0))
+    err = float((out.float().cpu()[:, 0].double() - ref[:, :, 0]).abs().max())
+    assert err <= 2.0 ** -8 * float(ref.abs().max())             # the slot returns bf16: half a unit in the last place
+    assert layer.kv_selection is sel
+    # the selection inside the captured decode step: same tokens as the eager loop
+    model = _small_model(640 + 24, layers=3)
+    model.enable_kv_selection(num_centroids=32, topk=96, num_iters=3)
+    eager = model.generate("SDPA", prompt, None, 12, verbose=False)
+    graphed = model.generate("SDPA", prompt, None, 12, verbose=False, use_graph=True)
+    assert eager == graphed
