@@ -162,7 +162,8 @@ int sq_index_add(const DLTensor* value, const DLTensor* idx, DLTensor* out, DLTe
 /*
  * Centroid-scored token selection: per group g = b*Hkv + kvh, clusters ranked by
  * max_{h in group} <query[b,h], centroids[g,c]> (ties -> lower c); whole clusters taken in rank order
- * until k tokens are emitted; missing tail = -1.  query bf16 [B,Hq,D]; out int32 [G,k].
+ * until k tokens are emitted; missing tail = -1.  query bf16 [B,Hq,D]; out int32 [G,k], rows contiguous and at least
+ * k apart (it may be the leading columns of a wider list that sq_decode_selected_fwd reads).
  */
 int sq_topk_select(const DLTensor* query, const DLTensor* centroids, const DLTensor* clusters,
                    const DLTensor* cluster_size, DLTensor* out, DLTensor* workspace, int32_t num_kv_groups,

@@ -63,7 +63,7 @@ class KVSelection:
         self.offset = torch.tensor([self.topk - n for n in prompt], dtype=torch.int32, device=dev)
         self.list_len = torch.zeros(B, dtype=torch.int32, device=dev)
         # buffers of a step, allocated once: the selection, the top-k scratch, the decode partials
-        self.picked = torch.empty(B * Hkv, self.topk, dtype=torch.int32, device=dev)
+        self.picked = self.ids[:, :self.topk]
         self.topk_ws = _workspace(B * Hkv, 1, self.num_centroids, dev)
         lib = N.lib()
         splits = lib.sq_decode_num_splits(B, Hkv, self.topk + self.room)
@@ -79,7 +79,6 @@ class KVSelection:
         """query_states [B, 1, Hq, D]; key_cache / value_cache [B, max_length, Hkv, D] -> [B, 1, Hq, D]."""
         st = self.layers[layer_idx]
         topk_select(query_states[:, 0], st["centroids"], st["clusters"], st["cluster_size"], self.topk, num_kv_groups,
-                    out=self.picked, workspace=self.topk_ws)
-        self.ids[:, :self.topk].copy_(self.picked)
+                    out=self.picked, workspace=self.topk_ws)      # straight into the leading columns of the lists
         return attn_decode_selected(query_states, key_cache, value_cache, self.ids, "NHD", query_states.dtype, seqlens=self.list_len,
                                     workspace=self.decode_ws)

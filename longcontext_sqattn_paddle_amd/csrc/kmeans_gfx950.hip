@@ -374,7 +374,8 @@ struct TopkArgs {
   const uint16_t* cent;    // [G,C,128] bf16
   const int32_t* clusters; // [G,C,M]
   const int32_t* size;     // [G,C]
-  int32_t* out;            // [G,k]
+  int32_t* out;            // [G,k], rows out_sg apart
+  int64_t out_sg;
   float* score;            // workspace [G,C]
   int32_t* start;          // workspace [G,C] start position of each cluster in rank order
   int64_t q_sb, q_sh, c_sg, c_sc, cl_sg, cl_sc;
@@ -490,7 +491,7 @@ __global__ __launch_bounds__(1024) void topk_emit_kernel(TopkArgs a) {
   if (t == 1023) pre[a.C] = part[1023];
   __syncthreads();
   const int total = pre[a.C];
-  int32_t* out = a.out + (int64_t)g * a.k;
+  int32_t* out = a.out + (int64_t)g * a.out_sg;
   for (int p = t; p < a.k; p += blockDim.x) {
     int32_t id = -1;
     if (p < total) {
@@ -704,9 +705,12 @@ extern "C" int sq_topk_select(const DLTensor* query, const DLTensor* centroids, 
   const int dev = query->device.device_id;
   int rc;
   if ((rc = check_gnd(query, "query", dev)) || (rc = check_gnd(centroids, "centroids", dev)) ||
-      (rc = check_i32(clusters, "clusters", 3, dev)) || (rc = check_i32(cluster_size, "cluster_size", 2, dev)) ||
-      (rc = check_i32(out, "out", 2, dev)))
+      (rc = check_i32(clusters, "clusters", 3, dev)) || (rc = check_i32(cluster_size, "cluster_size", 2, dev)))
     return rc;
+  // out may be the leading columns of a wider int32 matrix (a decode list that continues with other tokens)
+  SQ_REQUIRE(on_gpu(out) && out->device.device_id == dev, SQ_EDEVICE, "out is not on the same ROCm device");
+  SQ_REQUIRE(dtype_of(out) == DType::I32 && out->ndim == 2 && stride_of(out, 1) == 1 && stride_of(out, 0) >= out->shape[1], SQ_ESHAPE,
+             "out must be int32 [G, k] with contiguous rows");
   const int64_t B = query->shape[0], Hq = query->shape[1], G = centroids->shape[0], C = centroids->shape[1];
   const int64_t M = clusters->shape[2], k = out->shape[1];
   SQ_REQUIRE(num_kv_groups > 0 && Hq % num_kv_groups == 0, SQ_EINVAL, "sq_topk_select: num_kv_groups %d does not divide Hq", num_kv_groups);
@@ -726,6 +730,7 @@ extern "C" int sq_topk_select(const DLTensor* query, const DLTensor* centroids, 
   a.clusters = (const int32_t*)data_of(clusters);
   a.size = (const int32_t*)data_of(cluster_size);
   a.out = (int32_t*)data_of(out);
+  a.out_sg = stride_of(out, 0);
   a.score = (float*)(wsp + w.off_bytes + w.hist_bytes + w.order_bytes);
   a.start = (int32_t*)(wsp + w.off_bytes + w.hist_bytes + w.order_bytes + w.score_bytes);
   a.q_sb = stride_of(query, 0);
