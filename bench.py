@@ -391,7 +391,22 @@ def time_kmeans(torch, iters=10):
     us = e0.elapsed_time(e1) / iters * 1e3
     flops = 2.0 * N * C * D * G
     nbytes = G * (N * D * 2 * 2 + N * 4 * 3 + C * D * 2 * 2)   # K read by assign and by the cluster sums, idx/order, centroids
-    return us, flops, nbytes
+    # the selection that follows the clustering in the benchmark configuration: top-k = 4096 tokens for a 28-head query
+    from longcontext_sqattn_paddle_amd.cache_hub.kmeans import segment_k_means, topk_select
+
+    cent2, _, clusters, size = segment_k_means(key, key, C, num_iters=3)
+    q = torch.randn(1, 28, D, device=dev, generator=torch.Generator(device=dev).manual_seed(9)).bfloat16()
+    out = torch.empty(G, 4096, dtype=torch.int32, device=dev)
+    for _ in range(3):
+        topk_select(q, cent2, clusters, size, 4096, 7, out=out, workspace=ws)
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(20):
+        topk_select(q, cent2, clusters, size, 4096, 7, out=out, workspace=ws)
+    e1.record()
+    torch.cuda.synchronize()
+    assert int(out.min()) >= 0 and int(out.max()) < N
+    return us, flops, nbytes, e0.elapsed_time(e1) / 20 * 1e3
 
 
 def time_prepass(torch, N, want4, iters=10):
@@ -573,11 +588,13 @@ def main():
         result["e2e"] = [time_e2e(torch, N, new_tokens=args.e2e_new_tokens, **runs[r]) for r in args.e2e_runs.split(",")]
         log(f"[bench] end to end: {result['e2e']}")
     if not args.no_kmeans:
-        us, kflops, kbytes = time_kmeans(torch)
+        us, kflops, kbytes, topk_us = time_kmeans(torch)
         result["kmeans"] = {"us_per_iteration": round(us, 1), "TFLOP_per_s": round(kflops / us / 1e6, 1),
                             "frac_of_bf16_mfma_peak": round(kflops / us / 1e6 / PEAK_MFMA_BF16_TFLOPS, 4),
                             "GB_per_s": round(kbytes / us / 1e3, 1), "frac_of_hbm_peak": round(kbytes / us / 1e3 / PEAK_HBM_GBS, 4),
-                            "shape": "4 heads x 131072 tokens x 128, 1024 centroids, one Lloyd iteration"}
+                            "shape": "4 heads x 131072 tokens x 128, 1024 centroids, one Lloyd iteration",
+                            "topk_select_us": round(topk_us, 1),
+                            "topk_shape": "4096 tokens per kv head for one 28-head query, 1024 clusters per kv head"}
         log(f"[bench] kmeans iteration: {us:.0f} us")
     if not args.no_cpu_baseline:
         from oracle.cpu_baseline import time_cpu_baseline   # the checker's CPU path, timed as the baseline only
