@@ -235,7 +235,7 @@ def time_model_layers(torch, N):
     return out
 
 
-def time_e2e(torch, N, new_tokens=17, sqattn=False, kv_selection=False):
+def time_e2e(torch, N, new_tokens=17, sqattn=False, kv_selection=False, graph=False):
     """The whole 28-layer decoder of Qwen2.5-7B's shapes (random weights) through `generate`: prefill of one N-token
     prompt and greedy decoding, as the reference's latency logs measure them (model_hub/LLM.py:167-203).  With
     `sqattn`, layers 1..26 run the quantised sink/window closure of `process_model` with relative windows 0.25 / 0.5
@@ -268,13 +268,15 @@ def time_e2e(torch, N, new_tokens=17, sqattn=False, kv_selection=False):
     if kv_selection:
         model.enable_kv_selection(num_centroids=1024, topk=4096, num_iters=10)
     model.generate(model.attention_type, ids[:, :4096], None, 3, verbose=False)    # warm-up: library handles, GEMM heuristics
-    eager = model.generate(model.attention_type, ids, None, new_tokens, verbose=False)
+    eager = model.generate(model.attention_type, ids, None, new_tokens, verbose=False, use_graph=graph)
     res = {"prefill_s": round(model.prefill_latency, 3), "decode_ms_per_step": round(model.decode_latency * 1e3, 3),
            "tokens": N, "layers": cfg.num_hidden_layers, "attention": "SQAttn windows 0.25/0.5, sink 256" if sqattn else "exact causal"}
+    if graph:
+        res["decode_loop"] = "steps after the second replayed from a HIP graph"
     if kv_selection:
         res["decode"] = "k-means KV selection: 1024 clusters per kv head, 10 iterations, 4096 tokens per kv head and step"
         res["clustering_s"] = round(model.cluster_latency, 3)
-    if (not sqattn or kv_selection) and N <= 262144:   # (a second prefill of a longer prompt only for this check would take minutes)
+    if (not sqattn or kv_selection) and N <= 262144 and not graph:   # (a second prefill of a longer prompt only for this check would take minutes)
         # the same generation with the decode step replayed from a HIP graph: must produce the same tokens
         graphed = model.generate(model.attention_type, ids, None, new_tokens + 32, verbose=False, use_graph=True)
         assert graphed[0][:new_tokens] == eager[0], "graph-replayed decode diverged from the eager decode"
@@ -462,6 +464,8 @@ def main():
                     help="which end-to-end runs --e2e makes: exact attention, the SQAttn closure, the SQAttn closure with "
                          "k-means KV selection in the decode steps")
     ap.add_argument("--e2e-new-tokens", type=int, default=17, help="tokens generated by each end-to-end run")
+    ap.add_argument("--e2e-graph", action="store_true",
+                    help="the end-to-end runs replay their decode steps from a HIP graph (for prompts too long to prefill twice)")
     ap.add_argument("--e2e", action="store_true",
                     help="also run the whole 28-layer Qwen2.5-7B-shaped decoder (random weights): prefill latency and decode ms/step")
     args = ap.parse_args()
@@ -585,7 +589,7 @@ def main():
         torch.cuda.empty_cache()
     if args.e2e:
         runs = {"exact": dict(sqattn=False), "sqattn": dict(sqattn=True), "selection": dict(sqattn=True, kv_selection=True)}
-        result["e2e"] = [time_e2e(torch, N, new_tokens=args.e2e_new_tokens, **runs[r]) for r in args.e2e_runs.split(",")]
+        result["e2e"] = [time_e2e(torch, N, new_tokens=args.e2e_new_tokens, graph=args.e2e_graph, **runs[r]) for r in args.e2e_runs.split(",")]
         log(f"[bench] end to end: {result['e2e']}")
     if not args.no_kmeans:
         us, kflops, kbytes, topk_us = time_kmeans(torch)
