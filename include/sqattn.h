@@ -27,6 +27,8 @@
  *   sq_rmsnorm                model_hub/utils.py:15-19 (rmsnorm; caller model_hub/qwen.py:345-350)
  *   sq_silu_and_mul           model_hub/utils.py:4-13 (silu_and_mul; caller model_hub/qwen.py:319-326)
  *   sq_rope                   model_hub/utils.py:21-106 (apply_rope_with_cos_sin_cache_inplace; caller qwen.py:352-367)
+ *   sq_linear_rows            the matmuls of a decode step: model_hub/qwen.py:293-300 (lm), :302-312 (wqkv), :314-317 (wo),
+ *                             :319-326 (mlp), called from model_hub/LLM.py:88-116 (layer_decode)
  *   sq_fake_quant_prepass     sqattn/attn_replacer.py:334-365 (GQA expand, key centring and the five fake-quant
  *                             passes of mp_triton_wrapper's closure), sqattn/fake_quant.py:24-58, 98-125
  */
@@ -234,6 +236,19 @@ int sq_rmsnorm(const DLTensor* x, const DLTensor* weight, DLTensor* out, float e
  * operators each rounded to the tensor dtype.  bf16 or fp16; I a multiple of 8.
  */
 int sq_silu_and_mul(const DLTensor* x, DLTensor* out, void* stream);
+
+/*
+ * out = x . weight^T (+ bias) (+ residual) for 1 to 8 rows of x: the projections of a decode step, which the
+ * reference runs as tensor-library matmuls on a [batch, 1, hidden] activation (model_hub/qwen.py:302-326, lm head
+ * :293-300).  x [M, K], weight [N, K] (the layout of a Linear layer's weight), bias [N] or NULL, residual [M, N] or
+ * NULL, out [M, N]; bf16 or fp16, all of one dtype; K a multiple of 8; rows of x and weight 16-byte aligned (row
+ * strides free), last dimensions contiguous.  fp32 accumulation; the sum plus the bias is rounded once to the tensor
+ * dtype, and with a residual that rounded value plus the residual is rounded again (the two tensor operators of
+ * `residual + linear(x)`).  out may be the residual tensor itself; it must not overlap x.  M > 8 returns
+ * SQ_EUNSUPPORTED: such a product is a GEMM and belongs to the BLAS library.
+ */
+int sq_linear_rows(const DLTensor* x, const DLTensor* weight, const DLTensor* bias, const DLTensor* residual,
+                   DLTensor* out, void* stream);
 
 /*
  * Rotary position embedding of query [T, Hq * head_dim] and key [T, Hkv * head_dim] (T = batch * seq_len tokens)

@@ -1,0 +1,243 @@
+// The projections of a decode step for gfx950 (MI355X): y = x . W^T (+ bias) (+ residual) for at most eight rows of
+// x.  In the reference's runtime these are the tensor-library matmuls of wqkv, wo, mlp and lm
+// (model_hub/qwen.py:302-326, 293-300) on a [batch, 1, hidden] activation.  With one to eight activation rows the
+// product is a pass over the weights: every weight is read once from HBM and used `rows` times, so the kernel is
+// HBM-bound (algorithmic bytes = N x K weights x 2) and is laid out for that, not for the matrix cores: one wave
+// owns R output features, its 64 lanes walk the K axis in 16-byte steps (1 KB per wave and load, several loads in
+// flight), the activation rows sit in LDS, products go through the packed 16-bit dot instruction
+// (v_dot2c_f32_bf16 / v_dot2c_f32_f16: fp32 accumulation), and the R x rows partial sums of the 64 lanes are folded
+// by a transposing butterfly.  Rounding points: the fp32 sum plus the bias is rounded once to the tensor dtype (what
+// a GEMM with a bias epilogue gives); a residual is then added as a second tensor operator would (rounded again).
+#include "common.hpp"
+
+namespace sq {
+namespace {
+
+constexpr int kLinThreads = 256;   // four waves
+// Activation rows in LDS, K-chunk by K-chunk: up to 20480 elements of one row (a whole row of the widest projection,
+// four workgroups per CU), 5120 of each of four; with eight rows 2048 of each, which keeps five workgroups on a CU.
+constexpr int kLinLdsBytes = 40960, kLinLdsBytes8 = 32768;
+constexpr int kLinMaxRows = 8;
+
+struct LinArgs {
+  const char* x;
+  const char* w;
+  const char* bias;   // nullable
+  const char* res;    // nullable
+  char* y;
+  int64_t x_sr, w_sr, r_sr, y_sr;   // row strides in bytes
+  int32_t rows;                     // rows of x actually present (<= M)
+  int32_t n, k;
+  int32_t chunk;   // elements of every activation row per LDS pass (a multiple of 8)
+};
+
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2_t;
+
+template <bool BF16>
+__device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
+  if constexpr (BF16) return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b), c, false);
+  else return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, a), __builtin_bit_cast(f16x2_t, b), c, false);
+}
+template <bool BF16>
+__device__ __forceinline__ float ld16(const char* p) {
+  const uint32_t bits = *(const uint16_t*)p;
+  if constexpr (BF16) return bf16_bits_to_f32(bits);
+  else return (float)__builtin_bit_cast(_Float16, (uint16_t)bits);
+}
+template <bool BF16>
+__device__ __forceinline__ uint16_t st16(float x) {
+  if constexpr (BF16) return (uint16_t)f32_to_bf16_bits(x);
+  else return __builtin_bit_cast(uint16_t, (_Float16)x);
+}
+template <bool BF16>
+__device__ __forceinline__ float rnd16(float x) {
+  if constexpr (BF16) return bf16_bits_to_f32(f32_to_bf16_bits(x));
+  else return (float)(_Float16)x;
+}
+
+// M = activation rows the registers are sized for (1, 2, 4, 8), R = output features per wave (1, 2, 4),
+// U = 16-byte weight loads per feature a lane keeps in flight (eight loads per lane in all).
+template <bool BF16, int M, int R>
+__global__ __launch_bounds__(kLinThreads) void linear_rows_kernel(LinArgs a) {
+  constexpr int U = 8 / R;
+  extern __shared__ u32x4_t xs[];   // [M][chunk / 8]
+  const int kLinChunk = a.chunk, row16 = a.chunk / 8;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t feat0 = ((int64_t)blockIdx.x * (kLinThreads / 64) + wave) * R;
+  const bool live = feat0 < a.n;
+  const char* wrow[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int64_t f = (feat0 + r < a.n) ? feat0 + r : (int64_t)a.n - 1;   // features past the end re-read the last one
+    wrow[r] = a.w + f * a.w_sr;
+  }
+  float acc[R * M];
+#pragma unroll
+  for (int i = 0; i < R * M; ++i) acc[i] = 0.f;
+
+  for (int k0 = 0; k0 < a.k; k0 += kLinChunk) {
+    const int chunks = ((a.k - k0 < kLinChunk) ? (a.k - k0) : kLinChunk) / 8;
+    u32x4_t wv[R][U];
+    auto request = [&](int base) {   // base: the batch's first 16-byte step (wave-uniform)
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int cc = base + lane + 64 * u;
+        const int64_t off = ((int64_t)k0 + (int64_t)(cc < chunks ? cc : chunks - 1) * 8) * 2;   // past the end: re-read the last step
+#pragma unroll
+        for (int r = 0; r < R; ++r) wv[r][u] = __builtin_nontemporal_load((const u32x4_t*)(wrow[r] + off));
+      }
+    };
+    auto consume = [&](int base) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int cc = base + lane + 64 * u;
+        if (cc < chunks) {
+#pragma unroll
+          for (int m = 0; m < M; ++m) {
+            const u32x4_t xv = xs[m * row16 + cc];
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+#pragma unroll
+              for (int j = 0; j < 4; ++j) acc[r * M + m] = dot2<BF16>(wv[r][u][j], xv[j], acc[r * M + m]);
+          }
+        }
+      }
+    };
+    if (live) request(0);   // the first weights are on their way while the activations are staged
+    if (k0) __syncthreads();
+#pragma unroll
+    for (int m = 0; m < M; ++m) {
+      const char* xr = a.x + (int64_t)(m < a.rows ? m : a.rows - 1) * a.x_sr + (int64_t)k0 * 2;
+#pragma unroll 4
+      for (int c = threadIdx.x; c < chunks; c += kLinThreads) xs[m * row16 + c] = *(const u32x4_t*)(xr + c * 16);
+    }
+    __syncthreads();
+    if (live) {
+      for (int base = 0; base < chunks; base += 64 * U) {
+        if (base) request(base);
+        consume(base);
+      }
+    }
+  }
+  if (!live) return;
+
+  // Fold the 64 lanes.  While more than one value is left, a step over lane bit s halves the list: a lane keeps the
+  // even or the odd entry of each pair (by its bit s) and receives the partner's partial sum of that entry.  After
+  // log2(V) steps lane l holds entry (l mod V), summed over the low lane bits; plain butterflies finish the rest.
+  constexpr int V = R * M;
+  int width = V, s = 0;
+#pragma unroll
+  for (; (1 << s) < V; ++s) {
+    const bool odd = (lane >> s) & 1;
+#pragma unroll
+    for (int i = 0; i < width / 2; ++i) {
+      const float keep = odd ? acc[2 * i + 1] : acc[2 * i];
+      const float send = odd ? acc[2 * i] : acc[2 * i + 1];
+      acc[i] = keep + __shfl_xor(send, 1 << s);
+    }
+    width /= 2;
+  }
+#pragma unroll
+  for (; s < 6; ++s) acc[0] += __shfl_xor(acc[0], 1 << s);
+
+  const int idx = lane & (V - 1);
+  const int r = idx / M, m = idx % M;
+  const int64_t f = feat0 + r;
+  if (lane < V && f < a.n && m < a.rows) {
+    float v = acc[0];
+    if (a.bias) v += ld16<BF16>(a.bias + f * 2);
+    if (a.res) v = rnd16<BF16>(v) + ld16<BF16>(a.res + m * a.r_sr + f * 2);
+    *(uint16_t*)(a.y + m * a.y_sr + f * 2) = st16<BF16>(v);
+  }
+}
+
+template <bool BF16, int M>
+void launch_rows(LinArgs a, int R, hipStream_t stream) {
+  const int64_t waves = (a.n + R - 1) / R;
+  const dim3 grid((unsigned)((waves + kLinThreads / 64 - 1) / (kLinThreads / 64))), block(kLinThreads);
+  const int cap = (M == 8 ? kLinLdsBytes8 : kLinLdsBytes) / (2 * M) / 8 * 8;
+  a.chunk = a.k < cap ? a.k : cap;
+  const size_t lds = (size_t)M * a.chunk * 2;
+  if (R == 4) hipLaunchKernelGGL((linear_rows_kernel<BF16, M, 4>), grid, block, lds, stream, a);
+  else if (R == 2) hipLaunchKernelGGL((linear_rows_kernel<BF16, M, 2>), grid, block, lds, stream, a);
+  else hipLaunchKernelGGL((linear_rows_kernel<BF16, M, 1>), grid, block, lds, stream, a);
+}
+
+template <bool BF16>
+void launch(const LinArgs& a, hipStream_t stream) {
+  // Features per wave: more of them re-use each activation chunk read from LDS (and shrink the share of the
+  // LDS staging, which every workgroup repeats), fewer of them give more waves to a small matrix.
+  const int m = a.rows <= 1 ? 1 : a.rows <= 2 ? 2 : a.rows <= 4 ? 4 : 8;
+  int R = (a.n >= 32768) ? 4 : (a.n >= 12288) ? 2 : 1;
+  if (m >= 4 && R < 2) R = 2;
+  if (m == 8) R = 4;
+  switch (m) {
+    case 1: launch_rows<BF16, 1>(a, R, stream); break;
+    case 2: launch_rows<BF16, 2>(a, R, stream); break;
+    case 4: launch_rows<BF16, 4>(a, R, stream); break;
+    default: launch_rows<BF16, 8>(a, R, stream); break;
+  }
+}
+
+}  // namespace
+}  // namespace sq
+
+using namespace sq;
+
+extern "C" int sq_linear_rows(const DLTensor* x, const DLTensor* weight, const DLTensor* bias, const DLTensor* residual,
+                              DLTensor* out, void* stream) {
+  const char* fn = "sq_linear_rows";
+  SQ_REQUIRE(x && weight && out, SQ_EINVAL, "%s: null tensor argument", fn);
+  int rc;
+  if ((rc = check_tensor(x, "x", 2, x->device.device_id))) return rc;
+  const int dev = x->device.device_id;
+  const DType dt = dtype_of(x);
+  SQ_REQUIRE(dt == DType::BF16 || dt == DType::F16, SQ_EDTYPE, "%s: x must be bf16 or fp16", fn);
+  const int64_t M = x->shape[0], K = x->shape[1];
+  SQ_REQUIRE(M >= 1 && M <= kLinMaxRows, SQ_EUNSUPPORTED, "%s: x must have 1 to %d rows (got %lld); larger products belong to a GEMM", fn,
+             kLinMaxRows, (long long)M);
+  SQ_REQUIRE(K > 0 && K % 8 == 0, SQ_EUNSUPPORTED, "%s: the inner dimension must be a positive multiple of 8 (got %lld)", fn, (long long)K);
+  if ((rc = check_tensor(weight, "weight", 2, dev))) return rc;
+  const int64_t N = weight->shape[0];
+  SQ_REQUIRE(dtype_of(weight) == dt, SQ_EDTYPE, "%s: weight must have x's dtype", fn);
+  SQ_REQUIRE(N > 0 && N < (1ll << 31) && weight->shape[1] == K, SQ_ESHAPE, "%s: weight must be [N, %lld] (got [%lld, %lld])", fn, (long long)K,
+             (long long)N, (long long)weight->shape[1]);
+  if ((rc = check_tensor(out, "out", 2, dev))) return rc;
+  SQ_REQUIRE(dtype_of(out) == dt && out->shape[0] == M && out->shape[1] == N, SQ_ESHAPE, "%s: out must be [%lld, %lld] of x's dtype", fn,
+             (long long)M, (long long)N);
+  SQ_REQUIRE(stride_of(x, 1) == 1 && stride_of(weight, 1) == 1 && stride_of(out, 1) == 1, SQ_ESHAPE, "%s: the last dimension must be contiguous", fn);
+  SQ_REQUIRE((stride_of(x, 0) % 8 == 0 || M == 1) && (stride_of(weight, 0) % 8 == 0 || N == 1), SQ_ESHAPE, "%s: rows of x and weight must be 16-byte aligned",
+             fn);
+  SQ_REQUIRE(((uintptr_t)data_of(x) % 16 == 0) && ((uintptr_t)data_of(weight) % 16 == 0), SQ_ESHAPE, "%s: x and weight must be 16-byte aligned", fn);
+  if (bias) {
+    if ((rc = check_tensor(bias, "bias", 1, dev))) return rc;
+    SQ_REQUIRE(dtype_of(bias) == dt && bias->shape[0] == N && stride_of(bias, 0) == 1, SQ_ESHAPE, "%s: bias must be a contiguous [%lld] of x's dtype", fn,
+               (long long)N);
+  }
+  if (residual) {
+    if ((rc = check_tensor(residual, "residual", 2, dev))) return rc;
+    SQ_REQUIRE(dtype_of(residual) == dt && residual->shape[0] == M && residual->shape[1] == N && stride_of(residual, 1) == 1, SQ_ESHAPE,
+               "%s: residual must be [%lld, %lld] of x's dtype with a contiguous last dimension", fn, (long long)M, (long long)N);
+  }
+  int cur = -1;
+  SQ_HIP(hipGetDevice(&cur));
+  SQ_REQUIRE(cur == dev, SQ_EDEVICE, "%s: tensors live on device %d but the current device is %d", fn, dev, cur);
+  LinArgs a;
+  a.x = data_of(x);
+  a.w = data_of(weight);
+  a.bias = bias ? data_of(bias) : nullptr;
+  a.res = residual ? data_of(residual) : nullptr;
+  a.y = data_of(out);
+  a.x_sr = stride_of(x, 0) * 2;
+  a.w_sr = stride_of(weight, 0) * 2;
+  a.r_sr = residual ? stride_of(residual, 0) * 2 : 0;
+  a.y_sr = stride_of(out, 0) * 2;
+  a.rows = (int)M;
+  a.n = (int)N;
+  a.k = (int)K;
+  if (dt == DType::BF16) launch<true>(a, (hipStream_t)stream);
+  else launch<false>(a, (hipStream_t)stream);
+  SQ_HIP(hipGetLastError());
+  return SQ_OK;
+}

@@ -107,13 +107,10 @@ class LLM:
         attn_out = layer.decode_attention(query_states, key_states, value_states, None)
         if isinstance(attn_out, tuple):   # the slot `process_model(..., patch_decode=True)` binds returns a 1-tuple (LLM.py:105)
             attn_out = attn_out[0]
-        hidden_states = self.wo(attn_out, layer, bsz, seq_len, dim)
-        hidden_states = residual + hidden_states
-        residual = hidden_states
-        hidden_states = self.layernorm(hidden_states, layer.post_attention_layernorm_variance_epsilon,
+        residual = self.wo(attn_out, layer, bsz, seq_len, dim, residual=residual)   # residual + wo(...)
+        hidden_states = self.layernorm(residual, layer.post_attention_layernorm_variance_epsilon,
                                        layer.post_attention_layernorm_weight)
-        hidden_states = self.mlp(hidden_states, layer)
-        return residual + hidden_states
+        return self.mlp(hidden_states, layer, residual=residual)                     # residual + mlp(...)
 
     # ------------------------------------------------------------------ whole model
     def prefill_forward(self, inputs_ids):

@@ -17,7 +17,7 @@ from ..cache_hub.flash_attn_cache import flash_attn_cache
 from ..sqattn.attn_triton import attn_causal
 from ..sqattn.attn_triton_decode import attn_decode
 from .LLM import LLM
-from .utils import apply_rope_with_cos_sin_cache_inplace, rmsnorm, silu_and_mul, yarn_cos_sin_cache
+from .utils import apply_rope_with_cos_sin_cache_inplace, linear, rmsnorm, silu_and_mul, yarn_cos_sin_cache
 
 
 @dataclass
@@ -189,21 +189,22 @@ class QwenModel(LLM):
         return torch.nn.functional.embedding(inputs_id, self.embed_tokens)
 
     def lm(self, hidden_states):
-        return torch.nn.functional.linear(hidden_states, self.lm_head).float()
+        return linear(hidden_states, self.lm_head).float()
 
     def wqkv(self, hidden_states, layer):
         """qwen.py:302-312: one fused projection, split into views (no copies)."""
-        qkv = torch.nn.functional.linear(hidden_states, layer.wqkv, layer.bqkv)
+        qkv = linear(hidden_states, layer.wqkv, layer.bqkv)
         kv = self.hidden_size // self.num_key_value_groups
         return qkv.split([self.hidden_size, kv, kv], dim=-1)
 
-    def wo(self, hidden_states, layer, bsz, seq_len, dim):
-        return torch.nn.functional.linear(hidden_states.reshape(bsz, seq_len, dim), layer.wo)
+    def wo(self, hidden_states, layer, bsz, seq_len, dim, residual=None):
+        """qwen.py:314-317.  With `residual` the caller's `residual + wo(...)` is part of the same pass (same values)."""
+        return linear(hidden_states.reshape(bsz, seq_len, dim), layer.wo, None, residual)
 
-    def mlp(self, hidden_states, layer):
-        """qwen.py:319-326."""
-        hidden_states = torch.nn.functional.linear(hidden_states, layer.gate_up_proj)
-        return torch.nn.functional.linear(silu_and_mul(hidden_states), layer.down_proj)
+    def mlp(self, hidden_states, layer, residual=None):
+        """qwen.py:319-326.  `residual` as in `wo`."""
+        hidden_states = linear(hidden_states, layer.gate_up_proj)
+        return linear(silu_and_mul(hidden_states), layer.down_proj, None, residual)
 
     def layernorm(self, hidden_states, epsilon, weight):
         """qwen.py:345-350."""

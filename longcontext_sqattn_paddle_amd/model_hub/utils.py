@@ -36,6 +36,33 @@ def silu_and_mul(hidden_states: torch.Tensor, out: Optional[torch.Tensor] = None
     return out
 
 
+LINEAR_ROWS_MAX = 8   # sq_linear_rows takes 1 to 8 activation rows; more is a GEMM
+
+
+def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None, residual: Optional[torch.Tensor] = None,
+           max_rows: int = 4) -> torch.Tensor:
+    """`x @ weight.T (+ bias) (+ residual)` over the last dimension of x, weight [N, K] (the matmuls of
+    model_hub/qwen.py:293-326).  Up to `max_rows` rows of x (a decode step) go through the weight-streaming HIP
+    kernel; longer activations (a prompt) are a GEMM and go to the BLAS library.  The kernel takes up to
+    LINEAR_ROWS_MAX rows; from five rows on the library's GEMM is as fast, hence the default."""
+    _need_gpu(x, weight)
+    K = x.shape[-1]
+    rows = x.numel() // K
+    if rows > min(max_rows, LINEAR_ROWS_MAX) or K % 8 or weight.stride(-1) != 1 or weight.stride(0) % 8 or weight.data_ptr() % 16:
+        y = torch.nn.functional.linear(x, weight, bias)
+        return y if residual is None else residual + y
+    x2 = x.reshape(rows, K)
+    if x2.stride(-1) != 1 or (rows > 1 and x2.stride(0) % 8) or x2.data_ptr() % 16:
+        x2 = x2.contiguous()
+    n = weight.shape[0]
+    out = torch.empty(*x.shape[:-1], n, dtype=x.dtype, device=x.device)
+    b = [N.dl(x2), N.dl(weight), N.dl(bias) if bias is not None else None,
+         N.dl(residual.reshape(rows, n)) if residual is not None else None, N.dl(out.view(rows, n))]
+    N.check(N.lib().sq_linear_rows(N.ptr(b[0]), N.ptr(b[1]), N.ptr(b[2]) if b[2] is not None else None,
+                                   N.ptr(b[3]) if b[3] is not None else None, N.ptr(b[4]), N.current_stream(x.device)))
+    return out
+
+
 def rmsnorm(x: torch.Tensor, weight: torch.Tensor, epsilon: float = 1e-6, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """`x * rsqrt(mean(x^2, -1) + epsilon) * weight` over the last dimension (utils.py:15-19)."""
     _need_gpu(x, weight)

@@ -1,7 +1,8 @@
 """CPU restatement of the reference's element-wise layer helpers -- TEST INFRASTRUCTURE ONLY.
 
 Followed reference code: model_hub/utils.py:4-13 (`silu_and_mul`), :15-19 (`rmsnorm`), :21-106
-(`apply_rope_with_cos_sin_cache_inplace`).  The reference evaluates them as chains of tensor operators on 16-bit
+(`apply_rope_with_cos_sin_cache_inplace`); model_hub/qwen.py:293-326 (the `linear` calls of lm, wqkv, wo, mlp) with
+the residual additions of model_hub/LLM.py:88-116.  The reference evaluates them as chains of tensor operators on 16-bit
 tensors; every operator computes in fp32 and rounds its result to the tensor dtype, and an operator that meets the
 fp32 cos/sin table yields fp32.  The functions below spell out those rounding points one by one.
 
@@ -10,7 +11,8 @@ Pinned in tests/test_oracle_layer.py against torch's own 16-bit CPU operators ev
 preservation and position 0 of the rotation, scale equivariance of the normalisation).  Parity unpinned: whether
 PaddlePaddle's kernels round exactly at these points (it cannot be run here); the order of the fp32 accumulation
 inside `mean` (taken as exact here, which differs from any order only when the sum sits on a rounding boundary of
-the 16-bit variance).
+the 16-bit variance).  `linear` is pinned against torch's CPU matmul (fp32 and 16-bit), closed forms (identity and
+all-ones weights) and linearity; unpinned: the accumulation order of the reference's GEMM (taken as exact here).
 """
 from __future__ import annotations
 
@@ -33,6 +35,20 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, epsilon: float = 1e-6) -> tor
     r = _r(1.0 / torch.sqrt(ve), dt)                                       # paddle.rsqrt
     norm_x = _r(xf * r, dt)                                                # x * rsqrt(...)
     return (norm_x * weight.float()).to(dt)                                # norm_x * weight
+
+
+def linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None, residual: torch.Tensor | None = None) -> torch.Tensor:
+    """qwen.py:296-325 on a 16-bit x [..., K], weight [N, K] (the reference passes `w.T` of the same storage): exact
+    products and sums, the bias added before the one rounding of the matmul operator; `residual + linear(...)`
+    (LLM.py:107, 115) is a second operator and rounds again."""
+    dt = x.dtype
+    y = x.double() @ weight.double().T
+    if bias is not None:
+        y = y + bias.double()
+    y = y.to(torch.float32).to(dt)
+    if residual is not None:
+        y = (residual.float() + y.float()).to(dt)
+    return y
 
 
 def silu_and_mul(hidden_states: torch.Tensor) -> torch.Tensor:

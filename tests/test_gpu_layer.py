@@ -127,3 +127,94 @@ def test_layer_kernel_argument_errors():
         silu_and_mul(torch.zeros(4, 24, dtype=torch.bfloat16, device=DEV))
     with pytest.raises(RuntimeError, match="no CPU path"):
         silu_and_mul(torch.zeros(4, 32, dtype=torch.bfloat16))
+
+
+# ------------------------------------------------------------------------------------------ decode-step projections
+def _linear_case(M, N, K, dtype, seed, bias, residual):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(M, K, generator=g).to(dtype)
+    w = (torch.randn(N, K, generator=g) * K ** -0.5).to(dtype)
+    b = torch.randn(N, generator=g).to(dtype) if bias else None
+    r = torch.randn(M, N, generator=g).to(dtype) if residual else None
+    return x, w, b, r
+
+
+def _check_linear(out, x, w, b, r):
+    """fp32 accumulation over K terms in the kernel's order against the oracle's exact sum: the two round to the
+    same 16-bit value except where the exact sum lies within the accumulation error of a rounding boundary, and then
+    they are neighbours.  Bound on the fp32 error: K * 2^-24 * sum|x_k w_k| (far above what is observed)."""
+    ref = OL.linear(x, w, b, r)
+    o, f = out.float().cpu(), ref.float()
+    eps = 2.0 ** -8 if x.dtype == torch.bfloat16 else 2.0 ** -11       # half a spacing, relative
+    mag = (x.double().abs() @ w.double().abs().T).float() + (b.float().abs() if b is not None else 0)
+    spacing = torch.maximum(o.abs(), f.abs()).clamp_min(2.0 ** -14) * 2 * eps
+    tol = spacing * 1.01 + mag * x.shape[1] * 2.0 ** -24
+    if r is not None:   # a neighbouring 16-bit product moves the sum by the product's spacing, whatever the sum's size
+        tol = tol + OL.linear(x, w, b).float().abs().clamp_min(2.0 ** -14) * 2 * eps * 1.01
+    assert bool(((o - f).abs() <= tol).all()), float(((o - f).abs() / spacing).max())
+    assert float((o == f).float().mean()) >= 0.98
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,N,K,bias,residual", [(1, 4608, 3584, True, False), (1, 3584, 3584, False, True),
+                                                 (1, 37888, 3584, False, False), (1, 3584, 18944, False, True),
+                                                 (2, 1000, 512, True, True), (3, 33, 8, True, False), (4, 777, 4104, False, True),
+                                                 (5, 2050, 1024, True, True), (8, 4608, 3584, True, False), (8, 515, 18944, False, True),
+                                                 (7, 1, 8, False, False), (1, 40000, 128, True, True)])
+def test_linear_rows_matches_oracle(dtype, M, N, K, bias, residual):
+    from longcontext_sqattn_paddle_amd.model_hub.utils import linear
+
+    print(f"case linear {dtype} M={M} N={N} K={K} bias={bias} residual={residual}", flush=True)
+    x, w, b, r = _linear_case(M, N, K, dtype, 7 * M + N + K, bias, residual)
+    out = linear(x.to(DEV), w.to(DEV), b.to(DEV) if bias else None, r.to(DEV) if residual else None, max_rows=8)
+    torch.cuda.synchronize()
+    assert out.shape == (M, N) and out.dtype == dtype
+    _check_linear(out, x, w, b, r)
+
+
+def test_linear_rows_views_batch_shapes_and_the_gemm_hand_over():
+    from longcontext_sqattn_paddle_amd import _native as NV
+    from longcontext_sqattn_paddle_amd.model_hub.utils import linear
+
+    g = torch.Generator().manual_seed(2)
+    # [batch, 1, hidden] activations as the decode step passes them; the residual keeps that shape
+    x = torch.randn(4, 1, 512, generator=g).bfloat16()
+    w = (torch.randn(768, 512, generator=g) / 22).bfloat16()
+    r = torch.randn(4, 1, 768, generator=g).bfloat16()
+    out = linear(x.to(DEV), w.to(DEV), None, r.to(DEV))
+    assert out.shape == (4, 1, 768)
+    _check_linear(out.view(4, 768), x.view(4, 512), w, None, r.view(4, 768))
+    # strided rows of x (columns of a wider tensor) and of the weight (a slice of a fused projection)
+    wide = torch.randn(3, 1024, generator=g).bfloat16()
+    wfused = (torch.randn(900, 1024, generator=g) / 22).bfloat16()
+    out = linear(wide.to(DEV)[:, 256:768], wfused.to(DEV)[100:612, 512:])
+    _check_linear(out, wide[:, 256:768], wfused[100:612, 512:], None, None)
+    # in place on the residual
+    rd = r.to(DEV).clone()
+    b = [NV.dl(x.to(DEV).view(4, 512)), NV.dl(w.to(DEV)), NV.dl(rd.view(4, 768))]
+    NV.check(NV.lib().sq_linear_rows(NV.ptr(b[0]), NV.ptr(b[1]), None, NV.ptr(b[2]), NV.ptr(b[2]), NV.current_stream(rd.device)))
+    torch.cuda.synchronize()
+    _check_linear(rd.view(4, 768), x.view(4, 512), w, None, r.view(4, 768))
+    # nine rows and more are a GEMM: the wrapper hands them to the BLAS library, the entry point refuses them
+    x9 = torch.randn(9, 512, generator=g).bfloat16()
+    out9 = linear(x9.to(DEV), w.to(DEV))
+    assert float((out9.float().cpu() - OL.linear(x9, w).float()).abs().max()) <= 2.0 ** -6
+    o9 = torch.empty(9, 768, dtype=torch.bfloat16, device=DEV)
+    b = [NV.dl(x9.to(DEV)), NV.dl(w.to(DEV)), NV.dl(o9)]
+    with pytest.raises(ValueError):
+        NV.check(NV.lib().sq_linear_rows(NV.ptr(b[0]), NV.ptr(b[1]), None, None, NV.ptr(b[2]), NV.current_stream(o9.device)))
+    # mismatched shapes and dtypes
+    o4 = torch.empty(4, 768, dtype=torch.bfloat16, device=DEV)
+    xd, wd = x.to(DEV).view(4, 512), w.to(DEV)
+    for args in [(xd, wd[:, :256].contiguous(), None, None, o4),             # inner dimensions differ
+                 (xd, wd, torch.zeros(700, dtype=torch.bfloat16, device=DEV), None, o4),   # bias length
+                 (xd, wd, None, o4[:3], o4),                                    # residual rows
+                 (xd, wd, None, None, torch.empty(4, 700, dtype=torch.bfloat16, device=DEV))]:
+        bb = [NV.dl(t) for t in args]
+        with pytest.raises(AssertionError):
+            NV.check(NV.lib().sq_linear_rows(*[NV.ptr(t) for t in bb], NV.current_stream(o4.device)))
+    bb = [NV.dl(xd), NV.dl(wd.half()), NV.dl(o4)]
+    with pytest.raises(ValueError):
+        NV.check(NV.lib().sq_linear_rows(NV.ptr(bb[0]), NV.ptr(bb[1]), None, None, NV.ptr(bb[2]), NV.current_stream(o4.device)))
+    with pytest.raises(RuntimeError):
+        linear(x, w)                                                            # CPU tensors: there is no host path

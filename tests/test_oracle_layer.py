@@ -94,3 +94,34 @@ def test_yarn_table_properties():
     t = torch.arange(40000.0)
     assert torch.allclose(long[:100, 0], torch.cos(t[:100] * inv[0]) * factor, atol=1e-5)
     assert torch.allclose(long[:, 63], torch.cos(t * inv[63] / 4.0) * factor, atol=1e-4)
+
+
+def test_linear_closed_forms_and_library_matmul():
+    g = torch.Generator().manual_seed(12)
+    for dt in (torch.bfloat16, torch.float16):
+        x = torch.randn(3, 64, generator=g).to(dt)
+        w = (torch.randn(40, 64, generator=g) / 8).to(dt)
+        b = torch.randn(40, generator=g).to(dt)
+        res = torch.randn(3, 40, generator=g).to(dt)
+        # identity weight returns x; with a bias, the 16-bit sum of the two
+        eye = torch.eye(64).to(dt)
+        assert torch.equal(OL.linear(x, eye), x)
+        assert torch.equal(OL.linear(x, eye, x[0]), (x.float() + x[0].float()).to(dt))
+        # an all-ones row sums the activations: exact in fp64, rounded once
+        ones = torch.ones(2, 64).to(dt)
+        assert torch.equal(OL.linear(x, ones)[:, 0], x.double().sum(-1).float().to(dt))
+        # the library's matmul (fp32 accumulation in some order): equal up to one 16-bit spacing of the result
+        lib = torch.nn.functional.linear(x.float(), w.float(), b.float())
+        got = OL.linear(x, w, b)
+        spacing = lib.abs().clamp_min(2.0 ** -14) * (2.0 ** -7 if dt == torch.bfloat16 else 2.0 ** -10)
+        fp32_noise = (x.float().abs() @ w.float().abs().T + b.float().abs()) * 64 * 2.0 ** -24   # where the sum cancels
+        assert bool(((got.float() - lib).abs() <= spacing + fp32_noise).all())
+        assert float((got == lib.to(dt)).float().mean()) > 0.97
+        # a transposed weight or a dropped bias would not survive this: row i of the weight alone
+        for i in (0, 17, 39):
+            assert torch.equal(OL.linear(x, w, b)[:, i], OL.linear(x, w[i:i + 1], b[i:i + 1])[:, 0])
+        # the residual is a second rounding, not part of the first
+        two_step = (res.float() + OL.linear(x, w, b).float()).to(dt)
+        assert torch.equal(OL.linear(x, w, b, res), two_step)
+        one_step = (x.double() @ w.double().T + b.double() + res.double()).float().to(dt)
+        assert not torch.equal(two_step, one_step) or dt == torch.float16
