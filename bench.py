@@ -193,6 +193,60 @@ def time_layer_kernels(torch, N, iters=10):
     return out
 
 
+def time_decode_projections(torch, rows=1, iters=40, rounds=5):
+    """The matmuls of one decode step at Qwen2.5-7B's sizes through `sq_linear_rows` (one activation row: batch 1),
+    each with the BLAS library's time for the same product beside it.  Every call reads another copy of the weight
+    (about 1.2 GB of copies per shape), so the weights stream from HBM as they do across the 28 layers of a step."""
+    from longcontext_sqattn_paddle_amd.model_hub import utils as U
+
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(9)
+    shapes = [("wqkv", 4608, 3584, True, False), ("wo", 3584, 3584, False, True), ("gate_up_proj", 37888, 3584, False, False),
+              ("down_proj", 3584, 18944, False, True), ("lm_head", 152064, 3584, False, False)]
+    out = {}
+    for name, n, k, has_bias, has_res in shapes:
+        copies = max(2, min(12, int(1.2e9 // (n * k * 2))))
+        ws = [(torch.randn(n, k, device=dev, generator=g) * k ** -0.5).bfloat16() for _ in range(copies)]
+        x = torch.randn(rows, k, device=dev, generator=g).bfloat16()
+        bias = torch.randn(n, device=dev, generator=g).bfloat16() if has_bias else None
+        res = torch.randn(rows, n, device=dev, generator=g).bfloat16() if has_res else None
+
+        def blas(w):
+            y = torch.nn.functional.linear(x, w, bias)
+            return y if res is None else res + y
+
+        def timed(fn):
+            """`iters` calls captured into one HIP graph and replayed: kernel time without the host's launch cost,
+            as in the graph-replayed decode step."""
+            for i in range(3):
+                fn(ws[i % copies])
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                for i in range(iters):
+                    fn(ws[i % copies])
+            graph.replay()
+            torch.cuda.synchronize()
+            samples = []
+            for _ in range(rounds):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                graph.replay()
+                e1.record()
+                torch.cuda.synchronize()
+                samples.append(e0.elapsed_time(e1) / iters * 1e3)
+            del graph
+            return sorted(samples)[len(samples) // 2]
+
+        y = U.linear(x, ws[0], bias, res)
+        ref = blas(ws[0])
+        assert float((y.float() - ref.float()).abs().max()) <= 2.0 ** -5 * float(ref.float().abs().max())
+        out[name] = (timed(lambda w: U.linear(x, w, bias, res)), timed(blas), float(n) * k * 2)
+        del ws
+        torch.cuda.empty_cache()
+    return out
+
+
 def time_model_layers(torch, N):
     """Two decoder layers of Qwen2.5-7B's shapes (random weights) through the runtime mirror: prompt of N tokens
     (embedding, 2 x layer_prefill, final norm, lm head), then decode steps against the N-token cache."""
@@ -573,6 +627,14 @@ def main():
                          "frac_of_hbm_peak": round(nbytes / us / 1e3 / PEAK_HBM_GBS, 4), "bytes": nbytes}
             log(f"[bench] layer kernel {name}: {us:.0f} us, {nbytes / us / 1e3:.0f} GB/s")
         result["layer_kernels"] = lay
+        proj = {}
+        for name, (us, blas_us, nbytes) in time_decode_projections(torch).items():
+            proj[name] = {"us_per_call": round(us, 1), "GB_per_s": round(nbytes / us / 1e3, 1),
+                          "frac_of_hbm_peak": round(nbytes / us / 1e3 / PEAK_HBM_GBS, 4), "bytes": nbytes, "blas_us_per_call": round(blas_us, 1)}
+            log(f"[bench] decode projection {name}: {us:.1f} us, {nbytes / us / 1e3:.0f} GB/s (BLAS library: {blas_us:.1f} us)")
+        proj["note"] = ("one activation row (batch 1), bf16, bias / residual as in the decode step; 40 calls replayed from one HIP "
+                        "graph, each on another copy of the weight")
+        result["decode_projections"] = proj
     if not args.no_model:
         ml = time_model_layers(torch, N)
         result["model_layers"] = {k: round(v, 3) for k, v in ml.items()}
