@@ -29,6 +29,7 @@
  *   sq_rope                   model_hub/utils.py:21-106 (apply_rope_with_cos_sin_cache_inplace; caller qwen.py:352-367)
  *   sq_linear_rows            the matmuls of a decode step: model_hub/qwen.py:293-300 (lm), :302-312 (wqkv), :314-317 (wo),
  *                             :319-326 (mlp), called from model_hub/LLM.py:88-116 (layer_decode)
+ *   sq_linear_rows_silu_and_mul  model_hub/qwen.py:320-324 (gate_up_proj and silu_and_mul of mlp) on a decode step
  *   sq_fake_quant_prepass     sqattn/attn_replacer.py:334-365 (GQA expand, key centring and the five fake-quant
  *                             passes of mp_triton_wrapper's closure), sqattn/fake_quant.py:24-58, 98-125
  */
@@ -249,6 +250,15 @@ int sq_silu_and_mul(const DLTensor* x, DLTensor* out, void* stream);
  */
 int sq_linear_rows(const DLTensor* x, const DLTensor* weight, const DLTensor* bias, const DLTensor* residual,
                    DLTensor* out, void* stream);
+
+/*
+ * out = silu_and_mul(x . weight^T (+ bias)) for 1 to 8 rows of x: the first projection of the MLP and the activation
+ * behind it in one pass (model_hub/qwen.py:320-324 on a decode step's activation).  weight [2 I, K] = [gate | up] as
+ * the reference stores gate_up_proj, bias [2 I] or NULL, out [M, I] = up * (gate * sigmoid(gate)) with the values
+ * sq_linear_rows followed by sq_silu_and_mul give (the projection rounded to the tensor dtype, then the three
+ * rounded operators of the activation).  Other requirements as for sq_linear_rows.
+ */
+int sq_linear_rows_silu_and_mul(const DLTensor* x, const DLTensor* weight, const DLTensor* bias, DLTensor* out, void* stream);
 
 /*
  * Rotary position embedding of query [T, Hq * head_dim] and key [T, Hkv * head_dim] (T = batch * seq_len tokens)

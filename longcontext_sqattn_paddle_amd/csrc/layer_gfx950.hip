@@ -73,6 +73,13 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_kernel(NormArgs a) {
     const int ch = lane + c * 64;
     if (ch < chunks) v[c] = __builtin_nontemporal_load((const u32x4_t*)(xr + ch * 16));
   }
+  // (the weight does not depend on the row's sum: requested here, it arrives while the lanes fold)
+  u32x4_t wt[CHUNKS];
+#pragma unroll
+  for (int c = 0; c < CHUNKS; ++c) {
+    const int ch = lane + c * 64;
+    if (ch < chunks) wt[c] = *(const u32x4_t*)(a.w + ch * 16);
+  }
   float sum = 0.f;
 #pragma unroll
   for (int c = 0; c < CHUNKS; ++c) {
@@ -96,7 +103,7 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_kernel(NormArgs a) {
     if (ch < chunks) {
       float f[8], g[8];
       unpack8<BF16>(v[c], f);
-      unpack8<BF16>(*(const u32x4_t*)(a.w + ch * 16), g);
+      unpack8<BF16>(wt[c], g);
 #pragma unroll
       for (int e = 0; e < 8; ++e) f[e] = rnd<BF16>(f[e] * r) * g[e];
       __builtin_nontemporal_store(pack8<BF16>(f), (u32x4_t*)(orow + ch * 16));

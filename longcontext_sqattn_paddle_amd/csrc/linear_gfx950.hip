@@ -8,6 +8,10 @@
 // (v_dot2c_f32_bf16 / v_dot2c_f32_f16: fp32 accumulation), and the R x rows partial sums of the 64 lanes are folded
 // by a transposing butterfly.  Rounding points: the fp32 sum plus the bias is rounded once to the tensor dtype (what
 // a GEMM with a bias epilogue gives); a residual is then added as a second tensor operator would (rounded again).
+// The gated form (sq_linear_rows_silu_and_mul) is the first projection of the MLP together with the activation that
+// follows it (model_hub/qwen.py:320-324): a wave owns features f and f + N/2 of the [gate | up] weight, so both
+// halves of an output pair end in one wave and out[f] = up * (gate * sigmoid(gate)) leaves with the rounding points
+// of the stand-alone pass (the product, sigmoid and gate * sigmoid each rounded to the tensor dtype).
 #include "common.hpp"
 
 namespace sq {
@@ -56,21 +60,33 @@ __device__ __forceinline__ float rnd16(float x) {
   else return (float)(_Float16)x;
 }
 
+// x2 * (x1 * sigmoid(x1)) with sigmoid and x1 * sigmoid rounded to the tensor dtype: the formula of silu_mul_kernel
+// (same instructions, so the same bits; the caller rounds the last product)
+template <bool BF16>
+__device__ __forceinline__ float silu_mul_elem(float x1, float x2) {
+  const float sg = rnd16<BF16>(__builtin_amdgcn_rcpf(1.0f + __expf(-x1)));
+  return x2 * rnd16<BF16>(x1 * sg);
+}
+
 // M = activation rows the registers are sized for (1, 2, 4, 8), R = output features per wave (1, 2, 4),
 // U = 16-byte weight loads per feature a lane keeps in flight (eight loads per lane in all).
-template <bool BF16, int M, int R>
+// GATED: the wave's R features are R/2 pairs (f, f + n/2) and the output has n/2 columns.
+template <bool BF16, int M, int R, bool GATED = false>
 __global__ __launch_bounds__(kLinThreads) void linear_rows_kernel(LinArgs a) {
+  static_assert(!GATED || R % 2 == 0, "a gated wave owns whole pairs");
+  constexpr int RO = GATED ? R / 2 : R;   // output columns per wave
+  const int n_out = GATED ? a.n / 2 : a.n;
   constexpr int U = 8 / R;
   extern __shared__ u32x4_t xs[];   // [M][chunk / 8]
   const int kLinChunk = a.chunk, row16 = a.chunk / 8;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int64_t feat0 = ((int64_t)blockIdx.x * (kLinThreads / 64) + wave) * R;
-  const bool live = feat0 < a.n;
+  const int64_t feat0 = ((int64_t)blockIdx.x * (kLinThreads / 64) + wave) * RO;
+  const bool live = feat0 < n_out;
   const char* wrow[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
-    const int64_t f = (feat0 + r < a.n) ? feat0 + r : (int64_t)a.n - 1;   // features past the end re-read the last one
-    wrow[r] = a.w + f * a.w_sr;
+    const int64_t col = (feat0 + r % RO < n_out) ? feat0 + r % RO : (int64_t)n_out - 1;   // columns past the end re-read the last one
+    wrow[r] = a.w + (col + (r >= RO ? n_out : 0)) * a.w_sr;                               // second half of a pair: feature col + n/2
   }
   float acc[R * M];
 #pragma unroll
@@ -143,40 +159,51 @@ __global__ __launch_bounds__(kLinThreads) void linear_rows_kernel(LinArgs a) {
 
   const int idx = lane & (V - 1);
   const int r = idx / M, m = idx % M;
-  const int64_t f = feat0 + r;
-  if (lane < V && f < a.n && m < a.rows) {
-    float v = acc[0];
+  const int64_t col = feat0 + r % RO;
+  float v = acc[0];
+  if constexpr (GATED) {
+    const int64_t f = (col < n_out ? col : (int64_t)n_out - 1) + (r >= RO ? n_out : 0);
     if (a.bias) v += ld16<BF16>(a.bias + f * 2);
-    if (a.res) v = rnd16<BF16>(v) + ld16<BF16>(a.res + m * a.r_sr + f * 2);
-    *(uint16_t*)(a.y + m * a.y_sr + f * 2) = st16<BF16>(v);
+    v = rnd16<BF16>(v);                                    // the projection's own rounding
+    const float up = __shfl(v, (lane + RO * M) & 63);      // lane idx + (R/2) M holds the pair's second half for the same row
+    if (lane < RO * M && col < n_out && m < a.rows) *(uint16_t*)(a.y + m * a.y_sr + col * 2) = st16<BF16>(silu_mul_elem<BF16>(v, up));
+  } else {
+    if (lane < V && col < a.n && m < a.rows) {
+      if (a.bias) v += ld16<BF16>(a.bias + col * 2);
+      if (a.res) v = rnd16<BF16>(v) + ld16<BF16>(a.res + m * a.r_sr + col * 2);
+      *(uint16_t*)(a.y + m * a.y_sr + col * 2) = st16<BF16>(v);
+    }
   }
 }
 
 template <bool BF16, int M>
-void launch_rows(LinArgs a, int R, hipStream_t stream) {
-  const int64_t waves = (a.n + R - 1) / R;
+void launch_rows(LinArgs a, int R, bool gated, hipStream_t stream) {
+  const int64_t waves = gated ? (a.n / 2 + R / 2 - 1) / (R / 2) : (a.n + R - 1) / R;
   const dim3 grid((unsigned)((waves + kLinThreads / 64 - 1) / (kLinThreads / 64))), block(kLinThreads);
   const int cap = (M == 8 ? kLinLdsBytes8 : kLinLdsBytes) / (2 * M) / 8 * 8;
   a.chunk = a.k < cap ? a.k : cap;
   const size_t lds = (size_t)M * a.chunk * 2;
-  if (R == 4) hipLaunchKernelGGL((linear_rows_kernel<BF16, M, 4>), grid, block, lds, stream, a);
+  if (gated) {
+    if (R == 4) hipLaunchKernelGGL((linear_rows_kernel<BF16, M, 4, true>), grid, block, lds, stream, a);
+    else hipLaunchKernelGGL((linear_rows_kernel<BF16, M, 2, true>), grid, block, lds, stream, a);
+  } else if (R == 4) hipLaunchKernelGGL((linear_rows_kernel<BF16, M, 4>), grid, block, lds, stream, a);
   else if (R == 2) hipLaunchKernelGGL((linear_rows_kernel<BF16, M, 2>), grid, block, lds, stream, a);
   else hipLaunchKernelGGL((linear_rows_kernel<BF16, M, 1>), grid, block, lds, stream, a);
 }
 
 template <bool BF16>
-void launch(const LinArgs& a, hipStream_t stream) {
+void launch(const LinArgs& a, bool gated, hipStream_t stream) {
   // Features per wave: more of them re-use each activation chunk read from LDS (and shrink the share of the
   // LDS staging, which every workgroup repeats), fewer of them give more waves to a small matrix.
   const int m = a.rows <= 1 ? 1 : a.rows <= 2 ? 2 : a.rows <= 4 ? 4 : 8;
   int R = (a.n >= 32768) ? 4 : (a.n >= 12288) ? 2 : 1;
-  if (m >= 4 && R < 2) R = 2;
+  if ((m >= 4 || gated) && R < 2) R = 2;
   if (m == 8) R = 4;
   switch (m) {
-    case 1: launch_rows<BF16, 1>(a, R, stream); break;
-    case 2: launch_rows<BF16, 2>(a, R, stream); break;
-    case 4: launch_rows<BF16, 4>(a, R, stream); break;
-    default: launch_rows<BF16, 8>(a, R, stream); break;
+    case 1: launch_rows<BF16, 1>(a, R, gated, stream); break;
+    case 2: launch_rows<BF16, 2>(a, R, gated, stream); break;
+    case 4: launch_rows<BF16, 4>(a, R, gated, stream); break;
+    default: launch_rows<BF16, 8>(a, R, gated, stream); break;
   }
 }
 
@@ -185,9 +212,9 @@ void launch(const LinArgs& a, hipStream_t stream) {
 
 using namespace sq;
 
-extern "C" int sq_linear_rows(const DLTensor* x, const DLTensor* weight, const DLTensor* bias, const DLTensor* residual,
-                              DLTensor* out, void* stream) {
-  const char* fn = "sq_linear_rows";
+namespace {
+int linear_rows(const char* fn, bool gated, const DLTensor* x, const DLTensor* weight, const DLTensor* bias, const DLTensor* residual,
+                DLTensor* out, void* stream) {
   SQ_REQUIRE(x && weight && out, SQ_EINVAL, "%s: null tensor argument", fn);
   int rc;
   if ((rc = check_tensor(x, "x", 2, x->device.device_id))) return rc;
@@ -204,8 +231,10 @@ extern "C" int sq_linear_rows(const DLTensor* x, const DLTensor* weight, const D
   SQ_REQUIRE(N > 0 && N < (1ll << 31) && weight->shape[1] == K, SQ_ESHAPE, "%s: weight must be [N, %lld] (got [%lld, %lld])", fn, (long long)K,
              (long long)N, (long long)weight->shape[1]);
   if ((rc = check_tensor(out, "out", 2, dev))) return rc;
-  SQ_REQUIRE(dtype_of(out) == dt && out->shape[0] == M && out->shape[1] == N, SQ_ESHAPE, "%s: out must be [%lld, %lld] of x's dtype", fn,
-             (long long)M, (long long)N);
+  SQ_REQUIRE(!gated || N % 2 == 0, SQ_ESHAPE, "%s: the weight must hold two halves of equal size (got %lld rows)", fn, (long long)N);
+  const int64_t NO = gated ? N / 2 : N;
+  SQ_REQUIRE(dtype_of(out) == dt && out->shape[0] == M && out->shape[1] == NO, SQ_ESHAPE, "%s: out must be [%lld, %lld] of x's dtype", fn,
+             (long long)M, (long long)NO);
   SQ_REQUIRE(stride_of(x, 1) == 1 && stride_of(weight, 1) == 1 && stride_of(out, 1) == 1, SQ_ESHAPE, "%s: the last dimension must be contiguous", fn);
   SQ_REQUIRE((stride_of(x, 0) % 8 == 0 || M == 1) && (stride_of(weight, 0) % 8 == 0 || N == 1), SQ_ESHAPE, "%s: rows of x and weight must be 16-byte aligned",
              fn);
@@ -236,8 +265,18 @@ extern "C" int sq_linear_rows(const DLTensor* x, const DLTensor* weight, const D
   a.rows = (int)M;
   a.n = (int)N;
   a.k = (int)K;
-  if (dt == DType::BF16) launch<true>(a, (hipStream_t)stream);
-  else launch<false>(a, (hipStream_t)stream);
+  if (dt == DType::BF16) launch<true>(a, gated, (hipStream_t)stream);
+  else launch<false>(a, gated, (hipStream_t)stream);
   SQ_HIP(hipGetLastError());
   return SQ_OK;
+}
+}  // namespace
+
+extern "C" int sq_linear_rows(const DLTensor* x, const DLTensor* weight, const DLTensor* bias, const DLTensor* residual,
+                              DLTensor* out, void* stream) {
+  return linear_rows("sq_linear_rows", false, x, weight, bias, residual, out, stream);
+}
+
+extern "C" int sq_linear_rows_silu_and_mul(const DLTensor* x, const DLTensor* weight, const DLTensor* bias, DLTensor* out, void* stream) {
+  return linear_rows("sq_linear_rows_silu_and_mul", true, x, weight, bias, nullptr, out, stream);
 }

@@ -17,7 +17,7 @@ from ..cache_hub.flash_attn_cache import flash_attn_cache
 from ..sqattn.attn_triton import attn_causal
 from ..sqattn.attn_triton_decode import attn_decode
 from .LLM import LLM
-from .utils import apply_rope_with_cos_sin_cache_inplace, linear, rmsnorm, silu_and_mul, yarn_cos_sin_cache
+from .utils import apply_rope_with_cos_sin_cache_inplace, linear, linear_silu_and_mul, rmsnorm, yarn_cos_sin_cache
 
 
 @dataclass
@@ -203,8 +203,7 @@ class QwenModel(LLM):
 
     def mlp(self, hidden_states, layer, residual=None):
         """qwen.py:319-326.  `residual` as in `wo`."""
-        hidden_states = linear(hidden_states, layer.gate_up_proj)
-        return linear(silu_and_mul(hidden_states), layer.down_proj, None, residual)
+        return linear(linear_silu_and_mul(hidden_states, layer.gate_up_proj), layer.down_proj, None, residual)
 
     def layernorm(self, hidden_states, epsilon, weight):
         """qwen.py:345-350."""

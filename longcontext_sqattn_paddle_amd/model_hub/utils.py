@@ -63,6 +63,25 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
     return out
 
 
+def linear_silu_and_mul(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None, max_rows: int = 4) -> torch.Tensor:
+    """`silu_and_mul(x @ weight.T (+ bias))`, weight [2 I, K] = [gate | up] -> [..., I]: the first half of `mlp`
+    (model_hub/qwen.py:320-324).  Up to `max_rows` rows go through one HIP kernel whose waves own both halves of an
+    output pair (same values as `silu_and_mul(linear(x, weight, bias))`); longer activations take that route."""
+    _need_gpu(x, weight)
+    K = x.shape[-1]
+    rows = x.numel() // K
+    n = weight.shape[0]
+    if rows > min(max_rows, LINEAR_ROWS_MAX) or K % 8 or n % 2 or weight.stride(-1) != 1 or weight.stride(0) % 8 or weight.data_ptr() % 16:
+        return silu_and_mul(torch.nn.functional.linear(x, weight, bias))
+    x2 = x.reshape(rows, K)
+    if x2.stride(-1) != 1 or (rows > 1 and x2.stride(0) % 8) or x2.data_ptr() % 16:
+        x2 = x2.contiguous()
+    out = torch.empty(*x.shape[:-1], n // 2, dtype=x.dtype, device=x.device)
+    b = [N.dl(x2), N.dl(weight), N.dl(bias), N.dl(out.view(rows, n // 2))]
+    N.check(N.lib().sq_linear_rows_silu_and_mul(*[N.ptr(t) for t in b], N.current_stream(x.device)))
+    return out
+
+
 def rmsnorm(x: torch.Tensor, weight: torch.Tensor, epsilon: float = 1e-6, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """`x * rsqrt(mean(x^2, -1) + epsilon) * weight` over the last dimension (utils.py:15-19)."""
     _need_gpu(x, weight)

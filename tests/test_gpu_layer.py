@@ -218,3 +218,40 @@ def test_linear_rows_views_batch_shapes_and_the_gemm_hand_over():
         NV.check(NV.lib().sq_linear_rows(NV.ptr(bb[0]), NV.ptr(bb[1]), None, None, NV.ptr(bb[2]), NV.current_stream(o4.device)))
     with pytest.raises(RuntimeError):
         linear(x, w)                                                            # CPU tensors: there is no host path
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,I,K,bias", [(1, 18944, 3584, False), (1, 2000, 512, True), (2, 9000, 1024, True), (3, 333, 4104, False),
+                                        (4, 8192, 256, True), (8, 515, 2048, False), (5, 1, 8, True), (1, 7, 24, False)])
+def test_gated_projection_equals_projection_then_silu_and_mul(dtype, M, I, K, bias):
+    """One kernel for gate_up_proj and the activation: the bits of the two separate passes, each of which is checked
+    against the oracle above."""
+    from longcontext_sqattn_paddle_amd import _native as NV
+    from longcontext_sqattn_paddle_amd.model_hub.utils import linear, linear_silu_and_mul, silu_and_mul
+
+    print(f"case gated linear {dtype} M={M} I={I} K={K} bias={bias}", flush=True)
+    g = torch.Generator().manual_seed(M + I + K)
+    x = torch.randn(M, K, generator=g).to(dtype).to(DEV)
+    w = (torch.randn(2 * I, K, generator=g) * 2 * K ** -0.5).to(dtype).to(DEV)
+    b = torch.randn(2 * I, generator=g).to(dtype).to(DEV) if bias else None
+    fused = linear_silu_and_mul(x, w, b, max_rows=8)
+    torch.cuda.synchronize()
+    assert fused.shape == (M, I) and fused.dtype == dtype
+    if I % 8 == 0:   # (the stand-alone activation pass takes whole 16-byte steps)
+        two = silu_and_mul(linear(x, w, b, max_rows=8))
+        assert torch.equal(fused.view(torch.int16), two.view(torch.int16))
+    ref = OL.silu_and_mul(OL.linear(x.cpu(), w.cpu(), b.cpu() if bias else None))
+    assert float((fused.float().cpu() - ref.float()).abs().max()) <= 2.0 ** -6 * max(1.0, float(ref.float().abs().max()))
+    # an odd number of weight rows has no two halves; an output of the full width is the plain projection's
+    o = torch.empty(M, 2 * I, dtype=dtype, device=DEV)
+    bb = [NV.dl(x), NV.dl(w), NV.dl(o)]
+    with pytest.raises(AssertionError):
+        NV.check(NV.lib().sq_linear_rows_silu_and_mul(NV.ptr(bb[0]), NV.ptr(bb[1]), None, NV.ptr(bb[2]), NV.current_stream(o.device)))
+    if I > 1:
+        bb = [NV.dl(x), NV.dl(w[:2 * I - 1]), NV.dl(torch.empty(M, I, dtype=dtype, device=DEV))]
+        with pytest.raises(AssertionError):
+            NV.check(NV.lib().sq_linear_rows_silu_and_mul(NV.ptr(bb[0]), NV.ptr(bb[1]), None, NV.ptr(bb[2]), NV.current_stream(o.device)))
+    # more rows than the kernel takes: the wrapper runs the two passes
+    if I % 8 == 0:
+        x9 = torch.randn(9, K, generator=g).to(dtype).to(DEV)
+        assert torch.equal(linear_silu_and_mul(x9, w, b), silu_and_mul(torch.nn.functional.linear(x9, w, b)))
