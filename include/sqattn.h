@@ -30,6 +30,7 @@
  *   sq_linear_rows            the matmuls of a decode step: model_hub/qwen.py:293-300 (lm), :302-312 (wqkv), :314-317 (wo),
  *                             :319-326 (mlp), called from model_hub/LLM.py:88-116 (layer_decode)
  *   sq_linear_rows_silu_and_mul  model_hub/qwen.py:320-324 (gate_up_proj and silu_and_mul of mlp) on a decode step
+ *   sq_linear_rows_rope       model_hub/qwen.py:302-312 (wqkv) + :352-379 (rotary embedding of q and k) on a decode step
  *   sq_fake_quant_prepass     sqattn/attn_replacer.py:334-365 (GQA expand, key centring and the five fake-quant
  *                             passes of mp_triton_wrapper's closure), sqattn/fake_quant.py:24-58, 98-125
  */
@@ -259,6 +260,18 @@ int sq_linear_rows(const DLTensor* x, const DLTensor* weight, const DLTensor* bi
  * rounded operators of the activation).  Other requirements as for sq_linear_rows.
  */
 int sq_linear_rows_silu_and_mul(const DLTensor* x, const DLTensor* weight, const DLTensor* bias, DLTensor* out, void* stream);
+
+/*
+ * out = x . weight^T (+ bias) with the rotary embedding applied to the first rope_features output features, for 1 to 8
+ * rows of x: the fused q/k/v projection of a decode step and the rotation of its q and k parts in one pass
+ * (model_hub/qwen.py:302-312 wqkv, :352-379 apply_rotary_pos_emb / position_embedd).  The first rope_features
+ * features are whole heads of head_dim; feature i < head_dim / 2 of a head is rotated with feature i + head_dim / 2 by
+ * row position_ids[m] of cos_sin_cache (fp32 [max_position, head_dim], cos | sin), exactly as sq_rope rotates the
+ * rounded output of sq_linear_rows; the remaining features (v) are the plain projection.  position_ids: int32 or
+ * int64, one entry per row of x.  Other requirements as for sq_linear_rows.
+ */
+int sq_linear_rows_rope(const DLTensor* x, const DLTensor* weight, const DLTensor* bias, const DLTensor* position_ids,
+                        const DLTensor* cos_sin_cache, int32_t head_dim, int32_t rope_features, DLTensor* out, void* stream);
 
 /*
  * Rotary position embedding of query [T, Hq * head_dim] and key [T, Hkv * head_dim] (T = batch * seq_len tokens)

@@ -12,6 +12,10 @@
 // follows it (model_hub/qwen.py:320-324): a wave owns features f and f + N/2 of the [gate | up] weight, so both
 // halves of an output pair end in one wave and out[f] = up * (gate * sigmoid(gate)) leaves with the rounding points
 // of the stand-alone pass (the product, sigmoid and gate * sigmoid each rounded to the tensor dtype).
+// The rotary form (sq_linear_rows_rope) is the fused q/k/v projection together with the rotary embedding of its q
+// and k parts (model_hub/qwen.py:302-312, 352-379): a wave owns features i and i + head_dim/2 of one head, rotates
+// the pair by the position's cos/sin (fp32 products and sums without fused multiply-add, one rounding, as sq_rope
+// does) and stores both; the waves behind the rotated part produce plain features (v).
 #include "common.hpp"
 
 namespace sq {
@@ -33,7 +37,13 @@ struct LinArgs {
   int32_t rows;                     // rows of x actually present (<= M)
   int32_t n, k;
   int32_t chunk;   // elements of every activation row per LDS pass (a multiple of 8)
+  // rotary form only
+  const void* pos;       // [rows] int32 or int64
+  const float* table;    // [max_pos, head_dim]: cos | sin
+  int32_t pos_is_i64, max_pos, head_dim, rope_features;
 };
+
+enum { kModePlain = 0, kModeGated = 1, kModeRope = 2 };
 
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
 typedef __attribute__((ext_vector_type(2))) _Float16 f16x2_t;
@@ -70,24 +80,47 @@ __device__ __forceinline__ float silu_mul_elem(float x1, float x2) {
 
 // M = activation rows the registers are sized for (1, 2, 4, 8), R = output features per wave (1, 2, 4),
 // U = 16-byte weight loads per feature a lane keeps in flight (eight loads per lane in all).
-// GATED: the wave's R features are R/2 pairs (f, f + n/2) and the output has n/2 columns.
-template <bool BF16, int M, int R, bool GATED = false>
+// kModeGated: the wave's R features are R/2 pairs (f, f + n/2) and the output has n/2 columns.
+// kModeRope (R = 2): wave w < rope_features / 2 owns the pair (i, i + head_dim / 2) of a head, later waves two plain features.
+template <bool BF16, int M, int R, int MODE = kModePlain>
 __global__ __launch_bounds__(kLinThreads) void linear_rows_kernel(LinArgs a) {
+  constexpr bool GATED = MODE == kModeGated, ROPE = MODE == kModeRope;
   static_assert(!GATED || R % 2 == 0, "a gated wave owns whole pairs");
+  static_assert(!ROPE || R == 2, "a rotary wave owns one pair");
   constexpr int RO = GATED ? R / 2 : R;   // output columns per wave
   const int n_out = GATED ? a.n / 2 : a.n;
   constexpr int U = 8 / R;
   extern __shared__ u32x4_t xs[];   // [M][chunk / 8]
   const int kLinChunk = a.chunk, row16 = a.chunk / 8;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int64_t feat0 = ((int64_t)blockIdx.x * (kLinThreads / 64) + wave) * RO;
-  const bool live = feat0 < n_out;
+  int64_t feat0 = ((int64_t)blockIdx.x * (kLinThreads / 64) + wave) * RO;
   const char* wrow[R];
+  [[maybe_unused]] int64_t rope_f[2] = {0, 0};   // the two features of a rotary wave
+  [[maybe_unused]] bool paired = false;
+  [[maybe_unused]] int rope_i = 0;               // index of the pair inside its head
+  if constexpr (ROPE) {
+    const int64_t w = (int64_t)blockIdx.x * (kLinThreads / 64) + wave;
+    const int half = a.head_dim / 2;
+    paired = w < a.rope_features / 2;
+    if (paired) {
+      rope_i = (int)(w % half);
+      rope_f[0] = w / half * a.head_dim + rope_i;
+      rope_f[1] = rope_f[0] + half;
+    } else {
+      rope_f[0] = a.rope_features + (w - a.rope_features / 2) * 2;
+      rope_f[1] = rope_f[0] + 1;
+    }
+    feat0 = rope_f[0];
 #pragma unroll
-  for (int r = 0; r < R; ++r) {
-    const int64_t col = (feat0 + r % RO < n_out) ? feat0 + r % RO : (int64_t)n_out - 1;   // columns past the end re-read the last one
-    wrow[r] = a.w + (col + (r >= RO ? n_out : 0)) * a.w_sr;                               // second half of a pair: feature col + n/2
+    for (int r = 0; r < R; ++r) wrow[r] = a.w + (rope_f[r] < a.n ? rope_f[r] : (int64_t)a.n - 1) * a.w_sr;
+  } else {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int64_t col = (feat0 + r % RO < n_out) ? feat0 + r % RO : (int64_t)n_out - 1;   // columns past the end re-read the last one
+      wrow[r] = a.w + (col + (r >= RO ? n_out : 0)) * a.w_sr;                               // second half of a pair: feature col + n/2
+    }
   }
+  const bool live = feat0 < n_out;
   float acc[R * M];
 #pragma unroll
   for (int i = 0; i < R * M; ++i) acc[i] = 0.f;
@@ -167,6 +200,32 @@ __global__ __launch_bounds__(kLinThreads) void linear_rows_kernel(LinArgs a) {
     v = rnd16<BF16>(v);                                    // the projection's own rounding
     const float up = __shfl(v, (lane + RO * M) & 63);      // lane idx + (R/2) M holds the pair's second half for the same row
     if (lane < RO * M && col < n_out && m < a.rows) *(uint16_t*)(a.y + m * a.y_sr + col * 2) = st16<BF16>(silu_mul_elem<BF16>(v, up));
+  } else if constexpr (ROPE) {
+    const int64_t f = rope_f[r] < a.n ? rope_f[r] : (int64_t)a.n - 1;
+    if (a.bias) v += ld16<BF16>(a.bias + f * 2);
+    v = rnd16<BF16>(v);                                   // the projection's own rounding
+    const float second = __shfl(v, (lane + M) & 63);      // lane idx + M holds feature rope_f[1] of the same row
+    if (paired) {
+      if (lane < M && m < a.rows) {
+        int64_t p = a.pos_is_i64 ? ((const int64_t*)a.pos)[m] : (int64_t)((const int32_t*)a.pos)[m];
+        p = p < 0 ? 0 : (p >= a.max_pos ? a.max_pos - 1 : p);
+        const float* row = a.table + p * a.head_dim;
+        const float cs = row[rope_i], sn = row[a.head_dim / 2 + rope_i];
+        float o1, o2;
+        {
+          // separate fp32 products and sums, as the stand-alone rotary pass forms them
+#pragma clang fp contract(off)
+          const float a1 = v * cs, b1 = second * sn;
+          const float a2 = v * sn, b2 = second * cs;
+          o1 = a1 - b1;
+          o2 = a2 + b2;
+        }
+        *(uint16_t*)(a.y + m * a.y_sr + rope_f[0] * 2) = st16<BF16>(o1);
+        *(uint16_t*)(a.y + m * a.y_sr + rope_f[1] * 2) = st16<BF16>(o2);
+      }
+    } else if (lane < V && rope_f[r] < a.n && m < a.rows) {
+      *(uint16_t*)(a.y + m * a.y_sr + rope_f[r] * 2) = st16<BF16>(v);
+    }
   } else {
     if (lane < V && col < a.n && m < a.rows) {
       if (a.bias) v += ld16<BF16>(a.bias + col * 2);
@@ -177,22 +236,27 @@ __global__ __launch_bounds__(kLinThreads) void linear_rows_kernel(LinArgs a) {
 }
 
 template <bool BF16, int M>
-void launch_rows(LinArgs a, int R, bool gated, hipStream_t stream) {
-  const int64_t waves = gated ? (a.n / 2 + R / 2 - 1) / (R / 2) : (a.n + R - 1) / R;
+void launch_rows(LinArgs a, int R, int mode, hipStream_t stream) {
+  const bool gated = mode == kModeGated;
+  if (mode == kModeRope) R = 2;
+  const int64_t waves = mode == kModeRope ? a.rope_features / 2 + (a.n - a.rope_features + 1) / 2
+                                          : gated ? (a.n / 2 + R / 2 - 1) / (R / 2) : (a.n + R - 1) / R;
   const dim3 grid((unsigned)((waves + kLinThreads / 64 - 1) / (kLinThreads / 64))), block(kLinThreads);
   const int cap = (M == 8 ? kLinLdsBytes8 : kLinLdsBytes) / (2 * M) / 8 * 8;
   a.chunk = a.k < cap ? a.k : cap;
   const size_t lds = (size_t)M * a.chunk * 2;
-  if (gated) {
-    if (R == 4) hipLaunchKernelGGL((linear_rows_kernel<BF16, M, 4, true>), grid, block, lds, stream, a);
-    else hipLaunchKernelGGL((linear_rows_kernel<BF16, M, 2, true>), grid, block, lds, stream, a);
+  if (mode == kModeRope) hipLaunchKernelGGL((linear_rows_kernel<BF16, M, 2, kModeRope>), grid, block, lds, stream, a);
+  else if (gated) {
+    if (R == 4) hipLaunchKernelGGL((linear_rows_kernel<BF16, M, 4, kModeGated>), grid, block, lds, stream, a);
+    else hipLaunchKernelGGL((linear_rows_kernel<BF16, M, 2, kModeGated>), grid, block, lds, stream, a);
   } else if (R == 4) hipLaunchKernelGGL((linear_rows_kernel<BF16, M, 4>), grid, block, lds, stream, a);
   else if (R == 2) hipLaunchKernelGGL((linear_rows_kernel<BF16, M, 2>), grid, block, lds, stream, a);
   else hipLaunchKernelGGL((linear_rows_kernel<BF16, M, 1>), grid, block, lds, stream, a);
 }
 
 template <bool BF16>
-void launch(const LinArgs& a, bool gated, hipStream_t stream) {
+void launch(const LinArgs& a, int mode, hipStream_t stream) {
+  const bool gated = mode == kModeGated;
   // Features per wave: more of them re-use each activation chunk read from LDS (and shrink the share of the
   // LDS staging, which every workgroup repeats), fewer of them give more waves to a small matrix.
   const int m = a.rows <= 1 ? 1 : a.rows <= 2 ? 2 : a.rows <= 4 ? 4 : 8;
@@ -200,10 +264,10 @@ void launch(const LinArgs& a, bool gated, hipStream_t stream) {
   if ((m >= 4 || gated) && R < 2) R = 2;
   if (m == 8) R = 4;
   switch (m) {
-    case 1: launch_rows<BF16, 1>(a, R, gated, stream); break;
-    case 2: launch_rows<BF16, 2>(a, R, gated, stream); break;
-    case 4: launch_rows<BF16, 4>(a, R, gated, stream); break;
-    default: launch_rows<BF16, 8>(a, R, gated, stream); break;
+    case 1: launch_rows<BF16, 1>(a, R, mode, stream); break;
+    case 2: launch_rows<BF16, 2>(a, R, mode, stream); break;
+    case 4: launch_rows<BF16, 4>(a, R, mode, stream); break;
+    default: launch_rows<BF16, 8>(a, R, mode, stream); break;
   }
 }
 
@@ -213,8 +277,15 @@ void launch(const LinArgs& a, bool gated, hipStream_t stream) {
 using namespace sq;
 
 namespace {
-int linear_rows(const char* fn, bool gated, const DLTensor* x, const DLTensor* weight, const DLTensor* bias, const DLTensor* residual,
-                DLTensor* out, void* stream) {
+struct RopeSpec {
+  const DLTensor* position_ids;
+  const DLTensor* cos_sin_cache;
+  int32_t head_dim, rope_features;
+};
+
+int linear_rows(const char* fn, int mode, const DLTensor* x, const DLTensor* weight, const DLTensor* bias, const DLTensor* residual,
+                DLTensor* out, void* stream, const RopeSpec* rope = nullptr) {
+  const bool gated = mode == kModeGated;
   SQ_REQUIRE(x && weight && out, SQ_EINVAL, "%s: null tensor argument", fn);
   int rc;
   if ((rc = check_tensor(x, "x", 2, x->device.device_id))) return rc;
@@ -249,10 +320,36 @@ int linear_rows(const char* fn, bool gated, const DLTensor* x, const DLTensor* w
     SQ_REQUIRE(dtype_of(residual) == dt && residual->shape[0] == M && residual->shape[1] == N && stride_of(residual, 1) == 1, SQ_ESHAPE,
                "%s: residual must be [%lld, %lld] of x's dtype with a contiguous last dimension", fn, (long long)M, (long long)N);
   }
+  LinArgs a;
+  a.pos = nullptr;
+  a.table = nullptr;
+  a.pos_is_i64 = a.max_pos = a.head_dim = a.rope_features = 0;
+  if (mode == kModeRope) {
+    const DLTensor* pos = rope->position_ids;
+    const DLTensor* tab = rope->cos_sin_cache;
+    SQ_REQUIRE(pos && tab, SQ_EINVAL, "%s: null tensor argument", fn);
+    SQ_REQUIRE(rope->head_dim > 0 && rope->head_dim % 2 == 0, SQ_EUNSUPPORTED, "%s: head_dim must be even (got %d)", fn, (int)rope->head_dim);
+    SQ_REQUIRE(rope->rope_features >= 0 && rope->rope_features <= N && rope->rope_features % rope->head_dim == 0, SQ_ESHAPE,
+               "%s: rope_features must be whole heads of %d within the %lld output features (got %d)", fn, (int)rope->head_dim, (long long)N,
+               (int)rope->rope_features);
+    SQ_REQUIRE(on_gpu(pos) && pos->device.device_id == dev && on_gpu(tab) && tab->device.device_id == dev, SQ_EDEVICE,
+               "%s: position_ids and cos_sin_cache must live on the tensors' device", fn);
+    const bool i64 = pos->dtype.code == kDLInt && pos->dtype.bits == 64 && pos->dtype.lanes == 1;
+    SQ_REQUIRE((i64 || dtype_of(pos) == DType::I32) && numel_of(pos) == M && is_compact(pos), SQ_ESHAPE,
+               "%s: position_ids must be a contiguous int32 or int64 tensor of %lld entries", fn, (long long)M);
+    SQ_REQUIRE(dtype_of(tab) == DType::F32 && tab->ndim == 2 && tab->shape[1] == rope->head_dim && is_compact(tab) && tab->shape[0] > 0 &&
+                   tab->shape[0] < ((int64_t)1 << 31),
+               SQ_ESHAPE, "%s: cos_sin_cache must be a contiguous fp32 [max_position, %d] table (cos | sin)", fn, (int)rope->head_dim);
+    a.pos = data_of(pos);
+    a.table = (const float*)data_of(tab);
+    a.pos_is_i64 = i64 ? 1 : 0;
+    a.max_pos = (int)tab->shape[0];
+    a.head_dim = rope->head_dim;
+    a.rope_features = rope->rope_features;
+  }
   int cur = -1;
   SQ_HIP(hipGetDevice(&cur));
   SQ_REQUIRE(cur == dev, SQ_EDEVICE, "%s: tensors live on device %d but the current device is %d", fn, dev, cur);
-  LinArgs a;
   a.x = data_of(x);
   a.w = data_of(weight);
   a.bias = bias ? data_of(bias) : nullptr;
@@ -265,8 +362,8 @@ int linear_rows(const char* fn, bool gated, const DLTensor* x, const DLTensor* w
   a.rows = (int)M;
   a.n = (int)N;
   a.k = (int)K;
-  if (dt == DType::BF16) launch<true>(a, gated, (hipStream_t)stream);
-  else launch<false>(a, gated, (hipStream_t)stream);
+  if (dt == DType::BF16) launch<true>(a, mode, (hipStream_t)stream);
+  else launch<false>(a, mode, (hipStream_t)stream);
   SQ_HIP(hipGetLastError());
   return SQ_OK;
 }
@@ -274,9 +371,15 @@ int linear_rows(const char* fn, bool gated, const DLTensor* x, const DLTensor* w
 
 extern "C" int sq_linear_rows(const DLTensor* x, const DLTensor* weight, const DLTensor* bias, const DLTensor* residual,
                               DLTensor* out, void* stream) {
-  return linear_rows("sq_linear_rows", false, x, weight, bias, residual, out, stream);
+  return linear_rows("sq_linear_rows", kModePlain, x, weight, bias, residual, out, stream);
 }
 
 extern "C" int sq_linear_rows_silu_and_mul(const DLTensor* x, const DLTensor* weight, const DLTensor* bias, DLTensor* out, void* stream) {
-  return linear_rows("sq_linear_rows_silu_and_mul", true, x, weight, bias, nullptr, out, stream);
+  return linear_rows("sq_linear_rows_silu_and_mul", kModeGated, x, weight, bias, nullptr, out, stream);
+}
+
+extern "C" int sq_linear_rows_rope(const DLTensor* x, const DLTensor* weight, const DLTensor* bias, const DLTensor* position_ids,
+                                   const DLTensor* cos_sin_cache, int32_t head_dim, int32_t rope_features, DLTensor* out, void* stream) {
+  const RopeSpec rope{position_ids, cos_sin_cache, head_dim, rope_features};
+  return linear_rows("sq_linear_rows_rope", kModeRope, x, weight, bias, nullptr, out, stream, &rope);
 }

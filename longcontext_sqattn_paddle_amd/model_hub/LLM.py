@@ -98,10 +98,13 @@ class LLM:
         bsz, seq_len, dim = hidden_states.shape
         layer = self.layers[layer_idx]
         hidden_states = self.layernorm(hidden_states, layer.input_layernorm_variance_epsilon, layer.input_layernorm_weight)
-        query_states, key_states, value_states = self.wqkv(hidden_states, layer)
-        query_states, key_states = self.position_embedd(query_states, key_states)
-        query_states = query_states.view(bsz, -1, self.num_heads, self.head_dim)
-        key_states = key_states.view(bsz, -1, self.num_key_value_heads, self.head_dim)
+        if seq_len == 1 and hasattr(self, "wqkv_position_embedd"):   # projection and rotary embedding in one pass (same values)
+            query_states, key_states, value_states = self.wqkv_position_embedd(hidden_states, layer)
+        else:
+            query_states, key_states, value_states = self.wqkv(hidden_states, layer)
+            query_states, key_states = self.position_embedd(query_states, key_states)
+            query_states = query_states.view(bsz, -1, self.num_heads, self.head_dim)
+            key_states = key_states.view(bsz, -1, self.num_key_value_heads, self.head_dim)
         value_states = value_states.view(bsz, -1, self.num_key_value_heads, self.head_dim)
         key_states, value_states = self.kv_cache.decode_update_kv_cache(key_states, value_states, layer_idx)
         attn_out = layer.decode_attention(query_states, key_states, value_states, None)

@@ -17,7 +17,7 @@ from ..cache_hub.flash_attn_cache import flash_attn_cache
 from ..sqattn.attn_triton import attn_causal
 from ..sqattn.attn_triton_decode import attn_decode
 from .LLM import LLM
-from .utils import apply_rope_with_cos_sin_cache_inplace, linear, linear_silu_and_mul, rmsnorm, yarn_cos_sin_cache
+from .utils import apply_rope_with_cos_sin_cache_inplace, linear, linear_rope, linear_silu_and_mul, rmsnorm, yarn_cos_sin_cache
 
 
 @dataclass
@@ -196,6 +196,20 @@ class QwenModel(LLM):
         qkv = linear(hidden_states, layer.wqkv, layer.bqkv)
         kv = self.hidden_size // self.num_key_value_groups
         return qkv.split([self.hidden_size, kv, kv], dim=-1)
+
+    def wqkv_position_embedd(self, hidden_states, layer):
+        """`wqkv` followed by `position_embedd` for a decode step (qwen.py:302-312, 369-379) as one pass: returns
+        (query_states [bsz, 1, Hq, head_dim], key_states [bsz, 1, Hkv, head_dim], value_states [bsz, 1, kv_dim]),
+        q and k rotated, all three views of one projection output."""
+        bsz, seq_len, _ = hidden_states.shape
+        if getattr(self, "_graph_positions", None) is not None and seq_len == 1:
+            position_ids = self._graph_positions   # device-resident position of a captured decode step
+        else:
+            position_ids = self.position_ids[self.kv_cache.context:self.kv_cache.context + seq_len].unsqueeze(0).repeat(bsz, 1)
+        kv = self.hidden_size // self.num_key_value_groups
+        qkv = linear_rope(hidden_states, layer.wqkv, layer.bqkv, position_ids, self.head_dim, self.hidden_size + kv, self.cos_sin_cache)
+        q, k, v = qkv.split([self.hidden_size, kv, kv], dim=-1)
+        return q.view(bsz, seq_len, self.num_heads, self.head_dim), k.view(bsz, seq_len, self.num_key_value_heads, self.head_dim), v
 
     def wo(self, hidden_states, layer, bsz, seq_len, dim, residual=None):
         """qwen.py:314-317.  With `residual` the caller's `residual + wo(...)` is part of the same pass (same values)."""

@@ -82,6 +82,39 @@ def linear_silu_and_mul(x: torch.Tensor, weight: torch.Tensor, bias: Optional[to
     return out
 
 
+def linear_rope(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], position_ids: torch.Tensor, head_dim: int,
+                rope_features: int, cos_sin_cache: torch.Tensor, max_rows: int = 4) -> torch.Tensor:
+    """The fused q/k/v projection with the rotary embedding of its first `rope_features` output features (the q and
+    k heads) in one pass: x [batch, 1, K] -> [batch, 1, N], position_ids one position per row (model_hub/qwen.py:302-312
+    and :352-379 on a decode step).  Same values as `linear` followed by `apply_rope_with_cos_sin_cache_inplace`,
+    which is what longer activations (and more than `max_rows` rows) get."""
+    _need_gpu(x, weight, position_ids, cos_sin_cache)
+    K = x.shape[-1]
+    rows = x.numel() // K
+    n = weight.shape[0]
+    pos = position_ids.reshape(-1)
+    if pos.dtype not in (torch.int32, torch.int64):
+        pos = pos.to(torch.int64)
+    if rows > min(max_rows, LINEAR_ROWS_MAX) or K % 8 or weight.stride(-1) != 1 or weight.stride(0) % 8 or weight.data_ptr() % 16:
+        y = torch.nn.functional.linear(x, weight, bias)
+        if rope_features > 0:   # the rotation works head by head: any split of the rotated part into two groups of heads will do
+            flat = y.view(rows, n)
+            cut = max(rope_features - head_dim, head_dim) if rope_features > head_dim else rope_features
+            first, second = flat[:, :cut], flat[:, rope_features - head_dim:rope_features]
+            r1, r2 = apply_rope_with_cos_sin_cache_inplace(pos.view(rows, 1), first, second, head_dim, cos_sin_cache)
+            flat[:, :cut] = r1.reshape(rows, -1)
+            flat[:, rope_features - head_dim:rope_features] = r2.reshape(rows, -1)
+        return y
+    x2 = x.reshape(rows, K)
+    if x2.stride(-1) != 1 or (rows > 1 and x2.stride(0) % 8) or x2.data_ptr() % 16:
+        x2 = x2.contiguous()
+    out = torch.empty(*x.shape[:-1], n, dtype=x.dtype, device=x.device)
+    b = [N.dl(x2), N.dl(weight), N.dl(bias), N.dl(pos.contiguous()), N.dl(cos_sin_cache), N.dl(out.view(rows, n))]
+    N.check(N.lib().sq_linear_rows_rope(N.ptr(b[0]), N.ptr(b[1]), N.ptr(b[2]), N.ptr(b[3]), N.ptr(b[4]), int(head_dim), int(rope_features),
+                                        N.ptr(b[5]), N.current_stream(x.device)))
+    return out
+
+
 def rmsnorm(x: torch.Tensor, weight: torch.Tensor, epsilon: float = 1e-6, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """`x * rsqrt(mean(x^2, -1) + epsilon) * weight` over the last dimension (utils.py:15-19)."""
     _need_gpu(x, weight)

@@ -255,3 +255,52 @@ def test_gated_projection_equals_projection_then_silu_and_mul(dtype, M, I, K, bi
     if I % 8 == 0:
         x9 = torch.randn(9, K, generator=g).to(dtype).to(DEV)
         assert torch.equal(linear_silu_and_mul(x9, w, b), silu_and_mul(torch.nn.functional.linear(x9, w, b)))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,Hq,Hkv,D,K,bias", [(1, 28, 4, 128, 3584, True), (2, 4, 2, 64, 512, True), (3, 2, 1, 128, 264, False),
+                                               (4, 8, 8, 32, 1024, True), (8, 3, 1, 16, 4104, False), (1, 1, 1, 16, 8, True)])
+def test_rotary_projection_equals_projection_then_rope(dtype, M, Hq, Hkv, D, K, bias):
+    """One kernel for the fused q/k/v projection and the rotary embedding of q and k: the bits of sq_linear_rows
+    followed by sq_rope (each checked against the oracle above); v is the plain projection."""
+    from longcontext_sqattn_paddle_amd import _native as NV
+    from longcontext_sqattn_paddle_amd.model_hub.utils import apply_rope_with_cos_sin_cache_inplace, linear, linear_rope, yarn_cos_sin_cache
+
+    print(f"case rotary linear {dtype} M={M} Hq={Hq} Hkv={Hkv} D={D} K={K} bias={bias}", flush=True)
+    g = torch.Generator().manual_seed(M + Hq + D + K)
+    n = (Hq + 2 * Hkv) * D
+    x = torch.randn(M, 1, K, generator=g).to(dtype).to(DEV)
+    w = (torch.randn(n, K, generator=g) * 2 * K ** -0.5).to(dtype).to(DEV)
+    b = torch.randn(n, generator=g).to(dtype).to(DEV) if bias else None
+    table = yarn_cos_sin_cache(D, 1000000.0, 32768, 5000, DEV)
+    pos = torch.randint(0, 5000, (M, 1), generator=g).to(DEV)
+    fused = linear_rope(x, w, b, pos, D, (Hq + Hkv) * D, table, max_rows=8)
+    plain = linear(x, w, b, max_rows=8).view(M, n)
+    q_ref, k_ref = apply_rope_with_cos_sin_cache_inplace(pos, plain[:, :Hq * D], plain[:, Hq * D:(Hq + Hkv) * D], D, table)
+    torch.cuda.synchronize()
+    assert fused.shape == (M, 1, n) and fused.dtype == dtype
+    f = fused.view(M, n)
+    assert torch.equal(f[:, :Hq * D].contiguous().view(torch.int16), q_ref.reshape(M, -1).view(torch.int16))
+    assert torch.equal(f[:, Hq * D:(Hq + Hkv) * D].contiguous().view(torch.int16), k_ref.reshape(M, -1).view(torch.int16))
+    assert torch.equal(f[:, (Hq + Hkv) * D:].contiguous().view(torch.int16), plain[:, (Hq + Hkv) * D:].contiguous().view(torch.int16))
+    # int32 positions; nothing rotated = the plain projection
+    f32 = linear_rope(x, w, b, pos.to(torch.int32), D, (Hq + Hkv) * D, table, max_rows=8)
+    assert torch.equal(f32, fused)
+    assert torch.equal(linear_rope(x, w, b, pos, D, 0, table, max_rows=8).view(M, n), plain)
+    # more rows than the kernel takes: the two passes
+    x9 = torch.randn(9, 1, K, generator=g).to(dtype).to(DEV)
+    p9 = torch.randint(0, 5000, (9, 1), generator=g).to(DEV)
+    got = linear_rope(x9, w, b, p9, D, (Hq + Hkv) * D, table).view(9, n)
+    base = torch.nn.functional.linear(x9, w, b).view(9, n)
+    q9, k9 = apply_rope_with_cos_sin_cache_inplace(p9, base[:, :Hq * D], base[:, Hq * D:(Hq + Hkv) * D], D, table)
+    assert torch.equal(got[:, :Hq * D], q9.reshape(9, -1)) and torch.equal(got[:, Hq * D:(Hq + Hkv) * D], k9.reshape(9, -1))
+    assert torch.equal(got[:, (Hq + Hkv) * D:], base[:, (Hq + Hkv) * D:])
+    # argument errors: rotated width not whole heads, wrong number of positions, table of another head_dim
+    o = torch.empty(M, n, dtype=dtype, device=DEV)
+    x2 = x.view(M, K)
+    for args, hd, rf in [((x2, w, b, pos.view(-1), table, o), D, D // 2), ((x2, w, b, pos.view(-1)[:M - 1].contiguous() if M > 1 else torch.zeros(2, dtype=torch.int64, device=DEV), table, o), D, D),
+                         ((x2, w, b, pos.view(-1), table[:, :D // 2].contiguous(), o), D, D)]:
+        bb = [NV.dl(t) for t in args]
+        with pytest.raises(AssertionError):
+            NV.check(NV.lib().sq_linear_rows_rope(NV.ptr(bb[0]), NV.ptr(bb[1]), NV.ptr(bb[2]), NV.ptr(bb[3]), NV.ptr(bb[4]), hd, rf, NV.ptr(bb[5]),
+                                                  NV.current_stream(o.device)))
