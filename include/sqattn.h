@@ -269,9 +269,18 @@ int sq_linear_rows_silu_and_mul(const DLTensor* x, const DLTensor* weight, const
  * row position_ids[m] of cos_sin_cache (fp32 [max_position, head_dim], cos | sin), exactly as sq_rope rotates the
  * rounded output of sq_linear_rows; the remaining features (v) are the plain projection.  position_ids: int32 or
  * int64, one entry per row of x.  Other requirements as for sq_linear_rows.
+ *
+ * With key_cache / value_cache ([M, L, Hkv, head_dim], contiguous) and valid_length (int32 [M]) the output is
+ * [q | k | v] with k and v of Hkv * head_dim features each, and the rotated k and the v of row m are also written to
+ * row valid_length[m] of the caches -- the copies of sq_kv_cache_append (cache_hub/flash_attn_cache.py:248-252) --
+ * and attend_length (int32 [M], may be NULL) receives valid_length + 1.  valid_length itself is not changed: the
+ * reference advances it once per step after the last layer (:253-255), which stays with sq_kv_cache_append
+ * (advance != 0).  All four NULL: no cache.
  */
 int sq_linear_rows_rope(const DLTensor* x, const DLTensor* weight, const DLTensor* bias, const DLTensor* position_ids,
-                        const DLTensor* cos_sin_cache, int32_t head_dim, int32_t rope_features, DLTensor* out, void* stream);
+                        const DLTensor* cos_sin_cache, int32_t head_dim, int32_t rope_features, DLTensor* out,
+                        DLTensor* key_cache, DLTensor* value_cache, const DLTensor* valid_length, DLTensor* attend_length,
+                        void* stream);
 
 /*
  * Rotary position embedding of query [T, Hq * head_dim] and key [T, Hkv * head_dim] (T = batch * seq_len tokens)

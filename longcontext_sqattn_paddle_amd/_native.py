@@ -99,7 +99,7 @@ SYMBOLS = {
     "sq_rope": (ctypes.c_int, [_P] * 6 + [ctypes.c_int32, ctypes.c_void_p]),
     "sq_linear_rows": (ctypes.c_int, [_P] * 5 + [ctypes.c_void_p]),
     "sq_linear_rows_silu_and_mul": (ctypes.c_int, [_P] * 4 + [ctypes.c_void_p]),
-    "sq_linear_rows_rope": (ctypes.c_int, [_P] * 5 + [ctypes.c_int32, ctypes.c_int32, _P, ctypes.c_void_p]),
+    "sq_linear_rows_rope": (ctypes.c_int, [_P] * 5 + [ctypes.c_int32, ctypes.c_int32] + [_P] * 5 + [ctypes.c_void_p]),
     "sq_kv_cache_store": (ctypes.c_int, [_P] * 4 + [ctypes.c_int32, ctypes.c_int64, ctypes.c_void_p]),
     "sq_kv_cache_append": (ctypes.c_int, [_P] * 6 + [ctypes.c_int32, ctypes.c_void_p]),
     "sq_kv_cache_reorder": (ctypes.c_int, [_P] * 5 + [ctypes.c_void_p]),

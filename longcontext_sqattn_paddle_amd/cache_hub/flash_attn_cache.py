@@ -106,18 +106,27 @@ class flash_attn_cache(KV_Cache):
         """The current stream waits for the last prefill copy (flash_attn_cache.py:234-238)."""
         torch.cuda.current_stream(self.device).wait_event(self.copyevents[str(self.device)])
 
-    def decode_update_kv_cache(self, key_states, value_states, layer_idx):
+    def decode_append_targets(self, layer_idx):
+        """(key_cache, value_cache, valid_length, attend_length) of a layer, for a projection kernel that writes the
+        new token's k and v itself (`model_hub.utils.linear_rope`); `decode_update_kv_cache(..., appended=True)`
+        afterwards does the rest of the step's bookkeeping."""
+        self.check_room()
+        return self.key_cache[layer_idx], self.value_cache[layer_idx], self.valid_length, self.attend_length
+
+    def decode_update_kv_cache(self, key_states, value_states, layer_idx, appended=False):
         """Append one token per sequence at `valid_length` (flash_attn_cache.py:239-256).
 
         key_states/value_states [batch, 1, kv_heads, head_dim].  Returns the layer's whole cache buffers like the
         reference; `self.attend_length` (int32 [batch], on the device) holds how many of their rows are valid for
-        this step's attention.  `valid_length` and `context` advance after the last layer.
+        this step's attention.  `valid_length` and `context` advance after the last layer.  `appended`: the caller's
+        projection kernel has already written this layer's rows (see `decode_append_targets`).
         """
         self.check_room()
         last = layer_idx == self.layer_num - 1
-        b = [N.dl(t) for t in (key_states, value_states, self.key_cache[layer_idx], self.value_cache[layer_idx],
-                               self.valid_length, self.attend_length)]
-        N.check(self._lib.sq_kv_cache_append(*[N.ptr(x) for x in b], 1 if last else 0, N.current_stream(self.device)))
+        if not appended or last:   # appended: the rows and `attend_length` are in place; the last layer still advances the length
+            b = [N.dl(t) for t in (key_states, value_states, self.key_cache[layer_idx], self.value_cache[layer_idx],
+                                   self.valid_length, self.attend_length)]
+            N.check(self._lib.sq_kv_cache_append(*[N.ptr(x) for x in b], 1 if last else 0, N.current_stream(self.device)))
         if last:
             self.note_decode_step()
         return self.key_cache[layer_idx], self.value_cache[layer_idx]

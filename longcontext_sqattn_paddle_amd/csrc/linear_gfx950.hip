@@ -41,6 +41,13 @@ struct LinArgs {
   const void* pos;       // [rows] int32 or int64
   const float* table;    // [max_pos, head_dim]: cos | sin
   int32_t pos_is_i64, max_pos, head_dim, rope_features;
+  // rotary form with the KV cache behind it: the k and v features also go to row valid_length[m] of the caches
+  char* k_cache;                 // nullable
+  char* v_cache;
+  int64_t cache_sb;              // bytes per sequence of a cache
+  const int32_t* valid_length;   // [rows]
+  int32_t* attend_length;        // [rows] or null: receives valid_length + 1
+  int32_t max_length, q_features, kv_features;
 };
 
 enum { kModePlain = 0, kModeGated = 1, kModeRope = 2 };
@@ -222,9 +229,26 @@ __global__ __launch_bounds__(kLinThreads) void linear_rows_kernel(LinArgs a) {
         }
         *(uint16_t*)(a.y + m * a.y_sr + rope_f[0] * 2) = st16<BF16>(o1);
         *(uint16_t*)(a.y + m * a.y_sr + rope_f[1] * 2) = st16<BF16>(o2);
+        if (a.k_cache && rope_f[0] >= a.q_features) {   // a pair of a k head: its place in the new cache row
+          const int row = a.valid_length[m];
+          if (row >= 0 && row < a.max_length) {          // (a full sequence stays as it is, as in the append pass)
+            char* dst = a.k_cache + m * a.cache_sb + ((int64_t)row * a.kv_features - a.q_features) * 2;
+            *(uint16_t*)(dst + rope_f[0] * 2) = st16<BF16>(o1);
+            *(uint16_t*)(dst + rope_f[1] * 2) = st16<BF16>(o2);
+          }
+        }
       }
     } else if (lane < V && rope_f[r] < a.n && m < a.rows) {
       *(uint16_t*)(a.y + m * a.y_sr + rope_f[r] * 2) = st16<BF16>(v);
+      if (a.k_cache) {                                   // behind the rotated part: v
+        const int row = a.valid_length[m];
+        if (row >= 0 && row < a.max_length)
+          *(uint16_t*)(a.v_cache + m * a.cache_sb + ((int64_t)row * a.kv_features + rope_f[r] - a.rope_features) * 2) = st16<BF16>(v);
+      }
+    }
+    if (a.k_cache && a.attend_length && blockIdx.x == 0 && wave == 0 && lane < a.rows) {
+      const int row = a.valid_length[lane];
+      a.attend_length[lane] = row < a.max_length ? row + 1 : row;
     }
   } else {
     if (lane < V && col < a.n && m < a.rows) {
@@ -281,6 +305,10 @@ struct RopeSpec {
   const DLTensor* position_ids;
   const DLTensor* cos_sin_cache;
   int32_t head_dim, rope_features;
+  DLTensor* key_cache;       // all four null, or the cache behind the projection
+  DLTensor* value_cache;
+  const DLTensor* valid_length;
+  DLTensor* attend_length;   // may be null
 };
 
 int linear_rows(const char* fn, int mode, const DLTensor* x, const DLTensor* weight, const DLTensor* bias, const DLTensor* residual,
@@ -324,6 +352,11 @@ int linear_rows(const char* fn, int mode, const DLTensor* x, const DLTensor* wei
   a.pos = nullptr;
   a.table = nullptr;
   a.pos_is_i64 = a.max_pos = a.head_dim = a.rope_features = 0;
+  a.k_cache = a.v_cache = nullptr;
+  a.cache_sb = 0;
+  a.valid_length = nullptr;
+  a.attend_length = nullptr;
+  a.max_length = a.q_features = a.kv_features = 0;
   if (mode == kModeRope) {
     const DLTensor* pos = rope->position_ids;
     const DLTensor* tab = rope->cos_sin_cache;
@@ -346,6 +379,39 @@ int linear_rows(const char* fn, int mode, const DLTensor* x, const DLTensor* wei
     a.max_pos = (int)tab->shape[0];
     a.head_dim = rope->head_dim;
     a.rope_features = rope->rope_features;
+    if (rope->key_cache || rope->value_cache || rope->valid_length || rope->attend_length) {
+      const DLTensor* kc = rope->key_cache;
+      const DLTensor* vc = rope->value_cache;
+      const DLTensor* vl = rope->valid_length;
+      SQ_REQUIRE(kc && vc && vl, SQ_EINVAL, "%s: key_cache, value_cache and valid_length go together", fn);
+      const int64_t kvf = N - rope->rope_features;   // width of v = width of k
+      SQ_REQUIRE(kvf > 0 && kvf % rope->head_dim == 0 && rope->rope_features >= kvf, SQ_ESHAPE,
+                 "%s: the output must be [q | k | v] with k and v of equal width (rope_features %d of %lld)", fn, (int)rope->rope_features, (long long)N);
+      const DLTensor* both[2] = {kc, vc};
+      for (const DLTensor* t : both) {
+        int rc2;
+        if ((rc2 = check_tensor(t, "cache", 4, dev))) return rc2;
+        SQ_REQUIRE(dtype_of(t) == dt && is_compact(t) && t->shape[0] == M && t->shape[2] * t->shape[3] == kvf && t->shape[3] == rope->head_dim &&
+                       t->shape[1] == kc->shape[1] && t->shape[1] < ((int64_t)1 << 31),
+                   SQ_ESHAPE, "%s: the caches must be contiguous [%lld, L, Hkv, %d] of x's dtype with Hkv * %d = %lld", fn, (long long)M,
+                   (int)rope->head_dim, (int)rope->head_dim, (long long)kvf);
+      }
+      const DLTensor* lens[2] = {vl, rope->attend_length};
+      for (const DLTensor* t : lens) {
+        if (!t) continue;
+        SQ_REQUIRE(on_gpu(t) && t->device.device_id == dev, SQ_EDEVICE, "%s: length tensors must live on the cache's device", fn);
+        SQ_REQUIRE(dtype_of(t) == DType::I32 && t->ndim == 1 && t->shape[0] == M && is_compact(t), SQ_ESHAPE,
+                   "%s: length tensors must be contiguous int32 [%lld]", fn, (long long)M);
+      }
+      a.k_cache = data_of(kc);
+      a.v_cache = data_of(vc);
+      a.cache_sb = kc->shape[1] * kvf * 2;
+      a.valid_length = (const int32_t*)data_of(vl);
+      a.attend_length = rope->attend_length ? (int32_t*)data_of(rope->attend_length) : nullptr;
+      a.max_length = (int)kc->shape[1];
+      a.q_features = (int)(rope->rope_features - kvf);
+      a.kv_features = (int)kvf;
+    }
   }
   int cur = -1;
   SQ_HIP(hipGetDevice(&cur));
@@ -379,7 +445,9 @@ extern "C" int sq_linear_rows_silu_and_mul(const DLTensor* x, const DLTensor* we
 }
 
 extern "C" int sq_linear_rows_rope(const DLTensor* x, const DLTensor* weight, const DLTensor* bias, const DLTensor* position_ids,
-                                   const DLTensor* cos_sin_cache, int32_t head_dim, int32_t rope_features, DLTensor* out, void* stream) {
-  const RopeSpec rope{position_ids, cos_sin_cache, head_dim, rope_features};
+                                   const DLTensor* cos_sin_cache, int32_t head_dim, int32_t rope_features, DLTensor* out,
+                                   DLTensor* key_cache, DLTensor* value_cache, const DLTensor* valid_length, DLTensor* attend_length,
+                                   void* stream) {
+  const RopeSpec rope{position_ids, cos_sin_cache, head_dim, rope_features, key_cache, value_cache, valid_length, attend_length};
   return linear_rows("sq_linear_rows_rope", kModeRope, x, weight, bias, nullptr, out, stream, &rope);
 }

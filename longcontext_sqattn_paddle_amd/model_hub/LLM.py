@@ -98,15 +98,27 @@ class LLM:
         bsz, seq_len, dim = hidden_states.shape
         layer = self.layers[layer_idx]
         hidden_states = self.layernorm(hidden_states, layer.input_layernorm_variance_epsilon, layer.input_layernorm_weight)
-        if seq_len == 1 and hasattr(self, "wqkv_position_embedd"):   # projection and rotary embedding in one pass (same values)
-            query_states, key_states, value_states = self.wqkv_position_embedd(hidden_states, layer)
+        fused = None
+        if seq_len == 1 and hasattr(self, "wqkv_position_embedd"):
+            # projection, rotary embedding and the cache rows of the new token in one pass (same values)
+            targets = self.kv_cache.decode_append_targets(layer_idx) if hasattr(self.kv_cache, "decode_append_targets") else None
+            fused = self.wqkv_position_embedd(hidden_states, layer, cache=targets)
+            appended = fused is not None and targets is not None
+            if fused is None:
+                fused = self.wqkv_position_embedd(hidden_states, layer)
+        if fused is not None:
+            query_states, key_states, value_states = fused
         else:
+            appended = False
             query_states, key_states, value_states = self.wqkv(hidden_states, layer)
             query_states, key_states = self.position_embedd(query_states, key_states)
             query_states = query_states.view(bsz, -1, self.num_heads, self.head_dim)
             key_states = key_states.view(bsz, -1, self.num_key_value_heads, self.head_dim)
         value_states = value_states.view(bsz, -1, self.num_key_value_heads, self.head_dim)
-        key_states, value_states = self.kv_cache.decode_update_kv_cache(key_states, value_states, layer_idx)
+        if appended:
+            key_states, value_states = self.kv_cache.decode_update_kv_cache(key_states, value_states, layer_idx, appended=True)
+        else:
+            key_states, value_states = self.kv_cache.decode_update_kv_cache(key_states, value_states, layer_idx)
         attn_out = layer.decode_attention(query_states, key_states, value_states, None)
         if isinstance(attn_out, tuple):   # the slot `process_model(..., patch_decode=True)` binds returns a 1-tuple (LLM.py:105)
             attn_out = attn_out[0]

@@ -197,17 +197,21 @@ class QwenModel(LLM):
         kv = self.hidden_size // self.num_key_value_groups
         return qkv.split([self.hidden_size, kv, kv], dim=-1)
 
-    def wqkv_position_embedd(self, hidden_states, layer):
+    def wqkv_position_embedd(self, hidden_states, layer, cache=None):
         """`wqkv` followed by `position_embedd` for a decode step (qwen.py:302-312, 369-379) as one pass: returns
         (query_states [bsz, 1, Hq, head_dim], key_states [bsz, 1, Hkv, head_dim], value_states [bsz, 1, kv_dim]),
-        q and k rotated, all three views of one projection output."""
+        q and k rotated, all three views of one projection output.  `cache`: the layer's
+        `kv_cache.decode_append_targets(...)`; the pass then also appends k and v to the cache (None is returned if it
+        cannot, and nothing has been written)."""
         bsz, seq_len, _ = hidden_states.shape
         if getattr(self, "_graph_positions", None) is not None and seq_len == 1:
             position_ids = self._graph_positions   # device-resident position of a captured decode step
         else:
             position_ids = self.position_ids[self.kv_cache.context:self.kv_cache.context + seq_len].unsqueeze(0).repeat(bsz, 1)
         kv = self.hidden_size // self.num_key_value_groups
-        qkv = linear_rope(hidden_states, layer.wqkv, layer.bqkv, position_ids, self.head_dim, self.hidden_size + kv, self.cos_sin_cache)
+        qkv = linear_rope(hidden_states, layer.wqkv, layer.bqkv, position_ids, self.head_dim, self.hidden_size + kv, self.cos_sin_cache, cache=cache)
+        if qkv is None:
+            return None
         q, k, v = qkv.split([self.hidden_size, kv, kv], dim=-1)
         return q.view(bsz, seq_len, self.num_heads, self.head_dim), k.view(bsz, seq_len, self.num_key_value_heads, self.head_dim), v
 

@@ -83,11 +83,17 @@ def linear_silu_and_mul(x: torch.Tensor, weight: torch.Tensor, bias: Optional[to
 
 
 def linear_rope(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], position_ids: torch.Tensor, head_dim: int,
-                rope_features: int, cos_sin_cache: torch.Tensor, max_rows: int = 4) -> torch.Tensor:
+                rope_features: int, cos_sin_cache: torch.Tensor, max_rows: int = 4, cache=None) -> torch.Tensor:
     """The fused q/k/v projection with the rotary embedding of its first `rope_features` output features (the q and
     k heads) in one pass: x [batch, 1, K] -> [batch, 1, N], position_ids one position per row (model_hub/qwen.py:302-312
     and :352-379 on a decode step).  Same values as `linear` followed by `apply_rope_with_cos_sin_cache_inplace`,
-    which is what longer activations (and more than `max_rows` rows) get."""
+    which is what longer activations (and more than `max_rows` rows) get.
+
+    `cache` = (key_cache, value_cache, valid_length, attend_length) of the layer: the kernel also writes the rotated
+    k and the v of every row to row `valid_length` of the caches and sets `attend_length` (what
+    `flash_attn_cache.decode_update_kv_cache` does without advancing the length).  Returns None instead of the
+    output when `cache` is given but the call cannot go through the kernel: the caller then runs the separate
+    passes."""
     _need_gpu(x, weight, position_ids, cos_sin_cache)
     K = x.shape[-1]
     rows = x.numel() // K
@@ -96,6 +102,8 @@ def linear_rope(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tens
     if pos.dtype not in (torch.int32, torch.int64):
         pos = pos.to(torch.int64)
     if rows > min(max_rows, LINEAR_ROWS_MAX) or K % 8 or weight.stride(-1) != 1 or weight.stride(0) % 8 or weight.data_ptr() % 16:
+        if cache is not None:
+            return None
         y = torch.nn.functional.linear(x, weight, bias)
         if rope_features > 0:   # the rotation works head by head: any split of the rotated part into two groups of heads will do
             flat = y.view(rows, n)
@@ -110,8 +118,9 @@ def linear_rope(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tens
         x2 = x2.contiguous()
     out = torch.empty(*x.shape[:-1], n, dtype=x.dtype, device=x.device)
     b = [N.dl(x2), N.dl(weight), N.dl(bias), N.dl(pos.contiguous()), N.dl(cos_sin_cache), N.dl(out.view(rows, n))]
+    c = [N.dl(t) for t in cache] if cache is not None else [None] * 4
     N.check(N.lib().sq_linear_rows_rope(N.ptr(b[0]), N.ptr(b[1]), N.ptr(b[2]), N.ptr(b[3]), N.ptr(b[4]), int(head_dim), int(rope_features),
-                                        N.ptr(b[5]), N.current_stream(x.device)))
+                                        N.ptr(b[5]), *[N.ptr(t) for t in c], N.current_stream(x.device)))
     return out
 
 

@@ -303,4 +303,55 @@ def test_rotary_projection_equals_projection_then_rope(dtype, M, Hq, Hkv, D, K, 
         bb = [NV.dl(t) for t in args]
         with pytest.raises(AssertionError):
             NV.check(NV.lib().sq_linear_rows_rope(NV.ptr(bb[0]), NV.ptr(bb[1]), NV.ptr(bb[2]), NV.ptr(bb[3]), NV.ptr(bb[4]), hd, rf, NV.ptr(bb[5]),
-                                                  NV.current_stream(o.device)))
+                                                  None, None, None, None, NV.current_stream(o.device)))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,Hq,Hkv,D,K,L", [(1, 28, 4, 128, 3584, 300), (3, 4, 2, 64, 512, 40), (4, 2, 1, 16, 264, 9)])
+def test_rotary_projection_appends_to_the_kv_cache_like_the_append_pass(dtype, B, Hq, Hkv, D, K, L):
+    """With the layer's cache behind it the projection writes the new token's rotated k and its v to row
+    valid_length[b] and sets attend_length: the same cache bits as the projection followed by sq_kv_cache_append
+    (advance = 0); a full sequence is left alone; valid_length is not touched."""
+    from longcontext_sqattn_paddle_amd import _native as NV
+    from longcontext_sqattn_paddle_amd.model_hub.utils import linear_rope, yarn_cos_sin_cache
+
+    print(f"case rotary linear + cache {dtype} B={B} Hq={Hq} Hkv={Hkv} D={D} K={K} L={L}", flush=True)
+    g = torch.Generator().manual_seed(B + Hq + D + K)
+    n = (Hq + 2 * Hkv) * D
+    x = torch.randn(B, 1, K, generator=g).to(dtype).to(DEV)
+    w = (torch.randn(n, K, generator=g) * 2 * K ** -0.5).to(dtype).to(DEV)
+    b = torch.randn(n, generator=g).to(dtype).to(DEV)
+    table = yarn_cos_sin_cache(D, 1000000.0, 32768, 5000, DEV)
+    pos = torch.randint(0, 5000, (B, 1), generator=g).to(DEV)
+    lens = torch.randint(0, L, (B,), generator=g).to(torch.int32)
+    if B > 1:
+        lens[-1] = L                                     # a full sequence
+    base_k = torch.randn(B, L, Hkv, D, generator=g).to(dtype)
+    base_v = torch.randn(B, L, Hkv, D, generator=g).to(dtype)
+
+    kc1, vc1, vl1 = base_k.to(DEV), base_v.to(DEV), lens.to(DEV)
+    al1 = torch.full((B,), -7, dtype=torch.int32, device=DEV)
+    out = linear_rope(x, w, b, pos, D, (Hq + Hkv) * D, table, max_rows=8, cache=(kc1, vc1, vl1, al1))
+    assert out is not None
+    # the two passes
+    kc2, vc2, vl2 = base_k.to(DEV), base_v.to(DEV), lens.to(DEV)
+    al2 = torch.full((B,), -7, dtype=torch.int32, device=DEV)
+    plain = linear_rope(x, w, b, pos, D, (Hq + Hkv) * D, table, max_rows=8)
+    k_new = plain[..., Hq * D:(Hq + Hkv) * D].view(B, 1, Hkv, D)
+    v_new = plain[..., (Hq + Hkv) * D:].view(B, 1, Hkv, D)
+    bb = [NV.dl(t) for t in (k_new, v_new, kc2, vc2, vl2, al2)]
+    NV.check(NV.lib().sq_kv_cache_append(*[NV.ptr(t) for t in bb], 0, NV.current_stream(kc2.device)))
+    torch.cuda.synchronize()
+    assert torch.equal(out, plain)
+    assert torch.equal(kc1.view(torch.int16), kc2.view(torch.int16)) and torch.equal(vc1.view(torch.int16), vc2.view(torch.int16))
+    assert torch.equal(al1, al2) and torch.equal(vl1.cpu(), lens) and torch.equal(vl2.cpu(), lens)
+    assert not torch.equal(kc1.cpu(), base_k)            # something was written
+    if B > 1:
+        assert torch.equal(kc1[-1].cpu(), base_k[-1]) and int(al1[-1]) == L
+    # caches of another shape, a missing length tensor
+    with pytest.raises(AssertionError):
+        linear_rope(x, w, b, pos, D, (Hq + Hkv) * D, table, max_rows=8, cache=(kc1[:, :, :, :D // 2].contiguous(), vc1, vl1, al1))
+    with pytest.raises(AssertionError):
+        linear_rope(x, w, b, pos, D, (Hq + Hkv) * D, table, max_rows=8, cache=(kc1, vc1, vl1[:B - 1] if B > 1 else torch.zeros(2, dtype=torch.int32, device=DEV), al1))
+    with pytest.raises(ValueError):
+        linear_rope(x, w, b, pos, D, (Hq + Hkv) * D, table, max_rows=8, cache=(kc1, vc1, None, al1))
