@@ -21,7 +21,8 @@
 namespace sq {
 namespace {
 
-constexpr int kLinThreads = 256;   // four waves
+constexpr int kLinThreads = 256;   // four waves: the workgroup of a large matrix
+constexpr int kLinMaxWaves = 16;   // a matrix of at most 256 x 16 waves runs as one workgroup per CU
 // Activation rows in LDS, K-chunk by K-chunk: up to 20480 elements of one row (a whole row of the widest projection,
 // four workgroups per CU), 5120 of each of four; with eight rows 2048 of each, which keeps five workgroups on a CU.
 constexpr int kLinLdsBytes = 40960, kLinLdsBytes8 = 32768;
@@ -90,7 +91,7 @@ __device__ __forceinline__ float silu_mul_elem(float x1, float x2) {
 // kModeGated: the wave's R features are R/2 pairs (f, f + n/2) and the output has n/2 columns.
 // kModeRope (R = 2): wave w < rope_features / 2 owns the pair (i, i + head_dim / 2) of a head, later waves two plain features.
 template <bool BF16, int M, int R, int MODE = kModePlain>
-__global__ __launch_bounds__(kLinThreads) void linear_rows_kernel(LinArgs a) {
+__global__ __launch_bounds__(kLinMaxWaves * 64) void linear_rows_kernel(LinArgs a) {
   constexpr bool GATED = MODE == kModeGated, ROPE = MODE == kModeRope;
   static_assert(!GATED || R % 2 == 0, "a gated wave owns whole pairs");
   static_assert(!ROPE || R == 2, "a rotary wave owns one pair");
@@ -100,13 +101,13 @@ __global__ __launch_bounds__(kLinThreads) void linear_rows_kernel(LinArgs a) {
   extern __shared__ u32x4_t xs[];   // [M][chunk / 8]
   const int kLinChunk = a.chunk, row16 = a.chunk / 8;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  int64_t feat0 = ((int64_t)blockIdx.x * (kLinThreads / 64) + wave) * RO;
+  int64_t feat0 = ((int64_t)blockIdx.x * (blockDim.x >> 6) + wave) * RO;
   const char* wrow[R];
   [[maybe_unused]] int64_t rope_f[2] = {0, 0};   // the two features of a rotary wave
   [[maybe_unused]] bool paired = false;
   [[maybe_unused]] int rope_i = 0;               // index of the pair inside its head
   if constexpr (ROPE) {
-    const int64_t w = (int64_t)blockIdx.x * (kLinThreads / 64) + wave;
+    const int64_t w = (int64_t)blockIdx.x * (blockDim.x >> 6) + wave;
     const int half = a.head_dim / 2;
     paired = w < a.rope_features / 2;
     if (paired) {
@@ -166,7 +167,7 @@ __global__ __launch_bounds__(kLinThreads) void linear_rows_kernel(LinArgs a) {
     for (int m = 0; m < M; ++m) {
       const char* xr = a.x + (int64_t)(m < a.rows ? m : a.rows - 1) * a.x_sr + (int64_t)k0 * 2;
 #pragma unroll 4
-      for (int c = threadIdx.x; c < chunks; c += kLinThreads) xs[m * row16 + c] = *(const u32x4_t*)(xr + c * 16);
+      for (int c = threadIdx.x; c < chunks; c += blockDim.x) xs[m * row16 + c] = *(const u32x4_t*)(xr + c * 16);
     }
     __syncthreads();
     if (live) {
@@ -265,7 +266,12 @@ void launch_rows(LinArgs a, int R, int mode, hipStream_t stream) {
   if (mode == kModeRope) R = 2;
   const int64_t waves = mode == kModeRope ? a.rope_features / 2 + (a.n - a.rope_features + 1) / 2
                                           : gated ? (a.n / 2 + R / 2 - 1) / (R / 2) : (a.n + R - 1) / R;
-  const dim3 grid((unsigned)((waves + kLinThreads / 64 - 1) / (kLinThreads / 64))), block(kLinThreads);
+  // Waves per workgroup: a matrix that fits 256 workgroups of at most 16 waves runs as exactly one workgroup per
+  // CU (every CU gets the same number of waves and stages the activation rows once); larger ones as workgroups of
+  // four waves, which the dispatcher hands out as CUs free up.
+  const int64_t per_cu = (waves + 255) / 256;
+  const int wpw = per_cu <= kLinMaxWaves ? (int)(per_cu < 1 ? 1 : per_cu) : kLinThreads / 64;
+  const dim3 grid((unsigned)((waves + wpw - 1) / wpw)), block(wpw * 64);
   const int cap = (M == 8 ? kLinLdsBytes8 : kLinLdsBytes) / (2 * M) / 8 * 8;
   a.chunk = a.k < cap ? a.k : cap;
   const size_t lds = (size_t)M * a.chunk * 2;
