@@ -395,12 +395,12 @@ extern "C" int32_t sq_decode_num_splits(int64_t batch, int64_t num_kv_heads, int
   if (batch <= 0 || num_kv_heads <= 0 || max_len <= 0) return 1;
   // One workgroup per CU and never more workgroups than the 256 CUs: measured at batch 1, 256 workgroups stream a
   // 1M-token cache in 306 us, 512 in 324 us, and any count that is not a multiple of 256 leaves some CUs with twice
-  // the work of the others (320 workgroups: 425 us).  At least 256 tokens (4 waves x 4 tiles) per workgroup.
+  // the work of the others (320 workgroups: 425 us).  At least 64 tokens (4 waves x 1 tile) per workgroup.
   const int64_t target_blocks = 256;
   const int64_t hpw = (num_kv_heads % 4 == 0) ? 4 : ((num_kv_heads % 2 == 0) ? 2 : 1);
   const int64_t groups = batch * (num_kv_heads / hpw);
   int64_t s = target_blocks / groups;   // rounded down: 255 workgroups are fine, 257 are not
-  const int64_t max_s = (max_len * hpw + 255) / 256;   // at least 4 tiles of 16 tokens per wave
+  const int64_t max_s = (max_len * hpw + 63) / 64;   // at least one tile of 16 tokens per wave (4096 tokens: 256 workgroups 16.2 us, 64 workgroups 18.2 us)
   if (s > max_s) s = max_s;
   if (s < 1) s = 1;
   if (s > 4096) s = 4096;
