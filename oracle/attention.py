@@ -10,9 +10,11 @@ Followed reference code:
   * `attn_fwd_inner` + relative wrapper                    sqattn/attn_triton_mix_relative.py:8-99, 309-483
   * `_attn_fwd_inner` + absolute wrapper                   sqattn/attn_triton_mix_bad.py:9-98, 285-426
 
-Parity unpinned (build-defined, no reference counterpart; pinned only by their definitions' invariants in
-tests/test_oracle_attention.py and by exact attention): P modes `P_BLOCK_ABSMAX`, `P_STATIC448_GRID`, `P_MX_ROW`
-and `v_quant="e4m3_channel"`.
+Build-defined, no reference counterpart (the reference multiplies fp16 P by fp16 V, attn_triton.py:81-83), so no
+reference artefact can pin them: P modes `P_BLOCK_ABSMAX`, `P_STATIC448_GRID`, `P_MX_ROW` and `v_quant="e4m3_channel"`.
+tests/test_oracle_attention.py pins each against its written definition instead: hand-derived known answers on the e4m3
+grid, an independent scalar (grid-search) rounding loop, the exact power-of-two scale rule and its equivariance, and a
+scalar row-group brute force for the block-absmax mode.
 """
 from __future__ import annotations
 
@@ -153,6 +155,17 @@ class _RowState:
         return out, lse
 
 
+def quant_v_e4m3_channel(v: torch.Tensor):
+    """Build-defined V operand of the fp8 P.V product (no reference counterpart: the reference multiplies fp16 V,
+    attn_triton.py:83).  v [B,Hkv,N,D] -> (`e4m3(v * s) / s` as fp32, s [B,Hkv,1,D]) with one power-of-two scale per
+    (batch, kv head, channel): `s = 2^floor(log2(448 / amax))`, amax the channel's largest |v| over the tokens, so that
+    amax * s lies in (224, 448]; an all-zero channel takes s = 1 and stays zero."""
+    amax = v.float().abs().amax(dim=2, keepdim=True)
+    _, ex = torch.frexp(torch.where(amax > 0, 448.0 / amax, torch.ones_like(amax)))   # 448/amax = f * 2^ex, f in [1/2, 1)
+    sv = torch.ldexp(torch.ones_like(amax), ex - 1)                                    # 2^floor(log2(448/amax))
+    return (v.float() * sv).clamp(-448.0, 448.0).to(torch.float8_e4m3fn).float() / sv, sv
+
+
 def window_size_relative(ratio: float, kv_len: int) -> int:
     """`ceil128(int(float32(ratio) * kv_len))` (attn_triton_mix_relative.py:43-46)."""
     # the product is formed in fp32 on the device: float32(ratio) * float32(kv_len)
@@ -216,10 +229,7 @@ def prefill_blockwise(
     if v_quant is None:
         vf = v.to(torch.float16).float()
     elif v_quant == "e4m3_channel":
-        amax = v.float().abs().amax(dim=2, keepdim=True)
-        _, ex = torch.frexp(torch.where(amax > 0, 448.0 / amax, torch.ones_like(amax)))   # 448/amax = f * 2^ex
-        sv = torch.ldexp(torch.ones_like(amax), ex - 1)                                    # 2^floor(log2(448/amax))
-        vf = (v.float() * sv).clamp(-448.0, 448.0).to(torch.float8_e4m3fn).float() / sv
+        vf, _ = quant_v_e4m3_channel(v)
     else:
         raise ValueError(f"unknown v_quant {v_quant}")
     out = torch.zeros(B, Hq, Nq, D, dtype=torch.float32)

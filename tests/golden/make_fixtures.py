@@ -36,12 +36,19 @@ def randn(shape, seed, scale=1.0, dtype=torch.bfloat16):
 def prefill():
     q, k, v = randn((1, 4, 192, 128), 101), randn((1, 2, 192, 128), 102), randn((1, 2, 192, 128), 103)
     out = {"q": bits(q), "k": bits(k), "v": bits(v)}
-    for name, mode in (("none", A.P_NONE), ("e4m3_static", A.P_STATIC448)):
+    for name, mode in (("none", A.P_NONE), ("e4m3_static", A.P_STATIC448), ("e4m3_block", A.P_BLOCK_ABSMAX)):
         o, lse = A.prefill_blockwise(q, k, v, p_quant=mode, out_dtype=torch.float32)
+        out[f"out_{name}"], out[f"lse_{name}"] = o.numpy(), lse.numpy()
+    # the two fp8 P.V modes (e4m3 V with a per-channel power-of-two scale; P on the static grid / with a per-row tile scale)
+    for name, mode in (("fp8pv", A.P_STATIC448_GRID), ("mx_fp8pv", A.P_MX_ROW)):
+        o, lse = A.prefill_blockwise(q, k, v, p_quant=mode, v_quant="e4m3_channel", out_dtype=torch.float32)
         out[f"out_{name}"], out[f"lse_{name}"] = o.numpy(), lse.numpy()
     # sink 64 + per-head windows (8-bit 64 / 128 / 64 / 128 tokens, 4-bit 128 / 128 / 192 / 192), 64-row query blocks
     o, lse = A.prefill_blockwise(q, k, v, out_dtype=torch.float32, block_m=64, sink=64, w8=[64, 128, 64, 128], w4=[128, 128, 192, 192])
     out["out_window"], out["lse_window"] = o.numpy(), lse.numpy()
+    o, lse = A.prefill_blockwise(q, k, v, p_quant=A.P_MX_ROW, v_quant="e4m3_channel", out_dtype=torch.float32, block_m=64, sink=64,
+                                 w8=[64, 128, 64, 128], w4=[128, 128, 192, 192])
+    out["out_window_mx_fp8pv"], out["lse_window_mx_fp8pv"] = o.numpy(), lse.numpy()
     np.savez_compressed(os.path.join(HERE, "prefill_small.npz"), **out)
 
 
@@ -84,6 +91,7 @@ def window_search():
 
 
 if __name__ == "__main__":
-    for f in (prefill, decode, prepass, kmeans, window_search):
-        f()
-        print("wrote", f.__name__)
+    todo = {f.__name__: f for f in (prefill, decode, prepass, kmeans, window_search)}
+    for name in (sys.argv[1:] or list(todo)):   # optional arguments: the fixtures to rewrite
+        todo[name]()
+        print("wrote", name)

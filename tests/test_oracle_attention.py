@@ -258,3 +258,207 @@ def test_decode_closed_form_and_split_combine():
     oc, _ = A.exact_attention(q, kc, v, causal=False, kv_lens=lens)
     o0, _ = A.exact_attention(q, k.float(), v, causal=False, kv_lens=lens)
     assert torch.allclose(oc, o0, atol=1e-9)
+
+
+# ------------------------------------------------------------------ build-defined fp8 operands (no reference counterpart)
+def _e4m3_grid():
+    g = torch.arange(256, dtype=torch.uint8).view(torch.float8_e4m3fn).float().numpy().astype(np.float64)
+    return np.unique(g[np.isfinite(g) & (g >= 0)])   # -0 and +0 collapse: positions follow the positive encodings
+
+
+def _e4m3_scalar(x):
+    """Round-to-nearest-even onto the e4m3 value grid by search, element by element (no torch cast): an independent
+    restatement of the cast the oracle uses.  Even = even position in the sorted grid (positions follow the encodings)."""
+    grid = _e4m3_grid()
+    x = np.asarray(x, dtype=np.float64)
+    out = np.empty_like(x)
+    for i, t in np.ndenumerate(x):
+        a = min(abs(t), 448.0)
+        j = int(np.searchsorted(grid, a))
+        if j < len(grid) and grid[j] == a:
+            r = a
+        else:
+            lo, hi = grid[j - 1], grid[min(j, len(grid) - 1)]
+            if a - lo < hi - a:
+                r = lo
+            elif a - lo > hi - a:
+                r = hi
+            else:
+                r = lo if (j - 1) % 2 == 0 else hi
+        out[i] = np.copysign(r, t)
+    return out
+
+
+def test_static448_grid_known_answers():
+    """`P_STATIC448_GRID` = e4m3(448 p) / 448 in fp32.  Hand-derived on the e4m3 grid (3 mantissa bits: spacing 16 in
+    [128, 256), 32 in [256, 448]; subnormal spacing 2^-9 below 2^-6):
+      p = 1        -> 448            -> 448
+      p = 1/2      -> 224            -> 224
+      p = 0.3125   -> 140            -> 144   (128 | 144, nearer 144)
+      p = 0.296875 -> 133            -> 128
+      p = 0.375    -> 168 = tie of 160 | 176 -> 160 (mantissa 010 is even)
+      p = 0.40625  -> 182            -> 176
+      p = 0.9      -> 403.2          -> 416   (384 | 416)
+      p = 2^-6/448 -> 2^-6 (smallest normal), p = 2^-9/448 -> 2^-9 (smallest subnormal)
+      p = 2^-16    -> 7 * 2^-10 = tie of 3 | 4 * 2^-9 -> 4 * 2^-9 (even)
+      p = 2^-10/448 -> tie of 0 | 2^-9 -> 0;  p = 1.5 * 2^-10/448 -> 2^-9;  p = 0 -> 0."""
+    f = np.float32
+    cases = [(1.0, 448.0), (0.5, 224.0), (0.3125, 144.0), (0.296875, 128.0), (0.375, 160.0), (0.40625, 176.0), (0.9, 416.0),
+             (2.0 ** -6 / 448, 2.0 ** -6), (2.0 ** -9 / 448, 2.0 ** -9), (2.0 ** -16, 2.0 ** -7), (2.0 ** -10 / 448, 0.0),
+             (1.5 * 2.0 ** -10 / 448, 2.0 ** -9), (0.0, 0.0)]
+    p = torch.tensor([[c[0] for c in cases] + [0.0] * (64 - len(cases))], dtype=torch.float32)
+    # the subnormal cases need p * 448 exact in fp32: p = 2^-k / 448 is not a dyadic number, so check the products first
+    prod = (p * 448.0)[0, :len(cases)].double().numpy()
+    got = A._quant_p(p, A.P_STATIC448_GRID)[0, :len(cases)].numpy()
+    grid_pt = []
+    for (pv, want), x, y in zip(cases, prod, got):
+        if want in (2.0 ** -6, 2.0 ** -9) or pv in (2.0 ** -10 / 448,):
+            # p = 2^-k / 448 is not a dyadic number: the fp32 product may sit an ulp off the intended grid point / tie, and
+            # the answer must be the neighbour the product is nearest to, which the scalar search decides
+            want = float(_e4m3_scalar(x))
+        grid_pt.append(want)
+        assert y == f(want) / f(448.0), (pv, x, y, want)
+    # and the static mode of the reference is this grid followed by fp16(x / 448) in fp16 arithmetic (attn_triton.py:82)
+    ref1 = A._quant_p(p, A.P_STATIC448)[0, :len(cases)]
+    want1 = (torch.tensor(grid_pt, dtype=torch.float32).to(torch.float16) / 448).float()
+    assert torch.equal(ref1, want1)
+
+
+def test_static448_grid_matches_scalar_search_on_random_probabilities():
+    g = torch.Generator().manual_seed(31)
+    p = torch.cat([torch.rand(8, 64, generator=g), torch.rand(8, 64, generator=g) * 2.0 ** -8, torch.rand(8, 64, generator=g) * 2.0 ** -17])
+    want = _e4m3_scalar((p * 448.0).double().numpy()) / 448.0
+    got = A._quant_p(p, A.P_STATIC448_GRID).double().numpy()
+    assert np.array_equal(got, want.astype(np.float32).astype(np.float64))
+
+
+def test_v_e4m3_channel_scale_rule_and_values():
+    """`v_quant="e4m3_channel"` against what its definition fixes: the scale is the power of two with
+    224 < amax * s <= 448 per (batch, kv head, channel); the values equal an independent scalar rounding loop;
+    |v| >= 2^-6 amax keeps three mantissa bits; a zero channel stays zero without NaN."""
+    g = torch.Generator().manual_seed(41)
+    v = torch.randn(2, 3, 200, 16, generator=g)
+    v[..., 0] *= 1e-3
+    v[..., 1] *= 300.0
+    v[..., 2] = 0.0
+    v[0, 0, :, 3] = 0.0
+    v[0, 0, 7, 3] = -448.0            # amax * s == 448 exactly (upper end of the interval)
+    v[0, 1, :, 3] = 0.0
+    v[0, 1, 9, 3] = 224.0             # amax * s must go to 448, not stay at 224 (lower end is open)
+    v[1, 0, :, 4] = torch.linspace(-1, 1, 200) * 2.0 ** -20
+    v = v.bfloat16()
+    vq, s = A.quant_v_e4m3_channel(v)
+    assert vq.shape == v.shape and s.shape == (2, 3, 1, 16)
+    amax = v.float().abs().amax(dim=2, keepdim=True)
+    nz = amax > 0
+    assert torch.equal(torch.exp2(torch.round(torch.log2(s))), s)                          # a power of two
+    prod = (amax * s)[nz]
+    assert bool(((prod > 224.0) & (prod <= 448.0)).all())
+    assert float(s[0, 0, 0, 3]) == 1.0 and float(s[0, 1, 0, 3]) == 2.0
+    assert torch.equal(s[~nz], torch.ones_like(s[~nz])) and torch.equal(vq[..., 2], torch.zeros_like(vq[..., 2]))
+    assert bool(torch.isfinite(vq).all())
+    # values: independent scalar loop over every element
+    want = _e4m3_scalar((v.double() * s.double()).numpy()) / s.double().numpy()
+    assert np.array_equal(vq.double().numpy(), want)
+    # precision where the definition promises it
+    big = (v.float().abs() >= 2.0 ** -6 * amax) & nz
+    rel = ((vq - v.float()).abs() / v.float().abs())[big]
+    assert float(rel.max()) <= 2.0 ** -4
+    # scale equivariance: v * 2^j gives exactly vq * 2^j
+    for j in (-9, -1, 3, 11):
+        vj = (v.float() * 2.0 ** j).bfloat16()
+        assert torch.equal(vj.float(), v.float() * 2.0 ** j)   # exact in bf16
+        vqj, sj = A.quant_v_e4m3_channel(vj)
+        assert torch.equal(vqj, vq * 2.0 ** j) and torch.equal(sj[nz], s[nz] * 2.0 ** -j), j
+
+
+@pytest.mark.parametrize("mode", [A.P_STATIC448_GRID, A.P_MX_ROW, A.P_NONE])
+def test_prefill_with_v_quant_equals_prefill_on_prequantised_v(mode):
+    """The V quantisation is a pure pre-processing of V: running the blockwise algorithm with `v_quant` equals running
+    it without on a V that an independent scalar loop quantised beforehand (the quantised values have four significant
+    bits, so the bf16 tensor and the fp16 operand cast hold them exactly)."""
+    q, k, v = _rand(1, 4, 2, 200, 200, 32, 43)
+    v = (v.float() * torch.tensor([0.01, 1.0, 50.0, 3.0] * 8)).bfloat16()
+    a, la = A.prefill_blockwise(q, k, v, p_quant=mode, v_quant="e4m3_channel", out_dtype=torch.float32)
+    amax = v.double().abs().amax(dim=2, keepdim=True).numpy()
+    s = 2.0 ** np.floor(np.log2(448.0 / amax))
+    vq = torch.tensor(_e4m3_scalar(v.double().numpy() * s) / s).bfloat16()
+    b, lb = A.prefill_blockwise(q, k, vq, p_quant=mode, out_dtype=torch.float32)
+    assert torch.equal(a, b) and torch.equal(la, lb)
+
+
+def _scalar_block_absmax_prefill(q, k, v, D):
+    """Independent scalar restatement of the block-absmax FP8-P mode for ONE head: per (64 query rows x 64 keys) tile
+    the largest probability a of the tile (after each row's running-maximum update) sets the scale 448 / a,
+    P8 = e4m3(p * (448 / a)), and the product uses fp16(P8 * (a / 448)) with fp16 V; the denominator sums the
+    unquantised p.  Rows are processed in groups of 64, keys in ascending blocks of 64 up to the group's 128-row
+    tile end, with the additive -1e6 mask inside the diagonal tile (attn_triton.py:57-77 for the schedule)."""
+    f32 = np.float32
+    qf = A.fold_scale(q, D).float().numpy()
+    kf = k.float().numpy()
+    vf = v.to(torch.float16).float().numpy()
+    N = qf.shape[0]
+    out = np.zeros((N, D), dtype=f32)
+    lse = np.zeros(N, dtype=f32)
+    for g0 in range(0, N, 64):
+        rows = list(range(g0, min(g0 + 64, N)))
+        m = {i: f32(-np.inf) for i in rows}
+        l = {i: f32(1.0) for i in rows}
+        acc = {i: np.zeros(D, dtype=np.float64) for i in rows}
+        tile0 = (g0 // 128) * 128
+        for j0 in range(0, tile0 + 128, 64):
+            if j0 >= N:
+                break
+            p = {}
+            for i in rows:
+                s = np.zeros(64, dtype=f32)
+                for c in range(64):
+                    if j0 + c < N:
+                        s[c] = np.dot(qf[i].astype(np.float64), kf[j0 + c].astype(np.float64))
+                    if j0 >= tile0 and j0 + c > i:
+                        s[c] += f32(-1000000.0)
+                m_new = max(m[i], s.max())
+                p[i] = np.exp2((s - m_new).astype(np.float64)).astype(f32)
+                alpha = f32(np.exp2(np.float64(m[i] - m_new)))
+                l[i] = f32(l[i] * alpha + p[i].sum(dtype=f32))
+                acc[i] = acc[i] * np.float64(alpha)
+                m[i] = m_new
+            a = max(float(p[i].max()) for i in rows)
+            if a <= 0.0:
+                continue
+            sc, inv = f32(f32(448.0) / f32(a)), f32(f32(a) / f32(448.0))
+            for i in rows:
+                p8 = _e4m3_scalar(np.minimum((p[i] * sc).astype(f32), f32(448.0)).astype(np.float64))
+                pq = (p8.astype(f32) * inv).astype(np.float16).astype(np.float64)
+                for c in range(64):
+                    if j0 + c < N:
+                        acc[i] = acc[i] + pq[c] * vf[j0 + c]
+        for i in rows:
+            out[i] = (acc[i] / np.float64(l[i])).astype(f32)
+            lse[i] = np.log2(l[i]) + m[i]
+    return out, lse
+
+
+def test_block_absmax_matches_scalar_bruteforce():
+    """A wrong group size (per row, per 128 rows), a scale taken before the running-maximum update, or a missing
+    fp16 rounding of the dequantised P each move the result by e4m3 steps (~1e-2 of rms) and fail the 2e-5 band."""
+    D = 32
+    q, k, v = _rand(1, 1, 1, 200, 200, D, 47)
+    # make the scale matter: one dominant early key so that later tiles have a << 1 for most row groups
+    q[..., 0] = 3.0
+    k[0, 0, :, 0] *= 0.1
+    k[0, 0, 3, 0] = 9.0       # key 3 leads every row by about 2^7: the tiles behind the first hold a of 2^-7 .. 2^-3
+    out, lse = A.prefill_blockwise(q, k, v, p_quant=A.P_BLOCK_ABSMAX, out_dtype=torch.float32)
+    ref, lse_ref = _scalar_block_absmax_prefill(q[0, 0], k[0, 0], v[0, 0], D)
+    d = np.abs(out[0, 0].numpy() - ref)
+    rms = np.sqrt((ref ** 2).mean())
+    assert np.quantile(d, 0.999) < 2e-5 * max(rms, 1.0)
+    assert d.max() < 0.05
+    assert np.allclose(lse[0, 0].numpy(), lse_ref, atol=2e-5)
+    # the mode is not the static scale in disguise on this input
+    stat, _ = A.prefill_blockwise(q, k, v, p_quant=A.P_STATIC448, out_dtype=torch.float32)
+    assert float((stat - out).abs().max()) > 1e-3 * rms
+    # and a per-row or per-128-row group would differ
+    for gr in (1, 128):
+        other, _ = A.prefill_blockwise(q, k, v, p_quant=A.P_BLOCK_ABSMAX, out_dtype=torch.float32, group_rows=gr)
+        assert float((other - out).abs().max()) > 1e-3 * rms, gr
