@@ -14,6 +14,7 @@
  *                             sqattn/attn_triton_mix_relative.py:309-483 (launch :439-475),
  *                             sqattn/attn_triton_mix_bad.py:285-426 (launch :388-424)
  *   sq_decode_fwd             sqattn/attn_triton_decode.py:244-361 (decode launch :293-324)
+ *   sq_decode_fwd_noalloc     no reference counterpart: sq_decode_fwd for callers that cannot allocate device memory
  *   sq_decode_selected_fwd    no reference counterpart: the same decode over the tokens sq_topk_select picked
  *   sq_kmeans_train           cache_hub/kmeans.py:127-196 (assign launch :147-173, update launch :175-193)
  *   sq_reverse_index          cache_hub/kmeans.py:233-262
@@ -131,6 +132,21 @@ size_t sq_decode_workspace_bytes(int64_t batch, int64_t num_q_heads, int64_t hea
 int sq_decode_fwd(const DLTensor* q, const DLTensor* kcache, const DLTensor* vcache, const DLTensor* seqlens,
                   DLTensor* out, DLTensor* lse, DLTensor* workspace, const sq_decode_params* params,
                   void* stream);
+
+/*
+ * sq_decode_fwd without a workspace argument and without any allocation.  No counterpart in the reference: it is for
+ * callers that cannot allocate device memory -- code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc.  The split-KV partial results go to a device array inside the library
+ * (sq_decode_noalloc_scratch_bytes() = 8 MiB per GPU, held until the process ends) instead of a caller workspace; the
+ * kernels and the results are those of sq_decode_fwd with the same num_splits, bit for bit.  A call whose partials
+ * (batch * q heads * splits * 516 bytes) exceed the array returns SQ_EWORKSPACE.  q's device must be the current
+ * device.  The call allocates and frees nothing (the first call on a device looks the array's address up).  All calls
+ * on one GPU share that GPU's array: calls that overlap in time on one GPU (different streams, or threads) race;
+ * order them on one stream or with events.
+ */
+size_t sq_decode_noalloc_scratch_bytes(void);
+int sq_decode_fwd_noalloc(const DLTensor* q, const DLTensor* kcache, const DLTensor* vcache, const DLTensor* seqlens,
+                          DLTensor* out, DLTensor* lse, const sq_decode_params* params, void* stream);
 
 /*
  * The same decode over a selection of the cache (no reference counterpart; it consumes what sq_topk_select

@@ -86,6 +86,8 @@ SYMBOLS = {
     "sq_decode_num_splits": (ctypes.c_int32, [ctypes.c_int64] * 3),
     "sq_decode_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int32]),
     "sq_decode_fwd": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, _P, ctypes.POINTER(DecodeParams), ctypes.c_void_p]),
+    "sq_decode_noalloc_scratch_bytes": (ctypes.c_size_t, []),
+    "sq_decode_fwd_noalloc": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, ctypes.POINTER(DecodeParams), ctypes.c_void_p]),
     "sq_decode_selected_fwd": (ctypes.c_int, [_P] * 8 + [ctypes.POINTER(DecodeParams), ctypes.c_void_p]),
     "sq_kmeans_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int64] * 4),
     "sq_kmeans_train": (ctypes.c_int, [_P, _P, _P, _P, _P, ctypes.c_int32, ctypes.c_void_p]),

@@ -15,10 +15,22 @@
 //   O^T[d, head] += V^T . P^T  on v_mfma_f32_16x16x4_f32 with k = the 4 lane groups g: the A operand is
 //        the fp32 value of one loaded V element, the B operand is the lane's own p -- no transposition,
 //        no LDS, products in fp32 exactly as the reference's `p * v.to(float32)` (:234).
+#include <mutex>
+
 #include "common.hpp"
+
+// Scratch of sq_decode_fwd_noalloc: the split-KV partials of one call, in place of the caller's workspace.  One copy
+// per GPU the library is loaded on, held until the process ends; its contents are the last call's partials.  In host
+// code this name is only a handle for hipGetSymbolAddress; the device address is looked up once per device.
+constexpr size_t kNoAllocScratchBytes = 8u << 20;
+static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
+constexpr int kMaxDevices = 64;
+static void* g_scratch_ptr[kMaxDevices] = {};
+static std::mutex g_scratch_mutex;
 
 namespace sq {
 namespace {
+
 
 constexpr int kD = 128;          // head_dim handled by the kernels (the host pads smaller heads with zeros)
 constexpr int kWaves = 4;
@@ -415,9 +427,11 @@ extern "C" size_t sq_decode_workspace_bytes(int64_t batch, int64_t num_q_heads, 
 
 // Shared body of sq_decode_fwd (token_ids == null) and sq_decode_selected_fwd.  The messages keep the name of the
 // dense entry point for both.
+// Partials go to `workspace`, or, when `own_scratch` is given, to that device buffer of `own_scratch_bytes` bytes.
 static int decode_impl(const DLTensor* q, const DLTensor* kcache, const DLTensor* vcache, const DLTensor* seqlens,
                        const DLTensor* token_ids, DLTensor* out, DLTensor* lse, DLTensor* workspace,
-                       const sq_decode_params* params, void* stream) {
+                       const sq_decode_params* params, void* stream, void* own_scratch = nullptr,
+                       size_t own_scratch_bytes = 0) {
   SQ_REQUIRE(params, SQ_EINVAL, "sq_decode_fwd: params is null");
   SQ_REQUIRE(q && kcache && vcache && out, SQ_EINVAL, "sq_decode_fwd: q, kcache, vcache and out must be non-null");
   SQ_REQUIRE(params->layout == SQ_LAYOUT_HND || params->layout == SQ_LAYOUT_NHD, SQ_EINVAL,
@@ -475,11 +489,22 @@ static int decode_impl(const DLTensor* q, const DLTensor* kcache, const DLTensor
   int64_t chunk = (L + S - 1) / S;
   chunk = (chunk + kTile * kWaves - 1) / (kTile * kWaves) * (kTile * kWaves);
   const size_t need = sq_decode_workspace_bytes(B, Hq, D, S);
-  SQ_REQUIRE(workspace && on_gpu(workspace) && workspace->device.device_id == dev, SQ_EWORKSPACE,
-             "sq_decode_fwd: workspace missing or not on the device");
-  SQ_REQUIRE((size_t)numel_of(workspace) * (workspace->dtype.bits / 8) >= need && is_compact(workspace), SQ_EWORKSPACE,
-             "sq_decode_fwd: workspace too small: need %zu bytes", need);
-  SQ_REQUIRE(((uintptr_t)data_of(workspace) & 15) == 0, SQ_EWORKSPACE, "sq_decode_fwd: workspace not 16-byte aligned");
+  SQ_REQUIRE(S <= 4096, SQ_EINVAL, "sq_decode_fwd: num_splits %d above 4096", S);
+  float* ws_data;
+  if (own_scratch) {
+    SQ_REQUIRE(need <= own_scratch_bytes, SQ_EWORKSPACE,
+               "sq_decode_fwd_noalloc: batch %lld x %lld q heads x %d splits needs %zu bytes of partial results, the library's "
+               "scratch holds %zu; use sq_decode_fwd with a workspace (or fewer splits)",
+               (long long)B, (long long)Hq, S, need, own_scratch_bytes);
+    ws_data = (float*)own_scratch;
+  } else {
+    SQ_REQUIRE(workspace && on_gpu(workspace) && workspace->device.device_id == dev, SQ_EWORKSPACE,
+               "sq_decode_fwd: workspace missing or not on the device");
+    SQ_REQUIRE((size_t)numel_of(workspace) * (workspace->dtype.bits / 8) >= need && is_compact(workspace), SQ_EWORKSPACE,
+               "sq_decode_fwd: workspace too small: need %zu bytes", need);
+    SQ_REQUIRE(((uintptr_t)data_of(workspace) & 15) == 0, SQ_EWORKSPACE, "sq_decode_fwd: workspace not 16-byte aligned");
+    ws_data = (float*)data_of(workspace);
+  }
 
   const int64_t group = Hq / Hkv;
   DecodeArgs a;
@@ -490,7 +515,7 @@ static int decode_impl(const DLTensor* q, const DLTensor* kcache, const DLTensor
   a.ids = token_ids ? (const int32_t*)data_of(token_ids) : nullptr;
   a.ids_sg = token_ids ? stride_of(token_ids, 0) : 0;
   a.cache_len = (int32_t)Lcache;
-  a.part_o = (float*)data_of(workspace);
+  a.part_o = ws_data;
   a.part_lse = a.part_o + (size_t)B * Hq * S * kD;
   a.q_sb = stride_of(q, 0);
   a.q_sh = stride_of(q, hdim);
@@ -554,4 +579,30 @@ extern "C" int sq_decode_selected_fwd(const DLTensor* q, const DLTensor* kcache,
                                       DLTensor* workspace, const sq_decode_params* params, void* stream) {
   SQ_REQUIRE(token_ids, SQ_EINVAL, "sq_decode_selected_fwd: token_ids is null");
   return decode_impl(q, kcache, vcache, seqlens, token_ids, out, lse, workspace, params, stream);
+}
+
+extern "C" size_t sq_decode_noalloc_scratch_bytes(void) { return kNoAllocScratchBytes; }
+
+extern "C" int sq_decode_fwd_noalloc(const DLTensor* q, const DLTensor* kcache, const DLTensor* vcache, const DLTensor* seqlens,
+                                     DLTensor* out, DLTensor* lse, const sq_decode_params* params, void* stream) {
+  SQ_REQUIRE(q, SQ_EINVAL, "sq_decode_fwd_noalloc: q is null");
+  SQ_REQUIRE(on_gpu(q), SQ_EDEVICE, "sq_decode_fwd_noalloc: q is not on a ROCm device");
+  const int dev = q->device.device_id;
+  SQ_REQUIRE(dev >= 0 && dev < kMaxDevices, SQ_EDEVICE, "sq_decode_fwd_noalloc: device id %d out of range", dev);
+  int cur = -1;
+  SQ_HIP(hipGetDevice(&cur));
+  SQ_REQUIRE(cur == dev, SQ_EDEVICE, "sq_decode_fwd_noalloc: tensors live on device %d but the current device is %d", dev, cur);
+  void* ptr;
+  {
+    // every GPU holds its own copy of the array at its own address: looked up once per device, with that device current
+    std::lock_guard<std::mutex> guard(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+      void* p = nullptr;
+      SQ_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+      SQ_REQUIRE(p, SQ_EHIP, "sq_decode_fwd_noalloc: hipGetSymbolAddress returned a null address");
+      g_scratch_ptr[dev] = p;
+    }
+    ptr = g_scratch_ptr[dev];
+  }
+  return decode_impl(q, kcache, vcache, seqlens, nullptr, out, lse, nullptr, params, stream, ptr, kNoAllocScratchBytes);
 }

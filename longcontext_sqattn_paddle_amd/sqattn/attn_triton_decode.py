@@ -45,6 +45,23 @@ def attn_decode(q, k, v, tensor_layout="HND", output_dtype=torch.float16, return
     return (o, lse) if return_lse else o
 
 
+def attn_decode_noalloc(q, k, v, out, tensor_layout="NHD", lse: Optional[torch.Tensor] = None, is_P_fp8_quant=False,
+                        seqlens: Optional[torch.Tensor] = None, num_splits: int = 0):
+    """`attn_decode` for callers that must not allocate device memory (graph capture, serving loops): head_dim 128
+    tensors, caller-provided `out` (shape of q) and optional `lse` (fp32, B*Hq elements); the split-KV partials live
+    in the library's own 8 MiB device array instead of a workspace tensor.  No reference counterpart.  Calls that
+    overlap in time on one GPU share that array and race.  Returns `out`."""
+    if tensor_layout not in N.LAYOUT:
+        raise ValueError(f"tensor_layout {tensor_layout} not supported")
+    require_gpu(q, k, v)
+    if q.size(-1) != 128:
+        raise ValueError("attn_decode_noalloc needs head_dim 128 tensors (padding would allocate)")
+    params = N.DecodeParams(N.LAYOUT[tensor_layout], N.P_E4M3_STATIC if is_P_fp8_quant else N.P_NONE, num_splits, 128)
+    b = [N.dl(t) for t in (q, k, v, seqlens, out, lse)]
+    N.check(N.lib().sq_decode_fwd_noalloc(*[N.ptr(x) for x in b], params, N.current_stream(q.device)))
+    return out
+
+
 def attn_decode_selected(q, k, v, token_ids, tensor_layout="NHD", output_dtype=torch.float16, return_lse=False,
                          is_P_fp8_quant=False, seqlens: Optional[torch.Tensor] = None, num_splits: int = 0,
                          workspace: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None):
