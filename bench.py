@@ -39,17 +39,25 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def time_prefill(torch, N, steps, warmup, p_quant):
+def prefill_inputs(torch, N):
+    """BASELINE config 2's seeded inputs (CPU generator), uploaded once: q [1,28,N,128], k/v [1,4,N,128]."""
     from longcontext_sqattn_paddle_amd import workloads
+
+    dev = torch.device("cuda:0")
+    t0 = time.time()
+    q, k, v = workloads.prefill_inputs(1, 28, 4, N, 128, seed=2)
+    q, k, v = q.to(dev), k.to(dev), v.to(dev)
+    log(f"[bench] prefill inputs N={N} generated and uploaded in {time.time() - t0:.1f}s")
+    return q, k, v
+
+
+def time_prefill(torch, qkv, steps, warmup, p_quant):
     from longcontext_sqattn_paddle_amd.sqattn._prefill import prefill_workspace
     from longcontext_sqattn_paddle_amd.sqattn.attn_triton import attn_causal
 
-    dev = torch.device("cuda:0")
-    Hq, Hkv, D = 28, 4, 128
-    t0 = time.time()
-    q, k, v = workloads.prefill_inputs(1, Hq, Hkv, N, D, seed=2)
-    q, k, v = q.to(dev), k.to(dev), v.to(dev)
-    log(f"[bench] prefill inputs N={N} generated and uploaded in {time.time() - t0:.1f}s")
+    q, k, v = qkv
+    dev = q.device
+    Hq, Hkv, N, D = q.shape[1], k.shape[1], q.shape[2], q.shape[3]
     ws = prefill_workspace(1, Hkv, N, dev)
     out = torch.empty_like(q)
     stream = torch.cuda.current_stream(dev)
@@ -72,6 +80,58 @@ def time_prefill(torch, N, steps, warmup, p_quant):
     chk = out[0, :, -1, :].float()
     assert bool(torch.isfinite(chk).all()) and float(chk.abs().sum()) > 0
     return ms, flops
+
+
+def time_plugin(torch, qkv, steps=3):
+    """The path `ATTN_TYPE=SQAttn` dispatches to (sqattn/attn_replacer.py:423-448): the closure of `mp_triton_wrapper`
+    = operand pre-pass (key centring, int8 fake quantisation) + sink/window kernel with relative windows, at the prefill
+    benchmark shape in the plugin's [B,N,H,D] layout.  Window settings: the reference's shipped default (ratio 0.1 for
+    both windows, sink 256: sqattn/window_search.py:102-104, attn_replacer.py:24) and a wide one (0.25 / 0.5).  For each:
+    the whole closure call and the attention kernel alone on operands quantised beforehand."""
+    import types
+
+    from longcontext_sqattn_paddle_amd import workloads
+    from longcontext_sqattn_paddle_amd.sqattn._prefill import prefill_workspace
+    from longcontext_sqattn_paddle_amd.sqattn.attn_replacer import mp_triton_wrapper
+    from longcontext_sqattn_paddle_amd.sqattn.attn_triton_mix_relative import attn_hierarchical_relative_window, window_tokens
+    from longcontext_sqattn_paddle_amd.sqattn.fake_quant import fused_int_prepass
+
+    q, k, v = (t.permute(0, 2, 1, 3).contiguous() for t in qkv)   # the plugin boundary's layout
+    dev = q.device
+    N, Hq, D = q.shape[1], q.shape[2], q.shape[3]
+    layer = types.SimpleNamespace(num_key_value_groups=Hq // k.shape[2])
+    args = types.SimpleNamespace(qk_qtype="int", v_qtype="int", use_relative_distance=True)
+    ws = prefill_workspace(1, k.shape[2], N, dev)
+    out = {}
+
+    def timed(fn):
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / steps
+
+    for name, r8, r4, sink in (("default_ratio_0.1_sink_256", 0.1, 0.1, 256), ("ratio_0.25_0.5_sink_256", 0.25, 0.5, 256)):
+        closure = mp_triton_wrapper(1, r8, r4, sink, args)
+        call_ms = timed(lambda: closure(layer, q, k, v, None))
+        q8, _, k8, _, v8 = fused_int_prepass(q, k, v, want_4bit=False, tensor_layout="NHD")
+        o = torch.empty_like(q8)
+        kern_ms = timed(lambda: attn_hierarchical_relative_window(q8, k8, q8, k8, v8, r8, r4, sink, "NHD", torch.bfloat16, workspace=ws, out=o))
+        assert bool(torch.isfinite(o[0, -1].float()).all()) and float(o[0, -1].float().abs().sum()) > 0
+        flops = workloads.window_flops(N, D, sink, [window_tokens(r8, N)] * Hq, [window_tokens(r4, N)] * Hq, 64)
+        tf = flops / kern_ms / 1e9
+        out[name] = {"window_tokens": [window_tokens(r8, N), window_tokens(r4, N)], "flops": flops,
+                     "fraction_of_full_causal_flops": round(flops / (4.0 * N * N * D * Hq / 2), 4),
+                     "plugin_call_ms": round(call_ms, 3), "kernel_ms": round(kern_ms, 3),
+                     "roofline": {"bound": "mfma", "kernel": "prefill_kernel (sink + windows, fp16 P.V)", "achieved": round(tf, 1),
+                                  "peak": PEAK_MFMA_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / PEAK_MFMA_BF16_TFLOPS, 4)}}
+        del q8, k8, v8, o
+        torch.cuda.empty_cache()
+    return out
 
 
 def time_decode(torch, B, L, iters=10, warmup=5, rounds=7):
@@ -422,47 +482,57 @@ def time_calibration(torch, N, iters=3):
 
 
 def time_kmeans(torch, iters=10):
-    """One Lloyd iteration (assign + counting sort + exact cluster sums + centroid update) at the benchmark's
-    clustering shape: 4 kv heads x 131072 tokens x 128, 1024 centroids."""
+    """BASELINE config 4 at its shape (4 kv heads x 131072 tokens x 128, 1024 centroids): one Lloyd iteration (assign +
+    counting sort + exact cluster sums + centroid update), the whole `segment_k_means` of 10 iterations with its value sums
+    and reverse index, and the top-k selection behind it.  Two key sets alternate, so that a 134 MB key tensor does not
+    simply stay in the 256 MB Infinity Cache between iterations."""
     from longcontext_sqattn_paddle_amd import workloads
-    from longcontext_sqattn_paddle_amd.cache_hub.kmeans import _triton_k_means_train, _workspace
+    from longcontext_sqattn_paddle_amd.cache_hub.kmeans import _triton_k_means_train, _workspace, segment_k_means, topk_select
 
     dev = torch.device("cuda:0")
     G, N, C, D = 4, 131072, 1024, 128
-    key, _ = workloads.kmeans_inputs(G, N, D, seed=4)
-    key = key.to(dev)
     idx0 = (torch.arange(C, dtype=torch.float32) * (N / C) + N / C / 2).to(torch.int64).to(dev)
-    cent = key.index_select(1, idx0).contiguous()
+    sets = []
+    for seed in (4, 5):
+        key, value = workloads.kmeans_inputs(G, N, D, seed=seed)
+        key, value = key.to(dev), value.to(dev)
+        sets.append((key, value, key.index_select(1, idx0).contiguous()))
     ws = _workspace(G, N, C, dev)
     idx = torch.empty(G, N, dtype=torch.int32, device=dev)
-    for _ in range(2):
-        _triton_k_means_train(key, cent, max_idx=idx, workspace=ws)
+    for i in range(4):
+        _triton_k_means_train(sets[i % 2][0], sets[i % 2][2], max_idx=idx, workspace=ws)
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
-    for _ in range(iters):
-        _triton_k_means_train(key, cent, max_idx=idx, workspace=ws)
+    for i in range(iters):
+        _triton_k_means_train(sets[i % 2][0], sets[i % 2][2], max_idx=idx, workspace=ws)
     e1.record()
     torch.cuda.synchronize()
     us = e0.elapsed_time(e1) / iters * 1e3
     flops = 2.0 * N * C * D * G
-    nbytes = G * (N * D * 2 * 2 + N * 4 * 3 + C * D * 2 * 2)   # K read by assign and by the cluster sums, idx/order, centroids
-    # the selection that follows the clustering in the benchmark configuration: top-k = 4096 tokens for a 28-head query
-    from longcontext_sqattn_paddle_amd.cache_hub.kmeans import segment_k_means, topk_select
-
-    cent2, _, clusters, size = segment_k_means(key, key, C, num_iters=3)
+    nbytes = G * (N * D * 2 + N * 4 + C * D * 2 * 2 + C * 4)   # keys read once, assignment written, centroids read and written, counts
+    # the configuration as written: 10 Lloyd iterations (9 normalised + the final one), value sums, reverse index, then top-k
+    full = []
+    for i in range(4):
+        key, value, _ = sets[i % 2]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        cent, _, clusters, size = segment_k_means(key, value, C, num_iters=10)
+        torch.cuda.synchronize()
+        full.append((time.perf_counter() - t0) * 1e3)
+    assert int(size.sum()) == G * N
     q = torch.randn(1, 28, D, device=dev, generator=torch.Generator(device=dev).manual_seed(9)).bfloat16()
     out = torch.empty(G, 4096, dtype=torch.int32, device=dev)
     for _ in range(3):
-        topk_select(q, cent2, clusters, size, 4096, 7, out=out, workspace=ws)
+        topk_select(q, cent, clusters, size, 4096, 7, out=out, workspace=ws)
     torch.cuda.synchronize()
     e0.record()
     for _ in range(20):
-        topk_select(q, cent2, clusters, size, 4096, 7, out=out, workspace=ws)
+        topk_select(q, cent, clusters, size, 4096, 7, out=out, workspace=ws)
     e1.record()
     torch.cuda.synchronize()
     assert int(out.min()) >= 0 and int(out.max()) < N
-    return us, flops, nbytes, e0.elapsed_time(e1) / 20 * 1e3
+    return us, flops, nbytes, e0.elapsed_time(e1) / 20 * 1e3, sorted(full[1:])[1]
 
 
 def time_prepass(torch, N, want4, iters=10):
@@ -503,7 +573,8 @@ def main():
                          "3 e4m3 static 448 with the scale folded into the exponent, "
                          "4 = 3 plus e4m3 V so that P.V runs on the fp8 matrix pipe, "
                          "5 (default) = 4 with one power-of-two block scale per query row and 64-key tile on P")
-    ap.add_argument("--variants", action="store_true", help="also time P modes 1 and 3 (fp16 P.V) and report them")
+    ap.add_argument("--no-variants", action="store_true", help="skip the other P modes (0 - 4) of the prefill kernel")
+    ap.add_argument("--no-plugin", action="store_true", help="skip the plugin closure (pre-pass + sink/window kernel)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="run one 1 GiB device-to-device copy first: a kernel of known traffic for scaling FETCH_SIZE/WRITE_SIZE")
     ap.add_argument("--no-kmeans", action="store_true")
@@ -540,7 +611,8 @@ def main():
         torch.cuda.synchronize()
         del src, dst
         torch.cuda.empty_cache()
-    ms, flops = time_prefill(torch, N, args.steps, args.warmup, args.p_quant)
+    qkv = prefill_inputs(torch, N)
+    ms, flops = time_prefill(torch, qkv, args.steps, args.warmup, args.p_quant)
     tflops = flops / ms / 1e9
     log(f"[bench] prefill N={N}: {ms:.2f} ms/step, {tflops:.1f} TFLOP/s")
     if args.p_quant >= 4:
@@ -577,17 +649,35 @@ def main():
             "frac": round(tflops / peak, 4),
             "frac_of_bf16_peak": round(tflops / PEAK_MFMA_BF16_TFLOPS, 4),
             "traffic": PREFILL_TRAFFIC_BYTES_128K if (N == 131072 and args.p_quant >= 4) else None,
+            "traffic_note": "bytes per launch through the L2/fabric interface, a constant taken from the committed rocprofv3 FETCH_SIZE / "
+                            "WRITE_SIZE runs of this shape (profiles/prefill_kernel_128k.md), not re-measured by this run; null for other shapes",
+            "numerics": "P mode 5 is build-defined (the reference multiplies fp16 P by fp16 V): see `variants` for the reference's own modes",
         },
     }
-    if args.variants:
+    if not args.no_variants:
+        # the reference's own numerics (modes 0 and 1) and the other P modes, a few steps each: the kernel is the same,
+        # only the quantisation of P (and of V in mode 4) differs.  Each entry is priced against the peak of the matrix
+        # pipes it uses.
         result["variants"] = {}
-        for mode, name in ((4, "e4m3_P_static_scale_fp8_PV"), (3, "e4m3_P_fp16_PV"), (1, "e4m3_P_reference_rounding_fp16_PV")):
-            vms, _ = time_prefill(torch, N, args.steps, args.warmup, mode)
-            result["variants"][name] = {"p_quant": mode, "ms_per_step": round(vms, 3), "TFLOP_per_s": round(flops / vms / 1e9, 1)}
-            log(f"[bench] prefill variant {name}: {vms:.2f} ms")
+        for mode, name, note in ((0, "no_P_quant_fp16_PV", "attn_triton.py:83, is_P_fp8_quant=False (the reference's default)"),
+                                 (1, "e4m3_P_reference_rounding_fp16_PV", "attn_triton.py:81-82 op for op: fp16(fp16(e4m3(448 p)) / 448)"),
+                                 (3, "e4m3_P_folded_scale_fp16_PV", "the same e4m3 grid, 448 folded into the exponent (build-defined)"),
+                                 (2, "e4m3_P_block_absmax_fp16_PV", "per 64x64 block absmax scale on P (build-defined, BASELINE config 1)"),
+                                 (4, "e4m3_P_static_scale_fp8_PV", "e4m3 V and fp8 MFMA P.V with the static scale 448 (build-defined)")):
+            vms, _ = time_prefill(torch, qkv, 3, 1, mode)
+            vpeak = PEAK_MFMA_BLEND_TFLOPS if mode >= 4 else PEAK_MFMA_BF16_TFLOPS
+            vt = flops / vms / 1e9
+            result["variants"][name] = {"p_quant": mode, "ms_per_step": round(vms, 3), "TFLOP_per_s": round(vt, 1),
+                                        "peak": round(vpeak, 1), "frac": round(vt / vpeak, 4), "numerics": note}
+            log(f"[bench] prefill variant {name}: {vms:.2f} ms = {vt:.0f} TFLOP/s = {vt / vpeak:.3f} of {vpeak:.0f}")
+    if not args.no_plugin:
+        result["plugin"] = time_plugin(torch, qkv)
+        log(f"[bench] plugin closure: {result['plugin']}")
+    del qkv
+    torch.cuda.empty_cache()
     if not args.no_decode:
         dec = {}
-        for name, B, L in (("1M_b1", 1, 1048576), ("128K_b1", 1, 131072), ("128K_b8", 8, 131072)):
+        for name, B, L in (("1M_b1", 1, 1048576), ("128K_b1", 1, 131072), ("128K_b4", 4, 131072), ("128K_b8", 8, 131072)):
             us, nbytes = time_decode(torch, B, L)
             gbs = nbytes / us / 1e3
             dec[name] = {"us_per_call": round(us, 2), "GB_per_s": round(gbs, 1), "frac_of_hbm_peak": round(gbs / PEAK_HBM_GBS, 4),
@@ -654,28 +744,50 @@ def main():
         result["e2e"] = [time_e2e(torch, N, new_tokens=args.e2e_new_tokens, graph=args.e2e_graph, **runs[r]) for r in args.e2e_runs.split(",")]
         log(f"[bench] end to end: {result['e2e']}")
     if not args.no_kmeans:
-        us, kflops, kbytes, topk_us = time_kmeans(torch)
+        us, kflops, kbytes, topk_us, full_ms = time_kmeans(torch)
+        t_mfma, t_hbm = kflops / PEAK_MFMA_BF16_TFLOPS / 1e6, kbytes / PEAK_HBM_GBS / 1e3
         result["kmeans"] = {"us_per_iteration": round(us, 1), "TFLOP_per_s": round(kflops / us / 1e6, 1),
                             "frac_of_bf16_mfma_peak": round(kflops / us / 1e6 / PEAK_MFMA_BF16_TFLOPS, 4),
                             "GB_per_s": round(kbytes / us / 1e3, 1), "frac_of_hbm_peak": round(kbytes / us / 1e3 / PEAK_HBM_GBS, 4),
-                            "shape": "4 heads x 131072 tokens x 128, 1024 centroids, one Lloyd iteration",
+                            "bound_us": round(max(t_mfma, t_hbm), 1), "frac_of_bound": round(max(t_mfma, t_hbm) / us, 4),
+                            "bytes": kbytes, "flops": kflops,
+                            "shape": "4 heads x 131072 tokens x 128, 1024 centroids, one Lloyd iteration, two key sets alternating",
+                            "segment_k_means_10_iterations_ms": round(full_ms, 3),
+                            "segment_k_means_note": "10 iterations + value sums + reverse index, host wall clock including its one host "
+                                                    "synchronisation (the reference's Cnt.max().item(), cache_hub/kmeans.py:195)",
                             "topk_select_us": round(topk_us, 1),
                             "topk_shape": "4096 tokens per kv head for one 28-head query, 1024 clusters per kv head"}
         log(f"[bench] kmeans iteration: {us:.0f} us")
     if not args.no_cpu_baseline:
-        from oracle.cpu_baseline import time_cpu_baseline   # the checker's CPU path, timed as the baseline only
+        from oracle import cpu_baseline as CB   # the checker's CPU path, timed as the baseline only
 
-        cpu_tflops, threads, dt, n = time_cpu_baseline(budget_s=12.0)
+        cpu_tflops, threads, dt, n = CB.time_cpu_baseline(budget_s=6.0)
+        one_tflops, _, one_dt, one_n = CB.time_cpu_baseline(budget_s=4.0, threads=1)
+        pts, extrap_s = CB.time_prefill_points()
+        dec_gbs, dec_dt = CB.time_decode_cpu()
+        km_dt, km_tflops = CB.time_kmeans_iteration_cpu()
         result["cpu_baseline"] = {
             "value": round(cpu_tflops, 4),
             "unit": "TFLOP/s",
             "cores": threads,
             "kind": "port",
+            "cpu": f"{CB.cpu_model()}, {os.cpu_count()} logical CPUs visible, torch intra-op threads {threads}",
             "sample": f"config-1 shape (batch 1, 4 q heads on 1 kv head, head_dim 128, seq 4096, causal): GQA expand, K centring, "
                       f"int8/int4 fake-quant, torch CPU SDPA in bf16; {n} passes of {dt * 1e3:.1f} ms on {threads} threads "
                       f"({os.cpu_count()} logical CPUs)",
+            "one_thread": {"value": round(one_tflops, 4), "unit": "TFLOP/s", "cores": 1, "sample": f"the same shape, {one_n} passes of {one_dt * 1e3:.1f} ms"},
+            "config2_prefill_points": {"points": pts, "cores": threads,
+                                       "extrapolated_seconds_at_131072_tokens_28_heads": round(extrap_s, 1),
+                                       "note": "4 of the 28 query heads (one kv head) timed once per length, attention in 2048-row query chunks; "
+                                               "the 131072-token figure is EXTRAPOLATED from the largest point by (N ratio)^2 x 7, not measured"},
+            "config3_decode_128K_b1": {"value": round(dec_gbs, 2), "unit": "GB/s", "cores": threads, "seconds_per_call": round(dec_dt, 5),
+                                       "sample": "one query token, 28/4 heads, full 131072-token bf16 cache, 5 calls"},
+            "config4_kmeans_iteration": {"value": round(km_tflops, 4), "unit": "TFLOP/s", "cores": threads,
+                                         "seconds_per_iteration_4_heads": round(4 * km_dt, 3),
+                                         "sample": "one Lloyd iteration of one head (131072 x 128 keys, 1024 centroids, fp32), timed once, x 4 heads"},
         }
-        log(f"[bench] cpu baseline: {cpu_tflops:.3f} TFLOP/s on {threads} threads")
+        log(f"[bench] cpu baseline: {cpu_tflops:.3f} TFLOP/s on {threads} threads, {one_tflops:.3f} on one; C2 points {pts}; "
+            f"decode {dec_gbs:.1f} GB/s; k-means iteration {4 * km_dt:.2f} s")
     print(json.dumps(result), flush=True)
 
 

@@ -58,3 +58,19 @@ def kmeans_inputs(G=4, N=131072, D=128, *, n_modes=512, sigma=0.3, seed=4, dtype
     key = torch.gather(mu, 1, which[..., None].expand(G, N, D)) + sigma * torch.randn(G, N, D, generator=g)
     value = torch.randn(G, N, D, generator=g)
     return key.to(dtype), value.to(dtype)
+
+
+def window_flops(N: int, D: int, sink: int, w8, w4, block_m: int = 64) -> float:
+    """Algorithmic FLOPs of one sink + window prefill call: 4 * D * sum over heads and query blocks of
+    (rows x keys visited), the diagonal block counted as its causal half.  `w8` / `w4` are the per-head window sizes in
+    tokens; the key ranges are those of the reference's kernels (sink, 4-bit window, 8-bit window, own block:
+    sqattn/attn_triton_mix_relative.py:36-75)."""
+    total = 0.0
+    for a8, a4 in zip(w8, w4):
+        for qs in range(0, N, block_m):
+            qe = qs + block_m
+            rows = min(qe, N) - qs
+            left4, left8 = max(sink, qe - a4), max(sink, qe - a8)
+            keys = min(sink, qs) + max(left8 - left4, 0) + max(qs - left8, 0)
+            total += rows * keys + rows * (rows + 1) / 2
+    return 4.0 * D * total
