@@ -1109,6 +1109,9 @@ extern "C" int sq_prefill_fwd(const DLTensor* q, const DLTensor* k, const DLTens
              "qo_len and kv_len must be equal for causal attention (q_offset + qo_len = %lld, kv_len = %lld)",
              (long long)(p->q_offset + Nq), (long long)Nk);
   SQ_REQUIRE(Nk < (1ll << 31) - 65536, SQ_EUNSUPPORTED, "sq_prefill_fwd: more than 2^31 keys");
+  // a 64-key tile is copied with one 64-bit tile base and 32-bit per-lane byte offsets: a tile must span less than 4 GiB
+  SQ_REQUIRE(stride_of(k, ndim) > 0 && stride_of(k, ndim) < (1ll << 24) && stride_of(v, ndim) > 0 && stride_of(v, ndim) < (1ll << 31), SQ_EUNSUPPORTED,
+             "sq_prefill_fwd: token stride of k must be below 2^24 elements (got %lld)", (long long)stride_of(k, ndim));
   const DLTensor* ts[5] = {q, k, v, out, nullptr};
   for (int t = 0; t < 4; ++t)
     for (int i = 0; i < 3; ++i)

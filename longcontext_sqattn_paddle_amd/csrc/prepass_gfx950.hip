@@ -299,6 +299,9 @@ extern "C" int sq_fake_quant_prepass(const DLTensor* query, const DLTensor* key,
   const int64_t B = query->shape[0], N = query->shape[nd], Hq = query->shape[hd], Hkv = key->shape[hd];
   SQ_REQUIRE(B > 0 && N > 0 && Hq > 0 && Hkv > 0, SQ_ESHAPE, "sq_fake_quant_prepass: empty tensor");
   SQ_REQUIRE(B * N * Hq < (int64_t)1 << 40 && B * Hkv * kPD < (int64_t)1 << 24, SQ_EUNSUPPORTED, "sq_fake_quant_prepass: tensor too large");
+  // the kernels index tokens with 32-bit integers and the launches take 32-bit grid sizes (32 rows per workgroup)
+  SQ_REQUIRE(N < ((int64_t)1 << 31) - 65536 && B < ((int64_t)1 << 20) && B * N * Hq / 32 < ((int64_t)1 << 31) - 1, SQ_EUNSUPPORTED,
+             "sq_fake_quant_prepass: more than 2^31 tokens per sequence or 2^36 query rows");
   PrepassArgs a;
   memset(&a, 0, sizeof(a));
   if ((rc = make_view(query, "query", layout, dev, dt, B, N, Hq, &a.q)) || (rc = make_view(key, "key", layout, dev, dt, B, N, Hkv, &a.k)) ||

@@ -155,14 +155,53 @@ def mp_triton_wrapper(layer_idx, bit8_window_sizes=0, bit4_window_sizes=0, sink_
     return attention_fn
 
 
+def construct_mix_bit_mask(kv_len, bit8_window_sizes, bit4_window_sizes, sink_window_size, device):
+    """attn_replacer.py:63-112 (`construct_mix_bit_mask` and its per-head variant, called with seq_len = 2 * kv_len):
+    bool [kv_len, 2 kv_len] (or [H, kv_len, 2 kv_len] for per-head lists), True = attend; columns [0, kv_len) are the
+    8-bit keys, [kv_len, 2 kv_len) their 4-bit copies."""
+    L = 2 * kv_len
+    q_idx = torch.arange(L, device=device).unsqueeze(1)
+    kv_idx = torch.arange(L, device=device).unsqueeze(0)
+    w8, w4 = bit8_window_sizes, bit4_window_sizes
+    if isinstance(w8, list) or isinstance(w4, list):
+        w8 = torch.tensor(w8, device=device).view(-1, 1, 1)
+        w4 = torch.tensor(w4, device=device).view(-1, 1, 1)
+        q_idx, kv_idx = q_idx.unsqueeze(0), kv_idx.unsqueeze(0)
+    fp8_mask = (kv_idx <= q_idx) & ((kv_idx < sink_window_size) | (kv_idx > q_idx - w8))
+    kv_idx_4bit = kv_idx - L // 2
+    int4_mask = (kv_idx_4bit >= sink_window_size) & (kv_idx_4bit <= q_idx - w8) & (kv_idx_4bit > q_idx - w8 - w4)
+    is_bit8_part = kv_idx < L // 2
+    return ((is_bit8_part & fp8_mask) | (~is_bit8_part & int4_mask))[..., : L // 2, :]
+
+
 def delayed_sdpa_wrapper(layer_idx, bit8_window_sizes=0, bit4_window_sizes=0, sink_window_size=0, args=None):
-    """attn_replacer.py:36-250: the masked-SDPA emulation.  The reference's quantised branch is unfinished
-    (it stops in a debugger, :187-189); only its plain branch (`args.quant` false) is meaningful and kept."""
+    """attn_replacer.py:36-250: the masked-SDPA emulation of the mixed-precision windows, on dense [L, 2L] masks (a tool
+    for short sequences).  q, k, v are [B, H, L, D] here, heads already expanded as the reference's branch assumes.
+    Plain branch (`args.quant` false): SDPA with the caller's mask.  Quantised branch: the reference builds the
+    concatenated operands and the mask, then passes the unconcatenated operands to SDPA and stops in a debugger
+    (:173-189); this closure finishes what it sets up -- the 8-bit queries attend to [8-bit keys ; 4-bit keys] with values
+    [v8 ; v8] under the mask -- and returns [B, L, H * D]."""
+    bit8_window_sizes, bit4_window_sizes = _normalise_windows(bit8_window_sizes, bit4_window_sizes)
 
     def attention_fn(module, q, k, v, attn_mask, dropout=0.0, scaling=1.0, sliding_window=None, **kwargs):
-        if getattr(args, "quant", False):
-            raise NotImplementedError("the reference's quantised masked-SDPA emulation is unfinished (pdb.set_trace)")
-        return sdpa_attention_forward(module, q, k, v, attention_mask=attn_mask, dropout=dropout, scaling=scaling, **kwargs)
+        if not getattr(args, "quant", False):
+            return sdpa_attention_forward(module, q, k, v, attention_mask=attn_mask, dropout=dropout, scaling=scaling, **kwargs)
+        q_len, kv_len = q.shape[2], k.shape[2]
+        k = k - k.mean(dim=2, keepdim=True)
+        bit8_qk, bit4_qk, _ = _quantizers(args)
+        if args.v_qtype == "int":
+            bit8_v = IntegerQuantizer(8, False, "per_channel")          # this branch quantises V asymmetrically (:141)
+        else:
+            bit8_v = FloatQuantizer(args.v_qtype, True, "per_channel")
+        q_bit8 = bit8_qk.fake_quant_tensor(q)
+        k_bit8_bit4 = torch.cat([bit8_qk.fake_quant_tensor(k), bit4_qk.fake_quant_tensor(k)], dim=2)
+        v_bit8 = bit8_v.fake_quant_tensor(v)
+        v_bit8_bit8 = torch.cat([v_bit8, v_bit8], dim=2)
+        mask = construct_mix_bit_mask(kv_len, bit8_window_sizes, bit4_window_sizes, sink_window_size, q.device)[..., -q_len:, :]
+        if mask.ndim == 3:
+            mask = mask[None]
+        return sdpa_attention_forward(None, q_bit8, k_bit8_bit4, v_bit8_bit8, attention_mask=mask, dropout=dropout, scaling=scaling,
+                                      is_causal=False, tensor_layout="HND")
 
     return attention_fn
 

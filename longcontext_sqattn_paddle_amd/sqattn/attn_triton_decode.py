@@ -124,15 +124,30 @@ class DecodePlan:
 def attn_unified(q, k, v, tensor_layout="HND", output_dtype=torch.float16, return_lse=False, is_P_fp8_quant=False):
     """Unified interface (attn_triton_decode.py:244-361).
 
-    Decode: the per-channel K-mean subtraction of the reference (:268-269) is skipped, it shifts all
-    scores of a row equally and cannot change the softmax.  Prefill: K is centred with tensor ops as in
+    Decode: the per-channel K-mean subtraction of the reference (:268-269) is skipped in the kernel, it shifts all
+    scores of a row equally and cannot change the softmax; a returned log-sum-exp is moved into the reference's frame
+    (scores of the centred keys) afterwards.  Prefill: K is centred with tensor ops as in
     the reference (the bf16 rounding of the centred K is part of its result), then the prefill kernel runs.
     """
     if tensor_layout not in N.LAYOUT:
         raise ValueError(f"tensor_layout {tensor_layout} not supported")
     seq_dim = 1 if tensor_layout == "NHD" else 2
     if q.size(seq_dim) == 1:
-        return attn_decode(q, k, v, tensor_layout, output_dtype, return_lse, is_P_fp8_quant)
+        res = attn_decode(q, k, v, tensor_layout, output_dtype, return_lse, is_P_fp8_quant)
+        if not return_lse:
+            return res
+        # The reference subtracts the keys' token mean before the kernel (:268-269): the output is unchanged, but every
+        # score of a row, and with it the returned base-2 log-sum-exp, is lower by q~ . mean(k) (q~ = q * log2e / sqrt(D)
+        # rounded to the tensor dtype).  Put the log-sum-exp into that frame, the one the prefill branch below is in.
+        o, lse = res
+        head_dim = q.size(-1)
+        sm = torch.tensor(1.0 / head_dim ** 0.5 * 1.44269504, dtype=torch.float32, device=q.device)
+        q_folded = (q.float() * sm).to(q.dtype).float()
+        k_mean = k.float().mean(dim=seq_dim)                                   # [B, Hkv, D]
+        qh = q_folded.squeeze(seq_dim)                                         # [B, Hq, D]
+        groups = qh.size(1) // k_mean.size(1)
+        shift = (qh.view(qh.size(0), k_mean.size(1), groups, head_dim) * k_mean[:, :, None, :]).sum(-1).reshape(lse.shape)
+        return o, lse - shift
     from .attn_triton import attn_causal as _prefill
 
     k = k - k.mean(dim=seq_dim, keepdim=True)

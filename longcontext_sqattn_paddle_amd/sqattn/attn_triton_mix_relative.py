@@ -11,7 +11,7 @@ import numpy as np
 import torch
 
 from .. import _native as N
-from ._prefill import per_head, run_prefill
+from ._prefill import align_windows, per_head, run_prefill
 
 
 def window_tokens(ratio: float, kv_len: int) -> int:
@@ -32,9 +32,11 @@ def attn_hierarchical_relative_window(q_int8, k_int8, q_int4, k_int4, v, int8_wi
     r4 = per_head(int4_window_ratios, H, "int4_window_ratios")
     if not isinstance(sink_size, int) or sink_size < 0:
         raise ValueError(f"sink_size must be a non-negative integer, got {sink_size}")
-    window = {"block_m": 64, "sink": sink_size,
-              "w8": [window_tokens(float(r), kv_len) for r in r8],
-              "w4": [window_tokens(float(r), kv_len) for r in r4]}
+    # (ratios already give multiples of 128; the sink is rounded up to a 64-key block, and an 8-bit ratio of zero under
+    # a wider 4-bit window gets the query block, see align_windows)
+    w8, w4, sink_size = align_windows([window_tokens(float(r), kv_len) for r in r8], [window_tokens(float(r), kv_len) for r in r4],
+                                      sink_size, 64)
+    window = {"block_m": 64, "sink": sink_size, "w8": w8, "w4": w4}
     mode = p_quant if p_quant is not None else (N.P_E4M3_STATIC if is_P_fp8_quant else N.P_NONE)
     return run_prefill(q_int8, k_int8, v, tensor_layout=tensor_layout, output_dtype=output_dtype,
                        return_lse=return_lse, p_quant=mode, window=window, workspace=workspace, out=out)

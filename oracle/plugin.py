@@ -82,3 +82,46 @@ def plugin_attention(query, key, value, *, num_kv_groups, bit8, bit4, sink, rela
         out, _ = A.prefill_blockwise(q8, k8, v8, p_quant=p_quant, block_m=128, sink=sink,
                                      w8=[int(x) for x in b8], w4=[int(x) for x in b4], q4=q4, k4=k4)
     return out.transpose(1, 2).contiguous().view(B, N, Hq * D)
+
+
+# ------------------------------------------------------- masked-SDPA emulation (delayed_sdpa_wrapper, attn_replacer.py:36-250)
+def mix_bit_mask(kv_len: int, bit8_window, bit4_window, sink: int) -> torch.Tensor:
+    """`construct_mix_bit_mask` / `construct_mix_bit_mask_per_head` (attn_replacer.py:63-112) called with
+    `seq_len = 2 * kv_len` as the closure does (:152-165): a bool mask [kv_len, 2 * kv_len] (per head: [H, kv_len,
+    2 * kv_len] when the windows are lists), True = attend.  Columns [0, kv_len) are the 8-bit keys, columns
+    [kv_len, 2 kv_len) the 4-bit copies of the same keys.  Row i attends 8-bit key j iff j <= i and (j < sink or
+    j > i - w8), and the 4-bit copy of key j iff j >= sink and i - w8 - w4 < j <= i - w8."""
+    per_head = isinstance(bit8_window, (list, tuple)) or isinstance(bit4_window, (list, tuple))
+    L = 2 * kv_len
+    if per_head:
+        w8 = torch.tensor(bit8_window).view(-1, 1, 1)
+        w4 = torch.tensor(bit4_window).view(-1, 1, 1)
+        q_idx = torch.arange(L).view(1, L, 1)
+        kv_idx = torch.arange(L).view(1, 1, L)
+    else:
+        w8, w4 = bit8_window, bit4_window
+        q_idx = torch.arange(L).unsqueeze(1)
+        kv_idx = torch.arange(L).unsqueeze(0)
+    causal = kv_idx <= q_idx
+    fp8 = causal & ((kv_idx < sink) | (kv_idx > q_idx - w8))
+    kv4 = kv_idx - L // 2
+    int4 = (kv4 >= sink) & (kv4 <= q_idx - w8) & (kv4 > q_idx - w8 - w4)
+    is8 = kv_idx < L // 2
+    final = (is8 & fp8) | (~is8 & int4)
+    return final[..., : L // 2, :]
+
+
+def masked_sdpa_emulation(q, k, v, *, bit8_window, bit4_window, sink, qk_qtype="int", v_qtype="int"):
+    """What the quantised branch of `delayed_sdpa_wrapper`'s closure sets out to compute (attn_replacer.py:123-186; the
+    reference's own call passes the unconcatenated operands with the [L, 2L] mask and then stops in a debugger, :173-189):
+    exact softmax attention of the 8-bit queries over the concatenation [8-bit keys ; 4-bit keys] with the values
+    [v8 ; v8] under `mix_bit_mask`.  q, k, v [B,H,L,D] (heads already expanded).  K is centred over tokens first; V uses
+    the asymmetric 8-bit per-channel quantiser of this branch (:141).  fp64, returns [B,H,L,D]."""
+    kc = k - k.mean(dim=2, keepdim=True)
+    q8 = _qk_quant(q, qk_qtype, 8)
+    k8, k4 = _qk_quant(kc, qk_qtype, 8), _qk_quant(kc, qk_qtype, 4)
+    v8 = FQ.int_fake_quant(v, 8, False, "per_channel") if v_qtype == "int" else FQ.float_fake_quant(v, v_qtype, "per_channel")
+    L = k.shape[2]
+    mask = mix_bit_mask(L, bit8_window, bit4_window, sink)[..., -q.shape[2]:, :]
+    out, _ = A.exact_attention(q8, torch.cat([k8, k4], dim=2), torch.cat([v8, v8], dim=2), mask=mask if mask.ndim == 2 else mask[None])
+    return out

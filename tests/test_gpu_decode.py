@@ -261,3 +261,31 @@ def test_full_size_decode_against_closed_form(B, L):
             rms = float(ref.pow(2).mean().sqrt())
             assert float((got - ref).abs().max()) <= 2e-4 * rms + 1e-6
             assert torch.allclose(lse[b, kvh * 7:(kvh + 1) * 7, 0].cpu().double(), ref_lse, atol=2e-4)
+
+
+@pytest.mark.parametrize("layout", ["NHD", "HND"])
+def test_attn_unified_decode_lse_is_in_the_frame_of_the_centred_keys(layout):
+    """`attn_unified` subtracts the keys' token mean before its kernel (attn_triton_decode.py:268-269), so the
+    log-sum-exp it returns is that of the centred keys' scores; the prefill branch of the same function is in that
+    frame too.  The decode kernel here skips the subtraction (the output cannot change) and the wrapper moves the
+    log-sum-exp: it must equal the closed form over exactly centred keys (the reference rounds the centred keys to
+    the tensor dtype, which moves a score by about 3e-3 here and is not reproduced; tolerance 2e-3 against the
+    unrounded closed form, where 1.1 would be the error of not shifting at all)."""
+    from longcontext_sqattn_paddle_amd.sqattn.attn_triton_decode import attn_unified
+
+    print(f"case attn_unified decode lse {layout}", flush=True)
+    dev = torch.device("cuda:0")
+    q, kc, vc, _ = inputs.decode_inputs(2, 28, 4, 2000, 128, seed=77)
+    kc = (kc.float() + torch.linspace(-1.0, 1.0, 128)).bfloat16()        # a key mean worth noticing
+    qh, kh, vh = _to_hnd(q, kc, vc)
+    centred = kh.double() - kh.double().mean(dim=2, keepdim=True)
+    ref, lse_ref = A.exact_attention(A.fold_scale(qh, 128).double(), centred, vh.double(), causal=False, score_scale=math.log(2.0))
+    _, lse_plain = A.exact_attention(A.fold_scale(qh, 128), kh, vh, causal=False, score_scale=math.log(2.0))
+    assert float((lse_plain - lse_ref).abs().max()) > 0.5               # the two frames really differ on this input
+    args = (q, kc, vc) if layout == "NHD" else (qh, kh, vh)
+    out, lse = attn_unified(*[t.to(dev) for t in args], layout, torch.float32, return_lse=True)
+    torch.cuda.synchronize()
+    out = out.cpu()
+    out = out[:, 0] if layout == "NHD" else out[:, :, 0]
+    assert float((out.double() - ref[:, :, 0]).abs().max()) < 2e-4 * float(ref.pow(2).mean().sqrt()) + 1e-6
+    assert torch.allclose(lse.cpu().double().view(2, 28), lse_ref[:, :, 0], atol=2e-3)

@@ -85,6 +85,23 @@ def test_plugin_closure_matches_oracle(relative, bit8, bit4):
     assert float((o - r).abs().max()) <= 2 ** -7 * float(r.abs().max()) + 2e-3 * rms
 
 
+def test_process_model_takes_the_window_sizes_the_reference_calibration_writes():
+    """The reference's window search returns 1 token when a head's histogram is empty and the histogram's length when the
+    threshold is never reached (sqattn/window_search.py:90-128), and its configuration keeps a 256-token sink: a
+    configuration like that must run (sizes rounded as documented: 1 -> 128, 1000 -> 1024), not raise."""
+    from longcontext_sqattn_paddle_amd.sqattn.attn_replacer import process_model
+
+    q, k, v = inputs.plugin_inputs(1, 4, 1, 1536, 128, seed=3)
+    m = _Model(2, 4)
+    process_model(m, "SQAttn", {1: {"bit8": [1, 1, 1000, 5000], "bit4": [1, 1000, 1000, 5000], "sink": 256}}, _args(False))
+    out = m.layers[1].prefill_attention(q.to(DEV), k.to(DEV), v.to(DEV), None)
+    torch.cuda.synchronize()
+    ref = plugin.plugin_attention(q, k, v, num_kv_groups=4, bit8=[128, 128, 1024, 5120], bit4=[128, 1024, 1024, 5120], sink=256, relative=False)
+    o, r = out.float().cpu(), ref.float()
+    assert _cos(o, r) >= 0.99999
+    assert float((o - r).abs().max()) <= 2 ** -7 * float(r.abs().max()) + 2e-3 * float(r.pow(2).mean().sqrt())
+
+
 def test_config1_full_causal_with_block_fp8_p():
     """Benchmark configuration 1: seq 4096, 4 q-heads on 1 kv head, int8 fake-quant, windows >= N (full causal),
     P quantised to e4m3 with per-64x64-block absmax scales (a mode the reference closure itself never enables)."""

@@ -74,3 +74,67 @@ def test_calibration_host_logic_without_a_gpu():
         window_search.attention_histograms(q, q, window_search.ABSOLUTE, 8)
     assert (window_search.ABSOLUTE, window_search.RELATIVE, window_search.RELATIVE_SINK) == (0, 1, 2)
     assert compress.SINK_TOKENS == 256 and compress.MAX_SAMPLE_TOKENS == 5000
+
+
+def test_align_windows_rule():
+    from longcontext_sqattn_paddle_amd.sqattn._prefill import align_windows
+
+    # multiples stay; others go up to the next multiple of 128 (windows) / 64 (sink)
+    assert align_windows([0, 128, 13184], [0, 256, 13184], 256, 64) == ([0, 128, 13184], [0, 256, 13184], 256)
+    assert align_windows([1, 129, 1000], [1, 129, 1000], 100, 128) == ([128, 256, 1024], [128, 256, 1024], 128)
+    # 8-bit window below the query block under a wider 4-bit window: raised to the block
+    assert align_windows([0, 0, 64], [384, 0, 0], 0, 64) == ([64, 0, 128], [384, 0, 0], 0)
+    assert align_windows([0], [256], 0, 128) == ([128], [256], 0)
+
+
+def _brute_mix_mask(kv_len, w8, w4, sink):
+    """Element loop from the written semantics: row i sees 8-bit key j iff j <= i and (j < sink or j > i - w8); the
+    4-bit copy of key j iff j >= sink and i - w8 - w4 < j <= i - w8."""
+    m = torch.zeros(kv_len, 2 * kv_len, dtype=torch.bool)
+    for i in range(kv_len):
+        for j in range(kv_len):
+            m[i, j] = j <= i and (j < sink or j > i - w8)
+            m[i, kv_len + j] = j >= sink and (i - w8 - w4 < j <= i - w8)
+    return m
+
+
+def test_mix_bit_mask_restatements_against_element_loops():
+    from longcontext_sqattn_paddle_amd.sqattn.attn_replacer import construct_mix_bit_mask
+    from oracle import plugin
+
+    for kv_len, w8, w4, sink in ((24, 5, 7, 3), (17, 0, 4, 0), (16, 100, 100, 2), (9, 1, 0, 4)):
+        want = _brute_mix_mask(kv_len, w8, w4, sink)
+        assert torch.equal(plugin.mix_bit_mask(kv_len, w8, w4, sink), want)
+        assert torch.equal(construct_mix_bit_mask(kv_len, w8, w4, sink, "cpu"), want)
+    # every key is seen at most once per row (8-bit copy or 4-bit copy), and the row's own token always as 8-bit
+    m = plugin.mix_bit_mask(40, 6, 9, 4)
+    assert not bool((m[:, :40] & m[:, 40:]).any()) and bool(torch.diagonal(m[:, :40]).all())
+    # per-head lists
+    w8s, w4s = [5, 0, 12], [7, 3, 0]
+    want = torch.stack([_brute_mix_mask(20, a, b, 2) for a, b in zip(w8s, w4s)])
+    assert torch.equal(plugin.mix_bit_mask(20, w8s, w4s, 2), want)
+    assert torch.equal(construct_mix_bit_mask(20, w8s, w4s, 2, "cpu"), want)
+
+
+def test_delayed_sdpa_wrapper_quantised_branch_matches_the_oracle():
+    """The masked-SDPA emulation over [8-bit keys ; 4-bit keys] (attn_replacer.py:123-186), host code on torch: runs on
+    the CPU, so it is checked here against the oracle's float64 restatement."""
+    import types
+
+    from longcontext_sqattn_paddle_amd.sqattn.attn_replacer import delayed_sdpa_wrapper
+    from oracle import plugin
+
+    g = torch.Generator().manual_seed(5)
+    q, k, v = (torch.randn(1, 3, 48, 32, generator=g) for _ in range(3))
+    k = k + 0.7
+    args = types.SimpleNamespace(quant=True, qk_qtype="int", v_qtype="int", vis_attn=False)
+    for w8, w4 in ((6, 10), ([4, 9, 48], [8, 0, 5])):
+        out = delayed_sdpa_wrapper(0, w8, w4, 4, args)(None, q, k, v, None, scaling=1.0)
+        ref = plugin.masked_sdpa_emulation(q, k, v, bit8_window=w8, bit4_window=w4, sink=4)
+        assert out.shape == (1, 48, 3 * 32)
+        got = out.view(1, 48, 3, 32).permute(0, 2, 1, 3).double()
+        assert float((got - ref).abs().max()) < 1e-5
+    # the plain branch is SDPA with the caller's mask
+    plain = delayed_sdpa_wrapper(0, 0, 0, 0, types.SimpleNamespace(quant=False))(None, q, k, v, None, tensor_layout="HND")
+    want = torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True).transpose(1, 2).reshape(1, 48, 96)
+    assert torch.allclose(plain, want, atol=1e-6)
