@@ -507,6 +507,230 @@ __global__ __launch_bounds__(1024) void topk_emit_kernel(TopkArgs a) {
   }
 }
 
+
+// ---- the same selection in one launch, without ordering all clusters (at most 1024 clusters and 16 q heads per kv head;
+// other shapes take the two kernels above).  One workgroup of 1024 threads per group, one cluster per thread:
+//   1. scores of all clusters on the matrix cores (fp32 accumulation of exact bf16 products), maximum over the q heads;
+//   2. the clusters that can take part are found by a radix select on the top 16 bits of the order-preserving score key,
+//      weighted by cluster size: two rounds of a 256-bin histogram in LDS (sum of sizes per bin), each read from the top
+//      bin down by one wave until k tokens are covered.  Every cluster whose 16-bit key is at or above the pivot is a
+//      candidate: all clusters above the pivot together hold fewer than k tokens, those at the pivot complete them;
+//   3. only the candidates (a few dozen of 1024 for k = 4096) are ordered by (score descending, index ascending): a
+//      counting rank while there are at most 256 of them, the bitonic network otherwise;
+//   4. prefix of the sizes in rank order by one wave, then every output position finds its cluster by binary search.
+constexpr int kSelCount = 256;   // candidates ranked by counting; more go through the bitonic network
+
+// executed by the 64 lanes of one wave: the highest bin d with (weight of bins above d) < need <= (that + weight of bin d)
+__device__ __forceinline__ void find_pivot(const int32_t* hw, int need, int lane, int& digit, int& above) {
+  int w[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) w[i] = hw[4 * lane + i];
+  const int s = w[0] + w[1] + w[2] + w[3];
+  int suf = s;                                   // weight of this lane's bins and of all higher lanes'
+  for (int d = 1; d < 64; d <<= 1) {
+    const int v = __shfl_down(suf, d);
+    if (lane + d < 64) suf += v;
+  }
+  const unsigned long long m = __ballot(suf >= need);
+  int dg = -1, ab = 0;
+  if (m != 0) {
+    const int lp = 63 - __builtin_clzll(m);      // suf falls with the lane index: the highest lane that still reaches `need`
+    if (lane == lp) {
+      int cum = suf - s;
+      dg = 4 * lane;
+      ab = cum + w[3] + w[2] + w[1];
+#pragma unroll
+      for (int i = 3; i >= 1; --i) {
+        if (cum + w[i] >= need) {
+          dg = 4 * lane + i;
+          ab = cum;
+          break;
+        }
+        cum += w[i];
+      }
+    }
+    dg = __shfl(dg, lp);
+    ab = __shfl(ab, lp);
+  }
+  digit = dg;    // -1: all bins together hold fewer than `need`
+  above = ab;
+}
+
+__global__ __launch_bounds__(1024) void topk_select_kernel(TopkArgs a) {
+  __shared__ float sc[1024];
+  __shared__ unsigned long long ckey[1024];
+  __shared__ int32_t pre[1025], rank_cluster[1024], rank_size[1024], hw[256], misc[8];
+  const int g = blockIdx.x, t = threadIdx.x, lane = t & 63;
+  const int b = g / a.Hkv, kvh = g % a.Hkv;
+  const int nh = a.group;
+  if (t < 256) hw[t] = 0;
+  if (t == 0) misc[0] = 0;
+  const bool have = t < a.C;
+  const int sz = have ? min(a.size[(int64_t)g * a.C + t], a.M) : 0;   // requested ahead of the score phase
+  // ---- 1. scores on the matrix cores: wave w takes clusters 64 w .. 64 w + 63 in four blocks of 16; per block
+  // S[cluster, head] = centroids . queries^T on v_mfma_f32_16x16x32_bf16 (the group's q heads padded to 16 columns).
+  // Lane (r = lane % 16, q = lane / 16) feeds centroid row r, columns 32 kk + 8 q .. + 7 as the A operand and the same
+  // columns of query head r as the B operand, and receives S[cluster 4 q + i][head r], i < 4.
+  {
+    const int wave = t >> 6, r = lane & 15, q4 = lane >> 4;
+    typedef __attribute__((ext_vector_type(4))) float f32x4;
+    uint4 qf[4];
+    const uint16_t* qp = a.query + (int64_t)b * a.q_sb + (int64_t)(kvh * a.group + min(r, nh - 1)) * a.q_sh + 8 * q4;
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) qf[kk] = (r < nh) ? *(const uint4*)(qp + 32 * kk) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+    for (int blk = 0; blk < 4; ++blk) {
+      const int c0 = 64 * wave + 16 * blk;
+      const int row = min(c0 + r, a.C - 1);
+      const uint16_t* cp = a.cent + (int64_t)g * a.c_sg + (int64_t)row * a.c_sc + 8 * q4;
+      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) {
+        const uint4 cf = *(const uint4*)(cp + 32 * kk);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, cf), __builtin_bit_cast(bf16x8_t, qf[kk]), acc, 0, 0, 0);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float v = (r < nh) ? acc[i] : -INFINITY;   // the padded columns take no part in the maximum over the q heads
+        // maximum over the 16 lanes of a row by rotations within the row (DPP row_ror 1, 2, 4, 8): no LDS traffic
+        v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x121, 0xf, 0xf, false)));
+        v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x122, 0xf, 0xf, false)));
+        v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x124, 0xf, 0xf, false)));
+        v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xf, 0xf, false)));
+        if (r == 0) sc[c0 + 4 * q4 + i] = v;
+      }
+    }
+  }
+  __syncthreads();
+  uint32_t key32 = 0;
+  if (have) {
+    const uint32_t bits = __float_as_uint(sc[t] + 0.0f);    // -0.0 counts as +0.0
+    key32 = (bits & 0x80000000u) ? ~bits : (bits | 0x80000000u);
+  }
+  // ---- 2. radix select over the top 16 key bits, weighted by size
+  if (sz > 0) atomicAdd(&hw[key32 >> 24], sz);
+  __syncthreads();
+  if (t < 64) {
+    int d1, ab1;
+    find_pivot(hw, a.k, lane, d1, ab1);
+    if (t == 0) {
+      misc[1] = d1;
+      misc[2] = ab1;
+    }
+  }
+  __syncthreads();
+  const int d1 = misc[1], above1 = misc[2];
+  if (t < 256) hw[t] = 0;
+  __syncthreads();
+  if (sz > 0 && d1 >= 0 && (int)(key32 >> 24) == d1) atomicAdd(&hw[(key32 >> 16) & 255], sz);
+  __syncthreads();
+  if (t < 64 && d1 >= 0) {
+    int d2, ab2;
+    find_pivot(hw, a.k - above1, lane, d2, ab2);   // bin d1 holds at least k - above1 tokens, so d2 >= 0
+    if (t == 0) misc[3] = d2;
+  }
+  __syncthreads();
+  const uint32_t pivot16 = d1 >= 0 ? (((uint32_t)d1 << 8) | (uint32_t)misc[3]) : 0u;   // fewer than k tokens in all: everything
+  // ---- 3. candidates and their order
+  if (sz > 0 && (key32 >> 16) >= pivot16) {
+    const int pos = atomicAdd(&misc[0], 1);
+    ckey[pos] = ((unsigned long long)key32 << 32) | (0xffffffffu - (uint32_t)t);
+    rank_size[pos] = sz;    // by candidate slot for now
+  }
+  __syncthreads();
+  const int m = misc[0];
+  int my_rank = -1, my_cluster = 0, my_size = 0;
+  if (m <= kSelCount) {
+    if (t < m) {
+      const unsigned long long mine = ckey[t];
+      int r = 0;
+      for (int j = 0; j < m; ++j) r += ckey[j] > mine;
+      my_rank = r;
+      my_cluster = (int)(0xffffffffu - (uint32_t)mine);
+      my_size = rank_size[t];
+    }
+    __syncthreads();
+    if (my_rank >= 0) {
+      rank_cluster[my_rank] = my_cluster;
+      rank_size[my_rank] = my_size;
+    }
+  } else {
+    int P = 1;
+    while (P < m) P <<= 1;
+    if (t >= m && t < P) ckey[t] = 0;            // padding sorts behind every candidate
+    __syncthreads();
+    for (int len = 2; len <= P; len <<= 1)
+      for (int d = len >> 1; d > 0; d >>= 1) {
+        if (t < P / 2) {
+          const int lo = ((t & ~(d - 1)) << 1) | (t & (d - 1)), hi = lo | d;
+          const bool descending = (lo & len) == 0;
+          const unsigned long long x = ckey[lo], y = ckey[hi];
+          if ((x < y) == descending) {
+            ckey[lo] = y;
+            ckey[hi] = x;
+          }
+        }
+        __syncthreads();
+      }
+    if (t < m) {
+      const int c = (int)(0xffffffffu - (uint32_t)ckey[t]);
+      rank_cluster[t] = c;
+      rank_size[t] = min(a.size[(int64_t)g * a.C + c], a.M);
+    }
+  }
+  __syncthreads();
+  // ---- 4. exclusive prefix of the sizes in rank order (one wave), then the token ids
+  if (t < 64) {
+    const int per = (m + 63) / 64;
+    int run = 0;
+    for (int i = 0; i < per; ++i) {
+      const int r = lane * per + i;
+      if (r < m) run += rank_size[r];
+    }
+    int inc = run;
+    for (int d = 1; d < 64; d <<= 1) {
+      const int v = __shfl_up(inc, d);
+      if (lane >= d) inc += v;
+    }
+    int acc = inc - run;
+    for (int i = 0; i < per; ++i) {
+      const int r = lane * per + i;
+      if (r < m) {
+        pre[r] = acc;
+        acc += rank_size[r];
+      }
+    }
+    if (lane == 63) pre[m] = inc;
+  }
+  __syncthreads();
+  const int total = pre[m];
+  int32_t* out = a.out + (int64_t)g * a.out_sg;
+  constexpr int U = 4;   // positions per thread and round: their table reads are independent and overlap
+  for (int p0 = t; p0 < a.k; p0 += U * 1024) {
+    int64_t off[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int p = p0 + u * 1024;
+      off[u] = -1;
+      if (p < a.k && p < total) {
+        int lo = 0, hi = m;               // the rank r with pre[r] <= p < pre[r + 1]
+        while (hi - lo > 1) {
+          const int mid = (lo + hi) >> 1;
+          if (pre[mid] <= p) lo = mid;
+          else hi = mid;
+        }
+        off[u] = (int64_t)g * a.cl_sg + (int64_t)rank_cluster[lo] * a.cl_sc + (p - pre[lo]);
+      }
+    }
+    int32_t id[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) id[u] = off[u] >= 0 ? a.clusters[off[u]] : -1;
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (p0 + u * 1024 < a.k) out[p0 + u * 1024] = id[u];
+  }
+}
+
 struct WsLayout {
   size_t off_bytes, hist_bytes, order_bytes, score_bytes, start_bytes, total_bytes;
   int nT;
@@ -744,6 +968,11 @@ extern "C" int sq_topk_select(const DLTensor* query, const DLTensor* centroids, 
   a.k = (int)k;
   a.Hkv = (int)Hkv;
   a.group = num_kv_groups;
+  if (C <= 1024 && num_kv_groups <= 16) {   // one launch, only the clusters that can fill k are ordered
+    hipLaunchKernelGGL(topk_select_kernel, dim3((unsigned)G), dim3(1024), 0, st, a);
+    SQ_HIP(hipGetLastError());
+    return SQ_OK;
+  }
   hipLaunchKernelGGL(topk_score_kernel, dim3((unsigned)((C + 255) / 256), (unsigned)G), dim3(256), 0, st, a);
   int P = 1;
   while (P < C) P <<= 1;
