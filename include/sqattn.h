@@ -32,6 +32,7 @@
  *                             :319-326 (mlp), called from model_hub/LLM.py:88-116 (layer_decode)
  *   sq_linear_rows_silu_and_mul  model_hub/qwen.py:320-324 (gate_up_proj and silu_and_mul of mlp) on a decode step
  *   sq_linear_rows_rope       model_hub/qwen.py:302-312 (wqkv) + :352-379 (rotary embedding of q and k) on a decode step
+ *   sq_fake_quant_prepass_typed  the same with the float quantiser types of sqattn/attn_replacer.py:340-358
  *   sq_fake_quant_prepass     sqattn/attn_replacer.py:334-365 (GQA expand, key centring and the five fake-quant
  *                             passes of mp_triton_wrapper's closure), sqattn/fake_quant.py:24-58, 98-125
  */
@@ -205,6 +206,20 @@ size_t sq_fake_quant_prepass_workspace_bytes(int64_t batch, int64_t num_kv_heads
 int sq_fake_quant_prepass(const DLTensor* query, const DLTensor* key, const DLTensor* value, DLTensor* q8,
                           DLTensor* q4, DLTensor* k8, DLTensor* k4, DLTensor* v8, DLTensor* workspace,
                           int32_t layout, void* stream);
+
+/*
+ * The same pre-pass with the closure's other quantiser types (sqattn/attn_replacer.py:340-358): qk_qtype selects the
+ * 8-bit quantiser of query and centred key (SQ_QTYPE_INT: IntegerQuantizer(8, True, "per_token"); SQ_QTYPE_E4M3 /
+ * SQ_QTYPE_E5M2: FloatQuantizer(..., True, "per_token"), the float simulation of sqattn/fake_quant.py:151-204 with the
+ * scale absmax / 448 resp. / 57344), v_qtype the one of value ("per_channel").  The 4-bit outputs are always the
+ * integer quantiser's, as in the reference.  Outputs equal the formulas evaluated in fp32 on the host, except that the
+ * float simulation's exponent is read from the exponent field instead of floor(log2(.)): the two differ only where a
+ * library's fp32 log2 rounds a value just below a power of two up to the integer.
+ */
+enum { SQ_QTYPE_INT = 0, SQ_QTYPE_E4M3 = 1, SQ_QTYPE_E5M2 = 2 };
+int sq_fake_quant_prepass_typed(const DLTensor* query, const DLTensor* key, const DLTensor* value, DLTensor* q8,
+                                DLTensor* q4, DLTensor* k8, DLTensor* k4, DLTensor* v8, DLTensor* workspace,
+                                int32_t layout, int32_t qk_qtype, int32_t v_qtype, void* stream);
 
 /*
  * Prefill side of the KV cache (cache_hub/flash_attn_cache.py:153-232): rows [valid_start, T) of one sequence's

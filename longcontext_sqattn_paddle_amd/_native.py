@@ -18,6 +18,7 @@ SQ_OK, SQ_EINVAL, SQ_ESHAPE, SQ_EDEVICE, SQ_EDTYPE, SQ_EUNSUPPORTED, SQ_EHIP, SQ
 LAYOUT = {"HND": 0, "NHD": 1}
 P_NONE, P_E4M3_STATIC, P_E4M3_BLOCK, P_E4M3_STATIC_FAST, P_E4M3_FP8_PV, P_E4M3_MX_FP8_PV = 0, 1, 2, 3, 4, 5
 WINDOW_NONE, WINDOW_SIZES = 0, 1
+QTYPE = {"int": 0, "e4m3": 1, "e5m2": 2}
 
 
 class DLDevice(ctypes.Structure):
@@ -96,6 +97,7 @@ SYMBOLS = {
     "sq_topk_select": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, ctypes.c_int32, ctypes.c_void_p]),
     "sq_fake_quant_prepass_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int64] * 3),
     "sq_fake_quant_prepass": (ctypes.c_int, [_P] * 9 + [ctypes.c_int32, ctypes.c_void_p]),
+    "sq_fake_quant_prepass_typed": (ctypes.c_int, [_P] * 9 + [ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, ctypes.c_void_p]),
     "sq_rmsnorm": (ctypes.c_int, [_P, _P, _P, ctypes.c_float, ctypes.c_void_p]),
     "sq_silu_and_mul": (ctypes.c_int, [_P, _P, ctypes.c_void_p]),
     "sq_rope": (ctypes.c_int, [_P] * 6 + [ctypes.c_int32, ctypes.c_void_p]),

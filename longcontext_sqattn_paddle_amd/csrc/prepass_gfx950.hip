@@ -36,6 +36,7 @@ struct PrepassArgs {
   int32_t B, N, Hq, Hkv, is_bf16, nblk, tok_per_blk, want4;
 };
 
+
 template <bool BF16>
 __device__ __forceinline__ float ld(uint32_t bits16) {
   if constexpr (BF16) return bf16_bits_to_f32(bits16);
@@ -75,6 +76,42 @@ __device__ __forceinline__ float round_half_away(float t) { return copysignf(flo
 __device__ __forceinline__ float qdq(float x, const Divisor& s, float qmin, float qmax) {
   const float q = fminf(fmaxf(round_half_away(divide(x, s)) + 0.0f, qmin), qmax);
   return q * s.d;
+}
+
+// FloatQuantizer(e4m3 | e5m2, True, ...).fake_quant_tensor of one value (fake_quant.py:151-204, 231-248):
+// t = clamp(x / scale, +-fmax); E = floor(log2(|t| + 1e-30)); f = |t| / 2^E - 1; E' = clip(E, 1 - bias, bias);
+// f' = clip(round(f * 2^MB) / 2^MB, 0, 1 - 2^-MB); y = (1 + f') * 2^E' * sign(t), clipped to +-(2 - 2^-MB) * 2^bias, zero
+// kept; result y * scale.  Every step is the reference's fp32 operation (the divisions and multiplications by powers of
+// two are exact), except that E is read from the exponent field of |t| + 1e-30 instead of floor(log2(.)): the two agree
+// unless a library's fp32 log2 rounds a value a few units in the last place below a power of two up to the integer,
+// where the reference's own result depends on that library.
+template <int EB, int MB>
+__device__ __forceinline__ float qdq_float(float x, const Divisor& s) {
+  constexpr float fmax = EB == 4 ? 448.f : 57344.f;
+  constexpr int bias = (1 << (EB - 1)) - 1;
+  constexpr float eps = 1.0f / (1 << MB);
+  constexpr float max_val = (2.0f - eps) * (float)(1u << bias);
+  const float t = fminf(fmaxf(divide(x, s) + 0.0f, -fmax), fmax);
+  const float av = fabsf(t);
+  const int E = (int)((__float_as_uint(av + 1e-30f) >> 23) & 255u) - 127;
+  const float f = av * ldexpf(1.0f, -E) - 1.0f;
+  const int Ec = min(max(E, 1 - bias), bias);
+  const float fq = fminf(fmaxf(round_half_away(f * (float)(1 << MB)) * eps, 0.0f), 1.0f - eps);
+  float y = (1.0f + fq) * ldexpf(1.0f, Ec);
+  y = fminf(y, max_val);
+  y = (av == 0.0f) ? 0.0f : copysignf(y, t);
+  return y * s.d;
+}
+// the 8-bit quantiser of a call: 0 integer (symmetric, +-127 range), 1 e4m3, 2 e5m2
+template <int QT>
+__device__ __forceinline__ float qdq8(float x, const Divisor& s) {
+  if constexpr (QT == 1) return qdq_float<4, 3>(x, s);
+  else if constexpr (QT == 2) return qdq_float<5, 2>(x, s);
+  else return qdq(x, s, -128.f, 127.f);
+}
+template <int QT>
+__device__ __forceinline__ float scale_of(float amax) {
+  return amax / (QT == 1 ? 448.f : (QT == 2 ? 57344.f : 127.f));
 }
 
 // ---- key mean, stage 1: workgroup b sums tokens [b*tok_per_blk, ...) of every (batch, kv head, channel) in fp64.
@@ -155,7 +192,7 @@ __global__ __launch_bounds__(256) void prepass_kmean_kernel(PrepassArgs a) {
 }
 
 // ---- per-token 8-bit (and 4-bit) fake quantisation of the rows of q (CENTRE = false) or of k minus its mean
-template <bool BF16, bool CENTRE>
+template <bool BF16, bool CENTRE, int QT>
 __global__ __launch_bounds__(256) void prepass_rows_kernel(PrepassArgs a) {
   const View& src = CENTRE ? a.k : a.q;
   const View& d8 = CENTRE ? a.k8 : a.q8;
@@ -203,10 +240,10 @@ __global__ __launch_bounds__(256) void prepass_rows_kernel(PrepassArgs a) {
     amax = fmaxf(amax, 1e-5f);
     if (!live[u]) continue;
     {
-      const Divisor scale = make_divisor(amax / 127.f);
+      const Divisor scale = make_divisor(scale_of<QT>(amax));
       float y[8];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) y[e] = qdq(x[e], scale, -128.f, 127.f);
+      for (int e = 0; e < 8; ++e) y[e] = qdq8<QT>(x[e], scale);
       const uint4 o = pack8<BF16>(y);
       __builtin_nontemporal_store(u32x4_t{o.x, o.y, o.z, o.w}, (u32x4_t*)((uint16_t*)d8.p + off8[u]));
     }
@@ -222,7 +259,7 @@ __global__ __launch_bounds__(256) void prepass_rows_kernel(PrepassArgs a) {
 }
 
 // ---- value: one 8-bit scale per (token, channel) over batch and heads
-template <bool BF16>
+template <bool BF16, int QT>
 __global__ __launch_bounds__(256) void prepass_v_kernel(PrepassArgs a) {
   const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;   // (token, group of 8 channels)
   if (t >= (int64_t)a.N * (kPD / 8)) return;
@@ -239,14 +276,14 @@ __global__ __launch_bounds__(256) void prepass_v_kernel(PrepassArgs a) {
     }
   Divisor scale[8];
 #pragma unroll
-  for (int e = 0; e < 8; ++e) scale[e] = make_divisor(fmaxf(amax[e], 1e-5f) / 127.f);
+  for (int e = 0; e < 8; ++e) scale[e] = make_divisor(scale_of<QT>(fmaxf(amax[e], 1e-5f)));
   uint16_t* obase = (uint16_t*)a.v8.p + n * a.v8.sn + 8 * c8;
   for (int b = 0; b < a.B; ++b)
     for (int h = 0; h < a.Hkv; ++h) {
       float x[8], y[8];
       unpack8<BF16>(*(const uint4*)(base + b * a.v.sb + h * a.v.sh), x);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) y[e] = qdq(x[e], scale[e], -128.f, 127.f);
+      for (int e = 0; e < 8; ++e) y[e] = qdq8<QT>(x[e], scale[e]);
       *(uint4*)(obase + b * a.v8.sb + h * a.v8.sh) = pack8<BF16>(y);
     }
 }
@@ -282,9 +319,11 @@ extern "C" size_t sq_fake_quant_prepass_workspace_bytes(int64_t batch, int64_t n
   return (size_t)nblk * cols * sizeof(double) + ((cols * 2 + 255) & ~(size_t)255);
 }
 
-extern "C" int sq_fake_quant_prepass(const DLTensor* query, const DLTensor* key, const DLTensor* value, DLTensor* q8,
-                                     DLTensor* q4, DLTensor* k8, DLTensor* k4, DLTensor* v8, DLTensor* workspace,
-                                     int32_t layout, void* stream) {
+extern "C" int sq_fake_quant_prepass_typed(const DLTensor* query, const DLTensor* key, const DLTensor* value, DLTensor* q8,
+                                           DLTensor* q4, DLTensor* k8, DLTensor* k4, DLTensor* v8, DLTensor* workspace,
+                                           int32_t layout, int32_t qk_qtype, int32_t v_qtype, void* stream) {
+  SQ_REQUIRE(qk_qtype >= SQ_QTYPE_INT && qk_qtype <= SQ_QTYPE_E5M2 && v_qtype >= SQ_QTYPE_INT && v_qtype <= SQ_QTYPE_E5M2, SQ_EINVAL,
+             "Invalid quantization type: %d / %d", (int)qk_qtype, (int)v_qtype);
   SQ_REQUIRE(query && key && value && q8 && k8 && v8, SQ_EINVAL, "sq_fake_quant_prepass: null tensor argument");
   SQ_REQUIRE((q4 == nullptr) == (k4 == nullptr), SQ_EINVAL, "sq_fake_quant_prepass: q4 and k4 must be given together");
   SQ_REQUIRE(layout == SQ_LAYOUT_HND || layout == SQ_LAYOUT_NHD, SQ_EINVAL, "Unknown tensor layout: %d", (int)layout);
@@ -333,17 +372,33 @@ extern "C" int sq_fake_quant_prepass(const DLTensor* query, const DLTensor* key,
   a.mean = (uint16_t*)(data_of(workspace) + (size_t)a.nblk * cols * sizeof(double));
   hipStream_t s = (hipStream_t)stream;
   const int64_t qrows = B * N * Hq, krows = B * N * Hkv, vthreads = N * (kPD / 8);
-#define SQ_PREPASS_LAUNCH(BF)                                                                                  \
-  do {                                                                                                         \
-    hipLaunchKernelGGL(prepass_ksum_kernel<BF>, dim3(a.nblk), dim3(256), 0, s, a);                             \
+#define SQ_PREPASS_ROWS(BF, QT)                                                                                        \
+  do {                                                                                                                 \
+    hipLaunchKernelGGL((prepass_rows_kernel<BF, false, QT>), dim3((unsigned)((qrows + 31) / 32)), dim3(256), 0, s, a); \
+    hipLaunchKernelGGL((prepass_rows_kernel<BF, true, QT>), dim3((unsigned)((krows + 31) / 32)), dim3(256), 0, s, a);  \
+  } while (0)
+#define SQ_PREPASS_LAUNCH(BF)                                                                                       \
+  do {                                                                                                              \
+    hipLaunchKernelGGL(prepass_ksum_kernel<BF>, dim3(a.nblk), dim3(256), 0, s, a);                                  \
     hipLaunchKernelGGL(prepass_kmean_kernel<BF>, dim3((unsigned)((cols * 16 + 255) / 256)), dim3(256), 0, s, a);    \
-    hipLaunchKernelGGL((prepass_rows_kernel<BF, false>), dim3((unsigned)((qrows + 31) / 32)), dim3(256), 0, s, a); \
-    hipLaunchKernelGGL((prepass_rows_kernel<BF, true>), dim3((unsigned)((krows + 31) / 32)), dim3(256), 0, s, a);  \
-    hipLaunchKernelGGL(prepass_v_kernel<BF>, dim3((unsigned)((vthreads + 255) / 256)), dim3(256), 0, s, a);    \
+    if (qk_qtype == SQ_QTYPE_E4M3) SQ_PREPASS_ROWS(BF, 1);                                                          \
+    else if (qk_qtype == SQ_QTYPE_E5M2) SQ_PREPASS_ROWS(BF, 2);                                                     \
+    else SQ_PREPASS_ROWS(BF, 0);                                                                                    \
+    const dim3 vgrid((unsigned)((vthreads + 255) / 256));                                                           \
+    if (v_qtype == SQ_QTYPE_E4M3) hipLaunchKernelGGL((prepass_v_kernel<BF, 1>), vgrid, dim3(256), 0, s, a);         \
+    else if (v_qtype == SQ_QTYPE_E5M2) hipLaunchKernelGGL((prepass_v_kernel<BF, 2>), vgrid, dim3(256), 0, s, a);    \
+    else hipLaunchKernelGGL((prepass_v_kernel<BF, 0>), vgrid, dim3(256), 0, s, a);                                  \
   } while (0)
   if (a.is_bf16) SQ_PREPASS_LAUNCH(true);
   else SQ_PREPASS_LAUNCH(false);
 #undef SQ_PREPASS_LAUNCH
+#undef SQ_PREPASS_ROWS
   SQ_HIP(hipGetLastError());
   return SQ_OK;
+}
+
+extern "C" int sq_fake_quant_prepass(const DLTensor* query, const DLTensor* key, const DLTensor* value, DLTensor* q8,
+                                     DLTensor* q4, DLTensor* k8, DLTensor* k4, DLTensor* v8, DLTensor* workspace,
+                                     int32_t layout, void* stream) {
+  return sq_fake_quant_prepass_typed(query, key, value, q8, q4, k8, k4, v8, workspace, layout, SQ_QTYPE_INT, SQ_QTYPE_INT, stream);
 }

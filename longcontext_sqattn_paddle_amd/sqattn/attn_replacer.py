@@ -117,12 +117,15 @@ def mp_triton_wrapper(layer_idx, bit8_window_sizes=0, bit4_window_sizes=0, sink_
             return out.reshape(b, n, h * d)
         p_quant = kwargs.get("p_quant", None)
         relative = bool(args.use_relative_distance)
-        if args.qk_qtype == "int" and args.v_qtype == "int" and query.size(-1) == 128:
-            # one fused HIP pre-pass instead of the reference's tensor passes (:338-365).  The relative launch
-            # aliases the 4-bit operands to the 8-bit ones (attn_triton_mix_relative.py:441-444), so they are
-            # only produced for the absolute variant.
-            q_bit8, q_bit4, k_bit8, k_bit4, v_bit8 = fused_int_prepass(query, key, value, want_4bit=not relative,
-                                                                       tensor_layout=layout)
+        known = ("int", "e4m3", "e5m2")
+        if args.qk_qtype not in known or args.v_qtype not in known:
+            raise ValueError(f"Invalid quantization type: {args.qk_qtype if args.qk_qtype not in known else args.v_qtype}")
+        if query.size(-1) == 128:
+            # one fused HIP pre-pass instead of the reference's tensor passes (:338-365), for every quantiser type.  The
+            # relative launch aliases the 4-bit operands to the 8-bit ones (attn_triton_mix_relative.py:441-444), so
+            # they are only produced for the absolute variant.
+            q_bit8, q_bit4, k_bit8, k_bit4, v_bit8 = fused_int_prepass(query, key, value, want_4bit=not relative, tensor_layout=layout,
+                                                                       qk_qtype=args.qk_qtype, v_qtype=args.v_qtype)
         else:
             bit8_qk, bit4_qk, bit8_v = _quantizers(args)
             if nhd:   # the quantisers' "per_channel" range is over dims (0, 1) of [B,H,N,D]: quantise HND views

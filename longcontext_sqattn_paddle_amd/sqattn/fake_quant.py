@@ -140,10 +140,11 @@ class FloatQuantizer(BaseQuantizer):
         return float_quantize(scaled.float(), self.e_bits, self.m_bits, rounding="nearest")
 
 
-def fused_int_prepass(query, key, value, want_4bit=True, tensor_layout="NHD"):
-    """The operand pre-pass of `mp_triton_wrapper`'s closure (attn_replacer.py:334-365) for the integer quantiser
-    types, as one call into the HIP library: key centring, per-token 8-bit (and 4-bit) fake quantisation of
-    query and centred key, per-channel 8-bit fake quantisation of value -- without expanding the kv heads.
+def fused_int_prepass(query, key, value, want_4bit=True, tensor_layout="NHD", qk_qtype="int", v_qtype="int"):
+    """The operand pre-pass of `mp_triton_wrapper`'s closure (attn_replacer.py:334-365) as one call into the HIP
+    library: key centring, per-token 8-bit (and integer 4-bit) fake quantisation of query and centred key, per-channel
+    8-bit fake quantisation of value -- without expanding the kv heads.  `qk_qtype` / `v_qtype` pick the 8-bit
+    quantisers as the closure does (:340-358): "int", "e4m3" or "e5m2".
 
     query [B,N,Hq,D], key/value [B,N,Hkv,D] for "NHD" ([B,H,N,D] for "HND"), bf16 or fp16, D == 128.
     Returns (q8, q4, k8, k4, v8) in the layout of the inputs; q4 and k4 are None unless `want_4bit`.
@@ -166,5 +167,9 @@ def fused_int_prepass(query, key, value, want_4bit=True, tensor_layout="NHD"):
     need = lib.sq_fake_quant_prepass_workspace_bytes(B, Hkv, Nk)
     ws = torch.empty((need + 7) // 8, dtype=torch.float64, device=query.device)
     b = [N.dl(t) for t in (query, key, value, q8, q4, k8, k4, v8, ws)]
-    N.check(lib.sq_fake_quant_prepass(*[N.ptr(x) for x in b], N.LAYOUT[tensor_layout], N.current_stream(query.device)))
+    for name in (qk_qtype, v_qtype):
+        if name not in N.QTYPE:
+            raise ValueError(f"Invalid quantization type: {name}")
+    N.check(lib.sq_fake_quant_prepass_typed(*[N.ptr(x) for x in b], N.LAYOUT[tensor_layout], N.QTYPE[qk_qtype], N.QTYPE[v_qtype],
+                                            N.current_stream(query.device)))
     return q8, q4, k8, k4, v8

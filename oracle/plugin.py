@@ -42,15 +42,16 @@ def key_mean_exact(key_hnd: torch.Tensor) -> torch.Tensor:
     return (key_hnd.double().sum(dim=2, keepdim=True) / n).float().to(key_hnd.dtype)
 
 
-def int_prepass(query, key, value, want_4bit=True):
-    """CPU restatement of the operand pre-pass for the integer quantisers (attn_replacer.py:334-365) without the
-    GQA expansion (which repeats heads and changes no value): inputs NHD `[B,N,H,D]`, outputs NHD
-    `(q8, q4, k8, k4, v8)`; q4/k4 None unless `want_4bit`."""
+def int_prepass(query, key, value, want_4bit=True, qk_qtype="int", v_qtype="int"):
+    """CPU restatement of the operand pre-pass (attn_replacer.py:334-365) without the GQA expansion (which repeats
+    heads and changes no value): inputs NHD `[B,N,H,D]`, outputs NHD `(q8, q4, k8, k4, v8)`; q4/k4 None unless
+    `want_4bit`.  `qk_qtype` / `v_qtype` pick the 8-bit quantisers as the closure does (:340-358); the 4-bit ones are
+    always the integer quantiser."""
     q, k, v = (t.permute(0, 2, 1, 3) for t in (query, key, value))   # HND views, as the reference quantises them
     kc = k - key_mean_exact(k)
-    outs = [FQ.int_fake_quant(q, 8, True, "per_token"), FQ.int_fake_quant(q, 4, True, "per_token") if want_4bit else None,
-            FQ.int_fake_quant(kc, 8, True, "per_token"), FQ.int_fake_quant(kc, 4, True, "per_token") if want_4bit else None,
-            FQ.int_fake_quant(v, 8, True, "per_channel")]
+    outs = [_qk_quant(q, qk_qtype, 8), FQ.int_fake_quant(q, 4, True, "per_token") if want_4bit else None,
+            _qk_quant(kc, qk_qtype, 8), FQ.int_fake_quant(kc, 4, True, "per_token") if want_4bit else None,
+            _v_quant(v, v_qtype)]
     return tuple(None if t is None else t.permute(0, 2, 1, 3).contiguous() for t in outs)
 
 
@@ -68,7 +69,7 @@ def plugin_attention(query, key, value, *, num_kv_groups, bit8, bit4, sink, rela
     k = repeat_kv(key, num_kv_groups)
     v = repeat_kv(value, num_kv_groups)
     q = query.permute(0, 2, 1, 3)
-    k = k - (key_mean_exact(k) if qk_qtype == "int" and v_qtype == "int" else k.mean(dim=2, keepdim=True))
+    k = k - key_mean_exact(k)
     q8, q4 = _qk_quant(q, qk_qtype, 8), _qk_quant(q, qk_qtype, 4)
     k8, k4 = _qk_quant(k, qk_qtype, 8), _qk_quant(k, qk_qtype, 4)
     v8 = _v_quant(v, v_qtype)

@@ -85,6 +85,24 @@ def test_plugin_closure_matches_oracle(relative, bit8, bit4):
     assert float((o - r).abs().max()) <= 2 ** -7 * float(r.abs().max()) + 2e-3 * rms
 
 
+def test_plugin_closure_with_float_quantiser_types():
+    """qk_qtype / v_qtype e4m3 (sqattn/attn_replacer.py:340-358) through the fused pre-pass and the windowed kernel."""
+    from longcontext_sqattn_paddle_amd.sqattn.attn_replacer import process_model
+
+    q, k, v = inputs.plugin_inputs(1, 4, 1, 1024, 128, seed=4)
+    m = _Model(2, 4)
+    process_model(m, "SQAttn", {1: {"bit8": 0.25, "bit4": 0.25, "sink": 0}}, _args(True, "e4m3", "e4m3"))
+    out = m.layers[1].prefill_attention(q.to(DEV), k.to(DEV), v.to(DEV), None)
+    torch.cuda.synchronize()
+    ref = plugin.plugin_attention(q, k, v, num_kv_groups=4, bit8=0.25, bit4=0.25, sink=256, relative=True, qk_qtype="e4m3", v_qtype="e4m3")
+    o, r = out.float().cpu(), ref.float()
+    assert _cos(o, r) >= 0.9999
+    assert float((o - r).abs().max()) <= 2 ** -7 * float(r.abs().max()) + 5e-3 * float(r.pow(2).mean().sqrt())
+    with pytest.raises(ValueError):
+        process_model(m, "SQAttn", {1: {"bit8": 0.25, "bit4": 0.25, "sink": 0}}, _args(True, "fp4", "int"))
+        m.layers[1].prefill_attention(q.to(DEV), k.to(DEV), v.to(DEV), None)
+
+
 def test_process_model_takes_the_window_sizes_the_reference_calibration_writes():
     """The reference's window search returns 1 token when a head's histogram is empty and the histogram's length when the
     threshold is never reached (sqattn/window_search.py:90-128), and its configuration keeps a 256-token sink: a

@@ -42,6 +42,35 @@ def test_prepass_is_bit_exact(B, N, Hq, Hkv, dtype, want4):
         assert torch.equal(a.cpu().contiguous().view(torch.int16), b.contiguous().view(torch.int16)), name
 
 
+@pytest.mark.parametrize("qk,vq,dtype", [("e4m3", "e4m3", torch.bfloat16), ("e5m2", "int", torch.bfloat16), ("int", "e5m2", torch.float16)])
+def test_prepass_float_quantiser_types(qk, vq, dtype):
+    """The closure's e4m3 / e5m2 quantisers (sqattn/attn_replacer.py:340-358, float simulation of fake_quant.py:151-204)
+    in the fused pre-pass.  Every operation of the simulation is exact in fp32 except `floor(log2(|t| + 1e-30))`, which
+    the kernel reads from the exponent field: where a library's fp32 log2 rounds a value a few units in the last place
+    below a power of two up to the integer, the two differ by one grid step.  Stated tolerance: at most 1e-4 of the
+    elements differ, each by at most one step of its grid (2^-3 relative for e4m3, 2^-2 for e5m2); the integer outputs
+    of the same call stay bit-exact."""
+    from longcontext_sqattn_paddle_amd.sqattn.fake_quant import fused_int_prepass
+
+    print(f"case prepass float quantisers qk={qk} v={vq} {dtype}", flush=True)
+    q, k, v = _inputs(2, 700, 8, 2, seed=5, dtype=dtype)
+    got = fused_int_prepass(q.to(DEV), k.to(DEV), v.to(DEV), want_4bit=True, tensor_layout="NHD", qk_qtype=qk, v_qtype=vq)
+    torch.cuda.synchronize()
+    ref = plugin.int_prepass(q, k, v, want_4bit=True, qk_qtype=qk, v_qtype=vq)
+    for name, a, b, qt in zip(("q8", "q4", "k8", "k4", "v8"), got, ref, (qk, "int", qk, "int", vq)):
+        a = a.cpu()
+        if qt == "int":
+            assert torch.equal(a.contiguous().view(torch.int16), b.contiguous().view(torch.int16)), name
+            continue
+        diff = a != b
+        assert float(diff.float().mean()) <= 1e-4, (name, float(diff.float().mean()))
+        step = 2.0 ** -3 if qt == "e4m3" else 2.0 ** -2
+        rel = (a.float() - b.float()).abs() / b.float().abs().clamp(min=1e-30)
+        assert float(rel[diff].max()) <= step * 1.01 if bool(diff.any()) else True, name
+    with pytest.raises(ValueError):
+        fused_int_prepass(q.to(DEV), k.to(DEV), v.to(DEV), qk_qtype="e3m4")
+
+
 def test_prepass_hnd_views_and_strides():
     from longcontext_sqattn_paddle_amd.sqattn.fake_quant import fused_int_prepass
 

@@ -82,3 +82,20 @@ def test_index_ranges():
             n = (k * d) // 200
             pairs += [(np.float32(n), np.float32(d)), (np.float32(n + 1), np.float32(d))]
     _check(pairs)
+
+
+def test_float_quantiser_ranges():
+    """pre-pass with the e4m3 / e5m2 quantisers: d = max(absmax, 1e-5) / 448 or / 57344, |x / d| <= 448 (or 57344);
+    dividends also next to the mantissa-rounding boundaries (1 + (k + 1/2) / 2^m) * 2^e of the float simulation"""
+    rng = np.random.default_rng(3)
+    pairs = []
+    for _ in range(300):
+        amax = np.float32(10.0 ** rng.uniform(-5, 4.8))
+        for fmax, mbits in ((448.0, 3), (57344.0, 2)):
+            d = np.float32(amax / np.float32(fmax))
+            xs = (rng.uniform(-1, 1, 3) * amax).astype(np.float32)
+            xs = (xs.view(np.uint32) & 0xFFFF0000).view(np.float32)
+            pairs += [(x, d) for x in xs]
+            k, e = int(rng.integers(0, 2 ** mbits)), int(rng.integers(-6, 8))
+            pairs.append((np.float32((1 + (k + 0.5) / 2 ** mbits) * 2.0 ** e * float(d)), d))
+    _check(pairs)
