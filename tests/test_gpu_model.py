@@ -173,3 +173,65 @@ def test_kmeans_kv_selection_in_the_decode_steps():
     eager = model.generate("SDPA", prompt, None, 12, verbose=False)
     graphed = model.generate("SDPA", prompt, None, 12, verbose=False, use_graph=True)
     assert eager == graphed
+
+
+def test_end_to_end_configuration_sizes_three_layers_one_million_tokens():
+    """The benchmark's end-to-end configuration at its real sizes, with 3 of the 28 layers (every layer does the same
+    work; 28 of them take minutes): Qwen2.5-7B-shaped random weights (hidden 3584, 28/4 heads of 128), one prompt of
+    1 048 576 tokens prefilled through the runtime (MLP in 8192-token chunks, exact attention in the first and last
+    layer, the SQAttn closure with the reference's default windows in the middle one), the whole KV cache resident,
+    k-means clustering of the prompt's keys (1024 clusters, 10 iterations), then greedy decode steps over the 4096-token
+    selection replayed from a HIP graph.  Checked: the generated tokens and cache lengths, and -- against the CPU closed
+    form on the cache rows the step really holds -- one layer's attention over the selection list and its dense decode
+    attention over all 1 048 583 cached tokens."""
+    import math
+    import time
+    import types
+
+    from longcontext_sqattn_paddle_amd.model_hub.qwen import QwenConfig, QwenModel
+    from longcontext_sqattn_paddle_amd.sqattn.attn_replacer import process_model
+    from longcontext_sqattn_paddle_amd.sqattn.attn_triton_decode import attn_decode
+    from oracle import attention as A
+
+    print("case model 3 layers x 1M tokens", flush=True)
+    N, new = 1 << 20, 8
+    cfg = QwenConfig(num_hidden_layers=3)
+    model = QwenModel("Qwen2.5-7B-shaped", N + new + 32, torch.bfloat16, DEV, "SQAttn", config=cfg, seed=1)
+    args = types.SimpleNamespace(qk_qtype="int", v_qtype="int", use_relative_distance=True)
+    process_model(model, "SQAttn", {1: {"bit8": 0.1, "bit4": 0.1, "sink": 256}}, args)
+    model.enable_kv_selection(num_centroids=1024, topk=4096, num_iters=10)
+    ids = torch.randint(0, cfg.vocab_size, (1, N), device=DEV, generator=torch.Generator(device=DEV).manual_seed(2))
+    t0 = time.time()
+    out = model.generate("SQAttn", ids, None, new, verbose=False, use_graph=True)
+    torch.cuda.synchronize()
+    print(f"  prefill {model.prefill_latency:.1f} s, clustering {model.cluster_latency:.2f} s, decode {model.decode_latency * 1e3:.2f} ms/step, "
+          f"total {time.time() - t0:.1f} s", flush=True)
+    assert len(out) == 1 and len(out[0]) == new and all(0 <= t < cfg.vocab_size for t in out[0])
+    cache, sel = model.kv_cache, model.kv_selection
+    assert cache.valid_length.cpu().tolist() == [N + new - 1]
+    # layer 1's attention over the selection list, by hand
+    g = torch.Generator().manual_seed(3)
+    q = torch.randn(1, 1, 28, 128, generator=g).to(torch.bfloat16).to(DEV)
+    sel.begin_step(cache.attend_length)
+    got = sel.attend(1, q, cache.key_cache[1], cache.value_cache[1], 7)
+    torch.cuda.synchronize()
+    n_list = int(sel.list_len[0])
+    assert n_list == 4096 + int(cache.attend_length[0]) - N
+    lists = sel.ids[:, :n_list]
+    assert int(lists[:, :4096].max()) < N and int(lists[:, :4096].min()) >= 0
+    rows = lists.long().clamp(min=0)
+    kc = torch.stack([cache.key_cache[1][0, rows[h], h] for h in range(4)])[None].cpu()      # [1, 4, n_list, 128]
+    vc = torch.stack([cache.value_cache[1][0, rows[h], h] for h in range(4)])[None].cpu()
+    qh = q.cpu().permute(0, 2, 1, 3)
+    ref, _ = A.exact_attention(A.fold_scale(qh, 128), kc, vc, causal=False, score_scale=math.log(2.0))
+    err = float((got.float().cpu().view(28, 128).double() - ref[0, :, 0]).abs().max())
+    assert err <= 2.0 ** -8 * float(ref.abs().max()) + 1e-6, err
+    # the dense decode attention over the whole cache of the same layer
+    L = int(cache.attend_length[0])
+    dense = attn_decode(q, cache.key_cache[1], cache.value_cache[1], "NHD", torch.float32, seqlens=cache.attend_length)
+    torch.cuda.synchronize()
+    kf = cache.key_cache[1][0, :L].cpu().permute(1, 0, 2)[None]
+    vf = cache.value_cache[1][0, :L].cpu().permute(1, 0, 2)[None]
+    ref, _ = A.exact_attention(A.fold_scale(qh, 128), kf, vf, causal=False, score_scale=math.log(2.0))
+    err = float((dense.cpu().view(28, 128).double() - ref[0, :, 0]).abs().max())
+    assert err <= 2e-4 * float(ref.pow(2).mean().sqrt()) + 1e-6, err
