@@ -32,6 +32,9 @@
  *                             :319-326 (mlp), called from model_hub/LLM.py:88-116 (layer_decode)
  *   sq_linear_rows_silu_and_mul  model_hub/qwen.py:320-324 (gate_up_proj and silu_and_mul of mlp) on a decode step
  *   sq_linear_rows_rope       model_hub/qwen.py:302-312 (wqkv) + :352-379 (rotary embedding of q and k) on a decode step
+ *   sq_rmsnorm_linear_rows, sq_rmsnorm_linear_rows_silu_and_mul, sq_rmsnorm_linear_rows_rope
+ *                             the three forms above together with the RMS norm in front of them: model_hub/LLM.py:92-93 + :95
+ *                             (input_layernorm, wqkv), :110-114 (post_attention_layernorm, mlp), :161-163 (norm, lm)
  *   sq_fake_quant_prepass_typed  the same with the float quantiser types of sqattn/attn_replacer.py:340-358
  *   sq_fake_quant_prepass     sqattn/attn_replacer.py:334-365 (GQA expand, key centring and the five fake-quant
  *                             passes of mp_triton_wrapper's closure), sqattn/fake_quant.py:24-58, 98-125
@@ -312,6 +315,24 @@ int sq_linear_rows_rope(const DLTensor* x, const DLTensor* weight, const DLTenso
                         const DLTensor* cos_sin_cache, int32_t head_dim, int32_t rope_features, DLTensor* out,
                         DLTensor* key_cache, DLTensor* value_cache, const DLTensor* valid_length, DLTensor* attend_length,
                         void* stream);
+
+/*
+ * The three projections above applied to rmsnorm(x, norm_weight, epsilon) instead of x, in one pass: the layer norm in
+ * front of wqkv, of the MLP and of the lm head on a decode step (model_hub/qwen.py:345-350 called from
+ * model_hub/LLM.py:92-95, 110-114, 161-163).  norm_weight [K] of x's dtype, contiguous and 16-byte aligned.  The
+ * normalised rows have the bits sq_rmsnorm writes (same operator sequence, same summation order), so each call returns
+ * what sq_rmsnorm followed by the plain form returns.  K at most 8192 (sq_rmsnorm's limit) for one or two rows of x,
+ * 5120 for three or four, 2048 for five to eight: a normalised row has to fit the staging buffer (SQ_EUNSUPPORTED beyond).
+ * Other arguments and requirements as for the plain forms.
+ */
+int sq_rmsnorm_linear_rows(const DLTensor* x, const DLTensor* norm_weight, float epsilon, const DLTensor* weight, const DLTensor* bias,
+                           const DLTensor* residual, DLTensor* out, void* stream);
+int sq_rmsnorm_linear_rows_silu_and_mul(const DLTensor* x, const DLTensor* norm_weight, float epsilon, const DLTensor* weight,
+                                        const DLTensor* bias, DLTensor* out, void* stream);
+int sq_rmsnorm_linear_rows_rope(const DLTensor* x, const DLTensor* norm_weight, float epsilon, const DLTensor* weight, const DLTensor* bias,
+                                const DLTensor* position_ids, const DLTensor* cos_sin_cache, int32_t head_dim, int32_t rope_features,
+                                DLTensor* out, DLTensor* key_cache, DLTensor* value_cache, const DLTensor* valid_length,
+                                DLTensor* attend_length, void* stream);
 
 /*
  * Rotary position embedding of query [T, Hq * head_dim] and key [T, Hkv * head_dim] (T = batch * seq_len tokens)

@@ -104,6 +104,9 @@ SYMBOLS = {
     "sq_linear_rows": (ctypes.c_int, [_P] * 5 + [ctypes.c_void_p]),
     "sq_linear_rows_silu_and_mul": (ctypes.c_int, [_P] * 4 + [ctypes.c_void_p]),
     "sq_linear_rows_rope": (ctypes.c_int, [_P] * 5 + [ctypes.c_int32, ctypes.c_int32] + [_P] * 5 + [ctypes.c_void_p]),
+    "sq_rmsnorm_linear_rows": (ctypes.c_int, [_P, _P, ctypes.c_float] + [_P] * 4 + [ctypes.c_void_p]),
+    "sq_rmsnorm_linear_rows_silu_and_mul": (ctypes.c_int, [_P, _P, ctypes.c_float] + [_P] * 3 + [ctypes.c_void_p]),
+    "sq_rmsnorm_linear_rows_rope": (ctypes.c_int, [_P, _P, ctypes.c_float] + [_P] * 4 + [ctypes.c_int32, ctypes.c_int32] + [_P] * 5 + [ctypes.c_void_p]),
     "sq_kv_cache_store": (ctypes.c_int, [_P] * 4 + [ctypes.c_int32, ctypes.c_int64, ctypes.c_void_p]),
     "sq_kv_cache_append": (ctypes.c_int, [_P] * 6 + [ctypes.c_int32, ctypes.c_void_p]),
     "sq_kv_cache_reorder": (ctypes.c_int, [_P] * 5 + [ctypes.c_void_p]),

@@ -80,17 +80,20 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_kernel(NormArgs a) {
     const int ch = lane + c * 64;
     if (ch < chunks) wt[c] = *(const u32x4_t*)(a.w + ch * 16);
   }
+  // fixed association: the eight rounded squares of a chunk, the lane's chunk sums in ascending order, then the lanes
+  // (the projections that carry this norm in front of them, linear_rows_kernel, form the same sums spread over waves)
   float sum = 0.f;
 #pragma unroll
   for (int c = 0; c < CHUNKS; ++c) {
     if (lane + c * 64 < chunks) {
       float f[8];
       unpack8<BF16>(v[c], f);
+      float p = 0.f;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) sum += rnd<BF16>(f[e] * f[e]);
+      for (int e = 0; e < 8; ++e) p += rnd<BF16>(f[e] * f[e]);
+      sum += p;
     }
   }
-  // fixed-order reduction over the wave
 #pragma unroll
   for (int m = 32; m > 0; m >>= 1) sum += __shfl_xor(sum, m);
   const float var = rnd<BF16>(sum / (float)a.dim);

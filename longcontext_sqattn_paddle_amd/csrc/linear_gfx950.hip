@@ -16,6 +16,11 @@
 // and k parts (model_hub/qwen.py:302-312, 352-379): a wave owns features i and i + head_dim/2 of one head, rotates
 // the pair by the position's cos/sin (fp32 products and sums without fused multiply-add, one rounding, as sq_rope
 // does) and stores both; the waves behind the rotated part produce plain features (v).
+// The sq_rmsnorm_linear_rows* forms take the activation before its RMS norm (model_hub/qwen.py:345-350 in front of wqkv and
+// of mlp, and in front of lm): while the first weights are on their way, the workgroup's waves normalise the rows
+// into LDS with the operator sequence of the stand-alone pass (rmsnorm_kernel: the same association of the sum of
+// squares, the same roundings), so the result has the same bits and the norm's launch, its output tensor and its round
+// trip through memory go away.  Every workgroup repeats the norm of the few rows; that is 14 KB of L2 reads each.
 #include "common.hpp"
 
 namespace sq {
@@ -49,6 +54,9 @@ struct LinArgs {
   const int32_t* valid_length;   // [rows]
   int32_t* attend_length;        // [rows] or null: receives valid_length + 1
   int32_t max_length, q_features, kv_features;
+  // RMS norm of the activation rows in front of the product (null: none); needs chunk == k
+  const char* norm_w;   // [k]
+  float eps;
 };
 
 enum { kModePlain = 0, kModeGated = 1, kModeRope = 2 };
@@ -65,6 +73,11 @@ template <bool BF16>
 __device__ __forceinline__ float ld16(const char* p) {
   const uint32_t bits = *(const uint16_t*)p;
   if constexpr (BF16) return bf16_bits_to_f32(bits);
+  else return (float)__builtin_bit_cast(_Float16, (uint16_t)bits);
+}
+template <bool BF16>
+__device__ __forceinline__ float cv16(uint32_t bits) {   // the low 16 bits as a value
+  if constexpr (BF16) return bf16_bits_to_f32(bits & 0xffffu);
   else return (float)__builtin_bit_cast(_Float16, (uint16_t)bits);
 }
 template <bool BF16>
@@ -163,11 +176,93 @@ __global__ __launch_bounds__(kLinMaxWaves * 64) void linear_rows_kernel(LinArgs 
     };
     if (live) request(0);   // the first weights are on their way while the activations are staged
     if (k0) __syncthreads();
+    if (a.norm_w) {
+      // The sum of squares in the association of rmsnorm_kernel -- lane l owns the 16-byte chunks l, l + 64, ...; each
+      // chunk's eight rounded squares are summed on their own, the chunk sums are added in ascending order, the lanes
+      // fold by a fixed butterfly -- but spread over the waves: (row, chunk index) pairs go round the waves, the chunk
+      // sums meet in LDS, and every wave folds them for itself.  Then x * r (rounded) * weight (rounded by the pack).
+      const int nw = (int)(blockDim.x >> 6);
+      const int per_lane = (chunks + 63) >> 6;
+      const int tasks = M * per_lane;
+      float* part = (float*)(xs + M * row16);   // [M][per_lane][64]
+      auto x_chunk = [&](int t) {
+        const int m = t / per_lane, c = lane + 64 * (t % per_lane);
+        return *(const u32x4_t*)(a.x + (int64_t)(m < a.rows ? m : a.rows - 1) * a.x_sr + (c < chunks ? c : chunks - 1) * 16);
+      };
+      auto w_chunk = [&](int t) {
+        const int c = lane + 64 * (t % per_lane);
+        return *(const u32x4_t*)(a.norm_w + (c < chunks ? c : chunks - 1) * 16);
+      };
+      auto squares = [&](int t, const u32x4_t& v) {
+        float p = 0.f;
+        if (lane + 64 * (t % per_lane) < chunks) {
 #pragma unroll
-    for (int m = 0; m < M; ++m) {
-      const char* xr = a.x + (int64_t)(m < a.rows ? m : a.rows - 1) * a.x_sr + (int64_t)k0 * 2;
+          for (int j = 0; j < 4; ++j) {
+            const float lo = cv16<BF16>(v[j]), hi = cv16<BF16>(v[j] >> 16);
+            p += rnd16<BF16>(lo * lo);
+            p += rnd16<BF16>(hi * hi);
+          }
+        }
+        part[t * 64 + lane] = p;
+      };
+      // a wave's first two chunks and their weights stay in registers across the barrier; further ones are read again
+      constexpr int KEEP = 2;
+      u32x4_t xk[KEEP], gk[KEEP];
+#pragma unroll
+      for (int i = 0; i < KEEP; ++i) {
+        const int t = wave + i * nw;
+        if (t < tasks) {
+          xk[i] = x_chunk(t);
+          gk[i] = w_chunk(t);
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < KEEP; ++i) {
+        const int t = wave + i * nw;
+        if (t < tasks) squares(t, xk[i]);
+      }
+      for (int t = wave + KEEP * nw; t < tasks; t += nw) squares(t, x_chunk(t));
+      __syncthreads();
+      float r[M];
+#pragma unroll
+      for (int m = 0; m < M; ++m) {
+        float sum = 0.f;
+        for (int c = 0; c < per_lane; ++c) sum += part[(m * per_lane + c) * 64 + lane];
+#pragma unroll
+        for (int sft = 32; sft > 0; sft >>= 1) sum += __shfl_xor(sum, sft);
+        const float var = rnd16<BF16>(sum / (float)a.k);
+        const float ve = rnd16<BF16>(var + a.eps);
+        r[m] = rnd16<BF16>(1.0f / sqrtf(ve));
+      }
+      auto scale = [&](int t, const u32x4_t& v, const u32x4_t& g) {
+        const int m = t / per_lane, c = lane + 64 * (t % per_lane);
+        float rr = r[0];
+#pragma unroll
+        for (int i = 1; i < M; ++i) rr = (m == i) ? r[i] : rr;
+        if (c < chunks) {
+          u32x4_t o;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const float lo = cv16<BF16>(v[j]), hi = cv16<BF16>(v[j] >> 16);
+            const float glo = cv16<BF16>(g[j]), ghi = cv16<BF16>(g[j] >> 16);
+            o[j] = (uint32_t)st16<BF16>(rnd16<BF16>(lo * rr) * glo) | ((uint32_t)st16<BF16>(rnd16<BF16>(hi * rr) * ghi) << 16);
+          }
+          xs[m * row16 + c] = o;
+        }
+      };
+#pragma unroll
+      for (int i = 0; i < KEEP; ++i) {
+        const int t = wave + i * nw;
+        if (t < tasks) scale(t, xk[i], gk[i]);
+      }
+      for (int t = wave + KEEP * nw; t < tasks; t += nw) scale(t, x_chunk(t), w_chunk(t));
+    } else {
+#pragma unroll
+      for (int m = 0; m < M; ++m) {
+        const char* xr = a.x + (int64_t)(m < a.rows ? m : a.rows - 1) * a.x_sr + (int64_t)k0 * 2;
 #pragma unroll 4
-      for (int c = threadIdx.x; c < chunks; c += blockDim.x) xs[m * row16 + c] = *(const u32x4_t*)(xr + c * 16);
+        for (int c = threadIdx.x; c < chunks; c += blockDim.x) xs[m * row16 + c] = *(const u32x4_t*)(xr + c * 16);
+      }
     }
     __syncthreads();
     if (live) {
@@ -260,6 +355,10 @@ __global__ __launch_bounds__(kLinMaxWaves * 64) void linear_rows_kernel(LinArgs 
   }
 }
 
+// elements of one activation row the LDS staging buffer holds when the registers are sized for m rows (1, 2, 4, 8)
+constexpr int chunk_cap(int m) { return (m == 8 ? kLinLdsBytes8 : kLinLdsBytes) / (2 * m) / 8 * 8; }
+int max_chunk(int rows) { return chunk_cap(rows <= 1 ? 1 : rows <= 2 ? 2 : rows <= 4 ? 4 : 8); }
+
 template <bool BF16, int M>
 void launch_rows(LinArgs a, int R, int mode, hipStream_t stream) {
   const bool gated = mode == kModeGated;
@@ -272,9 +371,10 @@ void launch_rows(LinArgs a, int R, int mode, hipStream_t stream) {
   const int64_t per_cu = (waves + 255) / 256;
   const int wpw = per_cu <= kLinMaxWaves ? (int)(per_cu < 1 ? 1 : per_cu) : kLinThreads / 64;
   const dim3 grid((unsigned)((waves + wpw - 1) / wpw)), block(wpw * 64);
-  const int cap = (M == 8 ? kLinLdsBytes8 : kLinLdsBytes) / (2 * M) / 8 * 8;
+  constexpr int cap = chunk_cap(M);
   a.chunk = a.k < cap ? a.k : cap;
-  const size_t lds = (size_t)M * a.chunk * 2;
+  // (with the norm in front: the chunk sums of the rows behind the rows themselves)
+  const size_t lds = (size_t)M * a.chunk * 2 + (a.norm_w ? (size_t)M * ((a.k / 8 + 63) / 64) * 256 : 0);
   if (mode == kModeRope) hipLaunchKernelGGL((linear_rows_kernel<BF16, M, 2, kModeRope>), grid, block, lds, stream, a);
   else if (gated) {
     if (R == 4) hipLaunchKernelGGL((linear_rows_kernel<BF16, M, 4, kModeGated>), grid, block, lds, stream, a);
@@ -317,8 +417,13 @@ struct RopeSpec {
   DLTensor* attend_length;   // may be null
 };
 
+struct NormSpec {
+  const DLTensor* weight;
+  float epsilon;
+};
+
 int linear_rows(const char* fn, int mode, const DLTensor* x, const DLTensor* weight, const DLTensor* bias, const DLTensor* residual,
-                DLTensor* out, void* stream, const RopeSpec* rope = nullptr) {
+                DLTensor* out, void* stream, const RopeSpec* rope = nullptr, const NormSpec* norm = nullptr) {
   const bool gated = mode == kModeGated;
   SQ_REQUIRE(x && weight && out, SQ_EINVAL, "%s: null tensor argument", fn);
   int rc;
@@ -355,6 +460,20 @@ int linear_rows(const char* fn, int mode, const DLTensor* x, const DLTensor* wei
                "%s: residual must be [%lld, %lld] of x's dtype with a contiguous last dimension", fn, (long long)M, (long long)N);
   }
   LinArgs a;
+  a.norm_w = nullptr;
+  a.eps = 0.f;
+  if (norm) {
+    const DLTensor* nw = norm->weight;
+    SQ_REQUIRE(nw, SQ_EINVAL, "%s: null tensor argument", fn);
+    if ((rc = check_tensor(nw, "norm_weight", 1, dev))) return rc;
+    SQ_REQUIRE(dtype_of(nw) == dt && nw->shape[0] == K && stride_of(nw, 0) == 1 && (uintptr_t)data_of(nw) % 16 == 0, SQ_ESHAPE,
+               "%s: norm_weight must be a contiguous, 16-byte aligned [%lld] of x's dtype", fn, (long long)K);
+    const int64_t cap = max_chunk((int)M) < 8192 ? max_chunk((int)M) : 8192;   // (8192: the longest row of sq_rmsnorm)
+    SQ_REQUIRE(K <= cap, SQ_EUNSUPPORTED, "%s: with %lld activation rows the normalised row can have at most %lld elements (got %lld)",
+               fn, (long long)M, (long long)cap, (long long)K);
+    a.norm_w = data_of(nw);
+    a.eps = norm->epsilon;
+  }
   a.pos = nullptr;
   a.table = nullptr;
   a.pos_is_i64 = a.max_pos = a.head_dim = a.rope_features = 0;
@@ -456,4 +575,25 @@ extern "C" int sq_linear_rows_rope(const DLTensor* x, const DLTensor* weight, co
                                    void* stream) {
   const RopeSpec rope{position_ids, cos_sin_cache, head_dim, rope_features, key_cache, value_cache, valid_length, attend_length};
   return linear_rows("sq_linear_rows_rope", kModeRope, x, weight, bias, nullptr, out, stream, &rope);
+}
+
+extern "C" int sq_rmsnorm_linear_rows(const DLTensor* x, const DLTensor* norm_weight, float epsilon, const DLTensor* weight, const DLTensor* bias,
+                                      const DLTensor* residual, DLTensor* out, void* stream) {
+  const NormSpec norm{norm_weight, epsilon};
+  return linear_rows("sq_rmsnorm_linear_rows", kModePlain, x, weight, bias, residual, out, stream, nullptr, &norm);
+}
+
+extern "C" int sq_rmsnorm_linear_rows_silu_and_mul(const DLTensor* x, const DLTensor* norm_weight, float epsilon, const DLTensor* weight,
+                                                   const DLTensor* bias, DLTensor* out, void* stream) {
+  const NormSpec norm{norm_weight, epsilon};
+  return linear_rows("sq_rmsnorm_linear_rows_silu_and_mul", kModeGated, x, weight, bias, nullptr, out, stream, nullptr, &norm);
+}
+
+extern "C" int sq_rmsnorm_linear_rows_rope(const DLTensor* x, const DLTensor* norm_weight, float epsilon, const DLTensor* weight,
+                                           const DLTensor* bias, const DLTensor* position_ids, const DLTensor* cos_sin_cache, int32_t head_dim,
+                                           int32_t rope_features, DLTensor* out, DLTensor* key_cache, DLTensor* value_cache,
+                                           const DLTensor* valid_length, DLTensor* attend_length, void* stream) {
+  const RopeSpec rope{position_ids, cos_sin_cache, head_dim, rope_features, key_cache, value_cache, valid_length, attend_length};
+  const NormSpec norm{norm_weight, epsilon};
+  return linear_rows("sq_rmsnorm_linear_rows_rope", kModeRope, x, weight, bias, nullptr, out, stream, &rope, &norm);
 }

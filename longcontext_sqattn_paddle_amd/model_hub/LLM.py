@@ -97,19 +97,20 @@ class LLM:
         residual = hidden_states
         bsz, seq_len, dim = hidden_states.shape
         layer = self.layers[layer_idx]
-        hidden_states = self.layernorm(hidden_states, layer.input_layernorm_variance_epsilon, layer.input_layernorm_weight)
         fused = None
         if seq_len == 1 and hasattr(self, "wqkv_position_embedd"):
-            # projection, rotary embedding and the cache rows of the new token in one pass (same values)
+            # input norm, projection, rotary embedding and the cache rows of the new token in one pass (same values)
+            norm = (layer.input_layernorm_weight, layer.input_layernorm_variance_epsilon)
             targets = self.kv_cache.decode_append_targets(layer_idx) if hasattr(self.kv_cache, "decode_append_targets") else None
-            fused = self.wqkv_position_embedd(hidden_states, layer, cache=targets)
+            fused = self.wqkv_position_embedd(hidden_states, layer, cache=targets, norm=norm)
             appended = fused is not None and targets is not None
             if fused is None:
-                fused = self.wqkv_position_embedd(hidden_states, layer)
+                fused = self.wqkv_position_embedd(hidden_states, layer, norm=norm)
         if fused is not None:
             query_states, key_states, value_states = fused
         else:
             appended = False
+            hidden_states = self.layernorm(hidden_states, layer.input_layernorm_variance_epsilon, layer.input_layernorm_weight)
             query_states, key_states, value_states = self.wqkv(hidden_states, layer)
             query_states, key_states = self.position_embedd(query_states, key_states)
             query_states = query_states.view(bsz, -1, self.num_heads, self.head_dim)
@@ -123,6 +124,9 @@ class LLM:
         if isinstance(attn_out, tuple):   # the slot `process_model(..., patch_decode=True)` binds returns a 1-tuple (LLM.py:105)
             attn_out = attn_out[0]
         residual = self.wo(attn_out, layer, bsz, seq_len, dim, residual=residual)   # residual + wo(...)
+        if seq_len == 1:   # post-attention norm inside the gated projection (same values)
+            return self.mlp(residual, layer, residual=residual,
+                            norm=(layer.post_attention_layernorm_weight, layer.post_attention_layernorm_variance_epsilon))
         hidden_states = self.layernorm(residual, layer.post_attention_layernorm_variance_epsilon,
                                        layer.post_attention_layernorm_weight)
         return self.mlp(hidden_states, layer, residual=residual)                     # residual + mlp(...)
@@ -146,8 +150,7 @@ class LLM:
         hidden_states = self.word_embedding(inputs_ids)
         for ldx in range(self.num_layers):
             hidden_states = self.layer_decode(ldx, hidden_states)
-        hidden_states = self.layernorm(hidden_states[:, -1:, :], self.norm_variance_epsilon, self.norm_weight)
-        return self.lm(hidden_states)
+        return self.lm(hidden_states[:, -1:, :], norm=(self.norm_weight, self.norm_variance_epsilon))
 
     # ------------------------------------------------------------------ captured decode step (extension)
     def capture_decode_step(self, first_token):

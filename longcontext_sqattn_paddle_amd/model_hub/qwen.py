@@ -188,8 +188,9 @@ class QwenModel(LLM):
     def word_embedding(self, inputs_id):
         return torch.nn.functional.embedding(inputs_id, self.embed_tokens)
 
-    def lm(self, hidden_states):
-        return linear(hidden_states, self.lm_head).float()
+    def lm(self, hidden_states, norm=None):
+        """qwen.py:293-300.  `norm` = (weight, epsilon): the final norm in front of the head rides in the same pass."""
+        return linear(hidden_states, self.lm_head, norm=norm).float()
 
     def wqkv(self, hidden_states, layer):
         """qwen.py:302-312: one fused projection, split into views (no copies)."""
@@ -197,19 +198,21 @@ class QwenModel(LLM):
         kv = self.hidden_size // self.num_key_value_groups
         return qkv.split([self.hidden_size, kv, kv], dim=-1)
 
-    def wqkv_position_embedd(self, hidden_states, layer, cache=None):
+    def wqkv_position_embedd(self, hidden_states, layer, cache=None, norm=None):
         """`wqkv` followed by `position_embedd` for a decode step (qwen.py:302-312, 369-379) as one pass: returns
         (query_states [bsz, 1, Hq, head_dim], key_states [bsz, 1, Hkv, head_dim], value_states [bsz, 1, kv_dim]),
         q and k rotated, all three views of one projection output.  `cache`: the layer's
         `kv_cache.decode_append_targets(...)`; the pass then also appends k and v to the cache (None is returned if it
-        cannot, and nothing has been written)."""
+        cannot, and nothing has been written).  `norm` = (weight, epsilon): `hidden_states` is the layer's input before
+        `input_layernorm`, which then is part of the same pass (same values)."""
         bsz, seq_len, _ = hidden_states.shape
         if getattr(self, "_graph_positions", None) is not None and seq_len == 1:
             position_ids = self._graph_positions   # device-resident position of a captured decode step
         else:
             position_ids = self.position_ids[self.kv_cache.context:self.kv_cache.context + seq_len].unsqueeze(0).repeat(bsz, 1)
         kv = self.hidden_size // self.num_key_value_groups
-        qkv = linear_rope(hidden_states, layer.wqkv, layer.bqkv, position_ids, self.head_dim, self.hidden_size + kv, self.cos_sin_cache, cache=cache)
+        qkv = linear_rope(hidden_states, layer.wqkv, layer.bqkv, position_ids, self.head_dim, self.hidden_size + kv, self.cos_sin_cache, cache=cache,
+                          norm=norm)
         if qkv is None:
             return None
         q, k, v = qkv.split([self.hidden_size, kv, kv], dim=-1)
@@ -219,9 +222,10 @@ class QwenModel(LLM):
         """qwen.py:314-317.  With `residual` the caller's `residual + wo(...)` is part of the same pass (same values)."""
         return linear(hidden_states.reshape(bsz, seq_len, dim), layer.wo, None, residual)
 
-    def mlp(self, hidden_states, layer, residual=None):
-        """qwen.py:319-326.  `residual` as in `wo`."""
-        return linear(linear_silu_and_mul(hidden_states, layer.gate_up_proj), layer.down_proj, None, residual)
+    def mlp(self, hidden_states, layer, residual=None, norm=None):
+        """qwen.py:319-326.  `residual` as in `wo`; `norm` = (weight, epsilon): `hidden_states` comes before
+        `post_attention_layernorm`, which a decode step's first projection then applies in the same pass."""
+        return linear(linear_silu_and_mul(hidden_states, layer.gate_up_proj, norm=norm), layer.down_proj, None, residual)
 
     def layernorm(self, hidden_states, epsilon, weight):
         """qwen.py:345-350."""

@@ -39,16 +39,33 @@ def silu_and_mul(hidden_states: torch.Tensor, out: Optional[torch.Tensor] = None
 LINEAR_ROWS_MAX = 8   # sq_linear_rows takes 1 to 8 activation rows; more is a GEMM
 
 
+def _norm_fits(norm, rows: int, K: int, fuse_rows: int = 1) -> bool:
+    """Should the RMS norm in front of a projection ride inside the projection's kernel?  The kernel takes it for up to
+    four rows (8192 elements -- the stand-alone norm's limit -- of one or two rows, 5120 of three or four: the normalised
+    rows have to fit its staging buffer), but every workgroup repeats the norm of every row: with one row that saves the
+    norm's whole launch (gated projection of the decode step 47.1 -> 42.8 us, fused q/k/v 11.4 -> 10.6 us), with four rows
+    it costs more than it saves (52 -> 66 us), hence `fuse_rows`."""
+    w = norm[0]
+    cap = 8192 if rows <= 2 else 5120 if rows <= 4 else 2048
+    return rows <= fuse_rows and K <= cap and w.is_contiguous() and w.data_ptr() % 16 == 0 and w.shape == (K,)
+
+
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None, residual: Optional[torch.Tensor] = None,
-           max_rows: int = 4) -> torch.Tensor:
+           max_rows: int = 4, norm=None, fuse_norm_rows: int = 1) -> torch.Tensor:
     """`x @ weight.T (+ bias) (+ residual)` over the last dimension of x, weight [N, K] (the matmuls of
     model_hub/qwen.py:293-326).  Up to `max_rows` rows of x (a decode step) go through the weight-streaming HIP
     kernel; longer activations (a prompt) are a GEMM and go to the BLAS library.  The kernel takes up to
-    LINEAR_ROWS_MAX rows; from five rows on the library's GEMM is as fast, hence the default."""
+    LINEAR_ROWS_MAX rows; from five rows on the library's GEMM is as fast, hence the default.
+
+    `norm` = (weight, epsilon): the product is taken of `rmsnorm(x, weight, epsilon)`; with up to `fuse_norm_rows` rows
+    on the kernel's route the norm is part of the same pass (same values as the two calls)."""
     _need_gpu(x, weight)
     K = x.shape[-1]
     rows = x.numel() // K
-    if rows > min(max_rows, LINEAR_ROWS_MAX) or K % 8 or weight.stride(-1) != 1 or weight.stride(0) % 8 or weight.data_ptr() % 16:
+    on_kernel = not (rows > min(max_rows, LINEAR_ROWS_MAX) or K % 8 or weight.stride(-1) != 1 or weight.stride(0) % 8 or weight.data_ptr() % 16)
+    if norm is not None and not (on_kernel and _norm_fits(norm, rows, K, fuse_norm_rows)):
+        x, norm = rmsnorm(x, norm[0], norm[1]), None
+    if not on_kernel:
         y = torch.nn.functional.linear(x, weight, bias)
         return y if residual is None else residual + y
     x2 = x.reshape(rows, K)
@@ -58,32 +75,47 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
     out = torch.empty(*x.shape[:-1], n, dtype=x.dtype, device=x.device)
     b = [N.dl(x2), N.dl(weight), N.dl(bias) if bias is not None else None,
          N.dl(residual.reshape(rows, n)) if residual is not None else None, N.dl(out.view(rows, n))]
-    N.check(N.lib().sq_linear_rows(N.ptr(b[0]), N.ptr(b[1]), N.ptr(b[2]) if b[2] is not None else None,
-                                   N.ptr(b[3]) if b[3] is not None else None, N.ptr(b[4]), N.current_stream(x.device)))
+    tail = (N.ptr(b[1]), N.ptr(b[2]) if b[2] is not None else None, N.ptr(b[3]) if b[3] is not None else None, N.ptr(b[4]),
+            N.current_stream(x.device))
+    if norm is not None:
+        nw = N.dl(norm[0])
+        N.check(N.lib().sq_rmsnorm_linear_rows(N.ptr(b[0]), N.ptr(nw), float(norm[1]), *tail))
+    else:
+        N.check(N.lib().sq_linear_rows(N.ptr(b[0]), *tail))
     return out
 
 
-def linear_silu_and_mul(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None, max_rows: int = 4) -> torch.Tensor:
+def linear_silu_and_mul(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None, max_rows: int = 4, norm=None,
+                        fuse_norm_rows: int = 1) -> torch.Tensor:
     """`silu_and_mul(x @ weight.T (+ bias))`, weight [2 I, K] = [gate | up] -> [..., I]: the first half of `mlp`
     (model_hub/qwen.py:320-324).  Up to `max_rows` rows go through one HIP kernel whose waves own both halves of an
-    output pair (same values as `silu_and_mul(linear(x, weight, bias))`); longer activations take that route."""
+    output pair (same values as `silu_and_mul(linear(x, weight, bias))`); longer activations take that route.
+    `norm` as in `linear`."""
     _need_gpu(x, weight)
     K = x.shape[-1]
     rows = x.numel() // K
     n = weight.shape[0]
-    if rows > min(max_rows, LINEAR_ROWS_MAX) or K % 8 or n % 2 or weight.stride(-1) != 1 or weight.stride(0) % 8 or weight.data_ptr() % 16:
+    on_kernel = not (rows > min(max_rows, LINEAR_ROWS_MAX) or K % 8 or n % 2 or weight.stride(-1) != 1 or weight.stride(0) % 8 or weight.data_ptr() % 16)
+    if norm is not None and not (on_kernel and _norm_fits(norm, rows, K, fuse_norm_rows)):
+        x, norm = rmsnorm(x, norm[0], norm[1]), None
+    if not on_kernel:
         return silu_and_mul(torch.nn.functional.linear(x, weight, bias))
     x2 = x.reshape(rows, K)
     if x2.stride(-1) != 1 or (rows > 1 and x2.stride(0) % 8) or x2.data_ptr() % 16:
         x2 = x2.contiguous()
     out = torch.empty(*x.shape[:-1], n // 2, dtype=x.dtype, device=x.device)
     b = [N.dl(x2), N.dl(weight), N.dl(bias), N.dl(out.view(rows, n // 2))]
-    N.check(N.lib().sq_linear_rows_silu_and_mul(*[N.ptr(t) for t in b], N.current_stream(x.device)))
+    if norm is not None:
+        nw = N.dl(norm[0])
+        N.check(N.lib().sq_rmsnorm_linear_rows_silu_and_mul(N.ptr(b[0]), N.ptr(nw), float(norm[1]), *[N.ptr(t) for t in b[1:]],
+                                                            N.current_stream(x.device)))
+    else:
+        N.check(N.lib().sq_linear_rows_silu_and_mul(*[N.ptr(t) for t in b], N.current_stream(x.device)))
     return out
 
 
 def linear_rope(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], position_ids: torch.Tensor, head_dim: int,
-                rope_features: int, cos_sin_cache: torch.Tensor, max_rows: int = 4, cache=None) -> torch.Tensor:
+                rope_features: int, cos_sin_cache: torch.Tensor, max_rows: int = 4, cache=None, norm=None, fuse_norm_rows: int = 1) -> torch.Tensor:
     """The fused q/k/v projection with the rotary embedding of its first `rope_features` output features (the q and
     k heads) in one pass: x [batch, 1, K] -> [batch, 1, N], position_ids one position per row (model_hub/qwen.py:302-312
     and :352-379 on a decode step).  Same values as `linear` followed by `apply_rope_with_cos_sin_cache_inplace`,
@@ -93,7 +125,7 @@ def linear_rope(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tens
     k and the v of every row to row `valid_length` of the caches and sets `attend_length` (what
     `flash_attn_cache.decode_update_kv_cache` does without advancing the length).  Returns None instead of the
     output when `cache` is given but the call cannot go through the kernel: the caller then runs the separate
-    passes."""
+    passes.  `norm` as in `linear`."""
     _need_gpu(x, weight, position_ids, cos_sin_cache)
     K = x.shape[-1]
     rows = x.numel() // K
@@ -101,9 +133,12 @@ def linear_rope(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tens
     pos = position_ids.reshape(-1)
     if pos.dtype not in (torch.int32, torch.int64):
         pos = pos.to(torch.int64)
-    if rows > min(max_rows, LINEAR_ROWS_MAX) or K % 8 or weight.stride(-1) != 1 or weight.stride(0) % 8 or weight.data_ptr() % 16:
-        if cache is not None:
-            return None
+    on_kernel = not (rows > min(max_rows, LINEAR_ROWS_MAX) or K % 8 or weight.stride(-1) != 1 or weight.stride(0) % 8 or weight.data_ptr() % 16)
+    if not on_kernel and cache is not None:
+        return None
+    if norm is not None and not (on_kernel and _norm_fits(norm, rows, K, fuse_norm_rows)):
+        x, norm = rmsnorm(x, norm[0], norm[1]), None
+    if not on_kernel:
         y = torch.nn.functional.linear(x, weight, bias)
         if rope_features > 0:   # the rotation works head by head: any split of the rotated part into two groups of heads will do
             flat = y.view(rows, n)
@@ -119,8 +154,13 @@ def linear_rope(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tens
     out = torch.empty(*x.shape[:-1], n, dtype=x.dtype, device=x.device)
     b = [N.dl(x2), N.dl(weight), N.dl(bias), N.dl(pos.contiguous()), N.dl(cos_sin_cache), N.dl(out.view(rows, n))]
     c = [N.dl(t) for t in cache] if cache is not None else [None] * 4
-    N.check(N.lib().sq_linear_rows_rope(N.ptr(b[0]), N.ptr(b[1]), N.ptr(b[2]), N.ptr(b[3]), N.ptr(b[4]), int(head_dim), int(rope_features),
-                                        N.ptr(b[5]), *[N.ptr(t) for t in c], N.current_stream(x.device)))
+    tail = (N.ptr(b[1]), N.ptr(b[2]), N.ptr(b[3]), N.ptr(b[4]), int(head_dim), int(rope_features), N.ptr(b[5]), *[N.ptr(t) for t in c],
+            N.current_stream(x.device))
+    if norm is not None:
+        nw = N.dl(norm[0])
+        N.check(N.lib().sq_rmsnorm_linear_rows_rope(N.ptr(b[0]), N.ptr(nw), float(norm[1]), *tail))
+    else:
+        N.check(N.lib().sq_linear_rows_rope(N.ptr(b[0]), *tail))
     return out
 
 

@@ -355,3 +355,84 @@ def test_rotary_projection_appends_to_the_kv_cache_like_the_append_pass(dtype, B
         linear_rope(x, w, b, pos, D, (Hq + Hkv) * D, table, max_rows=8, cache=(kc1, vc1, vl1[:B - 1] if B > 1 else torch.zeros(2, dtype=torch.int32, device=DEV), al1))
     with pytest.raises(ValueError):
         linear_rope(x, w, b, pos, D, (Hq + Hkv) * D, table, max_rows=8, cache=(kc1, vc1, None, al1))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,N,K", [(1, 4608, 3584), (1, 152064, 3584), (2, 1000, 1024), (3, 520, 4104), (4, 37888, 3584), (1, 24, 8),
+                                   (1, 512, 8192), (2, 264, 8192), (4, 64, 5120)])
+def test_projections_with_the_norm_in_front_equal_norm_then_projection(dtype, M, N, K):
+    """sq_rmsnorm_linear_rows*: the RMS norm of the activation rows inside the projection's pass gives the bits of
+    sq_rmsnorm followed by the plain form (each checked against the oracle above), for the plain, the gated and the
+    rotary projection, with and without the cache rows."""
+    from longcontext_sqattn_paddle_amd.model_hub.utils import linear, linear_rope, linear_silu_and_mul, rmsnorm, yarn_cos_sin_cache
+
+    print(f"case norm + linear {dtype} M={M} N={N} K={K}", flush=True)
+    g = torch.Generator().manual_seed(M + N + K)
+    x = (torch.randn(M, 1, K, generator=g) * 3.0).to(dtype).to(DEV)
+    gamma = (1.0 + 0.2 * torch.randn(K, generator=g)).to(dtype).to(DEV)
+    w = (torch.randn(N, K, generator=g) * 2 * K ** -0.5).to(dtype).to(DEV)
+    b = torch.randn(N, generator=g).to(dtype).to(DEV)
+    res = torch.randn(M, 1, N, generator=g).to(dtype).to(DEV)
+    eps = 1e-6
+    xn = rmsnorm(x, gamma, eps)
+    for bias, residual in ((b, None), (None, res), (b, res)):
+        got = linear(x, w, bias, residual, max_rows=4, norm=(gamma, eps), fuse_norm_rows=4)
+        want = linear(xn, w, bias, residual, max_rows=4)
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    if N % 2 == 0:
+        got = linear_silu_and_mul(x, w, b, norm=(gamma, eps), fuse_norm_rows=4)
+        want = linear_silu_and_mul(xn, w, b)
+        assert got.shape == (M, 1, N // 2) and torch.equal(got.view(torch.int16), want.view(torch.int16))
+    D = 8 if N < 512 else 128
+    if N % (4 * D) == 0:     # [q (2 heads' worth) | k | v] of equal thirds would not be GQA: q = N/2, k = v = N/4
+        Hkv = N // (4 * D)
+        rope = N // 2 + Hkv * D
+        table = yarn_cos_sin_cache(D, 1000000.0, 32768, 5000, DEV)
+        pos = torch.randint(0, 5000, (M, 1), generator=g).to(DEV)
+        got = linear_rope(x, w, b, pos, D, rope, table, norm=(gamma, eps), fuse_norm_rows=4)
+        want = linear_rope(xn, w, b, pos, D, rope, table)
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+        L = 12
+        lens = torch.randint(0, L, (M,), generator=g).to(torch.int32)
+        base_k = torch.randn(M, L, Hkv, D, generator=g).to(dtype)
+        base_v = torch.randn(M, L, Hkv, D, generator=g).to(dtype)
+        c1 = (base_k.to(DEV), base_v.to(DEV), lens.to(DEV), torch.zeros(M, dtype=torch.int32, device=DEV))
+        c2 = (base_k.to(DEV), base_v.to(DEV), lens.to(DEV), torch.zeros(M, dtype=torch.int32, device=DEV))
+        got = linear_rope(x, w, b, pos, D, rope, table, cache=c1, norm=(gamma, eps), fuse_norm_rows=4)
+        want = linear_rope(xn, w, b, pos, D, rope, table, cache=c2)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want)
+        for t1, t2 in zip(c1, c2):
+            assert torch.equal(t1, t2)
+
+
+def test_norm_in_front_hand_over_and_errors():
+    """Rows or row lengths the fused pass does not take go through the two passes with the same result; the C entry
+    point itself refuses a row that does not fit its staging buffer, a norm weight of another length or dtype."""
+    from longcontext_sqattn_paddle_amd import _native as NV
+    from longcontext_sqattn_paddle_amd.model_hub.utils import linear, linear_silu_and_mul, rmsnorm, silu_and_mul
+
+    g = torch.Generator().manual_seed(8)
+    dtype = torch.bfloat16
+    for M, K in ((4, 8192), (3, 5128), (6, 512), (9, 512)):
+        x = torch.randn(M, K, generator=g).to(dtype).to(DEV)
+        gamma = (1.0 + 0.2 * torch.randn(K, generator=g)).to(dtype).to(DEV)
+        w = (torch.randn(256, K, generator=g) * K ** -0.5).to(dtype).to(DEV)
+        xn = rmsnorm(x, gamma, 1e-5)
+        assert torch.equal(linear(x, w, max_rows=8, norm=(gamma, 1e-5)), linear(xn, w, max_rows=8))
+        assert torch.equal(linear_silu_and_mul(x, w, max_rows=8, norm=(gamma, 1e-5)), linear_silu_and_mul(xn, w, max_rows=8))
+    x = torch.randn(4, 8192, generator=g).to(dtype).to(DEV)
+    w = torch.randn(64, 8192, generator=g).to(dtype).to(DEV)
+    o = torch.empty(4, 64, dtype=dtype, device=DEV)
+    good = torch.ones(8192, dtype=dtype, device=DEV)
+    for xx, gm in ((x, good),                                    # four rows of 8192 elements do not fit
+                   (x[:1], torch.ones(4096, dtype=dtype, device=DEV)),      # wrong length
+                   (x[:1], torch.ones(8192, dtype=torch.float16, device=DEV))):   # wrong dtype
+        bb = [NV.dl(xx), NV.dl(gm), NV.dl(w), NV.dl(o[:xx.shape[0]])]
+        with pytest.raises((AssertionError, NotImplementedError, TypeError, ValueError)):
+            NV.check(NV.lib().sq_rmsnorm_linear_rows(NV.ptr(bb[0]), NV.ptr(bb[1]), 1e-6, NV.ptr(bb[2]), None, None, NV.ptr(bb[3]),
+                                                     NV.current_stream(o.device)))
+    bb = [NV.dl(x[:1]), NV.dl(good), NV.dl(w), NV.dl(o[:1])]
+    NV.check(NV.lib().sq_rmsnorm_linear_rows(NV.ptr(bb[0]), NV.ptr(bb[1]), 1e-6, NV.ptr(bb[2]), None, None, NV.ptr(bb[3]), NV.current_stream(o.device)))
+    torch.cuda.synchronize()
+    assert torch.equal(o[:1], linear(rmsnorm(x[:1], good, 1e-6), w))
