@@ -82,6 +82,48 @@ def time_prefill(torch, qkv, steps, warmup, p_quant):
     return ms, flops
 
 
+def time_mfma_only(torch, qkv):
+    """What the matrix cores sustain when a kernel issues nothing but MFMAs (`sq_probe_mfma_rate`: one workgroup of
+    eight waves per CU, operands loaded once): with constant operands, and with operand registers that hold values like
+    this workload's -- bf16 words of the benchmark's own K tensor; e4m3 codes of uniform probabilities x 448 and of V.  The
+    published peaks are reached on constant operands only: on random ones the chip lowers its clock under the matrix
+    cores' switching power.  The last figure is the harmonic blend for half the FLOPs on each pipe, as in P mode 5."""
+    from longcontext_sqattn_paddle_amd import _native as NV
+
+    dev = qkv[1].device
+    lib = NV.lib()
+    nbytes = int(lib.sq_probe_mfma_operand_bytes())
+    sink = torch.empty(131072, dtype=torch.float32, device=dev)
+    k_words = qkv[1].reshape(-1)[:nbytes // 2].contiguous()
+    g = torch.Generator(device=dev).manual_seed(12)
+    p8 = (torch.rand(nbytes // 2, device=dev, generator=g) * 448.0).to(torch.float8_e4m3fn)
+    v8 = (qkv[2].reshape(-1)[:nbytes // 2].float() * 2.0 ** 12).to(torch.float8_e4m3fn)   # N(0,1)/sqrt(128) scaled into e4m3's range
+    f8 = torch.cat([p8.view(torch.uint8), v8.view(torch.uint8)]).contiguous()
+    sets = {"bf16_constant": (0, torch.ones(nbytes // 2, dtype=torch.bfloat16, device=dev)), "bf16_workload_values": (0, k_words),
+            "e4m3_constant": (1, torch.full((nbytes,), 0x38, dtype=torch.uint8, device=dev)), "e4m3_workload_values": (1, f8)}
+    out = {}
+    stream = torch.cuda.current_stream(dev)
+    for name, (kind, ops) in sets.items():
+        iters = 20000 if kind == 0 else 10000
+        b = [NV.dl(ops), NV.dl(sink)]
+        times = []
+        for rep in range(4):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            NV.check(lib.sq_probe_mfma_rate(kind, NV.ptr(b[0]), NV.ptr(b[1]), iters, NV.current_stream(dev)))
+            e1.record(stream)
+            torch.cuda.synchronize()
+            times.append(e0.elapsed_time(e1))
+        ms = sorted(times[1:])[1]
+        out[name] = round(int(lib.sq_probe_mfma_flops(kind, iters)) / ms / 1e9, 1)
+    out["blend_workload_values"] = round(1.0 / (0.5 / out["bf16_workload_values"] + 0.5 / out["e4m3_workload_values"]), 1)
+    out["unit"] = "TFLOP/s"
+    out["note"] = ("a loop of nothing but MFMAs, two waves per SIMD on all 256 CUs, about 10 ms per launch: the published peaks hold for "
+                   "constant operands; the figures on workload values are what this GPU sustains on operands like the benchmark's, "
+                   "before any load, LDS or vector instruction shares the power budget")
+    return out
+
+
 def time_plugin(torch, qkv, steps=3):
     """The path `ATTN_TYPE=SQAttn` dispatches to (sqattn/attn_replacer.py:423-448): the closure of `mp_triton_wrapper`
     = operand pre-pass (key centring, int8 fake quantisation) + sink/window kernel with relative windows, at the prefill
@@ -574,6 +616,7 @@ def main():
                          "4 = 3 plus e4m3 V so that P.V runs on the fp8 matrix pipe, "
                          "5 (default) = 4 with one power-of-two block scale per query row and 64-key tile on P")
     ap.add_argument("--no-variants", action="store_true", help="skip the other P modes (0 - 4) of the prefill kernel")
+    ap.add_argument("--no-mfma-probe", action="store_true", help="skip the MFMA-only loop (sustained matrix-core rate on constant / workload operands)")
     ap.add_argument("--no-plugin", action="store_true", help="skip the plugin closure (pre-pass + sink/window kernel)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="run one 1 GiB device-to-device copy first: a kernel of known traffic for scaling FETCH_SIZE/WRITE_SIZE")
@@ -654,6 +697,12 @@ def main():
             "numerics": "P mode 5 is build-defined (the reference multiplies fp16 P by fp16 V): see `variants` for the reference's own modes",
         },
     }
+    if not args.no_mfma_probe:
+        probe = time_mfma_only(torch, qkv)
+        ceiling = probe["blend_workload_values"] if args.p_quant >= 4 else probe["bf16_workload_values"]
+        result["roofline"]["mfma_only_loop"] = probe
+        result["roofline"]["frac_of_mfma_only_loop"] = round(tflops / ceiling, 4)
+        log(f"[bench] MFMA-only loop: {probe}")
     if not args.no_variants:
         # the reference's own numerics (modes 0 and 1) and the other P modes, a few steps each: the kernel is the same,
         # only the quantisation of P (and of V in mode 4) differs.  Each entry is priced against the peak of the matrix

@@ -35,6 +35,7 @@
  *   sq_rmsnorm_linear_rows, sq_rmsnorm_linear_rows_silu_and_mul, sq_rmsnorm_linear_rows_rope
  *                             the three forms above together with the RMS norm in front of them: model_hub/LLM.py:92-93 + :95
  *                             (input_layernorm, wqkv), :110-114 (post_attention_layernorm, mlp), :161-163 (norm, lm)
+ *   sq_probe_mfma_rate        no reference counterpart: measurement aid (the rate of a loop of nothing but MFMAs on given operands)
  *   sq_fake_quant_prepass_typed  the same with the float quantiser types of sqattn/attn_replacer.py:340-358
  *   sq_fake_quant_prepass     sqattn/attn_replacer.py:334-365 (GQA expand, key centring and the five fake-quant
  *                             passes of mp_triton_wrapper's closure), sqattn/fake_quant.py:24-58, 98-125
@@ -370,6 +371,19 @@ typedef struct sq_histogram_params {
   float softmax_scale;  /* 1/sqrt(head_dim before padding) (attn_replacer.py:260)            */
 } sq_histogram_params;
 int sq_attention_histogram(const DLTensor* q, const DLTensor* k, DLTensor* hist, const sq_histogram_params* p, void* stream);
+
+/*
+ * Measurement aid, no counterpart in the reference: runs a kernel that issues nothing but MFMAs -- one workgroup of
+ * eight waves on each of 256 CUs, `iters` x 16 instructions per wave on four accumulators, kind 0 =
+ * v_mfma_f32_32x32x16_bf16, kind 1 = v_mfma_f32_32x32x64_f8f6f4 on e4m3 -- with operand registers loaded once from
+ * `operands` (any dtype, at least sq_probe_mfma_operand_bytes() bytes: 64 bytes per lane and operand set, four sets per
+ * lane).  The time of the launch, taken by the caller, and sq_probe_mfma_flops(kind, iters) give the rate the matrix
+ * cores sustain on such operands: with constant operands the published peak, with random ones about a quarter less
+ * (the chip lowers its clock).  sink: fp32, at least 131072 elements, receives the accumulators' sums.
+ */
+size_t sq_probe_mfma_operand_bytes(void);
+int64_t sq_probe_mfma_flops(int32_t kind, int32_t iters);
+int sq_probe_mfma_rate(int32_t kind, const DLTensor* operands, DLTensor* sink, int32_t iters, void* stream);
 
 #ifdef __cplusplus
 }

@@ -9,7 +9,7 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 INCLUDE = os.path.join(os.path.dirname(PKG_DIR), "include")
 LIB_PATH = os.path.join(PKG_DIR, "libsqattn_hip.so")
-SOURCES = ["capi.hip", "decode_gfx950.hip", "prefill_gfx950.hip", "kmeans_gfx950.hip", "prepass_gfx950.hip", "kvcache_gfx950.hip", "layer_gfx950.hip", "linear_gfx950.hip", "calib_gfx950.hip"]
+SOURCES = ["capi.hip", "decode_gfx950.hip", "prefill_gfx950.hip", "kmeans_gfx950.hip", "prepass_gfx950.hip", "kvcache_gfx950.hip", "layer_gfx950.hip", "linear_gfx950.hip", "calib_gfx950.hip", "probe_gfx950.hip"]
 
 HIPCC_FLAGS = [
     "-O3", "-std=c++17", "--offload-arch=gfx950", "-fPIC", "-shared",

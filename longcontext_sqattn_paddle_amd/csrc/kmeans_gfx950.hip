@@ -86,9 +86,17 @@ __global__ __launch_bounds__(kAssignWaves * 64, 1) void kmeans_assign_kernel(Ass
       }
     }
   };
+  // Fragment number n = 8 half + kk of a block: centroid row 32 half + c32, 16-byte chunk (2 kk + g) ^ (row & 15).  The
+  // reads go through lds_read128 / lds_wait (explicit lgkmcnt counts): left to the compiler, every wait was a full
+  // lgkmcnt(0), i.e. also for the fragments requested a moment ago.
   const int ksw = c32 & 15;
-  auto frag = [&](const char* buf, int half, int kk) {
-    return __builtin_bit_cast(bf16x8_t, *(const uint4*)(buf + (32 * half + c32) * 256 + (((2 * kk + g) ^ ksw) << 4)));
+  const uint32_t smem_addr = (uint32_t)(uintptr_t)(lds_ptr_t)smem;
+  uint32_t fa[8];
+#pragma unroll
+  for (int kk = 0; kk < 8; ++kk) fa[kk] = smem_addr + c32 * 256 + (((2 * kk + g) ^ ksw) << 4);
+  auto frag = [&](uint32_t boff, auto NUM) {
+    constexpr int n = decltype(NUM)::value;
+    return lds_read128<(n >> 3) * 8192>(fa[n & 7] + boff);
   };
   // Running arg-max in ascending centroid order with strict '>' = lowest index on ties (kmeans.py:62-65), four scores
   // at a time: the group's maximum (v_max3 + v_max) is compared with the running best; a group that wins leaves its
@@ -110,29 +118,39 @@ __global__ __launch_bounds__(kAssignWaves * 64, 1) void kmeans_assign_kernel(Ass
   for (int tb = 0; tb < 2; ++tb)
 #pragma unroll
     for (int i = 0; i < 16; ++i) S[tb][1][i] = -INFINITY;   // "previous phase" of the very first one
-  auto group_max = [](const f32x16_t& P, int q) {
-    // (fmaxf would quiet each operand first, one more instruction per score; the scores are never signalling NaNs)
+  // One group of four scores against the running best, as one instruction block in the short encodings with the
+  // condition in VCC (the compiler's form of the same selects is a masked block of moves behind s_and_saveexec):
+  // VCC = not (m > best); a group that wins leaves its id and its first three scores behind.
+  auto group_step = [&](const f32x16_t& P, int tb, auto Q) {
+    constexpr int q = decltype(Q)::value;
     float m;
-    asm("v_max3_f32 %0, %1, %2, %3\n\tv_max_f32 %0, %0, %4" : "=&v"(m) : "v"(P[4 * q]), "v"(P[4 * q + 1]), "v"(P[4 * q + 2]), "v"(P[4 * q + 3]));
-    return m;
+    float &b = best[tb], &k0 = keep0[tb], &k1 = keep1[tb], &k2 = keep2[tb];
+    int& grp = bgrp[tb];
+    asm volatile(
+        "v_max3_f32 %[m], %[p0], %[p1], %[p2]\n\t"
+        "v_max_f32_e32 %[m], %[m], %[p3]\n\t"
+        "v_cmp_le_f32_e32 vcc, %[m], %[best]\n\t"
+        "v_cndmask_b32_e32 %[k0], %[p0], %[k0], vcc\n\t"
+        "v_cndmask_b32_e32 %[k1], %[p1], %[k1], vcc\n\t"
+        "v_cndmask_b32_e32 %[k2], %[p2], %[k2], vcc\n\t"
+        "v_cndmask_b32_e32 %[grp], %[qq], %[grp], vcc\n\t"
+        "v_max_f32_e32 %[best], %[best], %[m]"
+        : [m] "=&v"(m), [best] "+v"(b), [k0] "+v"(k0), [k1] "+v"(k1), [k2] "+v"(k2), [grp] "+v"(grp)
+        : [p0] "v"(P[4 * q]), [p1] "v"(P[4 * q + 1]), [p2] "v"(P[4 * q + 2]), [p3] "v"(P[4 * q + 3]), [qq] "n"(q)
+        : "vcc");
   };
-  auto group_take = [&](const f32x16_t& P, int tb, int q, float m, bool gt) {
-    best[tb] = gt ? m : best[tb];
-    bgrp[tb] = gt ? q : bgrp[tb];
-    keep0[tb] = gt ? P[4 * q] : keep0[tb];
-    keep1[tb] = gt ? P[4 * q + 1] : keep1[tb];
-    keep2[tb] = gt ? P[4 * q + 2] : keep2[tb];
-  };
-  auto phase = [&](auto H, const char* buf, int half_id) {
+  // The 16 centroid fragments of a block (half h, slice kk -> number 8 h + kk) are requested kFragAhead steps before
+  // the MFMA pair that uses them: an LDS read takes longer than one pair of MFMAs when eight waves read at once.
+  constexpr int kFragAhead = 3;
+  auto phase = [&](auto H, uint32_t boff, int half_id, u32x4_t (&fr)[16]) {
     constexpr int h = decltype(H)::value;   // centroid half computed now; the arg-max runs over half 1 - h
     const float before0 = best[0], before1 = best[1];
-    bf16x8_t af = frag(buf, h, 0);
-    float m = 0.f;
-    bool gt = false;
     static_for<0, 8>([&](auto KK) {
       constexpr int kk = decltype(KK)::value;
-      bf16x8_t nf = af;
-      if constexpr (kk < 7) nf = frag(buf, h, kk + 1);
+      constexpr int cur = 8 * h + kk, nxt = cur + kFragAhead;
+      if constexpr (nxt < 16) fr[nxt] = frag(boff, std::integral_constant<int, nxt>{});
+      lds_wait<(15 - cur < kFragAhead ? 15 - cur : kFragAhead)>(fr[cur]);
+      const bf16x8_t af = __builtin_bit_cast(bf16x8_t, fr[cur]);
       static_for<0, 2>([&](auto TB) {
         constexpr int tb = decltype(TB)::value;
         const bf16x8_t t = __builtin_bit_cast(bf16x8_t, tf[tb][kk]);
@@ -143,18 +161,12 @@ __global__ __launch_bounds__(kAssignWaves * 64, 1) void kmeans_assign_kernel(Ass
           S[tb][h] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, t, S[tb][h], 0, 0, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
-        // group kk of the previous phase's 8 groups (token set kk >> 2, scores 4 (kk & 3) .. + 3): its maximum under
-        // the first MFMA of the pair, the selects under the second
+        // group kk of the previous phase's 8 groups (token set kk >> 2, scores 4 (kk & 3) .. + 3), behind the first
+        // MFMA of the pair
         constexpr int ctb = kk >> 2, q = kk & 3;
-        if constexpr (tb == 0) {
-          m = group_max(S[ctb][1 - h], q);
-          gt = m > best[ctb];
-        } else {
-          group_take(S[ctb][1 - h], ctb, q, m, gt);
-        }
+        if constexpr (tb == 0) group_step(S[ctb][1 - h], ctb, std::integral_constant<int, q>{});
         __builtin_amdgcn_sched_barrier(0);
       });
-      af = nf;
     });
     // the scores just examined belong to the half before this one
     bhalf[0] = (best[0] > before0) ? half_id - 1 : bhalf[0];
@@ -167,20 +179,20 @@ __global__ __launch_bounds__(kAssignWaves * 64, 1) void kmeans_assign_kernel(Ass
     // block `chunk` has landed for every wave, and every wave has finished reading block chunk - 1, whose buffer the
     // next block may now overwrite; it has this block's 32 MFMAs per wave to arrive
     __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
     if (chunk + 1 < nchunks) stage(chunk + 1, (chunk + 1) & 1);
-    const char* buf = smem + (chunk & 1) * (kCB * 256);
-    phase(std::integral_constant<int, 0>{}, buf, 2 * chunk);
-    phase(std::integral_constant<int, 1>{}, buf, 2 * chunk + 1);
+    const uint32_t boff = (chunk & 1) * (kCB * 256);
+    u32x4_t fr[16];
+    static_for<0, kFragAhead>([&](auto I) { fr[decltype(I)::value] = frag(boff, I); });
+    __builtin_amdgcn_sched_barrier(0);
+    phase(std::integral_constant<int, 0>{}, boff, 2 * chunk, fr);
+    phase(std::integral_constant<int, 1>{}, boff, 2 * chunk + 1, fr);
   }
   {   // the last half block
     const float before0 = best[0], before1 = best[1];
-#pragma unroll
-    for (int tb = 0; tb < 2; ++tb)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const float m = group_max(S[tb][1], q);
-        group_take(S[tb][1], tb, q, m, m > best[tb]);
-      }
+    static_for<0, 2>([&](auto TB) {
+      static_for<0, 4>([&](auto Q) { group_step(S[decltype(TB)::value][1], decltype(TB)::value, Q); });
+    });
     bhalf[0] = (best[0] > before0) ? 2 * nchunks - 1 : bhalf[0];
     bhalf[1] = (best[1] > before1) ? 2 * nchunks - 1 : bhalf[1];
   }
