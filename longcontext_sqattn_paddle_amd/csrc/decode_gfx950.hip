@@ -334,48 +334,55 @@ constexpr int kCombineThreads = 1024;
 constexpr int kCombineChunk = 32;                       // output channels per workgroup
 constexpr int kCombineGroups = kCombineThreads / kCombineChunk;   // 32 groups of 32 threads, each sums every 32nd split
 
-// One workgroup per (q head, batch): weights of all splits are formed in parallel in LDS, then 8 groups of 128
-// threads (one thread per output channel) each sum an eighth of the splits with independent, unrolled loads.
+// One workgroup per (q head, batch, 32 output channels): 32 groups of 32 threads (one thread per channel), each sums
+// every 32nd split.  A thread's first eight partial outputs are requested before anything else, so that they travel while
+// the weights of the splits are formed (maximum and sum of 2^(lse - max): one shuffle reduction per wave, the 16 wave
+// results through LDS, three barriers in all).
 __global__ __launch_bounds__(kCombineThreads) void decode_combine_kernel(CombineArgs a) {
   extern __shared__ float s_w[];          // [num_splits] weights, then [32][32] partial outputs
-  __shared__ float s_red[kCombineThreads];
+  __shared__ float s_red[2][kCombineThreads / 64];
   const int h = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
   const int S = a.num_splits;
   const int64_t row0 = ((int64_t)b * a.Hq + h) * S;
+  const int dl = tid & (kCombineChunk - 1), grp = tid / kCombineChunk;
+  const int d = blockIdx.z * kCombineChunk + dl;
+  const float* po = a.part_o + row0 * kD + d;
+  constexpr int G = kCombineGroups;
+  constexpr int kPre = 8;
+  float x[kPre];
+#pragma unroll
+  for (int i = 0; i < kPre; ++i) x[i] = (grp + i * G < S) ? po[(int64_t)(grp + i * G) * kD] : 0.f;
   float mx = -INFINITY;
   for (int s = tid; s < S; s += kCombineThreads) mx = fmaxf(mx, a.part_lse[row0 + s]);
-  s_red[tid] = mx;
+#pragma unroll
+  for (int m = 32; m > 0; m >>= 1) mx = fmaxf(mx, __shfl_xor(mx, m));
+  if ((tid & 63) == 0) s_red[0][tid >> 6] = mx;
   __syncthreads();
-  for (int d = kCombineThreads / 2; d > 0; d >>= 1) {
-    if (tid < d) s_red[tid] = fmaxf(s_red[tid], s_red[tid + d]);
-    __syncthreads();
-  }
-  mx = s_red[0];
-  __syncthreads();
+#pragma unroll
+  for (int w = 0; w < kCombineThreads / 64; ++w) mx = fmaxf(mx, s_red[0][w]);
   float tot = 0.f;
   for (int s = tid; s < S; s += kCombineThreads) {
     const float w = (mx > -INFINITY) ? exp2f(a.part_lse[row0 + s] - mx) : 0.f;
     s_w[s] = w;
     tot += w;
   }
-  s_red[tid] = tot;
+#pragma unroll
+  for (int m = 32; m > 0; m >>= 1) tot += __shfl_xor(tot, m);
+  if ((tid & 63) == 0) s_red[1][tid >> 6] = tot;
   __syncthreads();
-  for (int d = kCombineThreads / 2; d > 0; d >>= 1) {
-    if (tid < d) s_red[tid] += s_red[tid + d];
-    __syncthreads();
-  }
-  tot = s_red[0];
-  const int dl = tid & (kCombineChunk - 1), grp = tid / kCombineChunk;
-  const int d = blockIdx.z * kCombineChunk + dl;
-  const float* po = a.part_o + row0 * kD + d;
-  constexpr int G = kCombineGroups;
+  tot = 0.f;
+#pragma unroll
+  for (int w = 0; w < kCombineThreads / 64; ++w) tot += s_red[1][w];   // the same order in every thread
   float o = 0.f;
-  int s = grp;
+#pragma unroll
+  for (int i = 0; i < kPre; ++i)
+    if (grp + i * G < S) o += s_w[grp + i * G] * x[i];                  // an empty split has weight 0 and a zero partial
+  int s = grp + kPre * G;
   for (; s + 3 * G < S; s += 4 * G) {   // 4 independent loads in flight
     const float w0 = s_w[s], w1 = s_w[s + G], w2 = s_w[s + 2 * G], w3 = s_w[s + 3 * G];
     const float x0 = po[(int64_t)s * kD], x1 = po[(int64_t)(s + G) * kD], x2 = po[(int64_t)(s + 2 * G) * kD],
                 x3 = po[(int64_t)(s + 3 * G) * kD];
-    o += w0 * x0 + w1 * x1 + w2 * x2 + w3 * x3;   // an empty split has weight 0 and a zero partial
+    o += w0 * x0 + w1 * x1 + w2 * x2 + w3 * x3;
   }
   for (; s < S; s += G) o += s_w[s] * po[(int64_t)s * kD];
   float* s_part = s_w + S;
