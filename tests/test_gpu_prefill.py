@@ -342,3 +342,57 @@ def test_full_size_128k_sampled_rows(mode):
             assert err <= (4e-3 if mode == 0 else 8e-2) * scale, (h, i, err, scale)
             assert abs(float(lse[0, h, i]) - ref_lse) <= 2e-3, (h, i, float(lse[0, h, i]), ref_lse)
     print(f"  worst relative row error {worst:.2e}", flush=True)
+
+
+def test_window_configurations_drawn_at_random():
+    """A seeded sweep over what the window entry points take: sequence lengths that are not multiples of the tile, sink
+    sizes from none to longer than the sequence, per-head windows from nothing to everything (8-bit wider or narrower than
+    4-bit), 1 to 7 q heads per kv head, both layouts, relative and absolute sizes -- each case against the oracle's
+    block-wise restatement over `kv_ranges` (2e-3 rms) and its LSE."""
+    from longcontext_sqattn_paddle_amd.sqattn.attn_triton_mix_bad import attn_hierarchical_window
+    from longcontext_sqattn_paddle_amd.sqattn.attn_triton_mix_relative import attn_hierarchical_relative_window
+
+    rng = torch.Generator().manual_seed(2024)
+
+    def pick(options):
+        return options[int(torch.randint(0, len(options), (1,), generator=rng))]
+
+    for case in range(24):
+        N = int(torch.randint(65, 2100, (1,), generator=rng))
+        group = pick([1, 2, 4, 7])
+        Hkv = pick([1, 2])
+        Hq = Hkv * group
+        sink = pick([0, 64, 128, 256, 512, 4096])
+        layout = pick(["HND", "NHD"])
+        relative = case % 2 == 0
+        q, k, v = _rand(1, Hq, Hkv, N, 128, 1000 + case)
+        if relative:
+            r8 = [pick([0.0, 0.05, 0.1, 0.25, 0.5, 1.0, 2.0]) for _ in range(Hq)]
+            r4 = [pick([0.0, 0.1, 0.3, 0.5, 1.0]) for _ in range(Hq)]
+            w8 = [A.window_size_relative(x, N) for x in r8]
+            w4 = [A.window_size_relative(x, N) for x in r4]
+            # the documented rule for a 4-bit window wider than an 8-bit window below the query block: the 8-bit window is
+            # raised to the block (the reference's ranges would read future keys unmasked there)
+            w8 = [max(a8, 64) if a4 > a8 else a8 for a8, a4 in zip(w8, w4)]
+            block_m = 64
+        else:
+            w8 = [pick([0, 128, 256, 384, 1024, 4096]) for _ in range(Hq)]
+            w4 = [pick([0, 128, 512, 640, 2048]) for _ in range(Hq)]
+            w8 = [max(a8, 128) if a4 > a8 else a8 for a8, a4 in zip(w8, w4)]   # (a 4-bit window wider than an 8-bit window below the query block is refused)
+            block_m = 128
+        print(f"case windows #{case}: N={N} Hq={Hq} Hkv={Hkv} sink={sink} {layout} {'relative' if relative else 'absolute'} w8={w8} w4={w4}", flush=True)
+        ref, lse_ref = A.prefill_blockwise(q, k, v, block_m=block_m, sink=sink, w8=w8, w4=w4, out_dtype=torch.float32)
+        if layout == "NHD":
+            qd, kd, vd = (t.permute(0, 2, 1, 3).contiguous().to(DEV) for t in (q, k, v))
+        else:
+            qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
+        if relative:
+            out, lse = attn_hierarchical_relative_window(qd, kd, qd, kd, vd, r8, r4, sink, layout, torch.float32, return_lse=True)
+        else:
+            out, lse = attn_hierarchical_window(qd, kd, qd, kd, vd, torch.tensor(w8, dtype=torch.int32), torch.tensor(w4, dtype=torch.int32),
+                                                sink, layout, torch.float32, return_lse=True)
+        torch.cuda.synchronize()
+        if layout == "NHD":
+            out = out.permute(0, 2, 1, 3)
+        _check(out, ref, False)
+        assert torch.allclose(lse.cpu(), lse_ref, atol=2e-4), case
