@@ -289,3 +289,36 @@ def test_attn_unified_decode_lse_is_in_the_frame_of_the_centred_keys(layout):
     out = out[:, 0] if layout == "NHD" else out[:, :, 0]
     assert float((out.double() - ref[:, :, 0]).abs().max()) < 2e-4 * float(ref.pow(2).mean().sqrt()) + 1e-6
     assert torch.allclose(lse.cpu().double().view(2, 28), lse_ref[:, :, 0], atol=2e-3)
+
+
+def test_decode_configurations_drawn_at_random():
+    """A seeded sweep over the decode entry point: batch sizes, GQA ratios from 1 to 20 q heads per kv head, cache lengths
+    that are not multiples of the 16-token tile, ragged valid lengths down to a single token, both layouts, explicit split
+    counts from 1 to more than there are tiles -- each against exact attention over the valid prefix."""
+    rng = torch.Generator().manual_seed(77)
+
+    def pick(options):
+        return options[int(torch.randint(0, len(options), (1,), generator=rng))]
+
+    for case in range(20):
+        B = pick([1, 2, 3, 5])
+        Hkv = pick([1, 2, 4])
+        Hq = Hkv * pick([1, 2, 7, 20])
+        L = int(torch.randint(1, 2600, (1,), generator=rng))
+        layout = pick(["NHD", "HND"])
+        splits = pick([None, 1, 2, 7, 64, 300])
+        q, kc, vc, _ = inputs.decode_inputs(B, Hq, Hkv, L, 128, seed=500 + case)
+        lens = [int(torch.randint(1, L + 1, (1,), generator=rng)) for _ in range(B)]
+        lens[0] = L if case % 3 else 1
+        print(f"case decode #{case}: B={B} Hq={Hq} Hkv={Hkv} L={L} lens={lens} {layout} splits={splits}", flush=True)
+        qh, kh, vh = _to_hnd(q, kc, vc)
+        ref, lse_ref = A.exact_attention(A.fold_scale(qh, 128), kh, vh, causal=False, kv_lens=lens, score_scale=math.log(2.0))
+        args = (q, kc, vc) if layout == "NHD" else (qh, kh, vh)
+        kw = {} if splits is None else {"num_splits": splits}
+        out, lse = _run(*args, lens, layout, output_dtype=torch.float32, return_lse=True, **kw)
+        out = out.cpu()
+        out = out[:, 0] if layout == "NHD" else out[:, :, 0]
+        rms = float(ref.pow(2).mean().sqrt())
+        err = float((out.double() - ref[:, :, 0]).abs().max())
+        assert err < 2e-4 * rms + 1e-6, (case, err, rms)
+        assert torch.allclose(lse.cpu()[:, :, 0].double(), lse_ref[:, :, 0], atol=2e-4), case

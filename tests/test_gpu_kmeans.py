@@ -139,3 +139,41 @@ def test_full_size_properties():
     assert bool((gap[differ] < NEAR_TIE).all())
     nrm = cd.cpu()[size > 0].float().norm(dim=-1)
     assert float((nrm - 1).abs().max()) < 1e-2
+
+
+def test_kmeans_configurations_drawn_at_random():
+    """A seeded sweep over the training step and the index helpers: 1 to 5 groups, token counts that are not multiples of the
+    256-token tile (down to fewer tokens than centroids), centroid counts from 32 to 1056 (multiples of 32, with and
+    without a half block at the end), normalised or not -- each against the oracle under the rules at the top."""
+    from longcontext_sqattn_paddle_amd.cache_hub.kmeans import _triton_k_means_train, triton_index_add, triton_reverse_index
+
+    rng = torch.Generator().manual_seed(99)
+
+    def pick(options):
+        return options[int(torch.randint(0, len(options), (1,), generator=rng))]
+
+    for case in range(12):
+        G = pick([1, 2, 3, 5])
+        C = 32 * pick([1, 2, 3, 5, 8, 17, 33])
+        N = int(torch.randint(max(40, C // 2), 6000, (1,), generator=rng))
+        normalize = bool(case % 2)
+        print(f"case kmeans #{case}: G={G} N={N} C={C} normalize={normalize}", flush=True)
+        key, value = inputs.kmeans_inputs(G, N, 128, n_modes=min(C, 40), seed=600 + case)
+        cent0 = key[:, torch.randint(0, N, (C,), generator=rng)].clone()   # repeated picks give duplicate centroids
+        ref_idx, gap = KM.assign(key, cent0)
+        cent_d = cent0.clone().to(DEV)
+        _, idx_d, max_cnt = _triton_k_means_train(key.to(DEV), cent_d, normalize_centroids=normalize, return_indices=True)
+        torch.cuda.synchronize()
+        idx = idx_d.cpu()
+        differ = idx != ref_idx
+        assert bool((gap[differ] < NEAR_TIE).all()), (case, int(differ.sum()))
+        S, cnt = KM.cluster_sums(key, idx, C)
+        assert max_cnt == int(cnt.max())
+        ulp = _bf16_ulp_diff(cent_d.cpu(), KM.update(cent0, S, cnt, normalize))
+        assert int(ulp.max()) <= 1 and float((ulp > 0).float().mean()) <= 1e-3, case
+        clusters, size = triton_reverse_index(idx_d, C, max_cnt)
+        vsum = triton_index_add(value.to(DEV), idx_d, C)
+        torch.cuda.synchronize()
+        rc, rs = KM.reverse_index(idx, C, max_cnt)
+        assert torch.equal(size.cpu(), rs) and torch.equal(clusters.cpu(), rc), case
+        assert torch.equal(vsum.cpu(), KM.index_add(value, idx, C)), case
