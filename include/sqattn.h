@@ -52,7 +52,7 @@
 extern "C" {
 #endif
 
-#define SQ_ABI_VERSION 1
+#define SQ_ABI_VERSION 2
 
 enum {
   SQ_OK = 0,
@@ -102,6 +102,11 @@ typedef struct sq_prefill_params {
   int32_t num_heads_w;   /* number of entries of w8/w4 (== Hq)                                            */
   const int32_t* w8;     /* HOST arrays: per-head 8-bit / 4-bit window sizes in tokens (multiples of 64). */
   const int32_t* w4;     /* The relative wrapper converts ratios with ceil128(int(f32(ratio)*kv_len)).    */
+  int32_t q_quant;       /* 0: q as given.  8: every row of q (not of q4) goes through the symmetric 8-bit  */
+                         /* per-token fake quantiser as it is loaded -- IntegerQuantizer(8, True,          */
+                         /* "per_token"), sqattn/fake_quant.py:33-35, 47-52, 114-125, the pass             */
+                         /* sqattn/attn_replacer.py:361 runs on the query -- with the bits the pass        */
+                         /* sq_fake_quant_prepass writes, so the closure need not write and re-read q8     */
 } sq_prefill_params;
 
 /* Bytes of device workspace sq_prefill_fwd needs (fp16 transposed V tiles). */
@@ -202,7 +207,8 @@ size_t sq_fake_quant_prepass_workspace_bytes(int64_t batch, int64_t num_kv_heads
  * heads: key_c = key - mean over tokens (mean = dtype(float(exact sum / N)), subtraction rounded to the tensor
  * dtype); q8/q4 = IntegerQuantizer(8|4, True, "per_token").fake_quant_tensor(query); k8/k4 the same of key_c;
  * v8 = IntegerQuantizer(8, True, "per_channel").fake_quant_tensor(value), whose scale is per (token, channel)
- * over batch and heads as in the reference (range over dims 0 and 1 of [B,H,N,D]).  q4 and k4 may both be null.
+ * over batch and heads as in the reference (range over dims 0 and 1 of [B,H,N,D]).  q4 and k4 may both be null; q8 may
+ * be null as well (with q4 and k4): the query is then left alone, for a caller that sets sq_prefill_params.q_quant = 8.
  * query/q8/q4 [B,N,Hq,128] and key/value/k8/k4/v8 [B,N,Hkv,128] for SQ_LAYOUT_NHD ([B,H,N,128] for
  * SQ_LAYOUT_HND), bf16 or fp16, all of one dtype; any strides with a contiguous last dimension and 16-byte
  * aligned rows.  Outputs are bit-identical to the formulas evaluated in fp32 on the host.

@@ -53,6 +53,7 @@ class PrefillParams(ctypes.Structure):
         ("num_heads_w", ctypes.c_int32),
         ("w8", ctypes.POINTER(ctypes.c_int32)),
         ("w4", ctypes.POINTER(ctypes.c_int32)),
+        ("q_quant", ctypes.c_int32),
     ]
 
 
@@ -132,7 +133,7 @@ def lib() -> ctypes.CDLL:
             fn = getattr(handle, name)
             fn.restype = res
             fn.argtypes = args
-        if handle.sq_abi_version() != 1:
+        if handle.sq_abi_version() != 2:
             raise RuntimeError("libsqattn_hip.so ABI version mismatch")
         _lib = handle
     return _lib

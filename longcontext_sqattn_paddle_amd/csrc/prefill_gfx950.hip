@@ -56,6 +56,7 @@ struct PrefillArgs {
   int32_t B, Hq, Hkv, group, Nq, Nk, nT, nQB;
   int32_t q_offset, p_quant, window_mode, block_m, sink, out_dtype;
   int32_t sched_mode, sched_xpp, sched_items, sched_pairs;
+  int32_t q_quant;   // 8: the rows of q (not of q4) are fake-quantised to 8 bits per token as they are loaded
   float sm;
   int32_t w8[kMaxHeads];
   int32_t w4[kMaxHeads];
@@ -207,6 +208,18 @@ __device__ __forceinline__ uint32_t pack_f16(float lo, float hi) {
   typedef __attribute__((ext_vector_type(2))) _Float16 f16x2_t;
   f32x2_t v = {lo, hi};
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2_t));
+}
+
+// one 16-bit element of the tensor dtype as a value, and back (round to nearest even)
+template <bool BF16>
+__device__ __forceinline__ float elem16(uint32_t bits) {
+  if constexpr (BF16) return bf16_bits_to_f32(bits & 0xffffu);
+  else return (float)__builtin_bit_cast(_Float16, (uint16_t)bits);
+}
+template <bool BF16>
+__device__ __forceinline__ uint32_t bits16(float x) {
+  if constexpr (BF16) return f32_to_bf16_bits(x);
+  else return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)x);
 }
 
 template <bool BF16>
@@ -457,12 +470,37 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
     const uint16_t* qp = (const uint16_t*)qbase + (int64_t)b * a.q_sb + (int64_t)head * a.q_sh;
     const int row = max(min(row_w0 + c32, a.Nq - 1), 0);
     const uint16_t* rp = qp + (int64_t)row * a.q_sn + 8 * g;
+    uint4 raw[8];
 #pragma unroll
-    for (int kk = 0; kk < 8; ++kk) {
-      const uint4 raw = *(const uint4*)(rp + 16 * kk);
-      qf[kk] = make_uint4(scale_pair<BF16>(raw.x, a.sm), scale_pair<BF16>(raw.y, a.sm), scale_pair<BF16>(raw.z, a.sm),
-                          scale_pair<BF16>(raw.w, a.sm));
+    for (int kk = 0; kk < 8; ++kk) raw[kk] = *(const uint4*)(rp + 16 * kk);
+    if (a.q_quant == 8 && qbase == a.q) {
+      // IntegerQuantizer(8, True, "per_token").fake_quant_tensor of the row (fake_quant.py:33-35, 47-52, 114-125) with the
+      // operations of the stand-alone pre-pass (prepass_rows_kernel: the same maximum, the same correctly rounded
+      // division, round half away, clamp, product, rounding to the tensor dtype), so the operand has the same bits as a
+      // row that went through that pass and memory.  The row's 128 elements sit in this lane and the lane 32 away.
+      float amax = 0.f;
+#pragma unroll
+      for (int kk = 0; kk < 8; ++kk) {
+        const uint32_t w[4] = {raw[kk].x, raw[kk].y, raw[kk].z, raw[kk].w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) amax = fmaxf(amax, fmaxf(fabsf(elem16<BF16>(w[j] & 0xffffu)), fabsf(elem16<BF16>(w[j] >> 16))));
+      }
+      amax = fmaxf(xor32_max(amax), 1e-5f);
+      const Divisor scale = make_divisor(amax / 127.f);
+      auto qdq_elem = [&](float x) {   // clamp(round(x / scale) + zero, -128, 127) * scale with zero = 0.0 (turns -0.0 into +0.0)
+        const float t = divide(x, scale);
+        return fminf(fmaxf(copysignf(floorf(fabsf(t) + 0.5f), t) + 0.0f, -128.f), 127.f) * scale.d;
+      };
+      auto qdq_word = [&](uint32_t w) {
+        return bits16<BF16>(qdq_elem(elem16<BF16>(w & 0xffffu))) | (bits16<BF16>(qdq_elem(elem16<BF16>(w >> 16))) << 16);
+      };
+#pragma unroll
+      for (int kk = 0; kk < 8; ++kk) raw[kk] = make_uint4(qdq_word(raw[kk].x), qdq_word(raw[kk].y), qdq_word(raw[kk].z), qdq_word(raw[kk].w));
     }
+#pragma unroll
+    for (int kk = 0; kk < 8; ++kk)
+      qf[kk] = make_uint4(scale_pair<BF16>(raw[kk].x, a.sm), scale_pair<BF16>(raw[kk].y, a.sm), scale_pair<BF16>(raw[kk].z, a.sm),
+                          scale_pair<BF16>(raw[kk].w, a.sm));
   };
   load_q(a.q);
   bool q_is4 = false;
@@ -1215,6 +1253,8 @@ extern "C" int sq_prefill_fwd(const DLTensor* q, const DLTensor* k, const DLTens
   local.nT = nT;
   const int rows_wg = waves * 32;
   local.nQB = (int)((Nq + rows_wg - 1) / rows_wg);
+  SQ_REQUIRE(p->q_quant == 0 || p->q_quant == 8, SQ_EINVAL, "sq_prefill_fwd: q_quant must be 0 or 8 (got %d)", (int)p->q_quant);
+  local.q_quant = p->q_quant;
   local.q_offset = (int)p->q_offset;
   local.p_quant = p->p_quant;
   local.window_mode = p->window_mode;

@@ -324,8 +324,11 @@ extern "C" int sq_fake_quant_prepass_typed(const DLTensor* query, const DLTensor
                                            int32_t layout, int32_t qk_qtype, int32_t v_qtype, void* stream) {
   SQ_REQUIRE(qk_qtype >= SQ_QTYPE_INT && qk_qtype <= SQ_QTYPE_E5M2 && v_qtype >= SQ_QTYPE_INT && v_qtype <= SQ_QTYPE_E5M2, SQ_EINVAL,
              "Invalid quantization type: %d / %d", (int)qk_qtype, (int)v_qtype);
-  SQ_REQUIRE(query && key && value && q8 && k8 && v8, SQ_EINVAL, "sq_fake_quant_prepass: null tensor argument");
+  SQ_REQUIRE(query && key && value && k8 && v8, SQ_EINVAL, "sq_fake_quant_prepass: null tensor argument");
   SQ_REQUIRE((q4 == nullptr) == (k4 == nullptr), SQ_EINVAL, "sq_fake_quant_prepass: q4 and k4 must be given together");
+  // q8 == NULL: the query rows are left alone (the attention kernel can quantise them as it loads them, q_quant = 8)
+  SQ_REQUIRE(q8 || !q4, SQ_EINVAL, "sq_fake_quant_prepass: without q8 there are no 4-bit operands either");
+  const bool skip_q = q8 == nullptr;
   SQ_REQUIRE(layout == SQ_LAYOUT_HND || layout == SQ_LAYOUT_NHD, SQ_EINVAL, "Unknown tensor layout: %d", (int)layout);
   int rc;
   if ((rc = check_tensor(query, "query", 4, query->device.device_id))) return rc;
@@ -344,7 +347,7 @@ extern "C" int sq_fake_quant_prepass_typed(const DLTensor* query, const DLTensor
   PrepassArgs a;
   memset(&a, 0, sizeof(a));
   if ((rc = make_view(query, "query", layout, dev, dt, B, N, Hq, &a.q)) || (rc = make_view(key, "key", layout, dev, dt, B, N, Hkv, &a.k)) ||
-      (rc = make_view(value, "value", layout, dev, dt, B, N, Hkv, &a.v)) || (rc = make_view(q8, "q8", layout, dev, dt, B, N, Hq, &a.q8)) ||
+      (rc = make_view(value, "value", layout, dev, dt, B, N, Hkv, &a.v)) || (!skip_q && (rc = make_view(q8, "q8", layout, dev, dt, B, N, Hq, &a.q8))) ||
       (rc = make_view(k8, "k8", layout, dev, dt, B, N, Hkv, &a.k8)) || (rc = make_view(v8, "v8", layout, dev, dt, B, N, Hkv, &a.v8)))
     return rc;
   if (q4 && ((rc = make_view(q4, "q4", layout, dev, dt, B, N, Hq, &a.q4)) || (rc = make_view(k4, "k4", layout, dev, dt, B, N, Hkv, &a.k4))))
@@ -374,7 +377,8 @@ extern "C" int sq_fake_quant_prepass_typed(const DLTensor* query, const DLTensor
   const int64_t qrows = B * N * Hq, krows = B * N * Hkv, vthreads = N * (kPD / 8);
 #define SQ_PREPASS_ROWS(BF, QT)                                                                                        \
   do {                                                                                                                 \
-    hipLaunchKernelGGL((prepass_rows_kernel<BF, false, QT>), dim3((unsigned)((qrows + 31) / 32)), dim3(256), 0, s, a); \
+    if (!skip_q)                                                                                                       \
+      hipLaunchKernelGGL((prepass_rows_kernel<BF, false, QT>), dim3((unsigned)((qrows + 31) / 32)), dim3(256), 0, s, a); \
     hipLaunchKernelGGL((prepass_rows_kernel<BF, true, QT>), dim3((unsigned)((krows + 31) / 32)), dim3(256), 0, s, a);  \
   } while (0)
 #define SQ_PREPASS_LAUNCH(BF)                                                                                       \

@@ -18,8 +18,9 @@ def prefill_workspace(B: int, Hkv: int, kv_len: int, device) -> torch.Tensor:
 
 def run_prefill(q, k, v, *, tensor_layout="HND", output_dtype=torch.float16, return_lse=False, p_quant=N.P_NONE,
                 q4=None, k4=None, window: Optional[dict] = None, q_offset: int = 0,
-                workspace: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None):
-    """window = None (full causal) or {"block_m": 64|128, "sink": int, "w8": [Hq ints], "w4": [Hq ints]}."""
+                workspace: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None, q_quant: int = 0):
+    """window = None (full causal) or {"block_m": 64|128, "sink": int, "w8": [Hq ints], "w4": [Hq ints]}.
+    q_quant = 8: the kernel applies the 8-bit per-token fake quantiser to the rows of q as it loads them."""
     if tensor_layout not in N.LAYOUT:
         raise ValueError(f"tensor_layout {tensor_layout} not supported")
     require_gpu(q, k, v, q4, k4)
@@ -39,6 +40,7 @@ def run_prefill(q, k, v, *, tensor_layout="HND", output_dtype=torch.float16, ret
     params.p_quant = p_quant
     params.head_dim_og = head_dim_og
     params.q_offset = q_offset
+    params.q_quant = int(q_quant)
     keep = []
     if window is None:
         params.window_mode = N.WINDOW_NONE

@@ -124,9 +124,15 @@ def mp_triton_wrapper(layer_idx, bit8_window_sizes=0, bit4_window_sizes=0, sink_
             # one fused HIP pre-pass instead of the reference's tensor passes (:338-365), for every quantiser type.  The
             # relative launch aliases the 4-bit operands to the 8-bit ones (attn_triton_mix_relative.py:441-444), so
             # they are only produced for the absolute variant.
+            # With the integer quantiser and relative windows the query does not go through the pre-pass at all: the
+            # attention kernel quantises its rows while loading them (same bits), which saves writing and re-reading q8.
+            q_in_kernel = relative and args.qk_qtype == "int"
             q_bit8, q_bit4, k_bit8, k_bit4, v_bit8 = fused_int_prepass(query, key, value, want_4bit=not relative, tensor_layout=layout,
-                                                                       qk_qtype=args.qk_qtype, v_qtype=args.v_qtype)
+                                                                       qk_qtype=args.qk_qtype, v_qtype=args.v_qtype, skip_query=q_in_kernel)
+            if q_in_kernel:
+                q_bit8 = query
         else:
+            q_in_kernel = False
             bit8_qk, bit4_qk, bit8_v = _quantizers(args)
             if nhd:   # the quantisers' "per_channel" range is over dims (0, 1) of [B,H,N,D]: quantise HND views
                 query, key, value = (t.permute(0, 2, 1, 3) for t in (query, key, value))
@@ -144,7 +150,7 @@ def mp_triton_wrapper(layer_idx, bit8_window_sizes=0, bit4_window_sizes=0, sink_
             attn_output = attn_hierarchical_relative_window(
                 q_bit8, k_bit8, q_bit8, k_bit8, v_bit8, int8_window_ratios=bit8_window_sizes,
                 int4_window_ratios=bit4_window_sizes, sink_size=sink_window_size, tensor_layout=layout,
-                output_dtype=torch.bfloat16, p_quant=p_quant)
+                output_dtype=torch.bfloat16, p_quant=p_quant, q_quant=8 if q_in_kernel else 0)
         else:
             attn_output = attn_hierarchical_window(
                 q_bit8, k_bit8, q_bit4, k_bit4, v_bit8, int8_window_sizes=bit8_window_sizes,

@@ -140,14 +140,16 @@ class FloatQuantizer(BaseQuantizer):
         return float_quantize(scaled.float(), self.e_bits, self.m_bits, rounding="nearest")
 
 
-def fused_int_prepass(query, key, value, want_4bit=True, tensor_layout="NHD", qk_qtype="int", v_qtype="int"):
+def fused_int_prepass(query, key, value, want_4bit=True, tensor_layout="NHD", qk_qtype="int", v_qtype="int", skip_query=False):
     """The operand pre-pass of `mp_triton_wrapper`'s closure (attn_replacer.py:334-365) as one call into the HIP
     library: key centring, per-token 8-bit (and integer 4-bit) fake quantisation of query and centred key, per-channel
     8-bit fake quantisation of value -- without expanding the kv heads.  `qk_qtype` / `v_qtype` pick the 8-bit
     quantisers as the closure does (:340-358): "int", "e4m3" or "e5m2".
 
     query [B,N,Hq,D], key/value [B,N,Hkv,D] for "NHD" ([B,H,N,D] for "HND"), bf16 or fp16, D == 128.
-    Returns (q8, q4, k8, k4, v8) in the layout of the inputs; q4 and k4 are None unless `want_4bit`.
+    Returns (q8, q4, k8, k4, v8) in the layout of the inputs; q4 and k4 are None unless `want_4bit`.  With `skip_query`
+    the query is left alone and q8 is None (the attention kernel applies the 8-bit integer quantiser while it loads the
+    rows, `q_quant=8`); not together with `want_4bit`.
     """
     from .. import _native as N
     from ._common import require_gpu
@@ -161,7 +163,10 @@ def fused_int_prepass(query, key, value, want_4bit=True, tensor_layout="NHD", qk
     hdim, ndim = (1, 2) if tensor_layout == "HND" else (2, 1)
     B, Hkv, Nk = key.size(0), key.size(hdim), key.size(ndim)
     lib = N.lib()
-    q8, k8, v8 = torch.empty_like(query), torch.empty_like(key), torch.empty_like(value)
+    if skip_query and want_4bit:
+        raise ValueError("skip_query leaves no query to derive the 4-bit operands from")
+    q8 = None if skip_query else torch.empty_like(query)
+    k8, v8 = torch.empty_like(key), torch.empty_like(value)
     q4 = torch.empty_like(query) if want_4bit else None
     k4 = torch.empty_like(key) if want_4bit else None
     need = lib.sq_fake_quant_prepass_workspace_bytes(B, Hkv, Nk)

@@ -149,3 +149,35 @@ def test_decode_slot():
                                kv_lens=[int(x) for x in lens])
     assert out.shape == (2, 1, 8 * 128)
     assert _cos(out.float().cpu(), ref.permute(0, 2, 1, 3).reshape(2, 1, 1024)) >= 0.9999
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("layout", ["NHD", "HND"])
+def test_query_quantised_while_loaded_equals_the_separate_pass(dtype, layout):
+    """sq_prefill_params.q_quant = 8: the 8-bit per-token fake quantisation of the query rows inside the attention kernel
+    gives the output bits of the same kernel on a query that went through sq_fake_quant_prepass -- for rows with large and
+    tiny ranges, an all-zero row, GQA, a length that is not a multiple of the tile."""
+    from longcontext_sqattn_paddle_amd.sqattn.attn_triton_mix_relative import attn_hierarchical_relative_window
+    from longcontext_sqattn_paddle_amd.sqattn.fake_quant import fused_int_prepass
+
+    B, N, Hq, Hkv, D = 2, 1100, 14, 2, 128
+    g = torch.Generator().manual_seed(321)
+    q = torch.randn(B, N, Hq, D, generator=g) * torch.logspace(-6, 2, N)[None, :, None, None]   # row ranges from 1e-6 to 100
+    q[0, 5] = 0.0
+    q[1, 7, 3] = 1e-7
+    k = torch.randn(B, N, Hkv, D, generator=g)
+    v = torch.randn(B, N, Hkv, D, generator=g)
+    q, k, v = (t.to(dtype).to(DEV) for t in (q, k, v))
+    if layout == "HND":
+        q, k, v = (t.permute(0, 2, 1, 3).contiguous() for t in (q, k, v))
+    q8, _, k8, _, v8 = fused_int_prepass(q, k, v, want_4bit=False, tensor_layout=layout)
+    none, _, k8b, _, v8b = fused_int_prepass(q, k, v, want_4bit=False, tensor_layout=layout, skip_query=True)
+    assert none is None and torch.equal(k8, k8b) and torch.equal(v8, v8b)
+    two, lse2 = attn_hierarchical_relative_window(q8, k8, q8, k8, v8, 0.25, 0.5, 128, layout, torch.float32, return_lse=True)
+    one, lse1 = attn_hierarchical_relative_window(q, k8, q, k8, v8, 0.25, 0.5, 128, layout, torch.float32, return_lse=True, q_quant=8)
+    torch.cuda.synchronize()
+    assert torch.equal(one.view(torch.int32), two.view(torch.int32)) and torch.equal(lse1.view(torch.int32), lse2.view(torch.int32))
+    with pytest.raises(ValueError):
+        attn_hierarchical_relative_window(q, k8, q, k8, v8, 0.25, 0.5, 128, layout, torch.float32, q_quant=4)
+    with pytest.raises(ValueError):
+        fused_int_prepass(q, k, v, want_4bit=True, tensor_layout=layout, skip_query=True)
