@@ -227,6 +227,16 @@ int sq_fake_quant_prepass(const DLTensor* query, const DLTensor* key, const DLTe
  * library's fp32 log2 rounds a value just below a power of two up to the integer.
  */
 enum { SQ_QTYPE_INT = 0, SQ_QTYPE_E4M3 = 1, SQ_QTYPE_E5M2 = 2 };
+/*
+ * The pre-pass for a real integer Q.K^T (sq_prefill_int8qk_fwd): key centring as above, then instead of the fake-
+ * quantised key its two factors -- k_codes int8 [like key] = clamp(round(key_c / scale), -128, 127), the codes
+ * IntegerQuantizer(8, True, "per_token") multiplies by its scale (sqattn/fake_quant.py:114-125), and k_scale fp32
+ * [B, Hkv, S >= N] = that scale per token (entries past N are left alone) -- and v8 as above.  The query is not touched:
+ * the attention kernel forms its codes and scale from the rows it loads.
+ */
+int sq_fake_quant_prepass_int8qk(const DLTensor* query, const DLTensor* key, const DLTensor* value, DLTensor* k_codes,
+                                 DLTensor* k_scale, DLTensor* v8, DLTensor* workspace, int32_t layout, void* stream);
+
 int sq_fake_quant_prepass_typed(const DLTensor* query, const DLTensor* key, const DLTensor* value, DLTensor* q8,
                                 DLTensor* q4, DLTensor* k8, DLTensor* k4, DLTensor* v8, DLTensor* workspace,
                                 int32_t layout, int32_t qk_qtype, int32_t v_qtype, void* stream);

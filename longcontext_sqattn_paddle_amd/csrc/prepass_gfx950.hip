@@ -34,6 +34,11 @@ struct PrepassArgs {
   double* part;     // [nblk, B*Hkv*128]
   uint16_t* mean;   // [B*Hkv*128] bits of the key mean in the tensor dtype
   int32_t B, N, Hq, Hkv, is_bf16, nblk, tok_per_blk, want4;
+  // integer operands of a real int8 Q.K^T (null: not wanted): the 8-bit codes of the centred key, laid out like key with
+  // one byte per element, and the per-token scales, fp32 [B, Hkv, scale_stride] (token index last)
+  View kcodes;
+  float* kscale;
+  int64_t scale_stride;
 };
 
 
@@ -239,13 +244,29 @@ __global__ __launch_bounds__(256) void prepass_rows_kernel(PrepassArgs a) {
     for (int sh = 1; sh < 16; sh <<= 1) amax = fmaxf(amax, __shfl_xor(amax, sh));
     amax = fmaxf(amax, 1e-5f);
     if (!live[u]) continue;
-    {
+    if (d8.p) {
       const Divisor scale = make_divisor(scale_of<QT>(amax));
       float y[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e) y[e] = qdq8<QT>(x[e], scale);
       const uint4 o = pack8<BF16>(y);
       __builtin_nontemporal_store(u32x4_t{o.x, o.y, o.z, o.w}, (u32x4_t*)((uint16_t*)d8.p + off8[u]));
+    }
+    if constexpr (CENTRE && QT == 0) {
+      if (a.kcodes.p) {   // the codes themselves (what qdq multiplies by the scale) and the scale
+        const Divisor scale = make_divisor(amax / 127.f);
+        uint32_t w[2] = {0, 0};
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int c = (int)fminf(fmaxf(round_half_away(divide(x[e], scale)) + 0.0f, -128.f), 127.f);
+          w[e >> 2] |= (uint32_t)(c & 0xff) << (8 * (e & 3));
+        }
+        const int64_t row = row0 + u;
+        const int h = (int)(row % H);
+        const int64_t n = (row / H) % a.N, b = row / ((int64_t)H * a.N);
+        *(uint2*)((char*)a.kcodes.p + b * a.kcodes.sb + n * a.kcodes.sn + h * a.kcodes.sh + 8 * l16) = make_uint2(w[0], w[1]);
+        if (l16 == 0) a.kscale[(b * H + h) * a.scale_stride + n] = scale.d;
+      }
     }
     if (a.want4) {
       const Divisor scale = make_divisor(amax / 7.f);
@@ -319,12 +340,32 @@ extern "C" size_t sq_fake_quant_prepass_workspace_bytes(int64_t batch, int64_t n
   return (size_t)nblk * cols * sizeof(double) + ((cols * 2 + 255) & ~(size_t)255);
 }
 
+namespace {
+int prepass_impl(const DLTensor* query, const DLTensor* key, const DLTensor* value, DLTensor* q8, DLTensor* q4, DLTensor* k8, DLTensor* k4,
+                 DLTensor* v8, DLTensor* workspace, int32_t layout, int32_t qk_qtype, int32_t v_qtype, void* stream, DLTensor* k_codes,
+                 DLTensor* k_scale);
+}
+
 extern "C" int sq_fake_quant_prepass_typed(const DLTensor* query, const DLTensor* key, const DLTensor* value, DLTensor* q8,
                                            DLTensor* q4, DLTensor* k8, DLTensor* k4, DLTensor* v8, DLTensor* workspace,
                                            int32_t layout, int32_t qk_qtype, int32_t v_qtype, void* stream) {
+  return prepass_impl(query, key, value, q8, q4, k8, k4, v8, workspace, layout, qk_qtype, v_qtype, stream, nullptr, nullptr);
+}
+
+extern "C" int sq_fake_quant_prepass_int8qk(const DLTensor* query, const DLTensor* key, const DLTensor* value, DLTensor* k_codes,
+                                            DLTensor* k_scale, DLTensor* v8, DLTensor* workspace, int32_t layout, void* stream) {
+  SQ_REQUIRE(k_codes && k_scale, SQ_EINVAL, "sq_fake_quant_prepass_int8qk: null tensor argument");
+  return prepass_impl(query, key, value, nullptr, nullptr, nullptr, nullptr, v8, workspace, layout, SQ_QTYPE_INT, SQ_QTYPE_INT, stream, k_codes,
+                      k_scale);
+}
+
+namespace {
+int prepass_impl(const DLTensor* query, const DLTensor* key, const DLTensor* value, DLTensor* q8, DLTensor* q4, DLTensor* k8, DLTensor* k4,
+                 DLTensor* v8, DLTensor* workspace, int32_t layout, int32_t qk_qtype, int32_t v_qtype, void* stream, DLTensor* k_codes,
+                 DLTensor* k_scale) {
   SQ_REQUIRE(qk_qtype >= SQ_QTYPE_INT && qk_qtype <= SQ_QTYPE_E5M2 && v_qtype >= SQ_QTYPE_INT && v_qtype <= SQ_QTYPE_E5M2, SQ_EINVAL,
              "Invalid quantization type: %d / %d", (int)qk_qtype, (int)v_qtype);
-  SQ_REQUIRE(query && key && value && k8 && v8, SQ_EINVAL, "sq_fake_quant_prepass: null tensor argument");
+  SQ_REQUIRE(query && key && value && (k8 || k_codes) && v8, SQ_EINVAL, "sq_fake_quant_prepass: null tensor argument");
   SQ_REQUIRE((q4 == nullptr) == (k4 == nullptr), SQ_EINVAL, "sq_fake_quant_prepass: q4 and k4 must be given together");
   // q8 == NULL: the query rows are left alone (the attention kernel can quantise them as it loads them, q_quant = 8)
   SQ_REQUIRE(q8 || !q4, SQ_EINVAL, "sq_fake_quant_prepass: without q8 there are no 4-bit operands either");
@@ -348,8 +389,26 @@ extern "C" int sq_fake_quant_prepass_typed(const DLTensor* query, const DLTensor
   memset(&a, 0, sizeof(a));
   if ((rc = make_view(query, "query", layout, dev, dt, B, N, Hq, &a.q)) || (rc = make_view(key, "key", layout, dev, dt, B, N, Hkv, &a.k)) ||
       (rc = make_view(value, "value", layout, dev, dt, B, N, Hkv, &a.v)) || (!skip_q && (rc = make_view(q8, "q8", layout, dev, dt, B, N, Hq, &a.q8))) ||
-      (rc = make_view(k8, "k8", layout, dev, dt, B, N, Hkv, &a.k8)) || (rc = make_view(v8, "v8", layout, dev, dt, B, N, Hkv, &a.v8)))
+      (k8 && (rc = make_view(k8, "k8", layout, dev, dt, B, N, Hkv, &a.k8))) || (rc = make_view(v8, "v8", layout, dev, dt, B, N, Hkv, &a.v8)))
     return rc;
+  if (k_codes) {
+    // int8 [like key]; rows of 128 bytes on 16-byte boundaries.  k_scale: fp32 [B, Hkv, >= N], contiguous
+    if ((rc = check_tensor(k_codes, "k_codes", 4, dev)) || (rc = check_tensor(k_scale, "k_scale", 3, dev))) return rc;
+    SQ_REQUIRE(k_codes->dtype.code == kDLInt && k_codes->dtype.bits == 8 && k_codes->dtype.lanes == 1, SQ_EDTYPE,
+               "sq_fake_quant_prepass_int8qk: k_codes must be int8");
+    SQ_REQUIRE(k_codes->shape[0] == B && k_codes->shape[nd] == N && k_codes->shape[hd] == Hkv && k_codes->shape[3] == kPD, SQ_ESHAPE,
+               "sq_fake_quant_prepass_int8qk: k_codes has the wrong shape");
+    for (int d = 0; d < 3; ++d)
+      SQ_REQUIRE(stride_of(k_codes, d) % 16 == 0 || k_codes->shape[d] == 1, SQ_ESHAPE, "sq_fake_quant_prepass_int8qk: rows of k_codes are not 16-byte aligned");
+    SQ_REQUIRE(dtype_of(k_scale) == DType::F32 && k_scale->shape[0] == B && k_scale->shape[1] == Hkv && k_scale->shape[2] >= N && is_compact(k_scale),
+               SQ_ESHAPE, "sq_fake_quant_prepass_int8qk: k_scale must be a contiguous fp32 [B, Hkv, >= N]");
+    a.kcodes.p = data_of(k_codes);
+    a.kcodes.sb = stride_of(k_codes, 0);
+    a.kcodes.sn = stride_of(k_codes, nd);
+    a.kcodes.sh = stride_of(k_codes, hd);
+    a.kscale = (float*)data_of(k_scale);
+    a.scale_stride = k_scale->shape[2];
+  }
   if (q4 && ((rc = make_view(q4, "q4", layout, dev, dt, B, N, Hq, &a.q4)) || (rc = make_view(k4, "k4", layout, dev, dt, B, N, Hkv, &a.k4))))
     return rc;
   const size_t need = sq_fake_quant_prepass_workspace_bytes(B, Hkv, N);
@@ -400,6 +459,7 @@ extern "C" int sq_fake_quant_prepass_typed(const DLTensor* query, const DLTensor
   SQ_HIP(hipGetLastError());
   return SQ_OK;
 }
+}  // namespace
 
 extern "C" int sq_fake_quant_prepass(const DLTensor* query, const DLTensor* key, const DLTensor* value, DLTensor* q8,
                                      DLTensor* q4, DLTensor* k8, DLTensor* k4, DLTensor* v8, DLTensor* workspace,

@@ -178,3 +178,30 @@ def fused_int_prepass(query, key, value, want_4bit=True, tensor_layout="NHD", qk
     N.check(lib.sq_fake_quant_prepass_typed(*[N.ptr(x) for x in b], N.LAYOUT[tensor_layout], N.QTYPE[qk_qtype], N.QTYPE[v_qtype],
                                             N.current_stream(query.device)))
     return q8, q4, k8, k4, v8
+
+
+def fused_int8qk_prepass(query, key, value, tensor_layout="NHD"):
+    """The operand pre-pass for the integer Q.K^T path (`attn_int8qk_relative_window`): key centring, then the 8-bit
+    per-token codes of the centred key (int8, laid out like `key`) and their fp32 scales `[B, Hkv, N rounded up to 64]`
+    (the tail zero), and the per-channel 8-bit fake quantisation of value.  The query passes through untouched.
+    Returns (k_codes, k_scale, v8)."""
+    from .. import _native as N
+    from ._common import require_gpu
+
+    if tensor_layout not in N.LAYOUT:
+        raise ValueError(f"tensor_layout {tensor_layout} not supported")
+    require_gpu(query, key, value)
+    assert query.stride(-1) == 1 and key.stride(-1) == 1 and value.stride(-1) == 1, "Last dim of qkv must be contiguous."
+    if query.size(-1) != 128:
+        raise ValueError(f"Unsupported head_dim for the fused pre-pass: {query.size(-1)}")
+    hdim, ndim = (1, 2) if tensor_layout == "HND" else (2, 1)
+    B, Hkv, Nk = key.size(0), key.size(hdim), key.size(ndim)
+    lib = N.lib()
+    k_codes = torch.empty(key.shape, dtype=torch.int8, device=key.device)
+    k_scale = torch.zeros(B, Hkv, (Nk + 63) // 64 * 64, dtype=torch.float32, device=key.device)
+    v8 = torch.empty_like(value)
+    need = lib.sq_fake_quant_prepass_workspace_bytes(B, Hkv, Nk)
+    ws = torch.empty((need + 7) // 8, dtype=torch.float64, device=query.device)
+    b = [N.dl(t) for t in (query, key, value, k_codes, k_scale, v8, ws)]
+    N.check(lib.sq_fake_quant_prepass_int8qk(*[N.ptr(x) for x in b], N.LAYOUT[tensor_layout], N.current_stream(query.device)))
+    return k_codes, k_scale, v8

@@ -38,6 +38,20 @@ def int_fake_quant(x: torch.Tensor, bit: int, symmetric: bool, granularity: str)
     return ((qv - zero) * scale).to(x.dtype)
 
 
+def int_quant_codes(x: torch.Tensor, bit: int = 8):
+    """The integer codes and the fp32 scale behind `IntegerQuantizer(bit, True, "per_token").fake_quant_tensor(x)`
+    (fake_quant.py:33-35, 47-52, 114-125): `codes = clamp(round(x / scale), qmin, qmax)` (fp32 tensor of whole numbers),
+    `scale = max(|x|) .clip(1e-5) / qmax` over the last dimension, so that `int_fake_quant(x, bit, True, "per_token") ==
+    (codes * scale).to(x.dtype)`.  This is what a real integer Q.K^T consumes: the codes go through the integer matrix
+    instruction and the two scales multiply the sum."""
+    x32 = x.float()
+    mn, mx = _minmax(x32, "per_token")
+    qmin, qmax = float(-(2 ** (bit - 1))), float(2 ** (bit - 1) - 1)
+    scale = torch.maximum(mx.abs(), mn.abs()).clamp(min=1e-5) / qmax
+    codes = (round_half_away(x32 / scale) + torch.tensor(0.0)).clamp(qmin, qmax)
+    return codes, scale
+
+
 def float_quantize(x: torch.Tensor, e_bits: int, m_bits: int) -> torch.Tensor:
     """The home-made float simulation, nearest rounding (fake_quant.py:151-204)."""
     bias = 2 ** (e_bits - 1) - 1

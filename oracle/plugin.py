@@ -56,7 +56,7 @@ def int_prepass(query, key, value, want_4bit=True, qk_qtype="int", v_qtype="int"
 
 
 def plugin_attention(query, key, value, *, num_kv_groups, bit8, bit4, sink, relative,
-                     qk_qtype="int", v_qtype="int", p_quant=A.P_NONE):
+                     qk_qtype="int", v_qtype="int", p_quant=A.P_NONE, int8_qk=False):
     """query [B,N,Hq,D], key/value [B,N,Hkv,D] (bf16) -> [B,N,Hq*D] bf16.
 
     Steps (attn_replacer.py:334-452): GQA expand + permute to HND; K minus its per-channel token
@@ -64,6 +64,12 @@ def plugin_attention(query, key, value, *, num_kv_groups, bit8, bit4, sink, rela
     fake-quant of V; windowed prefill (relative: 64-row blocks, 4-bit operands aliased to the 8-bit
     ones, attn_triton_mix_relative.py:423,441-444; absolute: 128-row blocks, real 4-bit operands,
     attn_triton_mix_bad.py:386-392); back to [B,N,Hq*D].  `bit8`/`bit4` are per-head lists or scalars.
+
+    `int8_qk` (build-defined, relative windows and the integer quantiser only): Q.K^T as a real integer product -- the
+    8-bit codes of query and centred key are multiplied and summed exactly and the sum is scaled by the two per-token
+    scales and by log2e / sqrt(D) in fp32.  The reference's path rounds `codes * scale` to bf16 (fake_quant.py:85) and
+    the scaled query once more (attn_triton.py:251) before its bf16 product; this one does not, which is its only
+    difference (restated here by handing the block-wise loop unrounded fp32 operands).
     """
     B, N, Hq, D = query.shape
     k = repeat_kv(key, num_kv_groups)
@@ -75,6 +81,12 @@ def plugin_attention(query, key, value, *, num_kv_groups, bit8, bit4, sink, rela
     v8 = _v_quant(v, v_qtype)
     per_head = lambda w: [w] * Hq if not isinstance(w, (list, tuple)) else list(w)
     b8, b4 = per_head(bit8), per_head(bit4)
+    if int8_qk:
+        if not relative or qk_qtype != "int":
+            raise ValueError("int8_qk: relative windows and the integer quantiser only")
+        qc, qs = FQ.int_quant_codes(q, 8)
+        kc, ks = FQ.int_quant_codes(k, 8)
+        q8, k8 = qc * qs, kc * ks          # fp32, not rounded to the tensor dtype
     if relative:
         w8 = [A.window_size_relative(float(r), N) for r in b8]
         w4 = [A.window_size_relative(float(r), N) for r in b4]

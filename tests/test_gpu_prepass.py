@@ -4,6 +4,7 @@ sampled rows at the benchmark shape."""
 import pytest
 import torch
 
+from oracle import fake_quant as FQ
 from oracle import plugin
 
 pytestmark = pytest.mark.gpu
@@ -124,3 +125,36 @@ def test_prepass_errors():
         fused_int_prepass(q, k.half(), v)             # mixed dtypes
     with pytest.raises(RuntimeError):
         fused_int_prepass(q.cpu(), k, v)
+
+
+@pytest.mark.parametrize("layout", ["NHD", "HND"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_int8qk_prepass_codes_and_scales_are_the_quantisers_factors(layout, dtype):
+    """sq_fake_quant_prepass_int8qk: the int8 codes and fp32 scales of the centred key equal the oracle's factors exactly
+    (codes * scale rounded to the tensor dtype is the fake-quantised key of the other pre-pass), v8 is unchanged, the query
+    is not touched."""
+    from longcontext_sqattn_paddle_amd.sqattn.fake_quant import fused_int8qk_prepass, fused_int_prepass
+
+    B, N, Hq, Hkv, D = 2, 333, 8, 2, 128
+    g = torch.Generator().manual_seed(17)
+    q = torch.randn(B, N, Hq, D, generator=g).to(dtype)
+    k = (torch.randn(B, N, Hkv, D, generator=g) * torch.logspace(-4, 1, N)[None, :, None, None] + 0.25).to(dtype)
+    v = torch.randn(B, N, Hkv, D, generator=g).to(dtype)
+    kh = k.permute(0, 2, 1, 3)
+    kc = kh - plugin.key_mean_exact(kh)
+    codes_ref, scale_ref = FQ.int_quant_codes(kc, 8)                      # HND
+    if layout == "HND":
+        qd, kd, vd = (t.permute(0, 2, 1, 3).contiguous().to(DEV) for t in (q, k, v))
+    else:
+        qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
+    q_before = qd.clone()
+    k_codes, k_scale, v8 = fused_int8qk_prepass(qd, kd, vd, layout)
+    _, _, k8, _, v8_ref = fused_int_prepass(qd, kd, vd, want_4bit=False, tensor_layout=layout)
+    torch.cuda.synchronize()
+    assert torch.equal(qd, q_before) and torch.equal(v8, v8_ref)
+    got_codes = k_codes.cpu() if layout == "HND" else k_codes.cpu().permute(0, 2, 1, 3)
+    assert k_codes.dtype == torch.int8 and torch.equal(got_codes.float(), codes_ref)
+    assert k_scale.shape == (B, Hkv, 384) and torch.equal(k_scale.cpu()[:, :, :N], scale_ref[..., 0]) and not bool(k_scale[:, :, N:].any())
+    deq = (got_codes.float() * k_scale.cpu()[:, :, :N, None]).to(dtype)
+    k8h = k8.cpu() if layout == "HND" else k8.cpu().permute(0, 2, 1, 3)
+    assert torch.equal(deq.view(torch.int16), k8h.contiguous().view(torch.int16))

@@ -77,3 +77,59 @@ def test_structure():
     # the value scale is shared by batch and heads: scaling one head changes the other heads' grid
     assert torch.equal(v8, FQ.int_fake_quant(v.permute(0, 2, 1, 3), 8, True, "per_channel").permute(0, 2, 1, 3))
     assert plugin.int_prepass(q, k, v, want_4bit=False)[1] is None
+
+
+def test_integer_codes_are_what_the_fake_quantiser_dequantises():
+    """`int_quant_codes`: whole numbers in [-128, 127], the row's largest element at +-127, and codes * scale rounded to
+    the tensor dtype is the fake quantiser's output bit for bit; known answer: (1, -2, 0.5) -> scale 2/127, codes
+    (64, -127, 32) (63.5 and 31.75 round half away / to nearest)."""
+    g = torch.Generator().manual_seed(8)
+    x = (torch.randn(2, 3, 50, 128, generator=g) * torch.logspace(-3, 2, 50)[None, None, :, None]).bfloat16()
+    x[0, 0, 7] = 0.0
+    codes, scale = FQ.int_quant_codes(x, 8)
+    assert torch.equal(codes, codes.round()) and float(codes.min()) >= -128 and float(codes.max()) <= 127
+    assert torch.equal(codes.abs().amax(dim=-1)[x.float().abs().amax(dim=-1) >= 1e-5], torch.full((2, 3, 50), 127.0)[x.float().abs().amax(dim=-1) >= 1e-5])
+    assert torch.equal((codes * scale).to(x.dtype), FQ.int_fake_quant(x, 8, True, "per_token"))
+    assert float(scale[0, 0, 7]) == torch.tensor(1e-5).float() / 127 and not bool(codes[0, 0, 7].any())
+    row = torch.zeros(1, 1, 1, 128).bfloat16()
+    row[0, 0, 0, :3] = _bf([1.0, -2.0, 0.5])
+    c, s = FQ.int_quant_codes(row, 8)
+    assert c[0, 0, 0, :3].tolist() == [64.0, -127.0, 32.0] and float(s) == float(torch.tensor(2.0) / 127)
+
+
+def test_integer_product_closure_against_a_scalar_loop_and_the_fake_quant_closure():
+    """`plugin_attention(..., int8_qk=True)`: every score is (sum of code products) x scale_q x scale_k x log2e / sqrt(D),
+    checked row by row against a float64 loop over exactly the keys `kv_ranges` lists; and it stays within the size of one
+    bf16 rounding per operand of the reference's fake-quantised bf16 product (cosine and a 1 % band)."""
+    import math
+
+    from oracle import attention as A
+
+    B, N, Hq, Hkv, D = 1, 200, 4, 2, 128
+    g = torch.Generator().manual_seed(21)
+    q = torch.randn(B, N, Hq, D, generator=g).bfloat16()
+    k = (torch.randn(B, N, Hkv, D, generator=g) + 0.5).bfloat16()
+    v = torch.randn(B, N, Hkv, D, generator=g).bfloat16()
+    kw = dict(num_kv_groups=2, bit8=0.4, bit4=0.2, sink=64, relative=True)
+    got = plugin.plugin_attention(q, k, v, int8_qk=True, **kw).view(B, N, Hq, D)
+    ref = plugin.plugin_attention(q, k, v, **kw).view(B, N, Hq, D)
+    cos = torch.nn.functional.cosine_similarity(got.double().flatten(), ref.double().flatten(), dim=0)
+    assert float(cos) > 0.9999 and float((got.double() - ref.double()).abs().max()) < 0.01 * float(ref.double().abs().max()) + 0.01
+    # scalar restatement of a few rows
+    kh = plugin.repeat_kv(k, 2)
+    kh = kh - plugin.key_mean_exact(kh)
+    qh = q.permute(0, 2, 1, 3)
+    qc, qs = FQ.int_quant_codes(qh, 8)
+    kc, ks = FQ.int_quant_codes(kh, 8)
+    v8 = FQ.int_fake_quant(plugin.repeat_kv(v, 2), 8, True, "per_channel").to(torch.float16).double()
+    w = A.window_size_relative(0.4, N)
+    sm = math.log2(math.e) / math.sqrt(D)
+    for h in (0, 3):
+        for i in (0, 63, 64, 130, 199):
+            qb = i // 64 * 64
+            keys = torch.cat([torch.arange(lo, min(hi, i + 1) if masked else hi) for lo, hi, _, masked in A.kv_ranges(qb, qb + 64, sink=64, w8=w, w4=w) if hi > lo])
+            dots = (kc[0, h, keys].double() @ qc[0, h, i].double())           # exact integers
+            s2 = dots * ks[0, h, keys, 0].double() * float(qs[0, h, i, 0]) * sm
+            p = torch.exp2(s2 - s2.max())
+            want = (p[:, None] * v8[0, h, keys]).sum(0) / p.sum()
+            assert float((got[0, i, h].double() - want).abs().max()) <= 2e-2 * float(want.abs().max()) + 2e-3, (h, i)
