@@ -171,7 +171,23 @@ def time_plugin(torch, qkv, steps=3):
                      "plugin_call_ms": round(call_ms, 3), "kernel_ms": round(kern_ms, 3),
                      "roofline": {"bound": "mfma", "kernel": "prefill_kernel (sink + windows, fp16 P.V)", "achieved": round(tf, 1),
                                   "peak": PEAK_MFMA_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / PEAK_MFMA_BF16_TFLOPS, 4)}}
-        del q8, k8, v8, o
+        # the same call with Q.K^T as a real integer product (args.int8_qk): blended peak = half the FLOPs on the int8 pipe
+        # (5.0 POP/s), half on the 16-bit pipe (2.5 PFLOP/s)
+        from longcontext_sqattn_paddle_amd.sqattn.fake_quant import fused_int8qk_prepass
+
+        args8 = types.SimpleNamespace(qk_qtype="int", v_qtype="int", use_relative_distance=True, int8_qk=True)
+        closure8 = mp_triton_wrapper(1, r8, r4, sink, args8)
+        call8_ms = timed(lambda: closure8(layer, q, k, v, None))
+        kc, ks, v8b = fused_int8qk_prepass(q, k, v, "NHD")
+        kern8_ms = timed(lambda: attn_hierarchical_relative_window(q, kc, q, kc, v8b, r8, r4, sink, "NHD", torch.bfloat16, workspace=ws, out=o,
+                                                                   k_scale=ks))
+        tf8 = flops / kern8_ms / 1e9
+        out[name]["int8_qk"] = {"plugin_call_ms": round(call8_ms, 3), "kernel_ms": round(kern8_ms, 3),
+                                "roofline": {"bound": "mfma", "kernel": "prefill_kernel (int8 Q.K^T, fp16 P.V, compiler-scheduled step)",
+                                             "achieved": round(tf8, 1), "peak": round(PEAK_MFMA_BLEND_TFLOPS, 1), "unit": "TFLOP/s",
+                                             "frac": round(tf8 / PEAK_MFMA_BLEND_TFLOPS, 4)},
+                                "note": "build-defined option, off by default: same visited keys and P.V, scores from the int8 MFMA"}
+        del q8, k8, v8, o, kc, ks, v8b
         torch.cuda.empty_cache()
     return out
 

@@ -13,6 +13,8 @@
  *   sq_prefill_fwd            sqattn/attn_triton.py:216-315 (attn_causal -> _attn_fwd launch :279-310),
  *                             sqattn/attn_triton_mix_relative.py:309-483 (launch :439-475),
  *                             sqattn/attn_triton_mix_bad.py:285-426 (launch :388-424)
+ *   sq_prefill_int8qk_fwd     the same launches with the query/key product on the int8 matrix instruction
+ *   sq_fake_quant_prepass_int8qk  sqattn/attn_replacer.py:338-339, 361-365 for that path (key codes and scales, v8)
  *   sq_decode_fwd             sqattn/attn_triton_decode.py:244-361 (decode launch :293-324)
  *   sq_decode_fwd_noalloc     no reference counterpart: sq_decode_fwd for callers that cannot allocate device memory
  *   sq_decode_selected_fwd    no reference counterpart: the same decode over the tokens sq_topk_select picked
@@ -121,6 +123,20 @@ size_t sq_prefill_workspace_bytes(int64_t batch, int64_t num_kv_heads, int64_t k
 int sq_prefill_fwd(const DLTensor* q, const DLTensor* k, const DLTensor* v, const DLTensor* q4,
                    const DLTensor* k4, DLTensor* out, DLTensor* lse, DLTensor* workspace,
                    const sq_prefill_params* params, void* stream);
+
+/*
+ * The same attention with Q.K^T as a real integer product (the second half of what sqattn/attn_replacer.py:334-365 and
+ * the launch sqattn/attn_triton_mix_relative.py:439-475 only simulate: they fake-quantise query and key to 8 bits and
+ * then multiply them as bf16).  k_codes: int8, laid out like k above, the per-token symmetric 8-bit codes of the
+ * (centred) key; k_scale: fp32 [B, Hkv, ceil64(Nk)], their scales (sq_fake_quant_prepass_int8qk writes both).  q is the
+ * raw query: the kernel forms each row's codes and scale as it loads the row (the quantiser of :361).  A score is
+ * (sum of code products, exact in int32) * scale_k * (scale_q * log2e / sqrt(D)) in fp32; the reference's path differs
+ * from it by the bf16 rounding of code * scale (fake_quant.py:85) and of the scaled query (attn_triton.py:251).
+ * Everything else -- ranges, masking, fp16 P, v, out, lse, workspace, params (p_quant and q_quant must be 0, no 4-bit
+ * operand set) -- as for sq_prefill_fwd.
+ */
+int sq_prefill_int8qk_fwd(const DLTensor* q, const DLTensor* k_codes, const DLTensor* k_scale, const DLTensor* v,
+                          DLTensor* out, DLTensor* lse, DLTensor* workspace, const sq_prefill_params* p, void* stream);
 
 /* ----------------------------------------------------------------------------------------- decode */
 typedef struct sq_decode_params {

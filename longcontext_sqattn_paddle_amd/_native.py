@@ -108,6 +108,7 @@ SYMBOLS = {
     "sq_rmsnorm_linear_rows": (ctypes.c_int, [_P, _P, ctypes.c_float] + [_P] * 4 + [ctypes.c_void_p]),
     "sq_rmsnorm_linear_rows_silu_and_mul": (ctypes.c_int, [_P, _P, ctypes.c_float] + [_P] * 3 + [ctypes.c_void_p]),
     "sq_rmsnorm_linear_rows_rope": (ctypes.c_int, [_P, _P, ctypes.c_float] + [_P] * 4 + [ctypes.c_int32, ctypes.c_int32] + [_P] * 5 + [ctypes.c_void_p]),
+    "sq_prefill_int8qk_fwd": (ctypes.c_int, [_P] * 7 + [ctypes.POINTER(PrefillParams), ctypes.c_void_p]),
     "sq_fake_quant_prepass_int8qk": (ctypes.c_int, [_P] * 7 + [ctypes.c_int32, ctypes.c_void_p]),
     "sq_probe_mfma_operand_bytes": (ctypes.c_size_t, []),
     "sq_probe_mfma_flops": (ctypes.c_int64, [ctypes.c_int32, ctypes.c_int32]),

@@ -56,6 +56,7 @@ struct PrefillArgs {
   int32_t B, Hq, Hkv, group, Nq, Nk, nT, nQB;
   int32_t q_offset, p_quant, window_mode, block_m, sink, out_dtype;
   int32_t sched_mode, sched_xpp, sched_items, sched_pairs;
+  const float* k_scale;   // MODE 6: per-token scales of the int8 key codes in `k`, fp32 [B, Hkv, nT * 64]
   int32_t q_quant;   // 8: the rows of q (not of q4) are fake-quantised to 8 bits per token as they are loaded
   float sm;
   int32_t w8[kMaxHeads];
@@ -406,6 +407,13 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
   constexpr int NT = WAVES * 64;
   constexpr int CH = (kBN * kD * 2 / 16) / NT;  // 16-byte chunks per thread and tile operand
   constexpr int ROWS = 32;                      // query rows per wave
+  // MODE 6: Q.K^T on the int8 matrix instruction -- `k` holds the 8-bit codes of the (centred) key, one byte per element,
+  // `k_scale` their per-token scales; the query rows' codes and scale are formed here as the rows are loaded.  The scores
+  // are sum(code products) x scale_k x (scale_q log2e / sqrt(D)); from there on the step is MODE 0's (fp16 P, fp16 V), on
+  // the plain schedule MODE 2 also uses (no hand-placed slots).
+  constexpr bool kQK8 = MODE == 6;
+  constexpr bool kPlain = MODE == 2 || MODE == 6;   // tile step left to the compiler's scheduling
+  constexpr bool kPV8 = MODE == 4 || MODE == 5;     // e4m3 V tiles, fp8 P.V
   extern __shared__ __attribute__((aligned(16))) char smem[];
   // MODE 2: tile maxima of the two waves of a 64-row group, behind the tile rings (which start at LDS address 0)
   float (*s_amax)[WAVES] = (float (*)[WAVES])(smem + 4 * kStageBytes);
@@ -502,7 +510,52 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
       qf[kk] = make_uint4(scale_pair<BF16>(raw[kk].x, a.sm), scale_pair<BF16>(raw[kk].y, a.sm), scale_pair<BF16>(raw[kk].z, a.sm),
                           scale_pair<BF16>(raw[kk].w, a.sm));
   };
-  load_q(a.q);
+  // MODE 6: the row's 8-bit codes as the B operand of v_mfma_i32_32x32x32_i8 -- k-step kk covers dimensions 32 kk .. +31,
+  // of which this lane holds 16 g .. +15 (the lane 32 away the rest; the K fragments are cut the same way, so the pairing
+  // of the products does not depend on how the instruction numbers its k index) -- and the row's scale times log2e / sqrt(D).
+  typedef __attribute__((ext_vector_type(4))) int i32x4_t;
+  typedef __attribute__((ext_vector_type(16))) int i32x16_t;
+  i32x4_t qc[4] = {};
+  float q_scale = 0.f;
+  if constexpr (kQK8) {
+    const uint16_t* qp = (const uint16_t*)a.q + (int64_t)b * a.q_sb + (int64_t)head * a.q_sh;
+    const int row = max(min(row_w0 + c32, a.Nq - 1), 0);
+    const uint16_t* rp = qp + (int64_t)row * a.q_sn + 16 * g;
+    uint4 raw[4][2];
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      raw[kk][0] = *(const uint4*)(rp + 32 * kk);
+      raw[kk][1] = *(const uint4*)(rp + 32 * kk + 8);
+    }
+    float amax = 0.f;
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk)
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf) {
+        const uint32_t w[4] = {raw[kk][hf].x, raw[kk][hf].y, raw[kk][hf].z, raw[kk][hf].w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) amax = fmaxf(amax, fmaxf(fabsf(elem16<BF16>(w[j] & 0xffffu)), fabsf(elem16<BF16>(w[j] >> 16))));
+      }
+    amax = fmaxf(xor32_max(amax), 1e-5f);
+    const Divisor scale = make_divisor(amax / 127.f);
+    auto code = [&](float x) {   // clamp(round(x / scale), -128, 127), fake_quant.py:114-116
+      const float t = divide(x, scale);
+      return (uint32_t)((int)fminf(fmaxf(copysignf(floorf(fabsf(t) + 0.5f), t) + 0.0f, -128.f), 127.f) & 0xff);
+    };
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk)
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf) {
+        const uint32_t w[4] = {raw[kk][hf].x, raw[kk][hf].y, raw[kk][hf].z, raw[kk][hf].w};
+#pragma unroll
+        for (int j = 0; j < 2; ++j)   // four elements (two words) per code word
+          qc[kk][2 * hf + j] = (int)(code(elem16<BF16>(w[2 * j] & 0xffffu)) | (code(elem16<BF16>(w[2 * j] >> 16)) << 8) |
+                                     (code(elem16<BF16>(w[2 * j + 1] & 0xffffu)) << 16) | (code(elem16<BF16>(w[2 * j + 1] >> 16)) << 24));
+      }
+    q_scale = scale.d * a.sm;
+  } else {
+    load_q(a.q);
+  }
   bool q_is4 = false;
 
   f32x16_t O[4];
@@ -513,7 +566,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
   // Online-softmax state of this lane's query row.  The score accumulators are *initialised* with
   // cinit = kC - m_run (kC = log2(448) in MODE 3, else 0), so the MFMA chain delivers S - m_run + kC and, as
   // long as the running maximum does not move, p (or 448 p) is a bare exp2 of the accumulator.
-  constexpr float kC = (MODE >= 3) ? kLog2_448 : 0.f;
+  constexpr float kC = (MODE >= 3 && MODE <= 5) ? kLog2_448 : 0.f;
   // Lazy re-centring (MODE 5): a row maximum may rise up to kLazy (in log2 units) above the reference before the
   // accumulators are rescaled; the block scale absorbs any power of two (its exponent then exceeds 127), while the
   // fp32 accumulators and the denominator carry the common factor until the division at the end.  A row is shifted
@@ -537,7 +590,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
   const int64_t k_head_off = (int64_t)b * a.k_sb + (int64_t)kvh * a.k_sh;
   char* const kbase_lds = smem;                     // 4 x 16 KB
   char* const vbase_lds = smem + 4 * kKTileBytes;   // 4 x 16 KB (8 KB used per buffer in the fp8 mode)
-  auto stage_k = [&](int j, int stage) {
+  auto stage_k16 = [&](int j, int stage) {
     char* kbuf = kbase_lds + stage * kKTileBytes;
     const uint16_t* kb = (const uint16_t*)(tile_uses4(j) ? a.k4 : a.k) + k_head_off;
 #pragma unroll
@@ -549,9 +602,31 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
       __builtin_amdgcn_global_load_lds((const void*)(kb + (int64_t)n * a.k_sn + 8 * kc), (lds_ptr_t)(kbuf + q * 1024), 16, 0, 0);
     }
   };
+  // MODE 6: a tile of key codes is 64 rows x 128 bytes = 8 KB (one wave instruction of 8 rows per 1 KB; 16-byte chunk c
+  // of row r lands in slot c ^ (r & 7)), followed by the tile's 64 scales (one 4-byte copy per lane of wave 0)
+  auto stage_k8 = [&](int j, int stage) {
+    char* kbuf = kbase_lds + stage * kKTileBytes;
+    const char* kb = (const char*)a.k + k_head_off;
+    constexpr int CH8 = CH / 2;
+#pragma unroll
+    for (int c = 0; c < CH8; ++c) {
+      const int q = wave * CH8 + c;
+      const int kr = 8 * q + (lane >> 3);
+      const int kc = (lane & 7) ^ (kr & 7);
+      const int n = min(j * kBN + kr, a.Nk - 1);
+      __builtin_amdgcn_global_load_lds((const void*)(kb + (int64_t)n * a.k_sn + 16 * kc), (lds_ptr_t)(kbuf + q * 1024), 16, 0, 0);
+    }
+    if (wave == 0)
+      __builtin_amdgcn_global_load_lds((const void*)(a.k_scale + (((int64_t)b * a.Hkv + kvh) * a.nT + j) * kBN + lane),
+                                       (lds_ptr_t)(kbuf + kBN * kD), 4, 0, 0);
+  };
+  auto stage_k = [&](int j, int stage) {
+    if constexpr (kQK8) stage_k8(j, stage);
+    else stage_k16(j, stage);
+  };
   auto stage_v = [&](int j, int stage) {
     char* vbuf = vbase_lds + stage * kVTileBytes;
-    if constexpr (MODE >= 4) {
+    if constexpr (kPV8) {
       // e4m3 tile: 128 rows x 64 bytes = 8 KB, one wave instruction per wave; 16-byte chunk c of row d -> slot
       // c ^ ((d >> 2) & 3), which spreads the 16 rows a quarter-wave reads over all 16 bank groups
       const uint8_t* vsrc8 = a.vt8 + (((int64_t)b * a.Hkv + kvh) * a.nT + j) * (int64_t)(kD * kBN);
@@ -602,7 +677,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
   const uint32_t kx0 = c32 * kKStride + ((g ^ ksw) << 4);
   // MODE 4 with the main loop unrolled over the four ring buffers: the LDS address of every fragment is a
   // per-lane constant plus an immediate offset, so the tile step spends no vector instruction on addresses
-  constexpr bool kStaticRing = SQ_STATIC_RING && MODE != 2;
+  constexpr bool kStaticRing = SQ_STATIC_RING && !kPlain;
   uint32_t kxr[8];
 #pragma unroll
   for (int kk = 0; kk < 8; ++kk) kxr[kk] = smem_addr + (kx0 ^ (kk << 5));
@@ -619,6 +694,30 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
 
   // S^T = K . Q~^T + Cinit for one tile: 16 MFMAs that nothing below depends on until the next step
   auto qk_tile = [&](const char* kbuf, f32x16_t (&S)[2]) {
+    if constexpr (kQK8) {
+      i32x16_t acc0 = {}, acc1 = {};
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) {
+        const i32x4_t a0 = *(const i32x4_t*)(kbuf + c32 * kD + (((2 * kk + g) ^ (c32 & 7)) << 4));
+        const i32x4_t a1 = *(const i32x4_t*)(kbuf + (32 + c32) * kD + (((2 * kk + g) ^ (c32 & 7)) << 4));
+        acc0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, qc[kk], acc0, 0, 0, 0);
+        acc1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, qc[kk], acc1, 0, 0, 0);
+      }
+      // accumulator element i of block bn is key 32 bn + 8 (i >> 2) + 4 g + (i & 3): four neighbouring scales per read
+      const float* sk = (const float*)(kbuf + kBN * kD);
+#pragma unroll
+      for (int q4i = 0; q4i < 4; ++q4i) {
+        const float4 s0 = *(const float4*)(sk + 8 * q4i + 4 * g);
+        const float4 s1 = *(const float4*)(sk + 32 + 8 * q4i + 4 * g);
+        const float f0[4] = {s0.x, s0.y, s0.z, s0.w}, f1[4] = {s1.x, s1.y, s1.z, s1.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          S[0][4 * q4i + e] = __builtin_fmaf((float)acc0[4 * q4i + e] * f0[e], q_scale, Cinit[4 * q4i + e]);
+          S[1][4 * q4i + e] = __builtin_fmaf((float)acc1[4 * q4i + e] * f1[e], q_scale, Cinit[4 * q4i + e]);
+        }
+      }
+      return;
+    }
     {
       const uint4 a0 = *(const uint4*)(kbuf + c32 * kKStride + ((g ^ ksw) << 4));
       const uint4 a1 = *(const uint4*)(kbuf + (32 + c32) * kKStride + ((g ^ ksw) << 4));
@@ -669,13 +768,13 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
     const uint32_t klane = smem_addr + (((it + 1) & 3) * kKTileBytes) + kx0;
     u32x4_t kf[16];
     // K fragments are requested this many MFMA slots ahead (even, 2..8); the fp16 P.V modes have fewer registers to spare
-    constexpr int kDepth = (MODE >= 4) ? SQ_LDS_DEPTH : SQ_LDS_DEPTH_F16;
+    constexpr int kDepth = kPV8 ? SQ_LDS_DEPTH : SQ_LDS_DEPTH_F16;
     auto kread = [&](auto I) {
       constexpr int i = decltype(I)::value;
       if constexpr (kStaticRing) kf[i] = lds_read128<((R + 1) & 3) * kKTileBytes + (i & 1) * 32 * kKStride>(kxr[i >> 1]);
       else kf[i] = lds_read128<(i & 1) * 32 * kKStride>(klane ^ ((i >> 1) << 5));
     };
-    if constexpr (MODE != 2) static_for<0, kDepth>(kread);
+    if constexpr (!kPlain) static_for<0, kDepth>(kread);
     if (masked) {  // causal mask inside the query block's own tiles (attn_triton.py:69-71)
       // One tile in thousands takes this branch.  The laundered copy of g keeps the branch a branch and stops
       // the compiler from hoisting 32 per-lane column constants out of the loop into precious registers.
@@ -691,7 +790,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
     // row maximum of S - m_run + kC; the row's other 32 keys live in lane^32
     float tmax;
     bool slow;
-    if constexpr (MODE != 2) {
+    if constexpr (!kPlain) {
       if (masked) {
         tmax_row = xor32_max(lane_max(S));
         moved = __any(tmax_row > kMove);
@@ -727,7 +826,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
       for (int i = 0; i < 16; ++i) Cinit[i] = c;
       first = false;
     }
-    if constexpr (MODE >= 4) {
+    if constexpr (kPV8) {
       // MODE 5: the pack divides by 2^-k, the MFMA multiplies this lane's 32 values by 2^-k again (E8M0 scale in
       // byte 0 of the operand).  MODE 4: k = 0.
       const int mfma_scale_b = (MODE == 5) ? e_row : 0x7f7f7f7f;
@@ -927,7 +1026,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
 #pragma unroll
     for (int bn = 0; bn < 2; ++bn)
 #pragma unroll
-      for (int t = 0; t < 2; ++t) P[bn][t] = quant_pack8<(MODE >= 4 ? 3 : MODE)>(S[bn], t, sc, inv);
+      for (int t = 0; t < 2; ++t) P[bn][t] = quant_pack8<(kPV8 ? 3 : (kQK8 ? 0 : MODE))>(S[bn], t, sc, inv);
     // O^T[d, row] += V^T[d, key] . P^T[key, row]
 #pragma unroll
     for (int bd = 0; bd < 4; ++bd)
@@ -987,7 +1086,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
   if (vis_cur) {
     switch_q(tile_of(0));
     qk_tile(kbase_lds, Sa);
-    if constexpr (MODE != 2) {
+    if constexpr (!kPlain) {
       mfma_settle(Sa[0], Sa[1]);
       tmax_row = xor32_max(lane_max(Sa));
       moved = __any(tmax_row > kMove);
@@ -999,7 +1098,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
     if ((t & 1) == 0) {   // start of a pair: refill the four buffers the previous pair released
       if (t + 4 < nFull) {
         const int j2 = tile_of(t + 2), j3 = tile_of(t + 3), j4 = tile_of(t + 4);
-        if constexpr (WAVES == 8) {
+        if constexpr (WAVES == 8 && !kQK8) {
           stage_k_full(j3, (t + 3) & 3);
           stage_k_full(j4, t & 3);
         } else {
@@ -1027,7 +1126,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
     } else {
       if (vis_nxt) {
         qk_tile(knext, Snxt);
-        if constexpr (MODE != 2) {
+        if constexpr (!kPlain) {
           mfma_settle(Snxt[0], Snxt[1]);
           tmax_row = xor32_max(lane_max(Snxt));
           moved = __any(tmax_row > kMove);
@@ -1068,7 +1167,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
       float v[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) v[e] = O[bd][4 * i4 + e] / l;
-      if constexpr (MODE >= 4) {  // undo the per-channel V scale
+      if constexpr (kPV8) {  // undo the per-channel V scale
         const float4 isc = *(const float4*)(a.v_inv_scale + ((int64_t)b * a.Hkv + kvh) * kD + d);
         v[0] *= isc.x;
         v[1] *= isc.y;
@@ -1087,7 +1186,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
       }
     }
   if (a.lse && g == 0) {
-    const float lt = (MODE >= 3) ? l * (1.0f / 448.0f) : l;
+    const float lt = (MODE >= 3 && MODE <= 5) ? l * (1.0f / 448.0f) : l;
     a.lse[((int64_t)b * a.Hq + head) * a.Nq + row] = log2f(lt) + m_run;
   }
 }
@@ -1104,9 +1203,27 @@ extern "C" size_t sq_prefill_workspace_bytes(int64_t batch, int64_t num_kv_heads
   return (size_t)(batch * num_kv_heads * nT) * (size_t)(kD * kBN) * sizeof(_Float16);
 }
 
+namespace {
+int prefill_impl(const DLTensor* q, const DLTensor* k, const DLTensor* v, const DLTensor* q4, const DLTensor* k4, DLTensor* out,
+                 DLTensor* lse, DLTensor* workspace, const sq_prefill_params* p, void* stream, const DLTensor* k_scale);
+}
+
 extern "C" int sq_prefill_fwd(const DLTensor* q, const DLTensor* k, const DLTensor* v, const DLTensor* q4,
                               const DLTensor* k4, DLTensor* out, DLTensor* lse, DLTensor* workspace,
                               const sq_prefill_params* p, void* stream) {
+  return prefill_impl(q, k, v, q4, k4, out, lse, workspace, p, stream, nullptr);
+}
+
+extern "C" int sq_prefill_int8qk_fwd(const DLTensor* q, const DLTensor* k_codes, const DLTensor* k_scale, const DLTensor* v,
+                                     DLTensor* out, DLTensor* lse, DLTensor* workspace, const sq_prefill_params* p, void* stream) {
+  SQ_REQUIRE(k_scale, SQ_EINVAL, "sq_prefill_int8qk_fwd: k_scale is null");
+  return prefill_impl(q, k_codes, v, nullptr, nullptr, out, lse, workspace, p, stream, k_scale);
+}
+
+namespace {
+// k_scale != null: `k` holds int8 codes and the scores come from the int8 matrix instruction (sq_prefill_int8qk_fwd)
+int prefill_impl(const DLTensor* q, const DLTensor* k, const DLTensor* v, const DLTensor* q4, const DLTensor* k4, DLTensor* out,
+                 DLTensor* lse, DLTensor* workspace, const sq_prefill_params* p, void* stream, const DLTensor* k_scale) {
   SQ_REQUIRE(p, SQ_EINVAL, "sq_prefill_fwd: params is null");
   SQ_REQUIRE(q && k && v && out, SQ_EINVAL, "sq_prefill_fwd: q, k, v and out must be non-null");
   SQ_REQUIRE(p->layout == SQ_LAYOUT_HND || p->layout == SQ_LAYOUT_NHD, SQ_EINVAL, "tensor_layout %d not supported", p->layout);
@@ -1120,7 +1237,14 @@ extern "C" int sq_prefill_fwd(const DLTensor* q, const DLTensor* k, const DLTens
   if (q4 && ((rc = check_tensor(q4, "q4", 4, dev)) || (rc = check_tensor(k4, "k4", 4, dev)))) return rc;
   const DType dt = dtype_of(q);
   SQ_REQUIRE(dt == DType::BF16 || dt == DType::F16, SQ_EDTYPE, "sq_prefill_fwd: q must be bf16 or fp16");
-  SQ_REQUIRE(dtype_of(k) == dt && dtype_of(v) == dt, SQ_EDTYPE, "sq_prefill_fwd: q, k, v dtypes differ");
+  if (k_scale) {
+    SQ_REQUIRE(k->dtype.code == kDLInt && k->dtype.bits == 8 && k->dtype.lanes == 1 && dtype_of(v) == dt, SQ_EDTYPE,
+               "sq_prefill_int8qk_fwd: k_codes must be int8 and v of q's dtype");
+    SQ_REQUIRE(p->p_quant == SQ_P_NONE && p->q_quant == 0, SQ_EINVAL,
+               "sq_prefill_int8qk_fwd: p_quant and q_quant must be 0 (the query's codes are formed by the kernel, P stays fp16)");
+  } else {
+    SQ_REQUIRE(dtype_of(k) == dt && dtype_of(v) == dt, SQ_EDTYPE, "sq_prefill_fwd: q, k, v dtypes differ");
+  }
   if (q4) SQ_REQUIRE(dtype_of(q4) == dt && dtype_of(k4) == dt, SQ_EDTYPE, "sq_prefill_fwd: q4/k4 dtype differs from q");
   const DType odt = dtype_of(out);
   SQ_REQUIRE(odt == DType::BF16 || odt == DType::F16 || odt == DType::F32, SQ_EDTYPE, "sq_prefill_fwd: out must be bf16, fp16 or fp32");
@@ -1230,6 +1354,18 @@ extern "C" int sq_prefill_fwd(const DLTensor* q, const DLTensor* k, const DLTens
   local.k = data_of(k);
   local.q4 = q4 ? data_of(q4) : nullptr;
   local.k4 = k4 ? data_of(k4) : nullptr;
+  local.k_scale = nullptr;
+  if (k_scale) {
+    int rc2;
+    if ((rc2 = check_tensor(k_scale, "k_scale", 3, dev))) return rc2;
+    SQ_REQUIRE(dtype_of(k_scale) == DType::F32 && k_scale->shape[0] == B && k_scale->shape[1] == Hkv && k_scale->shape[2] == (int64_t)nT * kBN &&
+                   is_compact(k_scale),
+               SQ_ESHAPE, "sq_prefill_int8qk_fwd: k_scale must be a contiguous fp32 [B, Hkv, %lld] (tokens rounded up to whole tiles)",
+               (long long)nT * kBN);
+    SQ_REQUIRE(stride_of(k, ndim) % 16 == 0 && stride_of(k, hdim) % 16 == 0 && stride_of(k, 0) % 16 == 0, SQ_ESHAPE,
+               "sq_prefill_int8qk_fwd: rows of k_codes must start on 16-byte boundaries");
+    local.k_scale = (const float*)data_of(k_scale);
+  }
   local.vt = pa.vt;
   local.vt8 = pa.vt8;
   local.v_inv_scale = pa.v_inv_scale;
@@ -1297,6 +1433,10 @@ extern "C" int sq_prefill_fwd(const DLTensor* q, const DLTensor* k, const DLTens
   } while (0)
 #define SQ_LAUNCH_MODE(BF, W)                                   \
   do {                                                          \
+    if (k_scale) {                                              \
+      SQ_LAUNCH_PREFILL(BF, W, 6);                              \
+      break;                                                    \
+    }                                                           \
     switch (p->p_quant) {                                       \
       case SQ_P_NONE: SQ_LAUNCH_PREFILL(BF, W, 0); break;        \
       case SQ_P_E4M3_STATIC: SQ_LAUNCH_PREFILL(BF, W, 1); break; \
@@ -1318,3 +1458,4 @@ extern "C" int sq_prefill_fwd(const DLTensor* q, const DLTensor* k, const DLTens
   SQ_HIP(hipGetLastError());
   return SQ_OK;
 }
+}  // namespace

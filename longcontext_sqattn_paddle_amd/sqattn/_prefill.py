@@ -18,14 +18,23 @@ def prefill_workspace(B: int, Hkv: int, kv_len: int, device) -> torch.Tensor:
 
 def run_prefill(q, k, v, *, tensor_layout="HND", output_dtype=torch.float16, return_lse=False, p_quant=N.P_NONE,
                 q4=None, k4=None, window: Optional[dict] = None, q_offset: int = 0,
-                workspace: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None, q_quant: int = 0):
+                workspace: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None, q_quant: int = 0,
+                k_scale: Optional[torch.Tensor] = None):
     """window = None (full causal) or {"block_m": 64|128, "sink": int, "w8": [Hq ints], "w4": [Hq ints]}.
-    q_quant = 8: the kernel applies the 8-bit per-token fake quantiser to the rows of q as it loads them."""
+    q_quant = 8: the kernel applies the 8-bit per-token fake quantiser to the rows of q as it loads them.
+    k_scale (fp32 [B, Hkv, ceil64(Nk)]): `k` holds the int8 codes of the key and Q.K^T runs as an integer product
+    (`sq_prefill_int8qk_fwd`; head_dim 128 only, no 4-bit operands, P not quantised)."""
     if tensor_layout not in N.LAYOUT:
         raise ValueError(f"tensor_layout {tensor_layout} not supported")
     require_gpu(q, k, v, q4, k4)
     head_dim_og = q.size(-1)
-    q, k, v, q4, k4 = pad_head_dim((q, k, v, q4, k4), head_dim_og)
+    if k_scale is not None:
+        if head_dim_og != 128 or q4 is not None or k4 is not None or p_quant != N.P_NONE or q_quant:
+            raise ValueError("the integer Q.K^T path takes head_dim 128, no 4-bit operands and no P or q quantisation mode")
+        if k.dtype != torch.int8:
+            raise ValueError(f"k must hold int8 codes when k_scale is given (got {k.dtype})")
+    else:
+        q, k, v, q4, k4 = pad_head_dim((q, k, v, q4, k4), head_dim_og)
     assert q.stride(-1) == 1 and k.stride(-1) == 1 and v.stride(-1) == 1, "Last dim of qkv must be contiguous."
     hdim, ndim = (1, 2) if tensor_layout == "HND" else (2, 1)
     B, Hq, Nq = q.size(0), q.size(hdim), q.size(ndim)
@@ -55,8 +64,12 @@ def run_prefill(q, k, v, *, tensor_layout="HND", output_dtype=torch.float16, ret
         params.num_heads_w = Hq
         params.w8 = ctypes.cast(w8, ctypes.POINTER(ctypes.c_int32))
         params.w4 = ctypes.cast(w4, ctypes.POINTER(ctypes.c_int32))
-    b = [N.dl(t) for t in (q, k, v, q4, k4, o, lse, workspace)]
-    N.check(lib.sq_prefill_fwd(*[N.ptr(x) for x in b], ctypes.byref(params), N.current_stream(q.device)))
+    if k_scale is not None:
+        b = [N.dl(t) for t in (q, k, k_scale, v, o, lse, workspace)]
+        N.check(lib.sq_prefill_int8qk_fwd(*[N.ptr(x) for x in b], ctypes.byref(params), N.current_stream(q.device)))
+    else:
+        b = [N.dl(t) for t in (q, k, v, q4, k4, o, lse, workspace)]
+        N.check(lib.sq_prefill_fwd(*[N.ptr(x) for x in b], ctypes.byref(params), N.current_stream(q.device)))
     o = o[..., :head_dim_og]
     return (o, lse) if return_lse else o
 

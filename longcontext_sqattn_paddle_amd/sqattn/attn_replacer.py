@@ -21,7 +21,7 @@ import torch
 from .attn_triton_decode import attn_decode
 from .attn_triton_mix_bad import attn_hierarchical_window
 from .attn_triton_mix_relative import attn_hierarchical_relative_window
-from .fake_quant import FloatQuantizer, IntegerQuantizer, fused_int_prepass
+from .fake_quant import FloatQuantizer, IntegerQuantizer, fused_int8qk_prepass, fused_int_prepass
 from .sdpa_attention import sdpa_attention_forward
 
 
@@ -127,6 +127,21 @@ def mp_triton_wrapper(layer_idx, bit8_window_sizes=0, bit4_window_sizes=0, sink_
             # With the integer quantiser and relative windows the query does not go through the pre-pass at all: the
             # attention kernel quantises its rows while loading them (same bits), which saves writing and re-reading q8.
             q_in_kernel = relative and args.qk_qtype == "int"
+            if getattr(args, "int8_qk", False):
+                # extension (off unless args.int8_qk is set): Q.K^T as a real integer product on the int8 matrix
+                # instruction -- the pre-pass hands over the key's codes and scales instead of the fake-quantised key
+                if not (q_in_kernel and args.v_qtype == "int"):
+                    raise ValueError("int8_qk needs use_relative_distance and the integer quantiser types")
+                k_codes, k_scale, v_bit8 = fused_int8qk_prepass(query, key, value, tensor_layout=layout)
+                attn_output = attn_hierarchical_relative_window(
+                    query, k_codes, query, k_codes, v_bit8, int8_window_ratios=bit8_window_sizes,
+                    int4_window_ratios=bit4_window_sizes, sink_size=sink_window_size, tensor_layout=layout,
+                    output_dtype=torch.bfloat16, k_scale=k_scale)
+                del query, key, value
+                if layout == "HND":
+                    attn_output = attn_output.transpose(1, 2).contiguous()
+                bs, seq_len, head, head_dim = attn_output.shape
+                return attn_output.reshape(bs, seq_len, head * head_dim)
             q_bit8, q_bit4, k_bit8, k_bit4, v_bit8 = fused_int_prepass(query, key, value, want_4bit=not relative, tensor_layout=layout,
                                                                        qk_qtype=args.qk_qtype, v_qtype=args.v_qtype, skip_query=q_in_kernel)
             if q_in_kernel:

@@ -22,9 +22,11 @@ def window_tokens(ratio: float, kv_len: int) -> int:
 
 def attn_hierarchical_relative_window(q_int8, k_int8, q_int4, k_int4, v, int8_window_ratios, int4_window_ratios,
                                       sink_size, tensor_layout="HND", output_dtype=torch.float16, return_lse=False,
-                                      is_P_fp8_quant=False, *, p_quant=None, workspace=None, out=None, q_quant=0):
+                                      is_P_fp8_quant=False, *, p_quant=None, workspace=None, out=None, q_quant=0, k_scale=None):
     """`q_quant=8` (extension): `q_int8` is the query before its 8-bit per-token fake quantisation, which the kernel
-    then applies while loading the rows (same bits as the separate pass)."""
+    then applies while loading the rows (same bits as the separate pass).
+    `k_scale` (extension, see `sqattn.fake_quant.fused_int8qk_prepass`): `k_int8` holds the key's int8 codes, `k_scale`
+    their per-token scales and `q_int8` the raw query; Q.K^T then is a real integer product."""
     if tensor_layout not in N.LAYOUT:
         raise ValueError(f"tensor_layout {tensor_layout} not supported")
     seq_dim = 1 if tensor_layout == "NHD" else 2
@@ -41,4 +43,5 @@ def attn_hierarchical_relative_window(q_int8, k_int8, q_int4, k_int4, v, int8_wi
     window = {"block_m": 64, "sink": sink_size, "w8": w8, "w4": w4}
     mode = p_quant if p_quant is not None else (N.P_E4M3_STATIC if is_P_fp8_quant else N.P_NONE)
     return run_prefill(q_int8, k_int8, v, tensor_layout=tensor_layout, output_dtype=output_dtype,
-                       return_lse=return_lse, p_quant=mode, window=window, workspace=workspace, out=out, q_quant=q_quant)
+                       return_lse=return_lse, p_quant=mode, window=window, workspace=workspace, out=out, q_quant=q_quant,
+                       k_scale=k_scale)

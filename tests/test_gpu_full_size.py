@@ -96,7 +96,7 @@ def test_prefill_1m_tokens_sampled_rows(mode, layout):
     print(f"  worst relative row error {worst:.2e}", flush=True)
 
 
-def _closure_rows(N, rows, seed, from_cpu_generator):
+def _closure_rows(N, rows, seed, from_cpu_generator, int8_qk=False):
     """The reference's shipped default -- relative windows 0.1 / 0.1 and a 256-token sink
     (sqattn/window_search.py:102-104, sqattn/attn_replacer.py:24) -- through `mp_triton_wrapper`'s closure, against the
     closed form over the oracle's key ranges on the oracle's fake-quantised operands."""
@@ -106,7 +106,7 @@ def _closure_rows(N, rows, seed, from_cpu_generator):
         q, k, v = (t.permute(0, 2, 1, 3).contiguous().to(DEV) for t in inputs.prefill_inputs(1, HQ, HKV, N, D, seed=seed))
     else:
         q, k, v = _device_inputs(N, seed, "NHD")
-    args = types.SimpleNamespace(qk_qtype="int", v_qtype="int", use_relative_distance=True)
+    args = types.SimpleNamespace(qk_qtype="int", v_qtype="int", use_relative_distance=True, int8_qk=int8_qk)
     layer = types.SimpleNamespace(num_key_value_groups=HQ // HKV)
     out = mp_triton_wrapper(1, 0.1, 0.1, 256, args)(layer, q, k, v, None)
     torch.cuda.synchronize()
@@ -119,14 +119,22 @@ def _closure_rows(N, rows, seed, from_cpu_generator):
     from oracle import plugin as OP
 
     kh, vh = k.cpu().permute(0, 2, 1, 3), v.cpu().permute(0, 2, 1, 3)      # HND views
-    k8 = FQ.int_fake_quant(kh - OP.key_mean_exact(kh), 8, True, "per_token")
+    if int8_qk:   # the integer product's operands: codes x scale, not rounded to the tensor dtype
+        kcodes, kscale = FQ.int_quant_codes(kh - OP.key_mean_exact(kh), 8)
+        k8 = kcodes * kscale
+    else:
+        k8 = FQ.int_fake_quant(kh - OP.key_mean_exact(kh), 8, True, "per_token")
     v8 = FQ.int_fake_quant(vh, 8, True, "per_channel")
     worst = 0.0
     for kvh in sorted({h // (HQ // HKV) for h in HEADS}):
         kc, vc = k8[0, kvh].double(), v8[0, kvh].double()
         for h in (x for x in HEADS if x // (HQ // HKV) == kvh):
             for i in rows:
-                q8 = FQ.int_fake_quant(q[0, i, h].cpu()[None, None, None], 8, True, "per_token")[0, 0]
+                if int8_qk:
+                    qcodes, qscale = FQ.int_quant_codes(q[0, i, h].cpu()[None, None, None], 8)
+                    q8 = (qcodes * qscale)[0, 0]
+                else:
+                    q8 = FQ.int_fake_quant(q[0, i, h].cpu()[None, None, None], 8, True, "per_token")[0, 0]
                 qi = A.fold_scale(q8, D).double()[0]
                 qs = i // 64 * 64
                 ranges = A.kv_ranges(qs, qs + 64, sink=256, w8=w, w4=w)
@@ -140,6 +148,14 @@ def test_plugin_closure_128k_default_windows():
     # first rows, sink edge, the first query block whose window no longer reaches the sink (qe - w > 256), block edges
     rows = [0, 63, 64, 255, 256, 319, 13184 + 255, 13184 + 256, 13184 + 320, 65535, 65536, 100000, N - 1]
     _closure_rows(N, rows, 2, True)
+
+
+def test_integer_qk_closure_128k_default_windows():
+    """The same closure with args.int8_qk (Q.K^T on the int8 matrix instruction) at the benchmark's prefill shape."""
+    print("case int8 qk plugin closure 128K ratio 0.1 sink 256", flush=True)
+    N = 131072
+    rows = [0, 63, 64, 255, 256, 319, 13184 + 255, 13184 + 256, 13184 + 320, 65535, 65536, 100000, N - 1]
+    _closure_rows(N, rows, 2, True, int8_qk=True)
 
 
 def test_plugin_closure_1m_default_windows():

@@ -181,3 +181,36 @@ def test_query_quantised_while_loaded_equals_the_separate_pass(dtype, layout):
         attn_hierarchical_relative_window(q, k8, q, k8, v8, 0.25, 0.5, 128, layout, torch.float32, q_quant=4)
     with pytest.raises(ValueError):
         fused_int_prepass(q, k, v, want_4bit=True, tensor_layout=layout, skip_query=True)
+
+
+@pytest.mark.parametrize("bit8,bit4,N,Hq,Hkv", [(0.1, 0.1, 2048, 4, 1), ([0.05, 0.1, 0.2, 0.3], [0.4, 0.1, 0.2, 0.5], 2048, 4, 2),
+                                                 (2.0, 2.0, 700, 14, 2), (0.25, 0.5, 4096, 4, 1)])
+def test_integer_qk_closure_matches_its_oracle(bit8, bit4, N, Hq, Hkv):
+    """args.int8_qk: Q.K^T on the int8 matrix instruction (codes of the query formed in the kernel, codes and scales of
+    the centred key from sq_fake_quant_prepass_int8qk) against the oracle's integer-product restatement: both round the
+    same fp32 result to bf16, so one bf16 step of the largest output plus kernel noise; and against the reference's
+    fake-quantised bf16 product it stays within the two bf16 roundings that path applies to its operands (cosine, 1 % band).
+    The last case is benchmark configuration 1's shape (4 q heads / 1 kv head, 4096 tokens) with windows."""
+    from longcontext_sqattn_paddle_amd.sqattn.attn_replacer import process_model
+
+    print(f"case int8 qk closure N={N} Hq={Hq} Hkv={Hkv} bit8={bit8} bit4={bit4}", flush=True)
+    q, k, v = inputs.plugin_inputs(1, Hq, Hkv, N, 128, seed=3)
+    args = _args(True)
+    args.int8_qk = True
+    m = _Model(2, Hq // Hkv)
+    process_model(m, "SQAttn", {1: {"bit8": bit8, "bit4": bit4, "sink": 0}}, args)
+    out = m.layers[1].prefill_attention(q.to(DEV), k.to(DEV), v.to(DEV), None)
+    torch.cuda.synchronize()
+    assert out.shape == (1, N, Hq * 128) and out.dtype == torch.bfloat16
+    ref = plugin.plugin_attention(q, k, v, num_kv_groups=Hq // Hkv, bit8=bit8, bit4=bit4, sink=256, relative=True, int8_qk=True)
+    o, r = out.float().cpu(), ref.float()
+    rms = float(r.pow(2).mean().sqrt())
+    assert _cos(o, r) >= 0.99999
+    assert float((o - r).abs().max()) <= 2 ** -7 * float(r.abs().max()) + 2e-3 * rms
+    fake = plugin.plugin_attention(q, k, v, num_kv_groups=Hq // Hkv, bit8=bit8, bit4=bit4, sink=256, relative=True).float()
+    assert _cos(o, fake) >= 0.9999 and float((o - fake).abs().max()) <= 0.01 * float(fake.abs().max()) + 0.02 * rms
+    with pytest.raises(ValueError):
+        bad = _args(False)
+        bad.int8_qk = True
+        process_model(m, "SQAttn", {1: {"bit8": 256, "bit4": 256, "sink": 0}}, bad)
+        m.layers[1].prefill_attention(q.to(DEV), k.to(DEV), v.to(DEV), None)
