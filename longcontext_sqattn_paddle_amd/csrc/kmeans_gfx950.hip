@@ -218,10 +218,9 @@ struct SortArgs {
   const int32_t* idx;     // [G,N]
   int32_t* tile_hist;     // [G,nT,C]  in: per-tile histogram, after scan: exclusive prefix over tiles
   int32_t* total;         // [G,C]     cluster sizes (written by the scan)
-  int32_t* off;           // [G,C+1]   exclusive prefix over clusters (train only)
-  int32_t* dst;           // order [G,N] (train) or clusters [G,C,M] (reverse index)
+  int32_t* dst;           // clusters [G,C,M]
   int64_t i_sg, dst_sg, dst_sc;
-  int32_t N, C, nT, M, use_off;
+  int32_t N, C, nT, M;
 };
 
 __global__ __launch_bounds__(kTileTok) void sort_hist_kernel(SortArgs a) {
@@ -270,36 +269,6 @@ __global__ __launch_bounds__(32 * kScanSegs) void sort_scan_tiles_kernel(SortArg
   if (seg == 0) a.total[(int64_t)g * a.C + c] = total;
 }
 
-__global__ __launch_bounds__(1024) void sort_scan_clusters_kernel(SortArgs a) {
-  __shared__ int32_t part[1024];
-  const int g = blockIdx.x, t = threadIdx.x;
-  const int per = (a.C + 1023) / 1024;
-  const int32_t* tot = a.total + (int64_t)g * a.C;
-  int s = 0;
-  for (int i = 0; i < per; ++i) {
-    const int c = t * per + i;
-    if (c < a.C) s += tot[c];
-  }
-  part[t] = s;
-  __syncthreads();
-  for (int d = 1; d < 1024; d <<= 1) {  // Hillis-Steele inclusive scan
-    const int v = (t >= d) ? part[t - d] : 0;
-    __syncthreads();
-    part[t] += v;
-    __syncthreads();
-  }
-  int run = part[t] - s;
-  int32_t* off = a.off + (int64_t)g * (a.C + 1);
-  for (int i = 0; i < per; ++i) {
-    const int c = t * per + i;
-    if (c < a.C) {
-      off[c] = run;
-      run += tot[c];
-    }
-  }
-  if (t == 1023) off[a.C] = part[1023];
-}
-
 __global__ __launch_bounds__(kTileTok) void sort_scatter_kernel(SortArgs a) {
   __shared__ int32_t cl[kTileTok];
   const int tile = blockIdx.x, g = blockIdx.y, t = threadIdx.x;
@@ -311,59 +280,261 @@ __global__ __launch_bounds__(kTileTok) void sort_scatter_kernel(SortArgs a) {
   int rank = 0;
   for (int u = 0; u < t; ++u) rank += (cl[u] == c);   // tokens of a tile keep their ascending order
   const int base = a.tile_hist[((int64_t)g * a.nT + tile) * a.C + c] + rank;
-  if (a.use_off) {
-    a.dst[(int64_t)g * a.dst_sg + a.off[(int64_t)g * (a.C + 1) + c] + base] = n;
-  } else if (base < a.M) {
-    a.dst[(int64_t)g * a.dst_sg + (int64_t)c * a.dst_sc + base] = n;
+  if (base < a.M) a.dst[(int64_t)g * a.dst_sg + (int64_t)c * a.dst_sc + base] = n;
+}
+
+// Grouping without a global order, for the callers that only sum the rows of a cluster afterwards (centroid update,
+// index_add): those sums are exact, so neither the order of the addends nor where a cluster's tokens lie matters.  A
+// workgroup sorts its own tile of kBigTile tokens by cluster and nothing else: LDS histogram (the atomic's return value is
+// the token's rank inside its (tile, cluster) range), exclusive prefix over the clusters, token ids written to
+// order[tile * kBigTile + start[c] + rank].  start[tile][0..C] goes to memory; the sum kernel of cluster c walks the
+// tiles and picks up order[tile][start[c] .. start[c + 1]) from each.  One launch, no pass that depends on all tiles.
+//
+// Clusters are summed by one workgroup each, so a cluster that has swallowed a large part of the tokens (the second
+// Lloyd iteration from evenly spaced seeds does that: 50 000 of 131 072 tokens in one cluster, 0.5 ms in one workgroup)
+// would hold up the whole step.  Tiles all have the same number of tokens, so the tile's workgroup takes that work: a
+// (tile, cluster) range of kHeavy tokens or more is summed right here, in fp64, into rec[tile][start / kHeavy][128]
+// (ranges that long cannot share a block of kHeavy positions, so the slot is unique), and the cluster's workgroup adds
+// the records instead of the rows.
+#ifndef SQ_KM_BIG_TOK
+#define SQ_KM_BIG_TOK 2
+#endif
+constexpr int kBigTok = SQ_KM_BIG_TOK;          // tokens per thread
+constexpr int kBigTile = 1024 * kBigTok;        // tokens per workgroup
+constexpr int kHeavy = 64;                      // tokens of one cluster in one tile from which the tile sums them itself
+constexpr int kSlots = kBigTile / kHeavy;
+
+struct GroupArgs {
+  const int32_t* idx;     // [G,N]
+  const uint16_t* src;    // [G,N,128] bf16 rows that will be summed
+  int32_t* start;         // [G,nT,C+1]
+  int32_t* order;         // [G,N]
+  double* rec;            // [G,nT,kSlots,128]
+  int64_t i_sg, s_sg, s_sn;
+  int32_t N, C, nT;
+};
+
+__device__ __forceinline__ void add_row_bf16(double (&acc)[8], const uint4& raw) {
+  const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const uint32_t bits = (e & 1) ? (w[e >> 1] >> 16) : (w[e >> 1] & 0xffffu);
+    acc[e] += (double)bf16_bits_to_f32(bits);
   }
+}
+
+__device__ __forceinline__ int wave_inclusive_scan(int v, int lane) {
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const int o = __shfl_up(v, d);
+    if (lane >= d) v += o;
+  }
+  return v;
+}
+
+constexpr int kMaxItems = 2 * kSlots;   // pieces of at most kHeavy rows: sum over ranges of ceil(m / kHeavy) <= kBigTile / kHeavy + ranges
+
+__global__ __launch_bounds__(1024) void tile_group_kernel(GroupArgs a) {
+  extern __shared__ double racc[];       // [kSlots][128] sums of the long ranges; then C counters / start positions; then the sorted ids
+  __shared__ int32_t wsum[16];
+  __shared__ int32_t item[kMaxItems][3]; // (first position, rows, slot) of a piece of a long range
+  __shared__ int32_t used[kSlots];
+  __shared__ int32_t n_items;
+  int32_t* hist = (int32_t*)(racc + kSlots * kD);
+  int32_t* ids = hist + a.C;
+  const int tile = blockIdx.x, g = blockIdx.y, t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  int c[kBigTok], rank[kBigTok];
+#pragma unroll
+  for (int u = 0; u < kBigTok; ++u) {
+    const int n = tile * kBigTile + u * 1024 + t;
+    c[u] = (n < a.N) ? a.idx[(int64_t)g * a.i_sg + n] : -1;
+    if (c[u] >= a.C) c[u] = -1;
+  }
+  for (int i = t; i < a.C; i += 1024) hist[i] = 0;
+  for (int i = t; i < kSlots * kD; i += 1024) racc[i] = 0;
+  if (t < kSlots) used[t] = 0;
+  if (t == 0) n_items = 0;
+  __syncthreads();
+#pragma unroll
+  for (int u = 0; u < kBigTok; ++u) rank[u] = (c[u] >= 0) ? atomicAdd(&hist[c[u]], 1) : 0;
+  __syncthreads();
+  int32_t* out = a.start + ((int64_t)g * a.nT + tile) * (a.C + 1);
+  int carry = 0;
+  for (int c0 = 0; c0 < a.C; c0 += 1024) {
+    const int i = c0 + t;
+    const int v = (i < a.C) ? hist[i] : 0;
+    const int inc = wave_inclusive_scan(v, lane);
+    if (lane == 63) wsum[wave] = inc;
+    __syncthreads();
+    int wbase = 0, all = 0;
+#pragma unroll
+    for (int w = 0; w < 16; ++w) {
+      const int x = wsum[w];
+      if (w < wave) wbase += x;
+      all += x;
+    }
+    const int ex = carry + wbase + inc - v;
+    if (i < a.C) {
+      hist[i] = ex;
+      out[i] = ex;
+      if (v >= kHeavy) {
+        const int pieces = (v + kHeavy - 1) / kHeavy, sl = ex / kHeavy;
+        const int first = atomicAdd(&n_items, pieces);
+        used[sl] = 1;
+        for (int k = 0; k < pieces; ++k) {
+          item[first + k][0] = ex + k * kHeavy;
+          item[first + k][1] = min(kHeavy, v - k * kHeavy);
+          item[first + k][2] = sl;
+        }
+      }
+    }
+    carry += all;
+    __syncthreads();
+  }
+  if (t == 0) out[a.C] = carry;
+  int32_t* ord = a.order + (int64_t)g * a.N + (int64_t)tile * kBigTile;
+#pragma unroll
+  for (int u = 0; u < kBigTok; ++u)
+    if (c[u] >= 0) {
+      const int pos = hist[c[u]] + rank[u], n = tile * kBigTile + u * 1024 + t;
+      ord[pos] = n;
+      ids[pos] = n;
+    }
+  __syncthreads();
+  const int ni = n_items;
+  if (ni == 0) return;
+  // a piece per wave: four rows at a time (16 lanes of 16 bytes each), all of a lane's rows requested before the first is used
+  const int o = lane & 15, rg = lane >> 4;
+  const uint16_t* sb = a.src + (int64_t)g * a.s_sg + 8 * o;
+  for (int it = wave; it < ni; it += 16) {
+    const int p0 = item[it][0], m = item[it][1], sl = item[it][2];
+    uint4 raw[kHeavy / 4];
+#pragma unroll
+    for (int u = 0; u < kHeavy / 4; ++u) {
+      const int i = rg + 4 * u;
+      raw[u] = make_uint4(0, 0, 0, 0);
+      if (i < m) raw[u] = *(const uint4*)(sb + (int64_t)ids[p0 + i] * a.s_sn);
+    }
+    double acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+    for (int u = 0; u < kHeavy / 4; ++u) add_row_bf16(acc, raw[u]);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      acc[e] += __shfl_xor(acc[e], 16);
+      acc[e] += __shfl_xor(acc[e], 32);
+    }
+    if (lane < 16) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) atomicAdd(&racc[sl * kD + 8 * o + e], acc[e]);   // exact sums: the order does not matter
+    }
+  }
+  __syncthreads();
+  double* rec = a.rec + ((int64_t)g * a.nT + tile) * kSlots * kD;
+  for (int i = t; i < kSlots * kD; i += 1024)
+    if (used[i / kD]) rec[i] = racc[i];
 }
 
 // ------------------------------------------------------------------------- per-cluster sum + update
 struct SumArgs {
   const uint16_t* src;    // [G,N,128] bf16 rows to sum (keys for the update, values for index_add)
-  const int32_t* order;   // [G,N] tokens sorted by cluster
-  const int32_t* off;     // [G,C+1]
+  const int32_t* order;   // [G,N] token ids, every tile of kBigTile tokens grouped by cluster
+  const int32_t* start;   // [G,nT,C+1] where a cluster's range begins inside its tile
+  const double* rec;      // [G,nT,kSlots,128] sums of the ranges of kHeavy tokens or more
   uint16_t* dst;          // [G,C,128] bf16: centroids (update) or value sums (index_add)
-  int64_t s_sg, s_sn, o_sg, d_sg, d_sc;
-  int32_t C, mode;        // mode 0: plain sum cast to bf16; 1: mean; 2: mean + L2 normalise (1,2: only where cnt > 0)
+  int32_t* cnt;           // [G,C] cluster sizes, or null
+  int64_t s_sg, s_sn, d_sg, d_sc;
+  int32_t N, C, nT, mode; // mode 0: plain sum cast to bf16; 1: mean; 2: mean + L2 normalise (1,2: only where cnt > 0)
 };
 
+#ifndef SQ_KM_LIST
+#define SQ_KM_LIST 2048
+#endif
+constexpr int kListCap = SQ_KM_LIST;   // token ids staged in LDS at a time
+
 __global__ __launch_bounds__(256) void cluster_sum_kernel(SumArgs a) {
-  __shared__ double red[16][kD];
+  __shared__ double red[4][kD];
   __shared__ double ss_red[kD];
-  const int c = blockIdx.x, g = blockIdx.y, t = threadIdx.x;
+  __shared__ int32_t list[kListCap];
+  __shared__ int32_t wsum[4], wbig[4];
+  __shared__ int32_t slot[64];
+  const int c = blockIdx.x, g = blockIdx.y, t = threadIdx.x, lane = t & 63, wave = t >> 6;
   const int o = t & 15, r = t >> 4;
-  const int32_t* off = a.off + (int64_t)g * (a.C + 1);
-  const int beg = off[c], cnt = off[c + 1] - beg;
-  const int32_t* ord = a.order + (int64_t)g * a.o_sg + beg;
+  const int32_t* st = a.start + (int64_t)g * a.nT * (a.C + 1) + c;
+  const int32_t* ord = a.order + (int64_t)g * a.N;
   const uint16_t* sb = a.src + (int64_t)g * a.s_sg + 8 * o;
   double acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-  for (int i0 = r; i0 < cnt; i0 += 64) {  // 4 rows in flight per thread
-    uint4 raw[4];
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int i = i0 + 16 * u;
-      raw[u] = make_uint4(0, 0, 0, 0);
-      if (i < cnt) raw[u] = *(const uint4*)(sb + (int64_t)ord[i] * a.s_sn);
+  double extra = 0;   // channel t of the ranges the tiles have summed already
+  int cnt = 0;
+  for (int tb = 0; tb < a.nT; tb += 64) {   // 64 tiles at a time, four threads per tile
+    const int tile = tb + (t >> 2), q = t & 3;
+    int s0 = 0, mine = 0, big = 0;
+    if (tile < a.nT) {
+      s0 = st[(int64_t)tile * (a.C + 1)];
+      mine = st[(int64_t)tile * (a.C + 1) + 1] - s0;
     }
+    if (mine >= kHeavy) {
+      big = mine;
+      mine = 0;
+    }
+    if (q == 0) slot[t >> 2] = big ? s0 / kHeavy : -1;
+    const int inc = wave_inclusive_scan(q == 0 ? mine : 0, lane);
+    const int binc = wave_inclusive_scan(q == 0 ? big : 0, lane);
+    if (lane == 63) {
+      wsum[wave] = inc;
+      wbig[wave] = binc;
+    }
+    __syncthreads();
+    int base = __shfl(inc, lane & ~3) - mine, all = 0, all_big = 0;   // where this tile's ids go in the list
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const uint32_t w[4] = {raw[u].x, raw[u].y, raw[u].z, raw[u].w};
+    for (int w = 0; w < 4; ++w) {
+      const int x = wsum[w];
+      if (w < wave) base += x;
+      all += x;
+      all_big += wbig[w];
+    }
+    if (all_big > 0 && t < kD) {
+      const int nt = min(64, a.nT - tb);
+      for (int j = 0; j < nt; ++j)
+        if (slot[j] >= 0) extra += a.rec[(((int64_t)g * a.nT + tb + j) * kSlots + slot[j]) * kD + t];
+    }
+    cnt += all_big;
+    const int32_t* mo = ord + (int64_t)tile * kBigTile + s0;
+    for (int w0 = 0; w0 < all; w0 += kListCap) {   // the ids of these tiles' tokens, kListCap at a time
+      const int jb = max(0, w0 - base), je = min(mine, w0 + kListCap - base);
+      for (int j = jb + q; j < je; j += 4) list[base + j - w0] = mo[j];
+      __syncthreads();
+      const int m = min(all - w0, kListCap);
+      for (int i0 = r; i0 < m; i0 += 64) {  // 4 rows in flight per thread
+        uint4 raw[4];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const uint32_t bits = (e & 1) ? (w[e >> 1] >> 16) : (w[e >> 1] & 0xffffu);
-        acc[e] += (double)bf16_bits_to_f32(bits);
+        for (int u = 0; u < 4; ++u) {
+          const int i = i0 + 16 * u;
+          raw[u] = make_uint4(0, 0, 0, 0);
+          if (i < m) raw[u] = *(const uint4*)(sb + (int64_t)list[i] * a.s_sn);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) add_row_bf16(acc, raw[u]);
       }
+      __syncthreads();
     }
+    cnt += all;
+    __syncthreads();
   }
 #pragma unroll
-  for (int e = 0; e < 8; ++e) red[r][8 * o + e] = acc[e];
+  for (int e = 0; e < 8; ++e) {   // the wave's four rows, then the four waves through LDS
+    acc[e] += __shfl_xor(acc[e], 16);
+    acc[e] += __shfl_xor(acc[e], 32);
+  }
+  if (lane < 16) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) red[wave][8 * o + e] = acc[e];
+  }
   __syncthreads();
   float x = 0.f;
   if (t < kD) {
-    double s = 0;
+    double s = extra;
 #pragma unroll
-    for (int rr = 0; rr < 16; ++rr) s += red[rr][t];
+    for (int rr = 0; rr < 4; ++rr) s += red[rr][t];
     x = (float)s;                                   // exact sum rounded once to fp32
     if (a.mode >= 1) x = x / (float)cnt;            // kmeans.py:121
     ss_red[t] = (double)x * (double)x;
@@ -378,6 +549,7 @@ __global__ __launch_bounds__(256) void cluster_sum_kernel(SumArgs a) {
   }
   if (t < kD && (a.mode == 0 || cnt > 0))           // empty clusters keep the old centroid (kmeans.py:120,124)
     a.dst[(int64_t)g * a.d_sg + (int64_t)c * a.d_sc + t] = (uint16_t)f32_to_bf16_bits(x);
+  if (a.cnt && t == 0) a.cnt[(int64_t)g * a.C + c] = cnt;
 }
 
 // ---------------------------------------------------------------------------------- top-k selection
@@ -744,21 +916,24 @@ __global__ __launch_bounds__(1024) void topk_select_kernel(TopkArgs a) {
 }
 
 struct WsLayout {
-  size_t off_bytes, hist_bytes, order_bytes, score_bytes, start_bytes, total_bytes;
-  int nT;
-  size_t all() const { return off_bytes + hist_bytes + order_bytes + score_bytes + start_bytes + total_bytes; }
+  size_t off_bytes, hist_bytes, order_bytes, score_bytes, start_bytes, total_bytes, rec_bytes;
+  int nT, C;
+  size_t rec_offset() const { return off_bytes + hist_bytes + order_bytes + score_bytes + start_bytes + total_bytes; }
+  size_t all() const { return rec_offset() + rec_bytes; }
 };
 
 WsLayout ws_layout(int64_t G, int64_t N, int64_t C) {
   WsLayout w;
   auto up = [](size_t x) { return (x + 255) / 256 * 256; };
   w.nT = (int)((N + kTileTok - 1) / kTileTok);
+  w.C = (int)C;
   w.off_bytes = up((size_t)G * (C + 1) * 4);
-  w.hist_bytes = up((size_t)G * w.nT * C * 4);
+  w.hist_bytes = up((size_t)G * w.nT * (C + 1) * 4);   // per-tile histograms of the ordered sort, or range starts of the grouping
   w.order_bytes = up((size_t)G * N * 4);
   w.score_bytes = up((size_t)G * C * 4);
   w.start_bytes = up((size_t)G * C * 4);
   w.total_bytes = up((size_t)G * C * 4);
+  w.rec_bytes = up((size_t)G * ((N + kBigTile - 1) / kBigTile) * kSlots * kD * 8);
   return w;
 }
 
@@ -777,15 +952,14 @@ int check_current_device(int dev, const char* who) {
   return SQ_OK;
 }
 
-// sorts tokens by cluster into `dst`; shared by train / index_add (order + offsets) and reverse_index
+// tokens of every cluster in ascending order into clusters[G,C,M] (reverse index), sizes into total_out
 int run_sort(const DLTensor* idx, char* wsp, const WsLayout& w, int32_t* dst, int64_t dst_sg, int64_t dst_sc, int M,
-             bool use_off, int32_t* total_out, int C, hipStream_t st) {
+             int32_t* total_out, int C, hipStream_t st) {
   const int64_t G = idx->shape[0], N = idx->shape[1];
   SortArgs s;
   s.idx = (const int32_t*)data_of(idx);
-  s.off = (int32_t*)wsp;
   s.tile_hist = (int32_t*)(wsp + w.off_bytes);
-  s.total = total_out ? total_out : (int32_t*)(wsp + w.off_bytes + w.hist_bytes + w.order_bytes + w.score_bytes + w.start_bytes);
+  s.total = total_out;
   s.dst = dst;
   s.i_sg = stride_of(idx, 0);
   s.dst_sg = dst_sg;
@@ -794,11 +968,60 @@ int run_sort(const DLTensor* idx, char* wsp, const WsLayout& w, int32_t* dst, in
   s.C = C;
   s.nT = w.nT;
   s.M = M;
-  s.use_off = use_off;
   hipLaunchKernelGGL(sort_hist_kernel, dim3(w.nT, (unsigned)G), dim3(kTileTok), (size_t)C * 4, st, s);
   hipLaunchKernelGGL(sort_scan_tiles_kernel, dim3((C + 31) / 32, (unsigned)G), dim3(32 * kScanSegs), 0, st, s);
-  if (use_off) hipLaunchKernelGGL(sort_scan_clusters_kernel, dim3((unsigned)G), dim3(1024), 0, st, s);
   hipLaunchKernelGGL(sort_scatter_kernel, dim3(w.nT, (unsigned)G), dim3(kTileTok), 0, st, s);
+  SQ_HIP(hipGetLastError());
+  return SQ_OK;
+}
+
+// every tile of kBigTile tokens grouped by cluster into `order`, the ranges' starts into the histogram region
+int run_group(const DLTensor* idx, const DLTensor* src, char* wsp, const WsLayout& w, hipStream_t st) {
+  const int64_t G = idx->shape[0], N = idx->shape[1];
+  GroupArgs s;
+  s.idx = (const int32_t*)data_of(idx);
+  s.src = (const uint16_t*)data_of(src);
+  s.start = (int32_t*)(wsp + w.off_bytes);
+  s.order = (int32_t*)(wsp + w.off_bytes + w.hist_bytes);
+  s.rec = (double*)(wsp + w.rec_offset());
+  s.i_sg = stride_of(idx, 0);
+  s.s_sg = stride_of(src, 0);
+  s.s_sn = stride_of(src, 1);
+  s.N = (int)N;
+  s.C = w.C;
+  s.nT = (int)((N + kBigTile - 1) / kBigTile);
+  const size_t lds = (size_t)kSlots * kD * 8 + ((size_t)w.C + kBigTile) * 4;
+  static bool raised[64] = {};
+  int dev = 0;
+  SQ_HIP(hipGetDevice(&dev));
+  if (dev >= 0 && dev < 64 && !raised[dev]) {   // up to 72 KB for 8192 clusters, above the default limit
+    SQ_HIP(hipFuncSetAttribute((const void*)tile_group_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)((size_t)kSlots * kD * 8 + ((size_t)kMaxC + kBigTile) * 4)));
+    raised[dev] = true;
+  }
+  hipLaunchKernelGGL(tile_group_kernel, dim3(s.nT, (unsigned)G), dim3(1024), lds, st, s);
+  SQ_HIP(hipGetLastError());
+  return SQ_OK;
+}
+
+// sums of `src` rows per cluster after run_group
+int run_cluster_sum(const DLTensor* src, char* wsp, const WsLayout& w, DLTensor* dst, int32_t* cnt, int mode, hipStream_t st) {
+  const int64_t G = src->shape[0], N = src->shape[1];
+  SumArgs s;
+  s.src = (const uint16_t*)data_of(src);
+  s.start = (const int32_t*)(wsp + w.off_bytes);
+  s.order = (const int32_t*)(wsp + w.off_bytes + w.hist_bytes);
+  s.rec = (const double*)(wsp + w.rec_offset());
+  s.dst = (uint16_t*)data_of(dst);
+  s.cnt = cnt;
+  s.s_sg = stride_of(src, 0);
+  s.s_sn = stride_of(src, 1);
+  s.d_sg = stride_of(dst, 0);
+  s.d_sc = stride_of(dst, 1);
+  s.N = (int)N;
+  s.C = w.C;
+  s.nT = (int)((N + kBigTile - 1) / kBigTile);
+  s.mode = mode;
+  hipLaunchKernelGGL(cluster_sum_kernel, dim3((unsigned)w.C, (unsigned)G), dim3(256), 0, st, s);
   SQ_HIP(hipGetLastError());
   return SQ_OK;
 }
@@ -863,23 +1086,8 @@ extern "C" int sq_kmeans_train(const DLTensor* data, DLTensor* centroids, DLTens
   a.C = (int)C;
   hipLaunchKernelGGL(kmeans_assign_kernel, dim3((unsigned)((N + kTileTok - 1) / kTileTok), (unsigned)G), dim3(kAssignWaves * 64), 0, st, a);
   SQ_HIP(hipGetLastError());
-  int32_t* order = (int32_t*)(wsp + w.off_bytes + w.hist_bytes);
-  if ((rc = run_sort(idx, wsp, w, order, N, 0, 0, true, (int32_t*)data_of(cnt), (int)C, st))) return rc;   // cnt = cluster sizes
-  SumArgs s;
-  s.src = a.data;
-  s.order = order;
-  s.off = (const int32_t*)wsp;
-  s.dst = (uint16_t*)data_of(centroids);
-  s.s_sg = a.d_sg;
-  s.s_sn = a.d_sn;
-  s.o_sg = N;
-  s.d_sg = a.c_sg;
-  s.d_sc = a.c_sc;
-  s.C = (int)C;
-  s.mode = normalize ? 2 : 1;
-  hipLaunchKernelGGL(cluster_sum_kernel, dim3((unsigned)C, (unsigned)G), dim3(256), 0, st, s);
-  SQ_HIP(hipGetLastError());
-  return SQ_OK;
+  if ((rc = run_group(idx, data, wsp, w, st))) return rc;
+  return run_cluster_sum(data, wsp, w, centroids, (int32_t*)data_of(cnt), normalize ? 2 : 1, st);   // cnt = cluster sizes
 }
 
 extern "C" int sq_reverse_index(const DLTensor* idx, DLTensor* clusters, DLTensor* cluster_size, DLTensor* workspace, void* stream) {
@@ -898,7 +1106,7 @@ extern "C" int sq_reverse_index(const DLTensor* idx, DLTensor* clusters, DLTenso
   if ((rc = check_ws(workspace, w.all(), dev, "sq_reverse_index")) || (rc = check_current_device(dev, "sq_reverse_index"))) return rc;
   hipStream_t st = (hipStream_t)stream;
   hipLaunchKernelGGL(fill_i32_kernel, dim3(256), dim3(256), 0, st, (int32_t*)data_of(clusters), G * C * M, 0);
-  return run_sort(idx, data_of(workspace), w, (int32_t*)data_of(clusters), C * M, M, (int)M, false,
+  return run_sort(idx, data_of(workspace), w, (int32_t*)data_of(clusters), C * M, M, (int)M,
                   (int32_t*)data_of(cluster_size), (int)C, st);
 }
 
@@ -915,23 +1123,8 @@ extern "C" int sq_index_add(const DLTensor* value, const DLTensor* idx, DLTensor
   if ((rc = check_ws(workspace, w.all(), dev, "sq_index_add")) || (rc = check_current_device(dev, "sq_index_add"))) return rc;
   hipStream_t st = (hipStream_t)stream;
   char* wsp = data_of(workspace);
-  int32_t* order = (int32_t*)(wsp + w.off_bytes + w.hist_bytes);
-  if ((rc = run_sort(idx, wsp, w, order, N, 0, 0, true, nullptr, (int)C, st))) return rc;
-  SumArgs s;
-  s.src = (const uint16_t*)data_of(value);
-  s.order = order;
-  s.off = (const int32_t*)wsp;
-  s.dst = (uint16_t*)data_of(out);
-  s.s_sg = stride_of(value, 0);
-  s.s_sn = stride_of(value, 1);
-  s.o_sg = N;
-  s.d_sg = stride_of(out, 0);
-  s.d_sc = stride_of(out, 1);
-  s.C = (int)C;
-  s.mode = 0;
-  hipLaunchKernelGGL(cluster_sum_kernel, dim3((unsigned)C, (unsigned)G), dim3(256), 0, st, s);
-  SQ_HIP(hipGetLastError());
-  return SQ_OK;
+  if ((rc = run_group(idx, value, wsp, w, st))) return rc;
+  return run_cluster_sum(value, wsp, w, out, nullptr, 0, st);
 }
 
 extern "C" int sq_topk_select(const DLTensor* query, const DLTensor* centroids, const DLTensor* clusters,

@@ -68,6 +68,25 @@ def test_reverse_index_and_index_add_exact():
     assert torch.equal(vsum.cpu(), KM.index_add(value, idx, C))
 
 
+def test_index_add_many_tiles_and_one_huge_cluster():
+    """The grouping behind the sums works tile by tile: more tiles than one pass of the sum kernel walks (256), a ragged
+    last tile, a cluster far larger than the id list the kernel stages at a time (the tiles sum its rows themselves), one
+    with just under 2048 tokens per pass, an empty cluster.  Sums are exact."""
+    from longcontext_sqattn_paddle_amd.cache_hub.kmeans import triton_index_add
+
+    G, N, C = 1, 600_001, 32
+    g = torch.Generator().manual_seed(17)
+    idx = torch.randint(0, C, (G, N), generator=g, dtype=torch.int32)
+    u = torch.rand(G, N, generator=g)
+    idx[u < 0.5] = 3                                      # about 300 000 tokens in one cluster
+    idx[(u >= 0.5) & (u < 0.5156)] = 9                    # about 64 per tile of 2048 tokens: either side of the size from which a tile sums a range itself
+    idx[idx == 5] = 6
+    value = torch.randn(G, N, 128, generator=g).bfloat16()
+    vsum = triton_index_add(value.to(DEV), idx.to(DEV), C)
+    torch.cuda.synchronize()
+    assert torch.equal(vsum.cpu(), KM.index_add(value, idx, C))
+
+
 @pytest.mark.parametrize("segments", [1, 2])
 def test_segment_k_means_end_to_end(segments):
     from longcontext_sqattn_paddle_amd.cache_hub.kmeans import segment_k_means
