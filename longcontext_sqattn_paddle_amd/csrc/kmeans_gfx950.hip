@@ -449,6 +449,7 @@ struct SumArgs {
 #ifndef SQ_KM_LIST
 #define SQ_KM_LIST 2048
 #endif
+constexpr int kSumRows = 4;   // rows in flight per thread (8: slower, 2: the same)
 constexpr int kListCap = SQ_KM_LIST;   // token ids staged in LDS at a time
 
 __global__ __launch_bounds__(256) void cluster_sum_kernel(SumArgs a) {
@@ -504,16 +505,16 @@ __global__ __launch_bounds__(256) void cluster_sum_kernel(SumArgs a) {
       for (int j = jb + q; j < je; j += 4) list[base + j - w0] = mo[j];
       __syncthreads();
       const int m = min(all - w0, kListCap);
-      for (int i0 = r; i0 < m; i0 += 64) {  // 4 rows in flight per thread
-        uint4 raw[4];
+      for (int i0 = r; i0 < m; i0 += 16 * kSumRows) {  // kSumRows rows in flight per thread
+        uint4 raw[kSumRows];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < kSumRows; ++u) {
           const int i = i0 + 16 * u;
           raw[u] = make_uint4(0, 0, 0, 0);
           if (i < m) raw[u] = *(const uint4*)(sb + (int64_t)list[i] * a.s_sn);
         }
 #pragma unroll
-        for (int u = 0; u < 4; ++u) add_row_bf16(acc, raw[u]);
+        for (int u = 0; u < kSumRows; ++u) add_row_bf16(acc, raw[u]);
       }
       __syncthreads();
     }
