@@ -2,6 +2,8 @@
 restatement of the reference closure (sqattn/attn_replacer.py:296-454), plus the fake quantisers."""
 import types
 
+import numpy as np
+
 import pytest
 import torch
 
@@ -214,3 +216,43 @@ def test_integer_qk_closure_matches_its_oracle(bit8, bit4, N, Hq, Hkv):
         bad.int8_qk = True
         process_model(m, "SQAttn", {1: {"bit8": 256, "bit4": 256, "sink": 0}}, bad)
         m.layers[1].prefill_attention(q.to(DEV), k.to(DEV), v.to(DEV), None)
+
+
+def test_integer_qk_closure_configurations_drawn_at_random():
+    """Eight closure configurations with args.int8_qk drawn from a seeded generator: batch, GQA ratio, ragged lengths,
+    per-head window ratios (4-bit wider or narrower than 8-bit), bf16 / fp16, query rows whose ranges span eight decades,
+    an all-zero query row and an all-zero key row; each against the integer-product oracle."""
+    from longcontext_sqattn_paddle_amd.sqattn.attn_replacer import process_model
+
+    rng = np.random.default_rng(20240611)
+    for case in range(8):
+        B = int(rng.choice([1, 2]))
+        Hkv = int(rng.choice([1, 2, 4]))
+        group = int(rng.choice([1, 2, 4, 7]))
+        Hq = Hkv * group
+        N = int(rng.integers(130, 1500))
+        dtype = torch.bfloat16 if rng.random() < 0.6 else torch.float16
+        bit8 = [float(rng.choice([0.05, 0.1, 0.25, 0.5, 1.0])) for _ in range(Hq)]
+        bit4 = [float(rng.choice([0.05, 0.1, 0.3, 0.6, 1.0])) for _ in range(Hq)]
+        print(f"case {case}: B={B} Hq={Hq} Hkv={Hkv} N={N} {dtype} bit8={bit8} bit4={bit4}", flush=True)
+        g = torch.Generator().manual_seed(1000 + case)
+        q = torch.randn(B, N, Hq, 128, generator=g) * torch.logspace(-4, 1.5, N)[torch.randperm(N, generator=g)][None, :, None, None]
+        k = torch.randn(B, N, Hkv, 128, generator=g) + 0.5 * torch.randn(1, 1, Hkv, 128, generator=g)
+        v = torch.randn(B, N, Hkv, 128, generator=g)
+        q[0, N // 3, 0] = 0.0
+        k[0, N // 2, 0] = 0.0
+        q, k, v = q.to(dtype), k.to(dtype), v.to(dtype)
+        args = _args(True)
+        args.int8_qk = True
+        m = _Model(2, group)
+        process_model(m, "SQAttn", {1: {"bit8": bit8, "bit4": bit4, "sink": 0}}, args)
+        out = m.layers[1].prefill_attention(q.to(DEV), k.to(DEV), v.to(DEV), None)
+        torch.cuda.synchronize()
+        assert out.shape == (B, N, Hq * 128) and out.dtype == torch.bfloat16   # attn_replacer.py:434: bf16 whatever the inputs
+        ref = plugin.plugin_attention(q, k, v, num_kv_groups=group, bit8=bit8, bit4=bit4, sink=256, relative=True, int8_qk=True)
+        o, r = out.float().cpu(), ref.to(torch.bfloat16).float()
+        assert torch.isfinite(o).all()
+        rms = float(r.pow(2).mean().sqrt())
+        assert _cos(o, r) >= 0.99999, case
+        assert float((o - r).abs().max()) <= 2 ** -7 * float(r.abs().max()) + 2e-3 * rms, case
+
