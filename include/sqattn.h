@@ -210,6 +210,10 @@ int sq_index_add(const DLTensor* value, const DLTensor* idx, DLTensor* out, DLTe
  * max_{h in group} <query[b,h], centroids[g,c]> (ties -> lower c); whole clusters taken in rank order
  * until k tokens are emitted; missing tail = -1.  query bf16 [B,Hq,D]; out int32 [G,k], rows contiguous and at least
  * k apart (it may be the leading columns of a wider list that sq_decode_selected_fwd reads).
+ * With 1024 clusters the workgroups of a group share its score phase and hand over through one arrival counter per
+ * group index g, kept in a device array inside the library (zero between calls: the last arriver sets it back).  Two
+ * calls that overlap in time on one GPU and use the same g would share that counter: order such calls on one stream
+ * or with events.
  */
 int sq_topk_select(const DLTensor* query, const DLTensor* centroids, const DLTensor* clusters,
                    const DLTensor* cluster_size, DLTensor* out, DLTensor* workspace, int32_t num_kv_groups,

@@ -741,11 +741,24 @@ __device__ __forceinline__ void find_pivot(const int32_t* hw, int need, int lane
   above = ab;
 }
 
+// The score phase pulls a head's whole centroid matrix (256 KB at 1024 clusters) through the one CU its workgroup runs
+// on, which is most of that phase's time.  With SQ_TOPK_PARTS workgroups per (sequence, kv head), each scores its share
+// of the clusters into the workspace, and the one that arrives last (a counter per head in a library-owned array that
+// is zero when the library is loaded and that the last arriver sets back) carries on alone with steps 2 - 4.  Nobody
+// waits for anybody.  Calls that overlap on one GPU for the same head index would share the counters: do not overlap them.
+#ifndef SQ_TOPK_PARTS
+#define SQ_TOPK_PARTS 4
+#endif
+constexpr int kTopkParts = SQ_TOPK_PARTS;   // divides 16: every part gets whole waves of 64 clusters
+constexpr int kTopkMaxGroups = 4096;
+__device__ int32_t topk_arrivals[kTopkMaxGroups];
+
 __global__ __launch_bounds__(1024) void topk_select_kernel(TopkArgs a) {
   __shared__ float sc[1024];
   __shared__ unsigned long long ckey[1024];
   __shared__ int32_t pre[1025], rank_cluster[1024], rank_size[1024], hw[256], misc[8];
   const int g = blockIdx.x, t = threadIdx.x, lane = t & 63;
+  const int parts = gridDim.y, part = blockIdx.y;
   const int b = g / a.Hkv, kvh = g % a.Hkv;
   const int nh = a.group;
   if (t < 256) hw[t] = 0;
@@ -756,8 +769,9 @@ __global__ __launch_bounds__(1024) void topk_select_kernel(TopkArgs a) {
   // S[cluster, head] = centroids . queries^T on v_mfma_f32_16x16x32_bf16 (the group's q heads padded to 16 columns).
   // Lane (r = lane % 16, q = lane / 16) feeds centroid row r, columns 32 kk + 8 q .. + 7 as the A operand and the same
   // columns of query head r as the B operand, and receives S[cluster 4 q + i][head r], i < 4.
-  {
-    const int wave = t >> 6, r = lane & 15, q4 = lane >> 4;
+  const int waves_per_part = 16 / parts;
+  if ((t >> 6) < waves_per_part) {
+    const int wave = part * waves_per_part + (t >> 6), r = lane & 15, q4 = lane >> 4;
     typedef __attribute__((ext_vector_type(4))) float f32x4;
     uint4 qf[4];
     const uint16_t* qp = a.query + (int64_t)b * a.q_sb + (int64_t)(kvh * a.group + min(r, nh - 1)) * a.q_sh + 8 * q4;
@@ -782,9 +796,24 @@ __global__ __launch_bounds__(1024) void topk_select_kernel(TopkArgs a) {
         v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x122, 0xf, 0xf, false)));
         v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x124, 0xf, 0xf, false)));
         v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xf, 0xf, false)));
-        if (r == 0) sc[c0 + 4 * q4 + i] = v;
+        if (r == 0) {
+          if (parts == 1) sc[c0 + 4 * q4 + i] = v;
+          else if (c0 + 4 * q4 + i < a.C) a.score[(int64_t)g * a.C + c0 + 4 * q4 + i] = v;
+        }
       }
     }
+  }
+  if (parts > 1) {
+    __syncthreads();
+    if (t == 0) {
+      __threadfence();                   // the workgroup's scores (ordered before this by the barrier) reach the device before it is counted
+      const int arrived = atomicAdd(&topk_arrivals[g], 1);
+      if (arrived == parts - 1) atomicExch(&topk_arrivals[g], 0);   // for the next call
+      misc[4] = arrived;
+    }
+    __syncthreads();
+    if (misc[4] != parts - 1) return;    // uniform: somebody else finishes the job
+    if (have) sc[t] = __hip_atomic_load(&a.score[(int64_t)g * a.C + t], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   __syncthreads();
   uint32_t key32 = 0;
@@ -1175,7 +1204,8 @@ extern "C" int sq_topk_select(const DLTensor* query, const DLTensor* centroids, 
   a.Hkv = (int)Hkv;
   a.group = num_kv_groups;
   if (C <= 1024 && num_kv_groups <= 16) {   // one launch, only the clusters that can fill k are ordered
-    hipLaunchKernelGGL(topk_select_kernel, dim3((unsigned)G), dim3(1024), 0, st, a);
+    const unsigned parts = (G <= kTopkMaxGroups && C >= 64 * 16) ? kTopkParts : 1;   // fewer clusters: not worth sharing
+    hipLaunchKernelGGL(topk_select_kernel, dim3((unsigned)G, parts), dim3(1024), 0, st, a);
     SQ_HIP(hipGetLastError());
     return SQ_OK;
   }
