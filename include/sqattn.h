@@ -142,7 +142,11 @@ int sq_prefill_int8qk_fwd(const DLTensor* q, const DLTensor* k_codes, const DLTe
 typedef struct sq_decode_params {
   int32_t layout;      /* SQ_LAYOUT_HND: q [B,Hq,1,D], caches [B,Hkv,L,D]; SQ_LAYOUT_NHD: [B,1,Hq,D], [B,L,Hkv,D] */
   int32_t p_quant;     /* SQ_P_NONE or SQ_P_E4M3_STATIC (attn_triton_decode.py:232-233)                        */
-  int32_t num_splits;  /* KV splits per (batch, kv head); 0 = let the library choose                            */
+  int32_t num_splits;  /* KV splits per (batch, kv head); 0 = let the library choose.  With 0, seqlens and a batch of
+                          2 .. 32 sequences the library deals its batch * splits workgroups to the sequences in
+                          proportion to their lengths (a ragged batch then ends when its data ends, not when its
+                          longest sequence does); a positive value gives every sequence exactly that many splits, and a
+                          sequence's result then does not depend on its batch mates.  The workspace is the same.        */
   int32_t head_dim_og; /* head_dim before zero-padding to 128 (0 = the tensors' D)                             */
 } sq_decode_params;
 

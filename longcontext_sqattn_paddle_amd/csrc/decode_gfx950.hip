@@ -52,8 +52,40 @@ struct DecodeArgs {
   int32_t B, Hq, Hkv, L, group, head_chunks, num_splits, chunk, p_quant;
   int32_t cache_len;  // gather mode: rows per sequence in the cache (L is then the length of the id lists)
   int32_t hpw;  // kv heads per workgroup (1, 2 or 4): 4/hpw waves share one kv head and interleave its tiles
+  int32_t by_length;  // 1: the B * num_splits workgroups of a head group are dealt to the sequences in proportion to their lengths
   float sm;  // log2e / sqrt(D_original), rounded to fp32
 };
+
+constexpr int kMaxShareBatch = 32;
+
+// Ragged batches: with the same number of splits for every sequence the longest sequence decides when the call ends
+// (lengths uniform in [96K, 128K]: 12 % of the time nothing but that tail).  Dealing the W = B * num_splits workgroups in
+// proportion to the lengths evens that out: every sequence gets one workgroup, the other W - B go by cumulative rounding
+// of (W - B) * (tokens up to and including the sequence) / (all tokens), so the shares add up to W exactly.  Sequence i
+// then owns workgroups [base, base + n) and the same slots of the partial results, which are laid out [Hq, W] in this
+// mode.  The split kernel (want_b < 0: finds the owner of workgroup w) and the combine kernel (want_b = its sequence)
+// both call this, so they agree by construction.
+__device__ __forceinline__ void share_of(const int32_t* seqlens, int B, int Lmax, int W, int want_b, int w, int& b, int& base, int& n) {
+  float total = 0.f;
+  for (int i = 0; i < B; ++i) total += (float)min(max(seqlens[i], 0), Lmax);
+  const float spare = (float)(W - B);
+  float cum = 0.f;
+  int e0 = 0;
+  b = 0;
+  base = 0;
+  n = 1;
+  for (int i = 0; i < B; ++i) {
+    cum += (float)min(max(seqlens[i], 0), Lmax);
+    const int e1 = (total > 0.f) ? (int)floorf(spare * (cum / total)) : 0;
+    const int bs = i + e0, ni = 1 + e1 - e0;
+    if (want_b >= 0 ? (i == want_b) : (w >= bs && w < bs + ni)) {
+      b = i;
+      base = bs;
+      n = ni;
+    }
+    e0 = e1;
+  }
+}
 
 // 16-byte load of cache data that is read exactly once: non-temporal, so it does not displace useful lines
 __device__ __forceinline__ uint4 stream_load(const uint16_t* p) {
@@ -112,10 +144,19 @@ __global__ __launch_bounds__(kWaves * 64) void decode_splitkv_kernel(DecodeArgs 
 
   // Workgroup = (token range, hpw kv heads, batch).  With hpw = 4 each wave streams one kv head over the same
   // token range, so the workgroup as a whole reads whole cache rows of an NHD cache ([B, L, Hkv, D]).
-  const int split = blockIdx.x;
+  int split = blockIdx.x, b = blockIdx.z, nsp = a.num_splits;
+  int64_t slot_stride = a.num_splits;     // partial rows: (b * Hq + hq) * num_splits + split, or hq * W + workgroup
+  int64_t slot0 = (int64_t)b * a.Hq * a.num_splits + split;
+  if (a.by_length) {
+    const int W = a.B * a.num_splits, w = (int)blockIdx.z * a.num_splits + (int)blockIdx.x;
+    int base;
+    share_of(a.seqlens, a.B, a.L, W, -1, w, b, base, nsp);
+    split = w - base;
+    slot_stride = W;
+    slot0 = w;
+  }
   const int hy = blockIdx.y / a.head_chunks;
   const int hc = blockIdx.y % a.head_chunks;
-  const int b = blockIdx.z;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r = lane & 15;
@@ -132,7 +173,7 @@ __global__ __launch_bounds__(kWaves * 64) void decode_splitkv_kernel(DecodeArgs 
   // sweeps the cache front to back, which HBM serves much better than hundreds of separate streams.
   const int t1 = Lb;
   const int ntiles_all = (Lb + kTile - 1) / kTile;
-  const int ntiles = (ntiles_all - split + a.num_splits - 1) / a.num_splits;   // tiles of this workgroup (<= 0: none)
+  const int ntiles = (ntiles_all - split + nsp - 1) / nsp;   // tiles of this workgroup (<= 0: none)
   const int h0 = hc * 16;                    // first head of this chunk inside the kv group
   const int nh = min(16, a.group - h0);      // heads handled here
   const int hq0 = kvh * a.group + h0;        // absolute first q head of this wave
@@ -141,8 +182,8 @@ __global__ __launch_bounds__(kWaves * 64) void decode_splitkv_kernel(DecodeArgs 
     for (int i = threadIdx.x; i < a.hpw * nh * kD; i += blockDim.x) {
       const int hs = i / (nh * kD), h = (i / kD) % nh, d = i % kD;
       const int hq = (hy * a.hpw + hs) * a.group + h0 + h;
-      a.part_o[(((int64_t)b * a.Hq + hq) * a.num_splits + split) * kD + d] = 0.f;
-      if (d == 0) a.part_lse[((int64_t)b * a.Hq + hq) * a.num_splits + split] = -INFINITY;
+      a.part_o[((int64_t)hq * slot_stride + slot0) * kD + d] = 0.f;
+      if (d == 0) a.part_lse[(int64_t)hq * slot_stride + slot0] = -INFINITY;
     }
     return;
   }
@@ -160,7 +201,7 @@ __global__ __launch_bounds__(kWaves * 64) void decode_splitkv_kernel(DecodeArgs 
   // says whether token n0 + 4g + i (the one whose score this lane holds in s[i]) takes part
   const int32_t* idp = GATHER ? a.ids + ((int64_t)b * a.Hkv + kvh) * a.ids_sg : nullptr;
   auto load_tile = [&](int tile, uint4 (&kf)[4], uint4 (&vf)[4], int& valid) {
-    const int n0 = (split + tile * a.num_splits) * kTile;
+    const int n0 = (split + tile * nsp) * kTile;
     int tk = min(n0 + r, t1 - 1);
     if constexpr (GATHER) tk = min(max(idp[tk], 0), a.cache_len - 1);
     const uint16_t* kp = kbase + (int64_t)tk * a.k_sn + 8 * g;
@@ -297,7 +338,7 @@ __global__ __launch_bounds__(kWaves * 64) void decode_splitkv_kernel(DecodeArgs 
     // one division per lane (the general path below divides every element, which a wave alone on its SIMD feels:
     // the two together took 4 us off every call).  The normalised partial differs from o / l by at most 1 ulp.
     if (r < nh) {
-      const int64_t row = ((int64_t)b * a.Hq + hq0 + r) * a.num_splits + split;
+      const int64_t row = (int64_t)(hq0 + r) * slot_stride + slot0;
       float* po = a.part_o + row * kD + 32 * g;
       const bool any = l > 0.f;
       const float inv = any ? 1.f / l : 0.f;
@@ -333,7 +374,7 @@ __global__ __launch_bounds__(kWaves * 64) void decode_splitkv_kernel(DecodeArgs 
       o += s_o[w0 + w][h][d] * sc;
     }
     const int hq = (hy * a.hpw + hs) * a.group + h0 + h;
-    const int64_t row = ((int64_t)b * a.Hq + hq) * a.num_splits + split;
+    const int64_t row = (int64_t)hq * slot_stride + slot0;
     a.part_o[row * kD + d] = (lt > 0.f) ? o / lt : 0.f;
     if (d == 0) a.part_lse[row] = (lt > 0.f) ? mm + log2f(lt) : -INFINITY;
   }
@@ -346,6 +387,8 @@ struct CombineArgs {
   float* lse;  // may be null
   int64_t o_sb, o_sh;
   int32_t Hq, num_splits, out_dtype;  // 0 bf16, 1 f16, 2 f32
+  const int32_t* seqlens;             // by_length: the lengths the split kernel dealt its workgroups by
+  int32_t B, L, by_length;
 };
 
 constexpr int kCombineThreads = 1024;
@@ -360,8 +403,14 @@ __global__ __launch_bounds__(kCombineThreads) void decode_combine_kernel(Combine
   extern __shared__ float s_w[];          // [num_splits] weights, then [32][32] partial outputs
   __shared__ float s_red[2][kCombineThreads / 64];
   const int h = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
-  const int S = a.num_splits;
-  const int64_t row0 = ((int64_t)b * a.Hq + h) * S;
+  int S = a.num_splits;
+  int64_t row0 = ((int64_t)b * a.Hq + h) * S;
+  if (a.by_length) {   // this sequence's slots among the W of the head
+    const int W = a.B * a.num_splits;
+    int bb, base;
+    share_of(a.seqlens, a.B, a.L, W, b, 0, bb, base, S);
+    row0 = (int64_t)h * W + base;
+  }
   const int dl = tid & (kCombineChunk - 1), grp = tid / kCombineChunk;
   const int d = blockIdx.z * kCombineChunk + dl;
   const float* po = a.part_o + row0 * kD + d;
@@ -558,6 +607,9 @@ static int decode_impl(const DLTensor* q, const DLTensor* kcache, const DLTensor
   a.head_chunks = (int32_t)((group + 15) / 16);
   a.hpw = (Hkv % 4 == 0) ? 4 : ((Hkv % 2 == 0) ? 2 : 1);
   a.num_splits = S;
+  // the library's own choice of splits on a ragged batch: workgroups in proportion to the lengths.  A caller that names
+  // num_splits gets exactly that many for every sequence (a sequence's partition then does not depend on its batch mates).
+  a.by_length = (seqlens && params->num_splits <= 0 && B > 1 && B <= kMaxShareBatch && S > 1 && B * (int64_t)S <= 4096) ? 1 : 0;
   a.chunk = (int32_t)chunk;
   a.p_quant = params->p_quant;
   const int64_t d_og = params->head_dim_og > 0 ? params->head_dim_og : D;
@@ -587,8 +639,13 @@ static int decode_impl(const DLTensor* q, const DLTensor* kcache, const DLTensor
   c.Hq = (int32_t)Hq;
   c.num_splits = S;
   c.out_dtype = odt == DType::BF16 ? 0 : (odt == DType::F16 ? 1 : 2);
+  c.seqlens = a.seqlens;
+  c.B = (int32_t)B;
+  c.L = (int32_t)L;
+  c.by_length = a.by_length;
+  const size_t max_slots = a.by_length ? (size_t)B * S : (size_t)S;   // a sequence may own up to all of a head's workgroups
   hipLaunchKernelGGL(decode_combine_kernel, dim3((unsigned)Hq, (unsigned)B, kD / kCombineChunk), dim3(kCombineThreads),
-                     (size_t)(S + kCombineGroups * kCombineChunk) * sizeof(float), st, c);
+                     (max_slots + kCombineGroups * kCombineChunk) * sizeof(float), st, c);
   SQ_HIP(hipGetLastError());
   return SQ_OK;
 }

@@ -21,6 +21,9 @@ def attn_decode(q, k, v, tensor_layout="HND", output_dtype=torch.float16, return
 
     Extensions over the reference (all optional): `seqlens` int32 [B] valid prefix per sequence,
     `num_splits` KV splits, caller-provided `workspace`/`out` so that a serving loop allocates nothing.
+    With `num_splits=0` the library chooses, and on a batch with `seqlens` it deals its workgroups to the sequences in
+    proportion to their lengths; a positive `num_splits` gives every sequence exactly that many splits, so that a
+    sequence's result does not depend on its batch mates.
     """
     if tensor_layout not in N.LAYOUT:
         raise ValueError(f"tensor_layout {tensor_layout} not supported")
@@ -37,7 +40,7 @@ def attn_decode(q, k, v, tensor_layout="HND", output_dtype=torch.float16, return
         workspace = torch.empty(need // 4, dtype=torch.float32, device=q.device)
     o = out if out is not None else torch.empty(q.shape, dtype=output_dtype, device=q.device)
     lse = torch.empty([B, Hq, 1], dtype=torch.float32, device=q.device) if return_lse else None
-    params = N.DecodeParams(N.LAYOUT[tensor_layout], N.P_E4M3_STATIC if is_P_fp8_quant else N.P_NONE, S, head_dim_og)
+    params = N.DecodeParams(N.LAYOUT[tensor_layout], N.P_E4M3_STATIC if is_P_fp8_quant else N.P_NONE, max(num_splits, 0), head_dim_og)
     bq, bk, bv, bs, bo, bl, bw = (N.dl(t) for t in (q, k, v, seqlens, o, lse, workspace))
     N.check(lib.sq_decode_fwd(N.ptr(bq), N.ptr(bk), N.ptr(bv), N.ptr(bs), N.ptr(bo), N.ptr(bl), N.ptr(bw),
                               params, N.current_stream(q.device)))
@@ -82,7 +85,7 @@ def attn_decode_selected(q, k, v, token_ids, tensor_layout="NHD", output_dtype=t
         workspace = torch.empty(need // 4, dtype=torch.float32, device=q.device)
     o = out if out is not None else torch.empty(q.shape, dtype=output_dtype, device=q.device)
     lse = torch.empty([B, Hq, 1], dtype=torch.float32, device=q.device) if return_lse else None
-    params = N.DecodeParams(N.LAYOUT[tensor_layout], N.P_E4M3_STATIC if is_P_fp8_quant else N.P_NONE, S, head_dim_og)
+    params = N.DecodeParams(N.LAYOUT[tensor_layout], N.P_E4M3_STATIC if is_P_fp8_quant else N.P_NONE, max(num_splits, 0), head_dim_og)
     b = [N.dl(t) for t in (q, k, v, token_ids, seqlens, o, lse, workspace)]
     N.check(lib.sq_decode_selected_fwd(*[N.ptr(x) for x in b], params, N.current_stream(q.device)))
     o = o[..., :head_dim_og]
@@ -110,7 +113,7 @@ class DecodePlan:
                                      device=q.device)
         self.out = torch.empty(q.shape, dtype=output_dtype, device=q.device)
         self.lse = torch.empty([B, Hq, 1], dtype=torch.float32, device=q.device) if return_lse else None
-        self._params = N.DecodeParams(N.LAYOUT[tensor_layout], N.P_E4M3_STATIC if is_P_fp8_quant else N.P_NONE, S, 128)
+        self._params = N.DecodeParams(N.LAYOUT[tensor_layout], N.P_E4M3_STATIC if is_P_fp8_quant else N.P_NONE, max(num_splits, 0), 128)
         self._b = [N.dl(t) for t in (q, k, v, seqlens, self.out, self.lse, self.workspace)]
         self._ptrs = [N.ptr(x) for x in self._b]
         self._device = q.device

@@ -55,6 +55,30 @@ def test_decode_split_invariance_and_bf16_out():
     assert torch.equal(ob, outs[0].to(torch.bfloat16)) or float((ob.float() - outs[0]).abs().max()) < 2 ** -8
 
 
+@pytest.mark.parametrize("lens", [[8192, 17, 3000, 1], [5, 8192], [8192, 0, 4000], [100] * 7 + [8192]])
+def test_decode_workgroups_dealt_by_length(lens):
+    """With num_splits left to the library a ragged batch's workgroups go to the sequences in proportion to their
+    lengths (one each at least): very uneven lengths, a one-token and an empty sequence, against the closed form, and
+    against the same call with a named split count (every sequence the same number of splits)."""
+    print(f"case decode by length lens={lens}", flush=True)
+    B, L = len(lens), 8192
+    q, kc, vc, _ = inputs.decode_inputs(B, 28, 4, L, 128, seed=77)
+    qh, kh, vh = _to_hnd(q, kc, vc)
+    ref, lse_ref = A.exact_attention(A.fold_scale(qh, 128), kh, vh, causal=False, kv_lens=[max(x, 1) for x in lens], score_scale=math.log(2.0))
+    out, lse = _run(q, kc, vc, lens, "NHD", output_dtype=torch.float32, return_lse=True)
+    named, lse_named = _run(q, kc, vc, lens, "NHD", output_dtype=torch.float32, return_lse=True, num_splits=8)
+    out, named, lse, lse_named = out.cpu()[:, 0], named.cpu()[:, 0], lse.cpu()[:, :, 0], lse_named.cpu()[:, :, 0]
+    rms = float(ref.pow(2).mean().sqrt())
+    for b, n in enumerate(lens):
+        if n == 0:   # nothing to attend to: zeros and -inf, from both partitions
+            assert float(out[b].abs().max()) == 0.0 and float(named[b].abs().max()) == 0.0
+            assert bool(torch.isinf(lse[b]).all()) and bool(torch.isinf(lse_named[b]).all())
+            continue
+        assert float((out[b].double() - ref[b, :, 0]).abs().max()) < 2e-4 * rms + 1e-6, b
+        assert float((out[b] - named[b]).abs().max()) < 1e-5, b
+        assert torch.allclose(lse[b].double(), lse_ref[b, :, 0], atol=2e-4)
+
+
 def test_decode_no_seqlens_fp16_and_small_head_dim():
     g = torch.Generator().manual_seed(5)
     q = torch.randn(2, 8, 1, 64, generator=g).half()
