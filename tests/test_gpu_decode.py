@@ -79,6 +79,34 @@ def test_decode_workgroups_dealt_by_length(lens):
         assert torch.allclose(lse[b].double(), lse_ref[b, :, 0], atol=2e-4)
 
 
+def test_decode_by_length_replayed_from_a_graph_with_changing_lengths():
+    """The length-proportional dealing is computed on the device from `seqlens`, so a captured launch follows the
+    lengths it finds at replay time: one graph, four sets of lengths written between the replays (with eager work in
+    between), each replay bit-identical to an eager call with those lengths."""
+    from longcontext_sqattn_paddle_amd.sqattn.attn_triton_decode import DecodePlan
+
+    dev = torch.device("cuda:0")
+    B, L = 3, 6000
+    q, kc, vc, _ = inputs.decode_inputs(B, 28, 4, L, 128, seed=91)
+    q, kc, vc = q.to(dev), kc.to(dev), vc.to(dev)
+    lens = torch.tensor([L, 100, 2500], dtype=torch.int32, device=dev)
+    plan = DecodePlan(q, kc, vc, "NHD", torch.float32, seqlens=lens)
+    plan.run()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        plan.run()
+    for case in ([L, 100, 2500], [1, L, 1], [3000, 3000, 3000], [17, 5999, 0]):
+        lens.copy_(torch.tensor(case, dtype=torch.int32))
+        graph.replay()
+        got = plan.out.clone()
+        scratch = torch.randn(1 << 20, device=dev).sum()          # eager work between the replays
+        torch.cuda.synchronize()
+        eager = _run(q, kc, vc, case, "NHD", output_dtype=torch.float32)
+        assert torch.equal(got.view(torch.int32), eager.view(torch.int32)), case
+        assert bool(torch.isfinite(scratch))
+
+
 def test_decode_no_seqlens_fp16_and_small_head_dim():
     g = torch.Generator().manual_seed(5)
     q = torch.randn(2, 8, 1, 64, generator=g).half()
