@@ -4,7 +4,9 @@
  * Every entry point takes borrowed DLPack tensors (device pointers, shapes, strides in elements), plain
  * scalars and a HIP stream handle (`hipStream_t` passed as `void*`, NULL = the null stream); it enqueues
  * work on that stream and returns without synchronising unless stated otherwise.  Nothing is retained
- * after the call returns; outputs and workspaces are allocated by the caller.  Return value: SQ_OK or a
+ * after the call returns; outputs and workspaces are allocated by the caller.  (Two pieces of device memory live
+ * inside the library and say so where they are declared: the partials array of sq_decode_fwd_noalloc and the
+ * arrival counters of sq_topk_select, which are zero again when a call has finished.)  Return value: SQ_OK or a
  * negative SQ_E* code; `sq_last_error()` then holds a message (thread-local).  No entry point throws or
  * aborts.  Tensors must live on one ROCm device (DLPack device type kDLROCM, or kDLCUDA as some
  * PyTorch-ROCm builds report), have a contiguous last dimension and a 16-byte aligned base address.
