@@ -91,10 +91,15 @@ typedef __attribute__((ext_vector_type(2))) int i32x2_t;
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t bits16) { return __uint_as_float(bits16 << 16); }
 
 // round-to-nearest-even fp32 -> bf16 bit pattern (finite inputs)
+// fp32 -> bf16, round to nearest even: gfx950 converts in hardware (v_cvt_pk_bf16_f32, two values per instruction),
+// with the same bits as the add-0x7fff-plus-lsb sequence for every finite input
 __device__ __forceinline__ uint32_t f32_to_bf16_bits(float x) {
-  uint32_t u = __float_as_uint(x);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return u >> 16;
+  return (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)x);
+}
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+  typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{lo, hi}, bf16x2_t));
 }
 
 // e4m3 (OCP, max 448) round trip of a non-negative value <= 448: fp32 -> fp8 (RNE) -> fp32

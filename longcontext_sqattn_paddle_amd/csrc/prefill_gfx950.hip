@@ -228,7 +228,7 @@ __device__ __forceinline__ uint32_t scale_pair(uint32_t w, float sm) {
   if constexpr (BF16) {
     const float lo = bf16_bits_to_f32(w & 0xffffu) * sm;
     const float hi = bf16_bits_to_f32(w >> 16) * sm;
-    return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+    return pack_bf16x2(lo, hi);
   } else {
     const float lo = (float)__builtin_bit_cast(_Float16, (uint16_t)(w & 0xffffu)) * sm;
     const float hi = (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> 16)) * sm;
@@ -1176,8 +1176,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
         v[3] *= isc.w;
       }
       if (a.out_dtype == 0) {
-        uint2 w = make_uint2(f32_to_bf16_bits(v[0]) | (f32_to_bf16_bits(v[1]) << 16),
-                             f32_to_bf16_bits(v[2]) | (f32_to_bf16_bits(v[3]) << 16));
+        uint2 w = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
         *(uint2*)((uint16_t*)a.out + obase + d) = w;
       } else if (a.out_dtype == 1) {
         uint2 w = make_uint2(pack_f16(v[0], v[1]), pack_f16(v[2], v[3]));

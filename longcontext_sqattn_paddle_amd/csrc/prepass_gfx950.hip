@@ -65,7 +65,10 @@ template <bool BF16>
 __device__ __forceinline__ uint4 pack8(const float (&x)[8]) {
   uint32_t w[4];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) w[i] = st<BF16>(x[2 * i]) | (st<BF16>(x[2 * i + 1]) << 16);
+  for (int i = 0; i < 4; ++i) {
+    if constexpr (BF16) w[i] = pack_bf16x2(x[2 * i], x[2 * i + 1]);
+    else w[i] = st<BF16>(x[2 * i]) | (st<BF16>(x[2 * i + 1]) << 16);
+  }
   return make_uint4(w[0], w[1], w[2], w[3]);
 }
 
