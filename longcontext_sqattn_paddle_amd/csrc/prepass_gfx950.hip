@@ -29,8 +29,26 @@ struct View {   // [B, N, H, 128] addressed by element strides (either memory la
   int64_t sb, sn, sh;
 };
 
+// x / d for x < 2^31 as one multiply-high, one add and one shift (d >= 1): m = ceil(2^(32+s) / d) - 2^32, s = ceil(log2 d).
+// The row kernels split a row number into (batch, token, head) with it: the 64-bit divisions they used before were
+// a few hundred vector instructions per row, more than the quantisation itself.
+struct FastDiv {
+  uint32_t m, s, d;
+};
+inline FastDiv make_fastdiv(uint32_t d) {
+  FastDiv f;
+  f.d = d;
+  f.s = 0;
+  while ((1ull << f.s) < d) ++f.s;
+  f.m = (uint32_t)((((1ull << (32 + f.s)) + d - 1) / d) - (1ull << 32));
+  return f;
+}
+__device__ __forceinline__ uint32_t fastdiv(uint32_t x, const FastDiv& f) { return (__umulhi(x, f.m) + x) >> f.s; }
+
 struct PrepassArgs {
   View q, k, v, q8, q4, k8, k4, v8;
+  FastDiv div_hq, div_hkv, div_n;
+  int32_t small;    // every row number is below 2^31: the splits use fastdiv
   double* part;     // [nblk, B*Hkv*128]
   uint16_t* mean;   // [B*Hkv*128] bits of the key mean in the tensor dtype
   int32_t B, N, Hq, Hkv, is_bf16, nblk, tok_per_blk, want4;
@@ -213,15 +231,30 @@ __global__ __launch_bounds__(256) void prepass_rows_kernel(PrepassArgs a) {
   const int64_t row0 = ((int64_t)blockIdx.x * (blockDim.x / 16) + (threadIdx.x >> 4)) * R;
   if (row0 >= rows) return;   // whole 16-lane groups leave together; the shuffles below stay inside a group
   uint4 raw[R], mraw[R];
-  int64_t off8[R], off4[R];
+  int64_t off8[R], off4[R], nn[R], bbv[R];
+  int hh[R];
   bool live[R];
 #pragma unroll
   for (int u = 0; u < R; ++u) {
     const int64_t row = row0 + u;
     live[u] = row < rows;
     const int64_t rr = live[u] ? row : row0;
-    const int h = (int)(rr % H);
-    const int64_t n = (rr / H) % a.N, b = rr / ((int64_t)H * a.N);
+    int h;
+    int64_t n, b;
+    if (a.small) {
+      const uint32_t t = fastdiv((uint32_t)rr, CENTRE ? a.div_hkv : a.div_hq);
+      h = (int)((uint32_t)rr - t * (uint32_t)H);
+      const uint32_t bb = fastdiv(t, a.div_n);
+      n = t - bb * (uint32_t)a.N;
+      b = bb;
+    } else {
+      h = (int)(rr % H);
+      n = (rr / H) % a.N;
+      b = rr / ((int64_t)H * a.N);
+    }
+    hh[u] = h;
+    nn[u] = n;
+    bbv[u] = b;
     {   // rows are read once and written once: non-temporal accesses keep them from displacing each other in L2
       const u32x4_t w = __builtin_nontemporal_load((const u32x4_t*)((const uint16_t*)src.p + b * src.sb + n * src.sn + h * src.sh + 8 * l16));
       raw[u] = make_uint4(w[0], w[1], w[2], w[3]);
@@ -264,9 +297,8 @@ __global__ __launch_bounds__(256) void prepass_rows_kernel(PrepassArgs a) {
           const int c = (int)fminf(fmaxf(round_half_away(divide(x[e], scale)) + 0.0f, -128.f), 127.f);
           w[e >> 2] |= (uint32_t)(c & 0xff) << (8 * (e & 3));
         }
-        const int64_t row = row0 + u;
-        const int h = (int)(row % H);
-        const int64_t n = (row / H) % a.N, b = row / ((int64_t)H * a.N);
+        const int h = hh[u];
+        const int64_t n = nn[u], b = bbv[u];
         *(uint2*)((char*)a.kcodes.p + b * a.kcodes.sb + n * a.kcodes.sn + h * a.kcodes.sh + 8 * l16) = make_uint2(w[0], w[1]);
         if (l16 == 0) a.kscale[(b * H + h) * a.scale_stride + n] = scale.d;
       }
@@ -429,6 +461,10 @@ int prepass_impl(const DLTensor* query, const DLTensor* key, const DLTensor* val
   a.Hq = (int)Hq;
   a.Hkv = (int)Hkv;
   a.is_bf16 = dt == DType::BF16;
+  a.div_hq = make_fastdiv((uint32_t)Hq);
+  a.div_hkv = make_fastdiv((uint32_t)Hkv);
+  a.div_n = make_fastdiv((uint32_t)N);
+  a.small = (B * N * (Hq > Hkv ? Hq : Hkv) < (1ll << 31)) ? 1 : 0;
   a.tok_per_blk = tokens_per_block(N);
   a.nblk = (int)((N + a.tok_per_blk - 1) / a.tok_per_blk);
   a.want4 = q4 != nullptr;
