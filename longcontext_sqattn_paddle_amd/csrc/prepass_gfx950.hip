@@ -29,22 +29,8 @@ struct View {   // [B, N, H, 128] addressed by element strides (either memory la
   int64_t sb, sn, sh;
 };
 
-// x / d for x < 2^31 as one multiply-high, one add and one shift (d >= 1): m = ceil(2^(32+s) / d) - 2^32, s = ceil(log2 d).
-// The row kernels split a row number into (batch, token, head) with it: the 64-bit divisions they used before were
-// a few hundred vector instructions per row, more than the quantisation itself.
-struct FastDiv {
-  uint32_t m, s, d;
-};
-inline FastDiv make_fastdiv(uint32_t d) {
-  FastDiv f;
-  f.d = d;
-  f.s = 0;
-  while ((1ull << f.s) < d) ++f.s;
-  f.m = (uint32_t)((((1ull << (32 + f.s)) + d - 1) / d) - (1ull << 32));
-  return f;
-}
-__device__ __forceinline__ uint32_t fastdiv(uint32_t x, const FastDiv& f) { return (__umulhi(x, f.m) + x) >> f.s; }
-
+// The row kernels split a row number into (batch, token, head) with FastDiv (common.hpp): the 64-bit divisions they
+// used before were a few hundred vector instructions per row, more than the quantisation itself.
 struct PrepassArgs {
   View q, k, v, q8, q4, k8, k4, v8;
   FastDiv div_hq, div_hkv, div_n;
