@@ -191,8 +191,19 @@ __global__ __launch_bounds__(256) void prepass_kmean_kernel(PrepassArgs a) {
   const int ncol = a.B * a.Hkv * kPD;
   const int c = (blockIdx.x * blockDim.x + threadIdx.x) >> 4, l = threadIdx.x & 15;
   double s = 0;
-  if (c < ncol)
-    for (int b = l; b < a.nblk; b += 16) s += a.part[(int64_t)b * ncol + c];
+  if (c < ncol) {   // four partial sums requested at a time (one after the other they were 32 dependent round trips)
+    double s4[4] = {0, 0, 0, 0};
+    int b = l;
+    for (; b + 48 < a.nblk; b += 64) {
+      double v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) v[u] = a.part[(int64_t)(b + 16 * u) * ncol + c];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) s4[u] += v[u];
+    }
+    for (; b < a.nblk; b += 16) s4[0] += a.part[(int64_t)b * ncol + c];
+    s = (s4[0] + s4[1]) + (s4[2] + s4[3]);
+  }
 #pragma unroll
   for (int sh = 8; sh >= 1; sh >>= 1) s += __shfl_xor(s, sh);
   if (c >= ncol || l != 0) return;
