@@ -320,6 +320,48 @@ __global__ __launch_bounds__(256) void prepass_v_kernel(PrepassArgs a) {
   const int64_t n = t / (kPD / 8);
   const uint16_t* base = (const uint16_t*)a.v.p + n * a.v.sn + 8 * c8;
   float amax[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  const int nrow = a.B * a.Hkv;
+  if (nrow <= 8) {
+    // few (batch, head) rows per token (Qwen2.5-7B: 4): all of them requested at once and kept in registers, so that V
+    // is read once and no load waits for the one before it
+    uint4 raw[8];
+    int64_t oo[8];
+    int b = 0, h = 0;
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      raw[r] = make_uint4(0, 0, 0, 0);
+      oo[r] = 0;
+      if (r < nrow) {
+        raw[r] = *(const uint4*)(base + b * a.v.sb + h * a.v.sh);
+        oo[r] = b * a.v8.sb + h * a.v8.sh;
+        if (++h == a.Hkv) {
+          h = 0;
+          ++b;
+        }
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      float x[8];
+      unpack8<BF16>(raw[r], x);   // rows past nrow are zeros: no effect on the maximum
+#pragma unroll
+      for (int e = 0; e < 8; ++e) amax[e] = fmaxf(amax[e], fabsf(x[e]));
+    }
+    Divisor sc[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) sc[e] = make_divisor(scale_of<QT>(fmaxf(amax[e], 1e-5f)));
+    uint16_t* ob = (uint16_t*)a.v8.p + n * a.v8.sn + 8 * c8;
+#pragma unroll
+    for (int r = 0; r < 8; ++r)
+      if (r < nrow) {
+        float x[8], y[8];
+        unpack8<BF16>(raw[r], x);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) y[e] = qdq8<QT>(x[e], sc[e]);
+        *(uint4*)(ob + oo[r]) = pack8<BF16>(y);
+      }
+    return;
+  }
   for (int b = 0; b < a.B; ++b)
     for (int h = 0; h < a.Hkv; ++h) {
       float x[8];
