@@ -185,17 +185,21 @@ __global__ __launch_bounds__(kLinMaxWaves * 64) void linear_rows_kernel(LinArgs 
       const int per_lane = (chunks + 63) >> 6;
       const int tasks = M * per_lane;
       float* part = (float*)(xs + M * row16);   // [M][per_lane][64]
+      // task t = (row t / per_lane, chunk index t % per_lane); with one row the division by a kernel argument (a software
+      // routine of some thirty instructions, on the path between the staging and the main loop) drops out
+      auto row_of = [&](int t) { return M == 1 ? 0 : t / per_lane; };
+      auto idx_of = [&](int t) { return M == 1 ? t : t % per_lane; };
       auto x_chunk = [&](int t) {
-        const int m = t / per_lane, c = lane + 64 * (t % per_lane);
+        const int m = row_of(t), c = lane + 64 * idx_of(t);
         return *(const u32x4_t*)(a.x + (int64_t)(m < a.rows ? m : a.rows - 1) * a.x_sr + (c < chunks ? c : chunks - 1) * 16);
       };
       auto w_chunk = [&](int t) {
-        const int c = lane + 64 * (t % per_lane);
+        const int c = lane + 64 * idx_of(t);
         return *(const u32x4_t*)(a.norm_w + (c < chunks ? c : chunks - 1) * 16);
       };
       auto squares = [&](int t, const u32x4_t& v) {
         float p = 0.f;
-        if (lane + 64 * (t % per_lane) < chunks) {
+        if (lane + 64 * idx_of(t) < chunks) {
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             const float lo = cv16<BF16>(v[j]), hi = cv16<BF16>(v[j] >> 16);
@@ -235,7 +239,7 @@ __global__ __launch_bounds__(kLinMaxWaves * 64) void linear_rows_kernel(LinArgs 
         r[m] = rnd16<BF16>(1.0f / sqrtf(ve));
       }
       auto scale = [&](int t, const u32x4_t& v, const u32x4_t& g) {
-        const int m = t / per_lane, c = lane + 64 * (t % per_lane);
+        const int m = row_of(t), c = lane + 64 * idx_of(t);
         float rr = r[0];
 #pragma unroll
         for (int i = 1; i < M; ++i) rr = (m == i) ? r[i] : rr;
