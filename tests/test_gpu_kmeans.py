@@ -87,6 +87,27 @@ def test_index_add_many_tiles_and_one_huge_cluster():
     assert torch.equal(vsum.cpu(), KM.index_add(value, idx, C))
 
 
+@pytest.mark.parametrize("C", [8192, 5000, 1025])
+def test_index_add_many_clusters(C):
+    """Cluster counts up to the supported maximum (8192: the grouping kernel's counters, ids and long-range sums then
+    take 72 KB of LDS, above the default limit; its prefix over the clusters runs in eight rounds) and counts that are
+    not multiples of anything: sums exact, reverse index exact."""
+    from longcontext_sqattn_paddle_amd.cache_hub.kmeans import triton_index_add, triton_reverse_index
+
+    G, N = 2, 30_000
+    g = torch.Generator().manual_seed(C)
+    idx = torch.randint(0, C, (G, N), generator=g, dtype=torch.int32)
+    idx[0, :3000] = C - 1                                  # one long range at the last cluster
+    value = torch.randn(G, N, 128, generator=g).bfloat16()
+    vsum = triton_index_add(value.to(DEV), idx.to(DEV), C)
+    msize = int(torch.stack([torch.bincount(idx[i].long(), minlength=C) for i in range(G)]).max())
+    clusters, size = triton_reverse_index(idx.to(DEV), C, msize)
+    torch.cuda.synchronize()
+    assert torch.equal(vsum.cpu(), KM.index_add(value, idx, C))
+    rc, rs = KM.reverse_index(idx, C, msize)
+    assert torch.equal(size.cpu(), rs) and torch.equal(clusters.cpu(), rc)
+
+
 @pytest.mark.parametrize("segments", [1, 2])
 def test_segment_k_means_end_to_end(segments):
     from longcontext_sqattn_paddle_amd.cache_hub.kmeans import segment_k_means
