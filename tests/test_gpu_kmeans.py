@@ -24,7 +24,7 @@ def _bf16_ulp_diff(a, b):
 
 
 @pytest.mark.parametrize("normalize", [True, False])
-@pytest.mark.parametrize("G,N,C", [(2, 3000, 64), (1, 4096, 160)])
+@pytest.mark.parametrize("G,N,C", [(2, 3000, 64), (1, 4096, 160), (1, 9000, 2048), (1, 20000, 8192)])
 def test_train_step_teacher_forced(G, N, C, normalize):
     from longcontext_sqattn_paddle_amd.cache_hub.kmeans import _triton_k_means_train
 
