@@ -65,25 +65,35 @@ constexpr int kMaxShareBatch = 32;
 // then owns workgroups [base, base + n) and the same slots of the partial results, which are laid out [Hq, W] in this
 // mode.  The split kernel (want_b < 0: finds the owner of workgroup w) and the combine kernel (want_b = its sequence)
 // both call this, so they agree by construction.
+// Every wave computes the whole table at once, one sequence per lane (B <= 32): one load, an integer prefix sum by
+// shuffles (lengths in units of 32 tokens, so that 32 sequences of 2^31 tokens fit 32 bits; integer sums keep the prefix
+// monotone, which a float prefix formed in a different association per lane would not), one division per lane.  A loop
+// over the sequences with a load and a division in every round took longer than the rest of the combine kernel.
 __device__ __forceinline__ void share_of(const int32_t* seqlens, int B, int Lmax, int W, int want_b, int w, int& b, int& base, int& n) {
-  float total = 0.f;
-  for (int i = 0; i < B; ++i) total += (float)min(max(seqlens[i], 0), Lmax);
+  const int lane = threadIdx.x & 63;
+  const uint32_t len = lane < B ? ((uint32_t)min(max(seqlens[lane], 0), Lmax) + 31u) >> 5 : 0u;
+  uint32_t cum = len;   // inclusive prefix
+#pragma unroll
+  for (int d = 1; d < kMaxShareBatch; d <<= 1) {
+    const uint32_t v = __shfl_up(cum, d);
+    if (lane >= d) cum += v;
+  }
+  const uint32_t total = __shfl(cum, B - 1);
   const float spare = (float)(W - B);
-  float cum = 0.f;
-  int e0 = 0;
+  const int e1 = total > 0u ? (int)floorf(spare * ((float)cum / (float)total)) : 0;   // spare exactly for the last sequence
+  int e0 = __shfl_up(e1, 1);
+  if (lane == 0) e0 = 0;
+  const int bs = lane + e0, ni = 1 + e1 - e0;
+  const bool mine = lane < B && (want_b >= 0 ? lane == want_b : (w >= bs && w < bs + ni));
+  const unsigned long long mask = __ballot(mine);
   b = 0;
   base = 0;
   n = 1;
-  for (int i = 0; i < B; ++i) {
-    cum += (float)min(max(seqlens[i], 0), Lmax);
-    const int e1 = (total > 0.f) ? (int)floorf(spare * (cum / total)) : 0;
-    const int bs = i + e0, ni = 1 + e1 - e0;
-    if (want_b >= 0 ? (i == want_b) : (w >= bs && w < bs + ni)) {
-      b = i;
-      base = bs;
-      n = ni;
-    }
-    e0 = e1;
+  if (mask) {
+    const int src = __ffsll((long long)mask) - 1;
+    b = src;
+    base = __shfl(bs, src);
+    n = __shfl(ni, src);
   }
 }
 
@@ -136,7 +146,9 @@ __device__ __forceinline__ f32x4_t mfma_pv16(const i32x2_t& a, const i32x2_t& b,
 // GATHER: token t of the stream is cache row ids[b * Hkv + kvh][t] instead of row t (attention over a selection of
 // the cache, e.g. the tokens of the best-scoring k-means clusters); entries that are negative or beyond the cache
 // are skipped.
-template <bool BF16, bool GATHER>
+// BYLEN: the workgroups of a ragged batch dealt by length (share_of); a template parameter so that the code of the other launches
+// is the code without it.
+template <bool BF16, bool GATHER, bool BYLEN>
 __global__ __launch_bounds__(kWaves * 64) void decode_splitkv_kernel(DecodeArgs a) {
   __shared__ float s_o[kWaves][16][kOStride];
   __shared__ float s_m[kWaves][16];
@@ -147,7 +159,7 @@ __global__ __launch_bounds__(kWaves * 64) void decode_splitkv_kernel(DecodeArgs 
   int split = blockIdx.x, b = blockIdx.z, nsp = a.num_splits;
   int64_t slot_stride = a.num_splits;     // partial rows: (b * Hq + hq) * num_splits + split, or hq * W + workgroup
   int64_t slot0 = (int64_t)b * a.Hq * a.num_splits + split;
-  if (a.by_length) {
+  if constexpr (BYLEN) {
     const int W = a.B * a.num_splits, w = (int)blockIdx.z * a.num_splits + (int)blockIdx.x;
     int base;
     share_of(a.seqlens, a.B, a.L, W, -1, w, b, base, nsp);
@@ -621,13 +633,19 @@ static int decode_impl(const DLTensor* q, const DLTensor* kcache, const DLTensor
   SQ_HIP(hipGetDevice(&cur));
   SQ_REQUIRE(cur == dev, SQ_EDEVICE, "sq_decode_fwd: tensors live on device %d but the current device is %d", dev, cur);
   const dim3 grid((unsigned)S, (unsigned)(Hkv / a.hpw * a.head_chunks), (unsigned)B);
+#define SQ_LAUNCH_DECODE(BF, GA)                                                                                        \
+  do {                                                                                                                 \
+    if (a.by_length) hipLaunchKernelGGL((decode_splitkv_kernel<BF, GA, true>), grid, dim3(kWaves * 64), 0, st, a);     \
+    else hipLaunchKernelGGL((decode_splitkv_kernel<BF, GA, false>), grid, dim3(kWaves * 64), 0, st, a);                \
+  } while (0)
   if (token_ids) {
-    if (dt == DType::BF16) hipLaunchKernelGGL((decode_splitkv_kernel<true, true>), grid, dim3(kWaves * 64), 0, st, a);
-    else hipLaunchKernelGGL((decode_splitkv_kernel<false, true>), grid, dim3(kWaves * 64), 0, st, a);
+    if (dt == DType::BF16) SQ_LAUNCH_DECODE(true, true);
+    else SQ_LAUNCH_DECODE(false, true);
   } else {
-    if (dt == DType::BF16) hipLaunchKernelGGL((decode_splitkv_kernel<true, false>), grid, dim3(kWaves * 64), 0, st, a);
-    else hipLaunchKernelGGL((decode_splitkv_kernel<false, false>), grid, dim3(kWaves * 64), 0, st, a);
+    if (dt == DType::BF16) SQ_LAUNCH_DECODE(true, false);
+    else SQ_LAUNCH_DECODE(false, false);
   }
+#undef SQ_LAUNCH_DECODE
   SQ_HIP(hipGetLastError());
   CombineArgs c;
   c.part_o = a.part_o;
