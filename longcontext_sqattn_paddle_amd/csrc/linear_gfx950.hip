@@ -146,6 +146,39 @@ __global__ __launch_bounds__(kLinMaxWaves * 64) void linear_rows_kernel(LinArgs 
 #pragma unroll
   for (int i = 0; i < R * M; ++i) acc[i] = 0.f;
 
+  // What the epilogue adds to or multiplies with the result does not depend on the result: the bias, the residual, the
+  // row's position with its cos / sin pair, the cache row's number.  Requested here, they arrive during the main loop;
+  // requested in the epilogue they were two dependent round trips at the end of a kernel that is a few microseconds long.
+  constexpr int V = R * M;
+  const int idx = lane & (V - 1);
+  const int r = idx / M, m = idx % M;
+  const int64_t col = feat0 + r % RO;
+  const bool row_ok = live && lane < V && m < a.rows;
+  float pf_bias = 0.f, pf_res = 0.f, pf_cs = 0.f, pf_sn = 0.f;
+  int pf_row = -1;
+  if constexpr (GATED) {
+    const int64_t f = (col < n_out ? col : (int64_t)n_out - 1) + (r >= RO ? n_out : 0);
+    if (a.bias && live) pf_bias = ld16<BF16>(a.bias + f * 2);
+  } else if constexpr (ROPE) {
+    const int64_t f = rope_f[r] < a.n ? rope_f[r] : (int64_t)a.n - 1;
+    if (a.bias && live) pf_bias = ld16<BF16>(a.bias + f * 2);
+    if (row_ok) {
+      if (paired && lane < M) {
+        int64_t p = a.pos_is_i64 ? ((const int64_t*)a.pos)[m] : (int64_t)((const int32_t*)a.pos)[m];
+        p = p < 0 ? 0 : (p >= a.max_pos ? a.max_pos - 1 : p);
+        const float* trow = a.table + p * a.head_dim;
+        pf_cs = trow[rope_i];
+        pf_sn = trow[a.head_dim / 2 + rope_i];
+      }
+      if (a.k_cache) pf_row = a.valid_length[m];
+    }
+  } else {
+    if (row_ok && col < a.n) {
+      if (a.bias) pf_bias = ld16<BF16>(a.bias + col * 2);
+      if (a.res) pf_res = ld16<BF16>(a.res + m * a.r_sr + col * 2);
+    }
+  }
+
   for (int k0 = 0; k0 < a.k; k0 += kLinChunk) {
     const int chunks = ((a.k - k0 < kLinChunk) ? (a.k - k0) : kLinChunk) / 8;
     u32x4_t wv[R][U];
@@ -281,7 +314,6 @@ __global__ __launch_bounds__(kLinMaxWaves * 64) void linear_rows_kernel(LinArgs 
   // Fold the 64 lanes.  While more than one value is left, a step over lane bit s halves the list: a lane keeps the
   // even or the odd entry of each pair (by its bit s) and receives the partner's partial sum of that entry.  After
   // log2(V) steps lane l holds entry (l mod V), summed over the low lane bits; plain butterflies finish the rest.
-  constexpr int V = R * M;
   int width = V, s = 0;
 #pragma unroll
   for (; (1 << s) < V; ++s) {
@@ -297,27 +329,19 @@ __global__ __launch_bounds__(kLinMaxWaves * 64) void linear_rows_kernel(LinArgs 
 #pragma unroll
   for (; s < 6; ++s) acc[0] += __shfl_xor(acc[0], 1 << s);
 
-  const int idx = lane & (V - 1);
-  const int r = idx / M, m = idx % M;
-  const int64_t col = feat0 + r % RO;
   float v = acc[0];
   if constexpr (GATED) {
-    const int64_t f = (col < n_out ? col : (int64_t)n_out - 1) + (r >= RO ? n_out : 0);
-    if (a.bias) v += ld16<BF16>(a.bias + f * 2);
+    if (a.bias) v += pf_bias;
     v = rnd16<BF16>(v);                                    // the projection's own rounding
     const float up = __shfl(v, (lane + RO * M) & 63);      // lane idx + (R/2) M holds the pair's second half for the same row
     if (lane < RO * M && col < n_out && m < a.rows) *(uint16_t*)(a.y + m * a.y_sr + col * 2) = st16<BF16>(silu_mul_elem<BF16>(v, up));
   } else if constexpr (ROPE) {
-    const int64_t f = rope_f[r] < a.n ? rope_f[r] : (int64_t)a.n - 1;
-    if (a.bias) v += ld16<BF16>(a.bias + f * 2);
+    if (a.bias) v += pf_bias;
     v = rnd16<BF16>(v);                                   // the projection's own rounding
     const float second = __shfl(v, (lane + M) & 63);      // lane idx + M holds feature rope_f[1] of the same row
     if (paired) {
       if (lane < M && m < a.rows) {
-        int64_t p = a.pos_is_i64 ? ((const int64_t*)a.pos)[m] : (int64_t)((const int32_t*)a.pos)[m];
-        p = p < 0 ? 0 : (p >= a.max_pos ? a.max_pos - 1 : p);
-        const float* row = a.table + p * a.head_dim;
-        const float cs = row[rope_i], sn = row[a.head_dim / 2 + rope_i];
+        const float cs = pf_cs, sn = pf_sn;
         float o1, o2;
         {
           // separate fp32 products and sums, as the stand-alone rotary pass forms them
@@ -330,7 +354,7 @@ __global__ __launch_bounds__(kLinMaxWaves * 64) void linear_rows_kernel(LinArgs 
         *(uint16_t*)(a.y + m * a.y_sr + rope_f[0] * 2) = st16<BF16>(o1);
         *(uint16_t*)(a.y + m * a.y_sr + rope_f[1] * 2) = st16<BF16>(o2);
         if (a.k_cache && rope_f[0] >= a.q_features) {   // a pair of a k head: its place in the new cache row
-          const int row = a.valid_length[m];
+          const int row = pf_row;
           if (row >= 0 && row < a.max_length) {          // (a full sequence stays as it is, as in the append pass)
             char* dst = a.k_cache + m * a.cache_sb + ((int64_t)row * a.kv_features - a.q_features) * 2;
             *(uint16_t*)(dst + rope_f[0] * 2) = st16<BF16>(o1);
@@ -341,7 +365,7 @@ __global__ __launch_bounds__(kLinMaxWaves * 64) void linear_rows_kernel(LinArgs 
     } else if (lane < V && rope_f[r] < a.n && m < a.rows) {
       *(uint16_t*)(a.y + m * a.y_sr + rope_f[r] * 2) = st16<BF16>(v);
       if (a.k_cache) {                                   // behind the rotated part: v
-        const int row = a.valid_length[m];
+        const int row = pf_row;
         if (row >= 0 && row < a.max_length)
           *(uint16_t*)(a.v_cache + m * a.cache_sb + ((int64_t)row * a.kv_features + rope_f[r] - a.rope_features) * 2) = st16<BF16>(v);
       }
@@ -352,8 +376,8 @@ __global__ __launch_bounds__(kLinMaxWaves * 64) void linear_rows_kernel(LinArgs 
     }
   } else {
     if (lane < V && col < a.n && m < a.rows) {
-      if (a.bias) v += ld16<BF16>(a.bias + col * 2);
-      if (a.res) v = rnd16<BF16>(v) + ld16<BF16>(a.res + m * a.r_sr + col * 2);
+      if (a.bias) v += pf_bias;
+      if (a.res) v = rnd16<BF16>(v) + pf_res;
       *(uint16_t*)(a.y + m * a.y_sr + col * 2) = st16<BF16>(v);
     }
   }
