@@ -627,6 +627,8 @@ def main():
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--seq-len", type=int, default=131072)
+    ap.add_argument("--settle", type=float, default=2.0,
+                    help="seconds of idle time before each leg after the headline one (they follow seconds of work at the power limit)")
     ap.add_argument("--p-quant", type=int, default=5,
                     help="0 none, 1 e4m3 static 448 exactly as the reference rounds it, 2 e4m3 block absmax, "
                          "3 e4m3 static 448 with the scale folded into the exponent, "
@@ -741,7 +743,17 @@ def main():
         log(f"[bench] plugin closure: {result['plugin']}")
     del qkv
     torch.cuda.empty_cache()
+
+    def settle():
+        # The prefill legs above run the matrix cores at the chip's power limit for several seconds; a leg measured
+        # right behind them inherits that state (the 1M-token decode reads 322 us then and 307 - 312 us from an idle
+        # chip).  Every leg below therefore starts after a short pause, like the headline leg, which starts the process.
+        torch.cuda.synchronize()
+        time.sleep(args.settle)
+
+    result["settle_s"] = args.settle
     if not args.no_decode:
+        settle()
         dec = {}
         for name, B, L in (("1M_b1", 1, 1048576), ("128K_b1", 1, 131072), ("128K_b4", 4, 131072), ("128K_b8", 8, 131072)):
             us, nbytes = time_decode(torch, B, L)
@@ -761,6 +773,7 @@ def main():
             torch.cuda.empty_cache()
         result["decode_selected"] = sel
     if not args.no_prepass:
+        settle()
         pre = {}
         for name, want4, skip_q in (("int8", False, False), ("int8_int4", True, False), ("int8_key_and_value_only", False, True)):
             us, nbytes = time_prepass(torch, N, want4, skip_query=skip_q)
@@ -770,6 +783,7 @@ def main():
             torch.cuda.empty_cache()
         result["plugin_prepass"] = pre
     if not args.no_kv_cache:
+        settle()
         sus, sbytes, aus = time_kv_cache(torch, N)
         result["kv_cache"] = {"store_us": round(sus, 1), "store_GB_per_s": round(sbytes / sus / 1e3, 1),
                               "store_frac_of_hbm_peak": round(sbytes / sus / 1e3 / PEAK_HBM_GBS, 4), "store_bytes": sbytes,
@@ -777,6 +791,7 @@ def main():
         log(f"[bench] kv cache: store of {N} tokens {sus:.0f} us ({sbytes / sus / 1e3:.0f} GB/s), append (batch 8) {aus:.1f} us")
         torch.cuda.empty_cache()
     if not args.no_layer:
+        settle()
         lay = {}
         for name, (us, nbytes) in time_layer_kernels(torch, N).items():
             lay[name] = {"us_per_call": round(us, 1), "GB_per_s": round(nbytes / us / 1e3, 1),
@@ -810,6 +825,7 @@ def main():
         result["e2e"] = [time_e2e(torch, N, new_tokens=args.e2e_new_tokens, graph=args.e2e_graph, **runs[r]) for r in args.e2e_runs.split(",")]
         log(f"[bench] end to end: {result['e2e']}")
     if not args.no_kmeans:
+        settle()
         us, kflops, kbytes, topk_us, full_ms = time_kmeans(torch)
         t_mfma, t_hbm = kflops / PEAK_MFMA_BF16_TFLOPS / 1e6, kbytes / PEAK_HBM_GBS / 1e3
         result["kmeans"] = {"us_per_iteration": round(us, 1), "TFLOP_per_s": round(kflops / us / 1e6, 1),
