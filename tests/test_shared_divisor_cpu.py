@@ -99,3 +99,34 @@ def test_float_quantiser_ranges():
             k, e = int(rng.integers(0, 2 ** mbits)), int(rng.integers(-6, 8))
             pairs.append((np.float32((1 + (k + 0.5) / 2 ** mbits) * 2.0 ** e * float(d)), d))
     _check(pairs)
+
+
+# ---- the integer counterpart: FastDiv (csrc/common.hpp) replaces x / d, d fixed per launch, by
+# ((x * m >> 32) + x) >> s with s = ceil(log2 d), m = ceil(2^(32+s) / d) - 2^32, for x < 2^31.  Replayed here in
+# Python integers (arbitrary precision), with the 32-bit wrap of the one addition the device code makes.
+def _make_fastdiv(d):
+    s = 0
+    while (1 << s) < d:
+        s += 1
+    m = ((1 << (32 + s)) + d - 1) // d - (1 << 32)
+    assert 0 <= m < (1 << 32), (d, m)
+    return m, s
+
+
+def _fastdiv(x, m, s):
+    return ((((x * m) >> 32) + x) & 0xFFFFFFFF) >> s
+
+
+def test_fastdiv_equals_integer_division_below_2_31():
+    rng = np.random.default_rng(7)
+    divisors = list(range(1, 70)) + [127, 128, 129, 448, 1000, 3584, 4608, 18944, 131072, 131073, 1048576, 2 ** 20 + 1,
+                                     2 ** 30 - 1, 2 ** 30, 2 ** 30 + 1, 2 ** 31 - 1] + [int(v) for v in rng.integers(1, 2 ** 31, 200)]
+    top = 2 ** 31 - 1
+    for d in divisors:
+        m, s = _make_fastdiv(d)
+        xs = {0, 1, d - 1, d, d + 1, top, top - 1, top - d, (top // d) * d, (top // d) * d - 1}
+        xs |= {int(k) * d + off for k in rng.integers(0, max(top // d, 1), 40) for off in (-1, 0, 1)}
+        xs |= {int(v) for v in rng.integers(0, top + 1, 200)}
+        for x in xs:
+            if 0 <= x <= top:
+                assert _fastdiv(x, m, s) == x // d, (x, d)
