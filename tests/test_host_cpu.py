@@ -138,3 +138,42 @@ def test_delayed_sdpa_wrapper_quantised_branch_matches_the_oracle():
     plain = delayed_sdpa_wrapper(0, 0, 0, 0, types.SimpleNamespace(quant=False))(None, q, k, v, None, tensor_layout="HND")
     want = torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True).transpose(1, 2).reshape(1, 48, 96)
     assert torch.allclose(plain, want, atol=1e-6)
+
+
+def test_decode_shares_by_length_add_up():
+    """The rule by which the decode kernels deal the W workgroups of a ragged batch to its sequences (csrc/decode_gfx950.hip,
+    share_of): every sequence one workgroup, the other W - B by cumulative rounding of (W - B) * prefix / total in fp32, the
+    lengths counted in units of 32 tokens.  Replayed in numpy float32: the shares are positive, add up to W exactly, never
+    exceed a sequence's proportional share by more than one, and follow the lengths."""
+    import numpy as np
+
+    rng = np.random.default_rng(11)
+    for case in range(300):
+        B = int(rng.integers(2, 33))
+        S = int(rng.integers(2, 129))
+        W = B * S
+        kind = case % 4
+        if kind == 0:
+            lens = rng.integers(0, 2 ** 31 - 1, B)
+        elif kind == 1:
+            lens = rng.integers(98304, 131073, B)
+        elif kind == 2:
+            lens = np.where(rng.random(B) < 0.5, 0, rng.integers(1, 5000, B))
+        else:
+            lens = np.full(B, int(rng.integers(1, 2 ** 20)))
+        units = (lens.astype(np.uint64) + 31) >> 5
+        cum = np.cumsum(units).astype(np.uint32)           # fits 32 bits: 32 sequences of 2^26 units
+        total = cum[-1]
+        spare = np.float32(W - B)
+        e1 = np.floor(spare * (cum.astype(np.float32) / np.float32(total))).astype(np.int64) if total > 0 else np.zeros(B, np.int64)
+        e0 = np.concatenate([[0], e1[:-1]])
+        n = 1 + e1 - e0
+        base = np.arange(B) + e0
+        assert (n >= 1).all()
+        if total > 0:
+            assert int(n.sum()) == W and int(base[-1] + n[-1]) == W
+            want = (W - B) * units.astype(np.float64) / float(total)
+            assert (np.abs((n - 1) - want) <= 1.0 + 1e-3 * (W - B)).all()
+        else:
+            assert (n == 1).all()
+        assert (base[1:] == base[:-1] + n[:-1]).all()
