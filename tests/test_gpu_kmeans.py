@@ -155,7 +155,7 @@ def test_topk_select_matches_oracle():
 
 def test_topk_select_shared_score_phase_repeated():
     """With 1024 clusters several workgroups share a head's score phase and the last to arrive finishes the selection,
-    handing the scores over through memory.  Two queries alternate over 120 calls; every call must reproduce its query's
+    handing the scores over through memory.  Two queries alternate over 1000 calls; every call must reproduce its query's
     oracle result exactly (a score that arrives late, or a counter that is not set back, would show)."""
     from longcontext_sqattn_paddle_amd.cache_hub.kmeans import _workspace, topk_select
 
@@ -171,7 +171,7 @@ def test_topk_select_shared_score_phase_repeated():
     dq = [q.to(DEV) for q in qs]
     dc, dcl, dsz = cent.to(DEV), clusters.to(DEV), size.to(DEV)
     ws = _workspace(G, 1, C, DEV)   # one workspace for all calls: a stale score would be the other query's
-    outs = [topk_select(dq[i % 2], dc, dcl, dsz, k, groups, workspace=ws) for i in range(120)]
+    outs = [topk_select(dq[i % 2], dc, dcl, dsz, k, groups, workspace=ws) for i in range(1000)]
     torch.cuda.synchronize()
     for i, o in enumerate(outs):
         assert torch.equal(o.cpu(), want[i % 2]), i
