@@ -91,7 +91,7 @@ def time_mfma_only(torch, qkv):
     from longcontext_sqattn_paddle_amd import _native as NV
 
     dev = qkv[1].device
-    lib = NV.lib()
+    lib = NV.probe_lib()
     nbytes = int(lib.sq_probe_mfma_operand_bytes())
     sink = torch.empty(131072, dtype=torch.float32, device=dev)
     k_words = qkv[1].reshape(-1)[:nbytes // 2].contiguous()
@@ -110,7 +110,7 @@ def time_mfma_only(torch, qkv):
         for rep in range(4):
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record(stream)
-            NV.check(lib.sq_probe_mfma_rate(kind, NV.ptr(b[0]), NV.ptr(b[1]), iters, NV.current_stream(dev)))
+            NV.check(lib.sq_probe_mfma_rate(kind, NV.ptr(b[0]), NV.ptr(b[1]), iters, NV.current_stream(dev)), lib)
             e1.record(stream)
             torch.cuda.synchronize()
             times.append(e0.elapsed_time(e1))

@@ -4,9 +4,8 @@
  * Every entry point takes borrowed DLPack tensors (device pointers, shapes, strides in elements), plain
  * scalars and a HIP stream handle (`hipStream_t` passed as `void*`, NULL = the null stream); it enqueues
  * work on that stream and returns without synchronising unless stated otherwise.  Nothing is retained
- * after the call returns; outputs and workspaces are allocated by the caller.  (Two pieces of device memory live
- * inside the library and say so where they are declared: the partials array of sq_decode_fwd_noalloc and the
- * arrival counters of sq_topk_select, which are zero again when a call has finished.)  Return value: SQ_OK or a
+ * after the call returns; outputs and workspaces are allocated by the caller.  (One piece of device memory lives
+ * inside the library and says so where it is declared: the partials array of sq_decode_fwd_noalloc.)  Return value: SQ_OK or a
  * negative SQ_E* code; `sq_last_error()` then holds a message (thread-local).  No entry point throws or
  * aborts.  Tensors must live on one ROCm device (DLPack device type kDLROCM, or kDLCUDA as some
  * PyTorch-ROCm builds report), have a contiguous last dimension and a 16-byte aligned base address.
@@ -19,6 +18,7 @@
  *   sq_fake_quant_prepass_int8qk  sqattn/attn_replacer.py:338-339, 361-365 for that path (key codes and scales, v8)
  *   sq_decode_fwd             sqattn/attn_triton_decode.py:244-361 (decode launch :293-324)
  *   sq_decode_fwd_noalloc     no reference counterpart: sq_decode_fwd for callers that cannot allocate device memory
+ *   sq_decode_noalloc_init    no reference counterpart: its one-off set-up, for callers that record HIP graphs
  *   sq_decode_selected_fwd    no reference counterpart: the same decode over the tokens sq_topk_select picked
  *   sq_kmeans_train           cache_hub/kmeans.py:127-196 (assign launch :147-173, update launch :175-193)
  *   sq_reverse_index          cache_hub/kmeans.py:233-262
@@ -39,7 +39,6 @@
  *   sq_rmsnorm_linear_rows, sq_rmsnorm_linear_rows_silu_and_mul, sq_rmsnorm_linear_rows_rope
  *                             the three forms above together with the RMS norm in front of them: model_hub/LLM.py:92-93 + :95
  *                             (input_layernorm, wqkv), :110-114 (post_attention_layernorm, mlp), :161-163 (norm, lm)
- *   sq_probe_mfma_rate        no reference counterpart: measurement aid (the rate of a loop of nothing but MFMAs on given operands)
  *   sq_fake_quant_prepass_typed  the same with the float quantiser types of sqattn/attn_replacer.py:340-358
  *   sq_fake_quant_prepass     sqattn/attn_replacer.py:334-365 (GQA expand, key centring and the five fake-quant
  *                             passes of mp_triton_wrapper's closure), sqattn/fake_quant.py:24-58, 98-125
@@ -56,7 +55,7 @@
 extern "C" {
 #endif
 
-#define SQ_ABI_VERSION 2
+#define SQ_ABI_VERSION 3
 
 enum {
   SQ_OK = 0,
@@ -172,11 +171,14 @@ int sq_decode_fwd(const DLTensor* q, const DLTensor* kcache, const DLTensor* vca
  * (sq_decode_noalloc_scratch_bytes() = 8 MiB per GPU, held until the process ends) instead of a caller workspace; the
  * kernels and the results are those of sq_decode_fwd with the same num_splits, bit for bit.  A call whose partials
  * (batch * q heads * splits * 516 bytes) exceed the array returns SQ_EWORKSPACE.  q's device must be the current
- * device.  The call allocates and frees nothing (the first call on a device looks the array's address up).  All calls
- * on one GPU share that GPU's array: calls that overlap in time on one GPU (different streams, or threads) race;
- * order them on one stream or with events.
+ * device.  The call allocates and frees nothing.  The first use on a device looks the array's address up, which may
+ * load the library's code object: call sq_decode_noalloc_init() once per device (with that device current) before
+ * recording a HIP graph that contains sq_decode_fwd_noalloc; without it the first sq_decode_fwd_noalloc call does the
+ * look-up itself.  All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (different
+ * streams, or threads) race; order them on one stream or with events.
  */
 size_t sq_decode_noalloc_scratch_bytes(void);
+int sq_decode_noalloc_init(void);
 int sq_decode_fwd_noalloc(const DLTensor* q, const DLTensor* kcache, const DLTensor* vcache, const DLTensor* seqlens,
                           DLTensor* out, DLTensor* lse, const sq_decode_params* params, void* stream);
 
@@ -216,10 +218,10 @@ int sq_index_add(const DLTensor* value, const DLTensor* idx, DLTensor* out, DLTe
  * max_{h in group} <query[b,h], centroids[g,c]> (ties -> lower c); whole clusters taken in rank order
  * until k tokens are emitted; missing tail = -1.  query bf16 [B,Hq,D]; out int32 [G,k], rows contiguous and at least
  * k apart (it may be the leading columns of a wider list that sq_decode_selected_fwd reads).
- * With 1024 clusters the workgroups of a group share its score phase and hand over through one arrival counter per
- * group index g, kept in a device array inside the library (zero between calls: the last arriver sets it back).  Two
- * calls that overlap in time on one GPU and use the same g would share that counter: order such calls on one stream
- * or with events.
+ * With 1024 clusters the workgroups of a group share its score phase and hand over through one arrival word per
+ * group in the workspace.  The workspace needs no initialisation (any contents are fine) and may be shared with the
+ * other k-means entry points; calls that overlap in time must use different workspaces, as for every entry point
+ * that takes one.
  */
 int sq_topk_select(const DLTensor* query, const DLTensor* centroids, const DLTensor* clusters,
                    const DLTensor* cluster_size, DLTensor* out, DLTensor* workspace, int32_t num_kv_groups,
@@ -413,19 +415,6 @@ typedef struct sq_histogram_params {
   float softmax_scale;  /* 1/sqrt(head_dim before padding) (attn_replacer.py:260)            */
 } sq_histogram_params;
 int sq_attention_histogram(const DLTensor* q, const DLTensor* k, DLTensor* hist, const sq_histogram_params* p, void* stream);
-
-/*
- * Measurement aid, no counterpart in the reference: runs a kernel that issues nothing but MFMAs -- one workgroup of
- * eight waves on each of 256 CUs, `iters` x 16 instructions per wave on four accumulators, kind 0 =
- * v_mfma_f32_32x32x16_bf16, kind 1 = v_mfma_f32_32x32x64_f8f6f4 on e4m3 -- with operand registers loaded once from
- * `operands` (any dtype, at least sq_probe_mfma_operand_bytes() bytes: 64 bytes per lane and operand set, four sets per
- * lane).  The time of the launch, taken by the caller, and sq_probe_mfma_flops(kind, iters) give the rate the matrix
- * cores sustain on such operands: with constant operands the published peak, with random ones about a quarter less
- * (the chip lowers its clock).  sink: fp32, at least 131072 elements, receives the accumulators' sums.
- */
-size_t sq_probe_mfma_operand_bytes(void);
-int64_t sq_probe_mfma_flops(int32_t kind, int32_t iters);
-int sq_probe_mfma_rate(int32_t kind, const DLTensor* operands, DLTensor* sink, int32_t iters, void* stream);
 
 #ifdef __cplusplus
 }

@@ -14,6 +14,7 @@ import torch
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG_DIR, "libsqattn_hip.so")
 
+ABI_VERSION = 3   # SQ_ABI_VERSION of include/sqattn.h
 SQ_OK, SQ_EINVAL, SQ_ESHAPE, SQ_EDEVICE, SQ_EDTYPE, SQ_EUNSUPPORTED, SQ_EHIP, SQ_EWORKSPACE = 0, -1, -2, -3, -4, -5, -6, -7
 LAYOUT = {"HND": 0, "NHD": 1}
 P_NONE, P_E4M3_STATIC, P_E4M3_BLOCK, P_E4M3_STATIC_FAST, P_E4M3_FP8_PV, P_E4M3_MX_FP8_PV = 0, 1, 2, 3, 4, 5
@@ -89,6 +90,7 @@ SYMBOLS = {
     "sq_decode_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int32]),
     "sq_decode_fwd": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, _P, ctypes.POINTER(DecodeParams), ctypes.c_void_p]),
     "sq_decode_noalloc_scratch_bytes": (ctypes.c_size_t, []),
+    "sq_decode_noalloc_init": (ctypes.c_int, []),
     "sq_decode_fwd_noalloc": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, ctypes.POINTER(DecodeParams), ctypes.c_void_p]),
     "sq_decode_selected_fwd": (ctypes.c_int, [_P] * 8 + [ctypes.POINTER(DecodeParams), ctypes.c_void_p]),
     "sq_kmeans_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int64] * 4),
@@ -110,16 +112,23 @@ SYMBOLS = {
     "sq_rmsnorm_linear_rows_rope": (ctypes.c_int, [_P, _P, ctypes.c_float] + [_P] * 4 + [ctypes.c_int32, ctypes.c_int32] + [_P] * 5 + [ctypes.c_void_p]),
     "sq_prefill_int8qk_fwd": (ctypes.c_int, [_P] * 7 + [ctypes.POINTER(PrefillParams), ctypes.c_void_p]),
     "sq_fake_quant_prepass_int8qk": (ctypes.c_int, [_P] * 7 + [ctypes.c_int32, ctypes.c_void_p]),
-    "sq_probe_mfma_operand_bytes": (ctypes.c_size_t, []),
-    "sq_probe_mfma_flops": (ctypes.c_int64, [ctypes.c_int32, ctypes.c_int32]),
-    "sq_probe_mfma_rate": (ctypes.c_int, [ctypes.c_int32, _P, _P, ctypes.c_int32, ctypes.c_void_p]),
     "sq_kv_cache_store": (ctypes.c_int, [_P] * 4 + [ctypes.c_int32, ctypes.c_int64, ctypes.c_void_p]),
     "sq_kv_cache_append": (ctypes.c_int, [_P] * 6 + [ctypes.c_int32, ctypes.c_void_p]),
     "sq_kv_cache_reorder": (ctypes.c_int, [_P] * 5 + [ctypes.c_void_p]),
     "sq_attention_histogram": (ctypes.c_int, [_P, _P, _P, ctypes.POINTER(HistogramParams), ctypes.c_void_p]),
 }
 
+# libsqattn_probe.so: a measurement aid (the rate of a loop of nothing but MFMAs), not part of the product's C ABI
+PROBE_LIB_PATH = os.path.join(_PKG_DIR, "libsqattn_probe.so")
+PROBE_SYMBOLS = {
+    "sq_last_error": (ctypes.c_char_p, []),
+    "sq_probe_mfma_operand_bytes": (ctypes.c_size_t, []),
+    "sq_probe_mfma_flops": (ctypes.c_int64, [ctypes.c_int32, ctypes.c_int32]),
+    "sq_probe_mfma_rate": (ctypes.c_int, [ctypes.c_int32, _P, _P, ctypes.c_int32, ctypes.c_void_p]),
+}
+
 _lib: Optional[ctypes.CDLL] = None
+_probe_lib: Optional[ctypes.CDLL] = None
 
 
 def lib() -> ctypes.CDLL:
@@ -135,10 +144,25 @@ def lib() -> ctypes.CDLL:
             fn = getattr(handle, name)
             fn.restype = res
             fn.argtypes = args
-        if handle.sq_abi_version() != 2:
+        if handle.sq_abi_version() != ABI_VERSION:
             raise RuntimeError("libsqattn_hip.so ABI version mismatch")
         _lib = handle
     return _lib
+
+
+def probe_lib() -> ctypes.CDLL:
+    """The measurement-aid library (bench.py and its test); errors of its calls go through `check(code, probe_lib())`."""
+    global _probe_lib
+    if _probe_lib is None:
+        if not os.path.exists(PROBE_LIB_PATH):
+            raise RuntimeError(f"{PROBE_LIB_PATH} is missing: build it with `python -m longcontext_sqattn_paddle_amd.build`")
+        handle = ctypes.CDLL(PROBE_LIB_PATH)
+        for name, (res, args) in PROBE_SYMBOLS.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _probe_lib = handle
+    return _probe_lib
 
 
 _capsule_ptr = ctypes.pythonapi.PyCapsule_GetPointer
@@ -168,11 +192,11 @@ def ptr(b: Optional[Borrowed]):
     return None if b is None else b.ptr
 
 
-def check(code: int) -> None:
+def check(code: int, library: Optional[ctypes.CDLL] = None) -> None:
     """Map a library error code to the exception type the reference raises for the same mistake."""
     if code == SQ_OK:
         return
-    msg = lib().sq_last_error().decode("utf-8", "replace")
+    msg = (library or lib()).sq_last_error().decode("utf-8", "replace")
     if code in (SQ_EINVAL, SQ_EUNSUPPORTED, SQ_EDTYPE):
         raise ValueError(msg)
     if code == SQ_ESHAPE:

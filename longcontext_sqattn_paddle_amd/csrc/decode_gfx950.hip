@@ -12,9 +12,10 @@
 //   S^T[token, head] = K . Q~^T  on v_mfma_f32_16x16x32 (bf16/f16 in, fp32 acc); Q~ (16 padded heads) lives
 //        in registers as the B operand; lane (r,g) ends up with head r, tokens n0+4g+i, i<4.
 //   V : 4 x 16-byte loads per lane, load i reads V[n0+4g+i][8r .. 8r+7] (full 256-byte rows per 16 lanes)
-//   O^T[d, head] += V^T . P^T  on v_mfma_f32_16x16x4_f32 with k = the 4 lane groups g: the A operand is
-//        the fp32 value of one loaded V element, the B operand is the lane's own p -- no transposition,
-//        no LDS, products in fp32 exactly as the reference's `p * v.to(float32)` (:234).
+//   O^T[d, head] += V^T . P^T  on v_mfma_f32_16x16x16 of the tensor dtype with k = the tile's 16 tokens: the A operand is
+//        eight channels of the lane's four V rows (two v_perm_b32 per channel offset), the B operand the lane's own p as
+//        hi + lo (p rounded to the tensor dtype plus the rounded remainder, relative error 2^-16 for bf16) -- no
+//        transposition, no LDS, V exact, standing in for the reference's fp32 `p * v.to(float32)` (:234).
 #include <mutex>
 
 #include "common.hpp"
@@ -66,9 +67,9 @@ constexpr int kMaxShareBatch = 32;
 // mode.  The split kernel (want_b < 0: finds the owner of workgroup w) and the combine kernel (want_b = its sequence)
 // both call this, so they agree by construction.
 // Every wave computes the whole table at once, one sequence per lane (B <= 32): one load, an integer prefix sum by
-// shuffles (lengths in units of 32 tokens, so that 32 sequences of 2^31 tokens fit 32 bits; integer sums keep the prefix
-// monotone, which a float prefix formed in a different association per lane would not), one division per lane.  A loop
-// over the sequences with a load and a division in every round took longer than the rest of the combine kernel.
+// shuffles (lengths in units of 32 tokens, so that 32 sequences of 2^31 tokens fit 32 bits), one 64-bit integer
+// division per lane -- exact arithmetic, so the two kernels cannot disagree whatever flags they are compiled with.  A
+// loop over the sequences with a load and a division in every round took longer than the rest of the combine kernel.
 __device__ __forceinline__ void share_of(const int32_t* seqlens, int B, int Lmax, int W, int want_b, int w, int& b, int& base, int& n) {
   const int lane = threadIdx.x & 63;
   const uint32_t len = lane < B ? ((uint32_t)min(max(seqlens[lane], 0), Lmax) + 31u) >> 5 : 0u;
@@ -79,8 +80,7 @@ __device__ __forceinline__ void share_of(const int32_t* seqlens, int B, int Lmax
     if (lane >= d) cum += v;
   }
   const uint32_t total = __shfl(cum, B - 1);
-  const float spare = (float)(W - B);
-  const int e1 = total > 0u ? (int)floorf(spare * ((float)cum / (float)total)) : 0;   // spare exactly for the last sequence
+  const int e1 = total > 0u ? (int)((uint64_t)(uint32_t)(W - B) * cum / total) : 0;   // W - B exactly for the last sequence
   int e0 = __shfl_up(e1, 1);
   if (lane == 0) e0 = 0;
   const int bs = lane + e0, ni = 1 + e1 - e0;
@@ -683,26 +683,39 @@ extern "C" int sq_decode_selected_fwd(const DLTensor* q, const DLTensor* kcache,
 
 extern "C" size_t sq_decode_noalloc_scratch_bytes(void) { return kNoAllocScratchBytes; }
 
+// The device address of `scratch` on the current device, looked up once per device (every GPU holds its own copy of the
+// array at its own address).  The look-up may load the library's code object on first use, so a caller that records
+// HIP graphs runs it beforehand (sq_decode_noalloc_init); afterwards it is a table read.
+static int noalloc_scratch(int dev, void** out) {
+  SQ_REQUIRE(dev >= 0 && dev < kMaxDevices, SQ_EDEVICE, "sq_decode_fwd_noalloc: device id %d out of range", dev);
+  std::lock_guard<std::mutex> guard(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    SQ_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    SQ_REQUIRE(p, SQ_EHIP, "sq_decode_fwd_noalloc: hipGetSymbolAddress returned a null address");
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return SQ_OK;
+}
+
+extern "C" int sq_decode_noalloc_init(void) {
+  int cur = -1;
+  SQ_HIP(hipGetDevice(&cur));
+  void* ptr;
+  return noalloc_scratch(cur, &ptr);
+}
+
 extern "C" int sq_decode_fwd_noalloc(const DLTensor* q, const DLTensor* kcache, const DLTensor* vcache, const DLTensor* seqlens,
                                      DLTensor* out, DLTensor* lse, const sq_decode_params* params, void* stream) {
   SQ_REQUIRE(q, SQ_EINVAL, "sq_decode_fwd_noalloc: q is null");
   SQ_REQUIRE(on_gpu(q), SQ_EDEVICE, "sq_decode_fwd_noalloc: q is not on a ROCm device");
   const int dev = q->device.device_id;
-  SQ_REQUIRE(dev >= 0 && dev < kMaxDevices, SQ_EDEVICE, "sq_decode_fwd_noalloc: device id %d out of range", dev);
   int cur = -1;
   SQ_HIP(hipGetDevice(&cur));
   SQ_REQUIRE(cur == dev, SQ_EDEVICE, "sq_decode_fwd_noalloc: tensors live on device %d but the current device is %d", dev, cur);
   void* ptr;
-  {
-    // every GPU holds its own copy of the array at its own address: looked up once per device, with that device current
-    std::lock_guard<std::mutex> guard(g_scratch_mutex);
-    if (!g_scratch_ptr[dev]) {
-      void* p = nullptr;
-      SQ_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
-      SQ_REQUIRE(p, SQ_EHIP, "sq_decode_fwd_noalloc: hipGetSymbolAddress returned a null address");
-      g_scratch_ptr[dev] = p;
-    }
-    ptr = g_scratch_ptr[dev];
-  }
+  int rc = noalloc_scratch(dev, &ptr);
+  if (rc) return rc;
   return decode_impl(q, kcache, vcache, seqlens, nullptr, out, lse, nullptr, params, stream, ptr, kNoAllocScratchBytes);
 }

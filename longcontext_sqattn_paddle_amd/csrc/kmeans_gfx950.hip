@@ -296,10 +296,7 @@ __global__ __launch_bounds__(kTileTok) void sort_scatter_kernel(SortArgs a) {
 // (tile, cluster) range of kHeavy tokens or more is summed right here, in fp64, into rec[tile][start / kHeavy][128]
 // (ranges that long cannot share a block of kHeavy positions, so the slot is unique), and the cluster's workgroup adds
 // the records instead of the rows.
-#ifndef SQ_KM_BIG_TOK
-#define SQ_KM_BIG_TOK 2
-#endif
-constexpr int kBigTok = SQ_KM_BIG_TOK;          // tokens per thread
+constexpr int kBigTok = 2;          // tokens per thread
 constexpr int kBigTile = 1024 * kBigTok;        // tokens per workgroup
 constexpr int kHeavy = 64;                      // tokens of one cluster in one tile from which the tile sums them itself
 constexpr int kSlots = kBigTile / kHeavy;
@@ -446,11 +443,8 @@ struct SumArgs {
   int32_t N, C, nT, mode; // mode 0: plain sum cast to bf16; 1: mean; 2: mean + L2 normalise (1,2: only where cnt > 0)
 };
 
-#ifndef SQ_KM_LIST
-#define SQ_KM_LIST 2048
-#endif
 constexpr int kSumRows = 4;   // rows in flight per thread (8: slower, 2: the same)
-constexpr int kListCap = SQ_KM_LIST;   // token ids staged in LDS at a time
+constexpr int kListCap = 2048;   // token ids staged in LDS at a time
 
 __global__ __launch_bounds__(256) void cluster_sum_kernel(SumArgs a) {
   __shared__ double red[4][kD];
@@ -562,7 +556,8 @@ struct TopkArgs {
   int32_t* out;            // [G,k], rows out_sg apart
   int64_t out_sg;
   float* score;            // workspace [G,C]
-  int32_t* start;          // workspace [G,C] start position of each cluster in rank order
+  int32_t* start;          // workspace [G,C] start position of each cluster in rank order (two-kernel path)
+  uint32_t* arrive;        // workspace [G] arrival words of the shared score phase (one-launch path; same memory as `start`)
   int64_t q_sb, q_sh, c_sg, c_sc, cl_sg, cl_sc;
   int32_t C, M, k, Hkv, group;
 };
@@ -742,16 +737,27 @@ __device__ __forceinline__ void find_pivot(const int32_t* hw, int need, int lane
 }
 
 // The score phase pulls a head's whole centroid matrix (256 KB at 1024 clusters) through the one CU its workgroup runs
-// on, which is most of that phase's time.  With SQ_TOPK_PARTS workgroups per (sequence, kv head), each scores its share
-// of the clusters into the workspace, and the one that arrives last (a counter per head in a library-owned array that
-// is zero when the library is loaded and that the last arriver sets back) carries on alone with steps 2 - 4.  Nobody
-// waits for anybody.  Calls that overlap on one GPU for the same head index would share the counters: do not overlap them.
-#ifndef SQ_TOPK_PARTS
-#define SQ_TOPK_PARTS 4
-#endif
-constexpr int kTopkParts = SQ_TOPK_PARTS;   // divides 16: every part gets whole waves of 64 clusters
-constexpr int kTopkMaxGroups = 4096;
-__device__ int32_t topk_arrivals[kTopkMaxGroups];
+// on, which is most of that phase's time.  With kTopkParts workgroups per (sequence, kv head), each scores its share
+// of the clusters into the workspace, and the one that arrives last carries on alone with steps 2 - 4.  Nobody waits
+// for anybody.
+//
+// The arrival counter of a head is a word in the caller's workspace, so calls that use different workspaces never meet.
+// It needs no initialisation and no reset: the word counts as "k workgroups have arrived" only while it reads
+// kArriveTag | k with 0 < k < parts; anything else -- whatever the memory held before, or the kArriveTag | parts a
+// finished call leaves behind -- counts as zero.  (Only a call that was cut short between two arrivals could leave a
+// live count behind; a launch that dies half-way takes the process's GPU context with it.)
+//
+// Ordering of the hand-over, step by step:
+//   1. every wave that stored scores waits for its own stores to be acknowledged (s_waitcnt vmcnt(0)): they are then
+//      in this XCD's L2, not somewhere between the wave and the L2;
+//   2. the workgroup barrier puts all of that before thread 0's next instruction;
+//   3. thread 0's device-scope fence writes the L2's dirty lines back, which covers every wave's scores of step 1,
+//      and orders them before its atomic on the counter (the atomic executes at device scope);
+//   4. the workgroup that reads parts - 1 earlier arrivals has thread 0 execute a device-scope fence after the atomic
+//      (acquire: stale lines of other XCDs' data leave its L2), then the barrier, and only then the scores are read,
+//      with device-scope loads that go past the CU's vector cache.
+constexpr int kTopkParts = 4;   // divides 16: every part gets whole waves of 64 clusters
+constexpr uint32_t kArriveTag = 0x5A70CB00u;   // low byte: number of arrivals so far
 
 __global__ __launch_bounds__(1024) void topk_select_kernel(TopkArgs a) {
   __shared__ float sc[1024];
@@ -804,12 +810,18 @@ __global__ __launch_bounds__(1024) void topk_select_kernel(TopkArgs a) {
     }
   }
   if (parts > 1) {
-    __syncthreads();
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // step 1: this wave's score stores have reached the L2
+    __syncthreads();                                    // step 2
     if (t == 0) {
-      __threadfence();                   // the workgroup's scores (ordered before this by the barrier) reach the device before it is counted
-      const int arrived = atomicAdd(&topk_arrivals[g], 1);
-      if (arrived == parts - 1) atomicExch(&topk_arrivals[g], 0);   // for the next call
-      misc[4] = arrived;
+      __threadfence();                                  // step 3
+      uint32_t* ctr = a.arrive + g;
+      uint32_t old = __hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT), before;
+      do {
+        before = ((old & ~0xffu) == kArriveTag && (old & 0xffu) < (uint32_t)parts) ? (old & 0xffu) : 0u;
+      } while (!__hip_atomic_compare_exchange_strong(ctr, &old, kArriveTag | (before + 1u), __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                                     __HIP_MEMORY_SCOPE_AGENT));
+      if ((int)before == parts - 1) __threadfence();    // step 4
+      misc[4] = (int)before;
     }
     __syncthreads();
     if (misc[4] != parts - 1) return;    // uniform: somebody else finishes the job
@@ -1192,6 +1204,7 @@ extern "C" int sq_topk_select(const DLTensor* query, const DLTensor* centroids, 
   a.out_sg = stride_of(out, 0);
   a.score = (float*)(wsp + w.off_bytes + w.hist_bytes + w.order_bytes);
   a.start = (int32_t*)(wsp + w.off_bytes + w.hist_bytes + w.order_bytes + w.score_bytes);
+  a.arrive = (uint32_t*)a.start;   // the one-launch path does not use `start`
   a.q_sb = stride_of(query, 0);
   a.q_sh = stride_of(query, 1);
   a.c_sg = stride_of(centroids, 0);
@@ -1204,7 +1217,7 @@ extern "C" int sq_topk_select(const DLTensor* query, const DLTensor* centroids, 
   a.Hkv = (int)Hkv;
   a.group = num_kv_groups;
   if (C <= 1024 && num_kv_groups <= 16) {   // one launch, only the clusters that can fill k are ordered
-    const unsigned parts = (G <= kTopkMaxGroups && C >= 64 * 16) ? kTopkParts : 1;   // fewer clusters: not worth sharing
+    const unsigned parts = (C >= 64 * 16) ? kTopkParts : 1;   // fewer clusters: not worth sharing
     hipLaunchKernelGGL(topk_select_kernel, dim3((unsigned)G, parts), dim3(1024), 0, st, a);
     SQ_HIP(hipGetLastError());
     return SQ_OK;

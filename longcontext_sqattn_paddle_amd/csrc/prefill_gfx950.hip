@@ -326,15 +326,6 @@ __device__ __forceinline__ float xor32_sum(float v) {
   return __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
 }
 
-#ifndef SQ_LDS_DEPTH
-#define SQ_LDS_DEPTH 4
-#endif
-#ifndef SQ_LDS_DEPTH_F16
-#define SQ_LDS_DEPTH_F16 2
-#endif
-#ifndef SQ_STATIC_RING
-#define SQ_STATIC_RING 1
-#endif
 constexpr float kLog2_448 = 8.807354922057604f;  // log2(448)
 
 // Quantise 8 probabilities (one k-step of the P.V MFMA) and pack them as fp16 B-operand registers.
@@ -677,7 +668,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
   const uint32_t kx0 = c32 * kKStride + ((g ^ ksw) << 4);
   // MODE 4 with the main loop unrolled over the four ring buffers: the LDS address of every fragment is a
   // per-lane constant plus an immediate offset, so the tile step spends no vector instruction on addresses
-  constexpr bool kStaticRing = SQ_STATIC_RING && !kPlain;
+  constexpr bool kStaticRing = !kPlain;
   uint32_t kxr[8];
 #pragma unroll
   for (int kk = 0; kk < 8; ++kk) kxr[kk] = smem_addr + (kx0 ^ (kk << 5));
@@ -768,7 +759,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
     const uint32_t klane = smem_addr + (((it + 1) & 3) * kKTileBytes) + kx0;
     u32x4_t kf[16];
     // K fragments are requested this many MFMA slots ahead (even, 2..8); the fp16 P.V modes have fewer registers to spare
-    constexpr int kDepth = kPV8 ? SQ_LDS_DEPTH : SQ_LDS_DEPTH_F16;
+    constexpr int kDepth = kPV8 ? 4 : 2;
     auto kread = [&](auto I) {
       constexpr int i = decltype(I)::value;
       if constexpr (kStaticRing) kf[i] = lds_read128<((R + 1) & 3) * kKTileBytes + (i & 1) * 32 * kKStride>(kxr[i >> 1]);

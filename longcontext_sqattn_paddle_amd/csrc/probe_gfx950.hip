@@ -9,6 +9,14 @@
 // 64 bytes once and then issues `iters` x 16 MFMAs on four accumulators: v_mfma_f32_32x32x16_bf16 (kind 0, a set = 16
 // bytes of A + 16 of B, the rest unused) or v_mfma_f32_32x32x64_f8f6f4 on e4m3 (kind 1, 32 bytes of A + 32 of B).  The
 // sums go to `sink` so that the loop cannot be removed; nothing else is written.
+//
+// Built into a library of its own, libsqattn_probe.so, next to the product library: it is loaded by the benchmark and
+// its test only and is not part of the C ABI a maintainer binds.  Entry points:
+//   size_t  sq_probe_mfma_operand_bytes(void)              bytes `operands` must hold (64 per lane and set, four sets per lane)
+//   int64_t sq_probe_mfma_flops(int32_t kind, int32_t iters)  floating-point operations of one launch
+//   int     sq_probe_mfma_rate(int32_t kind, const DLTensor* operands, DLTensor* sink, int32_t iters, void* stream)
+//           kind 0 = v_mfma_f32_32x32x16_bf16, 1 = v_mfma_f32_32x32x64_f8f6f4 on e4m3; sink: fp32, at least 131072 elements;
+//           iters at most kProbeMaxIters, which keeps one launch well under a second
 #include "common.hpp"
 
 namespace sq {
@@ -16,6 +24,7 @@ namespace {
 
 typedef __attribute__((ext_vector_type(8))) int i32x8_t;
 constexpr int kProbeGroups = 256, kProbeThreads = 512, kProbeSets = 4, kProbeSetBytes = 64;
+constexpr int kProbeMaxIters = 1 << 18;   // 4 M MFMAs per wave: about 0.15 s per launch
 
 template <int KIND>
 __global__ __launch_bounds__(kProbeThreads) void probe_mfma_kernel(const uint32_t* src, float* sink, int iters) {
@@ -46,7 +55,11 @@ __global__ __launch_bounds__(kProbeThreads) void probe_mfma_kernel(const uint32_
         asm volatile("v_mfma_f32_32x32x64_f8f6f4 %0, %1, %2, %0" : "+v"(acc[s & 3]) : "v"(a8[s & 3]), "v"(b8[(s >> 2) & 3]));
     }
   }
-  // (the accumulators are read by ordinary code: the compiler supplies the wait states after the last MFMA)
+  // The MFMAs above are opaque asm statements, so the compiler does not know that the matrix pipe is still writing the
+  // accumulators: the wait states between the last MFMA and the first read are supplied by hand (a 16-pass MFMA needs
+  // fewer than 32).
+#pragma unroll
+  for (int j = 0; j < 4; ++j) asm volatile("s_nop 15\n\ts_nop 15" : "+v"(acc[j]));
   float r = 0.f;
 #pragma unroll
   for (int j = 0; j < 4; ++j)
@@ -70,7 +83,7 @@ extern "C" int sq_probe_mfma_rate(int32_t kind, const DLTensor* operands, DLTens
   const char* fn = "sq_probe_mfma_rate";
   SQ_REQUIRE(kind == 0 || kind == 1, SQ_EINVAL, "%s: kind must be 0 (bf16 32x32x16) or 1 (e4m3 32x32x64), got %d", fn, (int)kind);
   SQ_REQUIRE(operands && sink, SQ_EINVAL, "%s: null tensor argument", fn);
-  SQ_REQUIRE(iters > 0 && iters <= (1 << 24), SQ_EINVAL, "%s: iters must be in 1 .. 2^24 (got %d)", fn, (int)iters);
+  SQ_REQUIRE(iters > 0 && iters <= kProbeMaxIters, SQ_EINVAL, "%s: iters must be in 1 .. %d (got %d)", fn, kProbeMaxIters, (int)iters);
   int rc;
   if ((rc = check_tensor(operands, "operands", 1, operands->device.device_id))) return rc;
   const int dev = operands->device.device_id;

@@ -89,19 +89,19 @@ def per_head(values, H: int, what: str) -> list:
 def align_windows(w8, w4, sink: int, block_m: int):
     """Window and sink sizes the kernels take, from arbitrary non-negative integers.
 
-    The reference's kernels walk 64-key blocks from range bounds they promise the compiler to be multiples of the query
-    block (`tl.multiple_of(lo, BLOCK_M)`, attn_triton_mix_bad.py:54, 66, 75): for sizes that are not multiples of 128 their
-    behaviour is undefined (taken literally, the block loop starts at an unaligned key and runs past the end of its
-    range, visiting keys of the next range twice).  Its relative entry point never produces such sizes: it rounds every
-    window up to a multiple of 128 (attn_triton_mix_relative.py:43-46).  This build applies that rule to absolute sizes
-    as well: windows are rounded up to the next multiple of 128, the sink up to the next multiple of 64.
+    The reference's kernels walk a range in 64-key blocks (`range(lo, hi, 64)`), so sizes that are multiples of 64 are
+    walked as written and pass through unchanged here (192 stays 192 under the 128-row query block of the absolute
+    variant too).  For sizes that are not multiples of 64 the reference has no defined behaviour (taken literally, the
+    block loop starts at an unaligned key and runs past the end of its range, visiting keys of the next range twice);
+    they are rounded up to the next multiple of 64, and so is the sink.  The relative entry point produces multiples of
+    128 by itself (attn_triton_mix_relative.py:43-46).
 
     A 4-bit window wider than an 8-bit window that is smaller than the query block makes the reference's 4-bit range
     run into the query block itself without the causal mask (it reads keys behind the query rows).  Here the 8-bit
     window is raised to the query block in that case: the 4-bit range then ends where the block starts, and the
     block's own keys are visited once, masked, as 8-bit operands."""
     up = lambda x, m: (int(x) + m - 1) // m * m
-    w8 = [up(x, 128) for x in w8]
-    w4 = [up(x, 128) for x in w4]
+    w8 = [up(x, 64) for x in w8]
+    w4 = [up(x, 64) for x in w4]
     w8 = [max(a, block_m) if b > a and a < block_m else a for a, b in zip(w8, w4)]
     return w8, w4, up(sink, 64)

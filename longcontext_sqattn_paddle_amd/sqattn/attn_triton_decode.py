@@ -146,7 +146,8 @@ def attn_unified(q, k, v, tensor_layout="HND", output_dtype=torch.float16, retur
         head_dim = q.size(-1)
         sm = torch.tensor(1.0 / head_dim ** 0.5 * 1.44269504, dtype=torch.float32, device=q.device)
         q_folded = (q.float() * sm).to(q.dtype).float()
-        k_mean = k.float().mean(dim=seq_dim)                                   # [B, Hkv, D]
+        # one pass over the keys in their own dtype with fp32 accumulation (no fp32 copy of the cache: 4 GB at 1M tokens)
+        k_mean = k.mean(dim=seq_dim, dtype=torch.float32)                      # [B, Hkv, D]
         qh = q_folded.squeeze(seq_dim)                                         # [B, Hq, D]
         groups = qh.size(1) // k_mean.size(1)
         shift = (qh.view(qh.size(0), k_mean.size(1), groups, head_dim) * k_mean[:, :, None, :]).sum(-1).reshape(lse.shape)

@@ -2,7 +2,7 @@
 
 Sink + hierarchical windows with absolute sizes (tokens), evaluated per 128-row query block; the 4-bit
 window range really uses `q_int4`/`k_int4` (:388-393).  Any non-negative window and sink sizes are accepted; sizes
-the reference's kernel has no defined behaviour for (not multiples of its blocks) are rounded up as
+the reference's kernel has no defined behaviour for (not multiples of its 64-key block) are rounded up as
 `_prefill.align_windows` states.
 """
 from __future__ import annotations

@@ -5,8 +5,10 @@ Followed reference code: model_hub/LLM.py:40-165 (`layer_prefill`, `layer_decode
 `layernorm`, `position_embedd`).  Built from the pinned pieces of this package: `layer.rmsnorm`, `layer.rope`,
 `layer.silu_and_mul`, `attention.exact_attention` (the reference's SDPA / flash attention stand-in), and torch's
 16-bit CPU `linear` for the projections (fp32 accumulation, one rounding; the GPU's GEMM accumulates in another
-order, which is what the tolerance of the model test covers).  Nothing here is new arithmetic, so the module has no
-pin of its own beyond a consistency check of prefill against token-by-token decoding.
+order, which is what the tolerance of the model test covers).  Nothing here is new arithmetic; the wiring (operator
+order, head mapping, halves of the rotary embedding and of the gated projection, the growing KV history) is pinned in
+tests/test_oracle_model.py: prefill at once equals token-by-token feeding, and both equal an independent float64
+transformer written out from the architecture (exactly, for float32 weights, where the rounding points are no-ops).
 """
 from __future__ import annotations
 

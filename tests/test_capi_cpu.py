@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(handle, n), f"{n} declared in include/sqattn.h but not exported"
     assert set(names) == set(N.SYMBOLS), "ctypes table and header disagree"
-    assert N.lib().sq_abi_version() == 2
+    assert N.lib().sq_abi_version() == 3
 
 
 def test_sizes_and_split_heuristic():

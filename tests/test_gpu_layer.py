@@ -439,27 +439,27 @@ def test_norm_in_front_hand_over_and_errors():
 
 
 def test_mfma_probe_runs_and_checks_its_arguments():
-    """sq_probe_mfma_rate (measurement aid): a launch on constant operands returns sums that are exact multiples of the
+    """sq_probe_mfma_rate (measurement aid, in its own library libsqattn_probe.so): a launch on constant operands returns sums that are exact multiples of the
     products it accumulates, and the argument checks hold."""
     from longcontext_sqattn_paddle_amd import _native as NV
 
-    lib = NV.lib()
+    lib = NV.probe_lib()
     nbytes = int(lib.sq_probe_mfma_operand_bytes())
     assert nbytes == 256 * 512 * 4 * 64 and int(lib.sq_probe_mfma_flops(0, 10)) == 256 * 8 * 10 * 16 * 32768
     assert int(lib.sq_probe_mfma_flops(1, 10)) == 4 * int(lib.sq_probe_mfma_flops(0, 10))
     ones = torch.ones(nbytes // 2, dtype=torch.bfloat16, device=DEV)
     sink = torch.zeros(131072, dtype=torch.float32, device=DEV)
     b = [NV.dl(ones), NV.dl(sink)]
-    NV.check(lib.sq_probe_mfma_rate(0, NV.ptr(b[0]), NV.ptr(b[1]), 3, NV.current_stream(sink.device)))
+    NV.check(lib.sq_probe_mfma_rate(0, NV.ptr(b[0]), NV.ptr(b[1]), 3, NV.current_stream(sink.device)), lib)
     torch.cuda.synchronize()
     # every MFMA adds 16 products of 1 x 1 to each of a lane's 16 accumulator entries: 3 x 16 MFMAs on 4 accumulators
     assert bool((sink == 3 * 16 * 16 * 16).all())
     e4 = torch.full((nbytes,), 0x38, dtype=torch.uint8, device=DEV)   # e4m3 1.0
     b = [NV.dl(e4), NV.dl(sink)]
-    NV.check(lib.sq_probe_mfma_rate(1, NV.ptr(b[0]), NV.ptr(b[1]), 2, NV.current_stream(sink.device)))
+    NV.check(lib.sq_probe_mfma_rate(1, NV.ptr(b[0]), NV.ptr(b[1]), 2, NV.current_stream(sink.device)), lib)
     torch.cuda.synchronize()
     assert bool((sink == 2 * 16 * 64 * 16).all())
-    for kind, ops, snk, iters in ((2, e4, sink, 1), (0, e4[:1024], sink, 1), (0, e4, sink[:100], 1), (0, e4, sink, 0)):
+    for kind, ops, snk, iters in ((2, e4, sink, 1), (0, e4[:1024], sink, 1), (0, e4, sink[:100], 1), (0, e4, sink, 0), (0, e4, sink, (1 << 18) + 1)):
         bb = [NV.dl(ops), NV.dl(snk)]
         with pytest.raises((AssertionError, ValueError)):
-            NV.check(lib.sq_probe_mfma_rate(kind, NV.ptr(bb[0]), NV.ptr(bb[1]), iters, NV.current_stream(sink.device)))
+            NV.check(lib.sq_probe_mfma_rate(kind, NV.ptr(bb[0]), NV.ptr(bb[1]), iters, NV.current_stream(sink.device)), lib)

@@ -184,7 +184,8 @@ def test_relative_window_matches_oracle(sink, r8, r4):
 
 
 @pytest.mark.parametrize("sink,w8,w4,distinct", [(128, 256, 512, True), (64, 128, 128, True), (256, [128, 384], [640, 384], True),
-                                                 (128, 256, 512, False), (0, 0, 0, False)])
+                                                 (128, 256, 512, False), (0, 0, 0, False),
+                                                 (64, 192, 320, True), (192, [192, 64], [320, 64], True)])   # multiples of 64 but not of 128: walked as written
 def test_absolute_window_matches_oracle(sink, w8, w4, distinct):
     from longcontext_sqattn_paddle_amd.sqattn.attn_triton_mix_bad import attn_hierarchical_window
     from oracle import fake_quant as FQ
@@ -208,7 +209,7 @@ def test_absolute_window_matches_oracle(sink, w8, w4, distinct):
 
 def test_unaligned_window_and_sink_sizes_follow_the_documented_rounding():
     """Sizes the reference's kernel has no defined behaviour for (its block loops promise multiples of the query block):
-    windows are rounded up to the next multiple of 128, the sink to the next multiple of 64, and an 8-bit window below
+    windows and the sink are rounded up to the next multiple of 64, and an 8-bit window below
     the query block under a wider 4-bit window is raised to the block (the reference's 4-bit range would read keys behind
     the query rows).  Expected values: the oracle on the sizes written out by hand."""
     from longcontext_sqattn_paddle_amd.sqattn.attn_triton_mix_bad import attn_hierarchical_window
@@ -219,11 +220,11 @@ def test_unaligned_window_and_sink_sizes_follow_the_documented_rounding():
     q, k, v = _rand(1, 2, 1, N, 128, 19)
     q4, k4 = FQ.int_fake_quant(q, 4, True, "per_token"), FQ.int_fake_quant(k, 4, True, "per_token")
     dev = [t.to(DEV) for t in (q, k, q4, k4, v)]
-    # absolute: sink 100 -> 128; windows (1, 1000) -> (128, 1024); (300, 200) -> (384, 256)
+    # absolute: sink 100 -> 128; windows (1, 1000) -> (64, 1024) -> 8-bit window raised to the 128-row block; (300, 200) -> (320, 256)
     out, lse = attn_hierarchical_window(*dev, torch.tensor([1, 300], dtype=torch.int32), torch.tensor([1000, 200], dtype=torch.int32), 100,
                                         "HND", torch.float32, return_lse=True)
     torch.cuda.synchronize()
-    ref, lse_ref = A.prefill_blockwise(q, k, v, block_m=128, sink=128, w8=[128, 384], w4=[1024, 256], q4=q4, k4=k4, out_dtype=torch.float32)
+    ref, lse_ref = A.prefill_blockwise(q, k, v, block_m=128, sink=128, w8=[128, 320], w4=[1024, 256], q4=q4, k4=k4, out_dtype=torch.float32)
     _check(out, ref, False)
     assert torch.allclose(lse.cpu(), lse_ref, atol=2e-4)
     # relative: ratios (0, 0.3) -> 8-bit window 0 raised to the 64-row query block, 4-bit window ceil128(345) = 384; sink 1 -> 64

@@ -79,11 +79,12 @@ def test_calibration_host_logic_without_a_gpu():
 def test_align_windows_rule():
     from longcontext_sqattn_paddle_amd.sqattn._prefill import align_windows
 
-    # multiples stay; others go up to the next multiple of 128 (windows) / 64 (sink)
+    # multiples of 64 stay as given (the reference walks them in 64-key blocks); others go up to the next multiple of 64
     assert align_windows([0, 128, 13184], [0, 256, 13184], 256, 64) == ([0, 128, 13184], [0, 256, 13184], 256)
-    assert align_windows([1, 129, 1000], [1, 129, 1000], 100, 128) == ([128, 256, 1024], [128, 256, 1024], 128)
+    assert align_windows([1, 129, 1000], [1, 129, 1000], 100, 128) == ([64, 192, 1024], [64, 192, 1024], 128)
+    assert align_windows([192, 64, 320], [320, 64, 192], 192, 128) == ([192, 64, 320], [320, 64, 192], 192)
     # 8-bit window below the query block under a wider 4-bit window: raised to the block
-    assert align_windows([0, 0, 64], [384, 0, 0], 0, 64) == ([64, 0, 128], [384, 0, 0], 0)
+    assert align_windows([0, 0, 64], [384, 0, 0], 0, 64) == ([64, 0, 64], [384, 0, 0], 0)
     assert align_windows([0], [256], 0, 128) == ([128], [256], 0)
 
 
@@ -142,9 +143,9 @@ def test_delayed_sdpa_wrapper_quantised_branch_matches_the_oracle():
 
 def test_decode_shares_by_length_add_up():
     """The rule by which the decode kernels deal the W workgroups of a ragged batch to its sequences (csrc/decode_gfx950.hip,
-    share_of): every sequence one workgroup, the other W - B by cumulative rounding of (W - B) * prefix / total in fp32, the
-    lengths counted in units of 32 tokens.  Replayed in numpy float32: the shares are positive, add up to W exactly, never
-    exceed a sequence's proportional share by more than one, and follow the lengths."""
+    share_of): every sequence one workgroup, the other W - B by cumulative rounding down of (W - B) * prefix / total in
+    64-bit integers, the lengths counted in units of 32 tokens.  Replayed in Python integers: the shares are positive, add
+    up to W exactly, stay within one of a sequence's proportional share, and follow the lengths."""
     import numpy as np
 
     rng = np.random.default_rng(11)
@@ -164,8 +165,8 @@ def test_decode_shares_by_length_add_up():
         units = (lens.astype(np.uint64) + 31) >> 5
         cum = np.cumsum(units).astype(np.uint32)           # fits 32 bits: 32 sequences of 2^26 units
         total = cum[-1]
-        spare = np.float32(W - B)
-        e1 = np.floor(spare * (cum.astype(np.float32) / np.float32(total))).astype(np.int64) if total > 0 else np.zeros(B, np.int64)
+        assert (W - B) * int(total) < 2 ** 64              # the kernel's product fits its 64-bit integer
+        e1 = np.array([(W - B) * int(c) // int(total) for c in cum], dtype=np.int64) if total > 0 else np.zeros(B, np.int64)
         e0 = np.concatenate([[0], e1[:-1]])
         n = 1 + e1 - e0
         base = np.arange(B) + e0
@@ -173,7 +174,7 @@ def test_decode_shares_by_length_add_up():
         if total > 0:
             assert int(n.sum()) == W and int(base[-1] + n[-1]) == W
             want = (W - B) * units.astype(np.float64) / float(total)
-            assert (np.abs((n - 1) - want) <= 1.0 + 1e-3 * (W - B)).all()
+            assert (np.abs((n - 1) - want) < 1.0 + 1e-9).all()
         else:
             assert (n == 1).all()
         assert (base[1:] == base[:-1] + n[:-1]).all()

@@ -462,3 +462,115 @@ def test_block_absmax_matches_scalar_bruteforce():
     for gr in (1, 128):
         other, _ = A.prefill_blockwise(q, k, v, p_quant=A.P_BLOCK_ABSMAX, out_dtype=torch.float32, group_rows=gr)
         assert float((other - out).abs().max()) > 1e-3 * rms, gr
+
+
+# ------------------------------------------------------------------ the last corners: decode fp8-P, the lazy reference point
+def _scalar_fp8_decode(q, k, v, L, D):
+    """Independent scalar restatement of attn_triton_decode.py:204-241 with the fp8 option (:232-233) for ONE head: the
+    64-token blocks in ascending order, running maximum, the denominator summed from the *unquantised* p, then
+    p <- fp16(fp16(e4m3(448 p)) / 448) (the e4m3 cast as a search on the value grid) times the fp32 value rows."""
+    f32 = np.float32
+    qf = A.fold_scale(q, D).float().numpy()
+    kf, vf = k.float().numpy(), v.float().numpy()
+    m, l, acc = f32(-np.inf), f32(0.0), np.zeros(D, dtype=np.float64)
+    for j0 in range(0, L, 64):
+        j1 = min(j0 + 64, L)
+        s = np.array([np.dot(qf.astype(np.float64), kf[j].astype(np.float64)) for j in range(j0, j1)], dtype=f32)
+        m_new = max(m, s.max())
+        p = np.exp2((s - m_new).astype(np.float64)).astype(f32)
+        alpha = f32(np.exp2(np.float64(m - m_new)))
+        l = f32(l * alpha + p.sum(dtype=f32))
+        acc = acc * np.float64(alpha)
+        p8 = _e4m3_scalar((p * f32(448.0)).astype(np.float64))
+        pq = (p8.astype(np.float16) / np.float16(448.0)).astype(np.float16).astype(np.float64)   # fp16 / fp16 -> fp16
+        for c, j in enumerate(range(j0, j1)):
+            acc = acc + pq[c] * vf[j].astype(np.float64)
+        m = m_new
+    return (acc / np.float64(l)).astype(f32), f32(np.log2(l) + m)
+
+
+def test_decode_fp8_p_matches_scalar_bruteforce():
+    """`decode_blockwise(p_quant=P_STATIC448)` -- what the GPU decode test with the fp8 option compares against -- pinned
+    by the scalar loop above: quantising before the denominator is summed, quantising the accumulated output instead of
+    p, or a bf16 instead of an fp16 round trip each move the result by e4m3 steps (1e-2 of rms) or shift the LSE."""
+    B, Hq, Hkv, L, D = 2, 4, 2, 333, 32
+    g = torch.Generator().manual_seed(61)
+    q = torch.randn(B, Hq, 1, D, generator=g).bfloat16()
+    k = torch.randn(B, Hkv, L, D, generator=g).bfloat16()
+    v = torch.randn(B, Hkv, L, D, generator=g).bfloat16()
+    lens = [333, 130]
+    out, lse = A.decode_blockwise(q, k, v, lens, p_quant=A.P_STATIC448)
+    plain, lse_plain = A.decode_blockwise(q, k, v, lens)
+    for b in range(B):
+        for h in range(Hq):
+            ref, lref = _scalar_fp8_decode(q[b, h, 0], k[b, h // 2], v[b, h // 2], lens[b], D)
+            d = np.abs(out[b, h].numpy() - ref)
+            assert d.max() < 3e-5 * max(float(np.abs(ref).max()), 1.0), (b, h, d.max())
+            assert abs(float(lse[b, h]) - float(lref)) < 2e-5
+    assert torch.equal(lse, lse_plain)                                    # the quantisation never enters the LSE
+    rms = float(plain.pow(2).mean().sqrt())
+    assert 1e-3 * rms < float((out - plain).abs().max()) < 0.2 * rms      # and it is not a no-op
+
+
+def _scalar_mx_row(scores, vals):
+    """Independent per-row scalar restatement of the `P_MX_ROW` state: scores [blocks][64] (fp32, base-2 logits of one
+    query row), vals [blocks][64] (one output channel).  Written from the definition, not from the oracle's tensors:
+      * reference point r: the first block's maximum; a later block's maximum replaces it only when it exceeds r by more
+        than 16, otherwise r stays;
+      * p = 2^(s - r); the denominator sums p as it is; the block scale is 2^k, k = floor(-log2(max p)) clamped to
+        [-16, 60]; the product uses e4m3(p 448 2^k) / (448 2^k);
+      * when r moves by d, numerator and denominator are multiplied by 2^-d first."""
+    f32 = np.float32
+    r, num, den = None, 0.0, f32(0.0)
+    moves = []
+    for s, v in zip(scores, vals):
+        mx = f32(max(s))
+        if r is None:
+            r = mx
+        elif float(mx) - float(r) > 16.0:
+            alpha = f32(np.exp2(np.float64(r) - np.float64(mx)))
+            num, den = num * float(alpha), f32(den * alpha)
+            moves.append(float(mx) - float(r))
+            r = mx
+        p = np.exp2((np.asarray(s, dtype=f32) - r).astype(np.float64)).astype(f32)
+        den = f32(den + p.sum(dtype=f32))
+        kk = min(max(np.floor(-np.log2(np.float64(p.max()))), -16.0), 60.0)
+        sc = 448.0 * 2.0 ** kk
+        pq = _e4m3_scalar((p.astype(np.float64) * sc).astype(np.float32).astype(np.float64)) / sc
+        num = num + float(np.dot(pq, np.asarray(v, dtype=np.float64)))
+    return num / float(den), float(np.log2(np.float64(den)) + np.float64(r)), moves
+
+
+def test_lazy_reference_point_matches_scalar_row_loop():
+    """`_RowState.update` in `P_MX_ROW` against the scalar loop above, on rows whose maximum rises in one block by 15.9
+    (the reference point stays: p up to 2^15.9, block exponent -15), by 16.1 (it moves) and by 40 (it moves), then falls
+    back; one row per case plus a row that creeps up by 6 per block (moves once the lead passes 16)."""
+    g = torch.Generator().manual_seed(71)
+    blocks, D = 6, 4
+    rises = [15.9, 16.1, 40.0, None]
+    S = torch.randn(len(rises), blocks, 64, generator=g) * 2.0 - 3.0
+    for i, rise in enumerate(rises):
+        top0 = float(S[i, 0].max())
+        if rise is None:
+            for b in range(1, blocks):
+                S[i, b, 7] = top0 + 6.0 * b
+        else:
+            S[i, 1:] = torch.minimum(S[i, 1:], torch.tensor(top0 - 0.5))     # nothing else leads the first block
+            S[i, 2, 11] = top0 + rise
+    V = torch.randn(blocks, 64, D, generator=g).to(torch.float16).float()
+    st = A._RowState(len(rises), D)
+    for b in range(blocks):
+        st.update(S[:, b].contiguous(), V[b], A.P_MX_ROW, 64)
+    out, lse = st.finish()
+    expect_moves = [0, 1, 1, None]
+    for i, rise in enumerate(rises):
+        for d in range(D):
+            ref, lref, moves = _scalar_mx_row(S[i].numpy(), V[:, :, d].numpy())
+            assert abs(float(out[i, d]) - ref) <= 2e-5 * max(abs(ref), 1.0), (i, d, float(out[i, d]), ref)
+        assert abs(float(lse[i]) - lref) <= 2e-5 * max(abs(lref), 1.0)
+        if expect_moves[i] is not None:
+            assert len(moves) == expect_moves[i], (rise, moves)
+        else:
+            assert len(moves) == 1 and abs(moves[0] - 18.0) < 1e-4      # leads of 6 and 12 are tolerated, 18 is not
+    # the row that rose by 15.9 really kept its reference point: its m is still the first block's maximum
+    assert float(st.m[0]) == float(S[0, 0].max()) and float(st.m[1]) == float(S[1, 2, 11])

@@ -1,7 +1,9 @@
 """`sq_decode_fwd_noalloc` (the entry point for callers that cannot allocate device memory) against `sq_decode_fwd`:
 same kernels, partials in the library's own device array instead of a workspace, so the outputs must be equal bit for
 bit.  Two calls in a row, the second on a smaller input (the array then still holds the first call's partials), and
-the size limit."""
+the size limit.  "Allocates nothing" is checked against the driver's own count of free device memory
+(`hipMemGetInfo`, which also sees a `hipMalloc` made inside the library), not only against torch's allocator; and the
+call is recorded into a HIP graph after `sq_decode_noalloc_init` and replayed."""
 import ctypes
 
 import pytest
@@ -46,11 +48,14 @@ def test_noalloc_decode_equals_workspace_decode_twice_second_smaller():
         (q, k, v, sl), (out_a, lse_a, ws), (out_b, lse_b), S = _case(B, Hq, Hkv, L, lens, seed)
         rc, msg = _call("sq_decode_fwd", q, k, v, sl, out_a, lse_a, 0, ws)
         assert rc == 0, msg
-        before = torch.cuda.memory_allocated()
+        assert lib.sq_decode_noalloc_init() == 0, lib.sq_last_error().decode()   # the one-off look-up, outside the measured call
+        torch.cuda.synchronize()
+        before, free_before = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
         rc, msg = _call("sq_decode_fwd_noalloc", q, k, v, sl, out_b, lse_b, 0)
         assert rc == 0, msg
         torch.cuda.synchronize()
         assert torch.cuda.memory_allocated() == before
+        assert torch.cuda.mem_get_info()[0] == free_before      # the driver's count: no hipMalloc inside the library either
         assert bool(torch.isfinite(out_b).all())
         assert torch.equal(out_a, out_b) and torch.equal(lse_a, lse_b)
 
@@ -65,3 +70,30 @@ def test_noalloc_decode_rejects_sizes_beyond_its_array():
     assert rc == 0, msg
     torch.cuda.synchronize()
     assert bool(torch.isfinite(out_b).all())
+
+
+def test_noalloc_decode_recorded_into_a_graph_and_replayed():
+    """What the entry point is for: after `sq_decode_noalloc_init` and one eager call it is recorded into a HIP graph;
+    every replay -- with the cache contents changed and eager work in between -- equals the eager `sq_decode_fwd`."""
+    lib = N.lib()
+    assert lib.sq_decode_noalloc_init() == 0, lib.sq_last_error().decode()
+    (q, k, v, sl), (out_a, lse_a, ws), (out_b, lse_b), S = _case(2, 28, 4, 6000, [6000, 4321], 5)
+    rc, msg = _call("sq_decode_fwd_noalloc", q, k, v, sl, out_b, lse_b, 0)    # warm-up outside the capture
+    assert rc == 0, msg
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        rc, msg = _call("sq_decode_fwd_noalloc", q, k, v, sl, out_b, lse_b, 0)
+    assert rc == 0, msg
+    g = torch.Generator(device=DEV).manual_seed(9)
+    for rep in range(4):
+        k.copy_(torch.randn(k.shape, device=DEV, generator=g).bfloat16())
+        sl.copy_(torch.tensor([6000 - 100 * rep, 4321 + rep], dtype=torch.int32, device=DEV))
+        junk = torch.randn(256, 256, device=DEV) @ torch.randn(256, 256, device=DEV)   # eager work between the replays
+        torch.cuda.synchronize()
+        out_b.fill_(float("nan"))
+        graph.replay()
+        rc, msg = _call("sq_decode_fwd", q, k, v, sl, out_a, lse_a, 0, ws)
+        assert rc == 0, msg
+        torch.cuda.synchronize()
+        assert torch.equal(out_a, out_b) and torch.equal(lse_a, lse_b) and bool(torch.isfinite(junk).all()), rep
