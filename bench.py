@@ -189,6 +189,27 @@ def time_plugin(torch, qkv, steps=3):
                                 "note": "build-defined option, off by default: same visited keys and P.V, scores from the int8 MFMA"}
         del q8, k8, v8, o, kc, ks, v8b
         torch.cuda.empty_cache()
+    # the absolute-window launch (sqattn/attn_triton_mix_bad.py:285-426, args.use_relative_distance false): 128-row query
+    # blocks, the 4-bit window range on its own 4-bit fake-quantised operands -- the one launch that runs 4-wave workgroups
+    from longcontext_sqattn_paddle_amd.sqattn.attn_triton_mix_bad import attn_hierarchical_window
+
+    w8, w4, sink = 8192, 32768, 256
+    args_abs = types.SimpleNamespace(qk_qtype="int", v_qtype="int", use_relative_distance=False)
+    closure = mp_triton_wrapper(1, w8, w4, sink, args_abs)
+    call_ms = timed(lambda: closure(layer, q, k, v, None))
+    q8, q4, k8, k4, v8 = fused_int_prepass(q, k, v, want_4bit=True, tensor_layout="NHD")
+    o = torch.empty_like(q8)
+    kern_ms = timed(lambda: attn_hierarchical_window(q8, k8, q4, k4, v8, w8, w4, sink, "NHD", torch.bfloat16, workspace=ws, out=o))
+    assert bool(torch.isfinite(o[0, -1].float()).all()) and float(o[0, -1].float().abs().sum()) > 0
+    flops = workloads.window_flops(N, D, sink, [w8] * Hq, [w4] * Hq, 128)
+    tf = flops / kern_ms / 1e9
+    out["absolute_w8_8192_w4_32768_sink_256"] = {
+        "window_tokens": [w8, w4], "flops": flops, "fraction_of_full_causal_flops": round(flops / (4.0 * N * N * D * Hq / 2), 4),
+        "plugin_call_ms": round(call_ms, 3), "kernel_ms": round(kern_ms, 3),
+        "roofline": {"bound": "mfma", "kernel": "prefill_kernel (sink + absolute windows, separate 4-bit operands, 4-wave workgroups, fp16 P.V)",
+                     "achieved": round(tf, 1), "peak": PEAK_MFMA_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / PEAK_MFMA_BF16_TFLOPS, 4)}}
+    del q8, q4, k8, k4, v8, o
+    torch.cuda.empty_cache()
     return out
 
 
@@ -458,6 +479,105 @@ def time_e2e(torch, N, new_tokens=17, sqattn=False, kv_selection=False, graph=Fa
     return res
 
 
+def time_config5(torch, new_tokens=128):
+    """The benchmark's end-to-end configuration as written: the 28-layer Qwen2.5-7B-shaped decoder (random weights,
+    bf16), one prompt of 1 048 576 seeded random tokens prefilled through `generate` (MLP in 8192-token chunks; exact
+    attention in the first and last layer, the SQAttn closure of `process_model` with the reference's shipped windows --
+    ratio 0.1 / 0.1, sink 256 -- in layers 1..26), the whole KV cache resident in HBM, k-means clustering of the prompt's
+    keys (1024 clusters per kv head, 10 iterations), then `new_tokens` greedy tokens with the decode step replayed from a
+    HIP graph over the 4096-token selection (model_hub/LLM.py:40-116, 167-203).  Beside it: where the prefill's time goes
+    (HIP events around the attention slot and around the projections / MLP), and the dense decode step over the same
+    cache."""
+    import types
+
+    from longcontext_sqattn_paddle_amd import workloads
+    from longcontext_sqattn_paddle_amd.model_hub.qwen import QwenConfig, QwenModel
+    from longcontext_sqattn_paddle_amd.sqattn.attn_replacer import process_model
+    from longcontext_sqattn_paddle_amd.sqattn.attn_triton_mix_relative import window_tokens
+
+    dev, N = "cuda:0", 1 << 20
+    free_gib = torch.cuda.mem_get_info()[0] / 2.0 ** 30
+    if free_gib < 150.0:
+        return {"skipped": f"needs 150 GiB of free HBM (60 GiB cache x 1.3 headroom, weights, a layer's activations); {free_gib:.0f} GiB free"}
+    cfg = QwenConfig()
+    model = QwenModel("Qwen2.5-7B-shaped", N + new_tokens + 32, torch.bfloat16, dev, "SQAttn", config=cfg, seed=1)
+    ratio, sink = 0.1, 256
+    process_model(model, "SQAttn", {i: {"bit8": ratio, "bit4": ratio, "sink": sink} for i in range(1, cfg.num_hidden_layers - 1)},
+                  types.SimpleNamespace(qk_qtype="int", v_qtype="int", use_relative_distance=True))
+    model.enable_kv_selection(num_centroids=1024, topk=4096, num_iters=10)
+    spans = {"attention": [], "projections_and_mlp": []}
+
+    def timed(kind, fn, is_prefill):
+        def wrapper(*a, **kw):
+            if not is_prefill(*a, **kw):
+                return fn(*a, **kw)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            out = fn(*a, **kw)
+            e1.record()
+            spans[kind].append((e0, e1))
+            return out
+        return wrapper
+
+    for layer in model.layers:   # the slots process_model bound (layers 1..26) and the exact ones (0, 27)
+        layer.prefill_attention = timed("attention", layer.prefill_attention, lambda *a, **kw: True)
+    model.wqkv = timed("projections_and_mlp", model.wqkv, lambda h, layer: h.shape[1] > 1)
+    model.wo = timed("projections_and_mlp", model.wo, lambda h, layer, bsz, seq_len, dim, residual=None: seq_len > 1)
+    model.mlp = timed("projections_and_mlp", model.mlp, lambda h, layer, residual=None, norm=None: h.shape[1] > 1)
+    inner = model.layer_prefill
+
+    def layer_prefill(layer_idx, start_bdx, hidden_states):
+        out = inner(layer_idx, start_bdx, hidden_states)
+        if hidden_states.shape[1] == N and layer_idx % 4 == 3:
+            torch.cuda.synchronize()
+            log(f"[bench] config 5: layer {layer_idx + 1} of {cfg.num_hidden_layers} prefilled")
+        return out
+
+    model.layer_prefill = layer_prefill
+    ids = torch.randint(0, cfg.vocab_size, (1, N), device=dev, generator=torch.Generator(device=dev).manual_seed(5))
+    model.generate("SQAttn", ids[:, :4096], None, 3, verbose=False)    # warm-up: library handles, GEMM heuristics
+    for v in spans.values():
+        v.clear()
+    out = model.generate("SQAttn", ids, None, new_tokens, verbose=False, use_graph=True)
+    torch.cuda.synchronize()
+    assert len(out[0]) == new_tokens and model.kv_cache.valid_length.cpu().tolist() == [N + new_tokens - 1]
+    share = {k: sum(e0.elapsed_time(e1) for e0, e1 in v) / 1e3 for k, v in spans.items()}
+    w = window_tokens(ratio, N)
+    attn_flops = 2 * (4.0 * N * N * 128 * 28 / 2) + (cfg.num_hidden_layers - 2) * workloads.window_flops(N, 128, sink, [w] * 28, [w] * 28, 64)
+    res = {"config": f"{cfg.num_hidden_layers} layers, hidden {cfg.hidden_size}, 28/4 heads of 128, bf16 random weights; prompt {N} tokens, "
+                     f"{new_tokens} greedy tokens; SQAttn closure (ratio {ratio}/{ratio}, sink {sink}) in layers 1..{cfg.num_hidden_layers - 2}, exact "
+                     "attention in the first and last; 1024 clusters per kv head, 10 Lloyd iterations, 4096 selected tokens per kv head and step",
+           "prefill_s": round(model.prefill_latency, 2), "clustering_s": round(model.cluster_latency, 3),
+           "decode_ms_per_step_selection_hip_graph": round(model.decode_latency * 1e3, 3),
+           "prefill_seconds_by_part": {"attention_calls": round(share["attention"], 2), "projections_and_mlp": round(share["projections_and_mlp"], 2),
+                                       "other": round(model.prefill_latency - share["attention"] - share["projections_and_mlp"], 2),
+                                       "note": "HIP events around the attention slot of every layer (pre-pass + kernel) and around wqkv, wo and "
+                                               "the chunked MLP (hipBLASLt GEMMs + SiLU*mul); other = norms, rotary embedding, cache rows, embedding, host"},
+           "prefill_attention_TFLOP_per_s": round(attn_flops / share["attention"] / 1e12, 1),
+           "kv_cache_GB": round(2 * cfg.num_hidden_layers * N * 4 * 128 * 2 / 1e9, 1)}
+    # the dense decode step over the same cache, replayed from a graph as well.  The cache holds exactly prompt + new
+    # tokens, so it is rewound to the prompt first: the steps rewrite rows that are already there.
+    model.disable_kv_selection()
+    cache = model.kv_cache
+    cache.valid_length.fill_(N)
+    cache._host_valid, cache.context = [N], N
+    tok = torch.tensor([[out[0][0]]], device=dev)
+    tok = model.decode_forward(tok).argmax(dim=-1)
+    tok = model.capture_decode_step(tok).argmax(dim=-1)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(8):
+        tok = model.replay_decode_step(tok).argmax(dim=-1)
+    e1.record()
+    torch.cuda.synchronize()
+    model.release_decode_graph()
+    res["decode_ms_per_step_dense_hip_graph"] = round(e0.elapsed_time(e1) / 8, 3)
+    del model
+    torch.cuda.empty_cache()
+    return res
+
+
 def time_kv_cache(torch, N, iters=10):
     """The KV cache's two row movements at the benchmark shape (4 kv heads x 128, bf16): the store of an N-token
     prompt (K and V, each read once and written once) and the append of one token per sequence at batch 8."""
@@ -653,6 +773,8 @@ def main():
     ap.add_argument("--e2e-new-tokens", type=int, default=17, help="tokens generated by each end-to-end run")
     ap.add_argument("--e2e-graph", action="store_true",
                     help="the end-to-end runs replay their decode steps from a HIP graph (for prompts too long to prefill twice)")
+    ap.add_argument("--no-config5", action="store_true",
+                    help="skip the end-to-end configuration as written (28 layers, 1 048 576-token prompt, 128 graph-replayed steps: about two minutes)")
     ap.add_argument("--e2e", action="store_true",
                     help="also run the whole 28-layer Qwen2.5-7B-shaped decoder (random weights): prefill latency and decode ms/step")
     args = ap.parse_args()
@@ -822,8 +944,8 @@ def main():
         torch.cuda.empty_cache()
     if args.e2e:
         runs = {"exact": dict(sqattn=False), "sqattn": dict(sqattn=True), "selection": dict(sqattn=True, kv_selection=True)}
-        result["e2e"] = [time_e2e(torch, N, new_tokens=args.e2e_new_tokens, graph=args.e2e_graph, **runs[r]) for r in args.e2e_runs.split(",")]
-        log(f"[bench] end to end: {result['e2e']}")
+        result["e2e_runs"] = [time_e2e(torch, N, new_tokens=args.e2e_new_tokens, graph=args.e2e_graph, **runs[r]) for r in args.e2e_runs.split(",")]
+        log(f"[bench] end to end: {result['e2e_runs']}")
     if not args.no_kmeans:
         settle()
         us, kflops, kbytes, topk_us, full_ms = time_kmeans(torch)
@@ -840,6 +962,14 @@ def main():
                             "topk_select_us": round(topk_us, 1),
                             "topk_shape": "4096 tokens per kv head for one 28-head query, 1024 clusters per kv head"}
         log(f"[bench] kmeans iteration: {us:.0f} us")
+    if not args.no_config5:
+        settle()
+        try:
+            result["e2e"] = time_config5(torch)
+        except Exception as exc:   # the headline line must come out whatever happens to this leg
+            result["e2e"] = {"error": f"{type(exc).__name__}: {exc}"[:500]}
+            torch.cuda.empty_cache()
+        log(f"[bench] config 5 end to end: {result['e2e']}")
     if not args.no_cpu_baseline:
         from oracle import cpu_baseline as CB   # the checker's CPU path, timed as the baseline only
 

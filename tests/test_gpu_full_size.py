@@ -165,8 +165,95 @@ def test_plugin_closure_1m_default_windows():
     _closure_rows(N, rows, 7, False)
 
 
+def _mixed_row_reference(q8_row, q4_row, k8_head, k4_head, v_head, ranges, i):
+    """Closed form of one query row whose 4-bit window range uses its own operands (attn_triton_mix_bad.py:37-74): the
+    scores of keys in a range flagged `use4` are q4 . k4, all others q8 . k8; one softmax over the union, float64."""
+    parts = []
+    for lo, hi, use4, masked in ranges:
+        hi = min(hi, i + 1) if masked else hi
+        if hi > lo:
+            idx = torch.arange(lo, hi)
+            parts.append((idx, (k4_head if use4 else k8_head)[idx] @ (q4_row if use4 else q8_row)))
+    idx = torch.cat([p[0] for p in parts])
+    s = torch.cat([p[1] for p in parts])
+    m = s.max()
+    p = torch.exp2(s - m)
+    return (p[:, None] * v_head[idx]).sum(0) / p.sum(), idx.numel()
+
+
+@pytest.mark.parametrize("w8,w4", [(8192, 32768), ([8192, 4096, 128, 131072] * 7, [32768, 4096, 640, 131072] * 7)])
+def test_absolute_windows_with_4bit_operands_128k(w8, w4):
+    """The absolute-window launch with separate 4-bit operands (attn_triton_mix_bad.py:285-426) at the prefill benchmark
+    shape, through the closure `mp_triton_wrapper` builds for `use_relative_distance = False`: 128-row query blocks, the
+    4-bit range really multiplied with the 4-bit fake-quantised query and key.  It is the one configuration that runs
+    the 4-wave workgroups; here their 64-bit tile bases, the switch of the query operand set at the edges of the 4-bit
+    range and the per-head windows (one head with both windows equal, one with a 128-token 8-bit window, one wider than
+    the sequence) run at N = 131072.  Sampled rows against the float64 closed form over the oracle's key ranges on the
+    oracle's fake-quantised operands."""
+    from longcontext_sqattn_paddle_amd.sqattn.attn_replacer import mp_triton_wrapper
+    from oracle import plugin as OP
+
+    N = 131072
+    print(f"case absolute windows with 4-bit operands 128K w8={w8 if isinstance(w8, int) else 'per head'}", flush=True)
+    q, k, v = (t.permute(0, 2, 1, 3).contiguous().to(DEV) for t in inputs.prefill_inputs(1, HQ, HKV, N, D, seed=2))
+    args = types.SimpleNamespace(qk_qtype="int", v_qtype="int", use_relative_distance=False)
+    layer = types.SimpleNamespace(num_key_value_groups=HQ // HKV)
+    out = mp_triton_wrapper(1, w8, w4, 256, args)(layer, q, k, v, None)
+    torch.cuda.synchronize()
+    assert out.shape == (1, N, HQ * D) and out.dtype == torch.bfloat16 and bool(torch.isfinite(out).all())
+    out = out.view(1, N, HQ, D)
+    kh, vh = k.cpu().permute(0, 2, 1, 3), v.cpu().permute(0, 2, 1, 3)
+    kc = kh - OP.key_mean_exact(kh)
+    k8, k4 = FQ.int_fake_quant(kc, 8, True, "per_token"), FQ.int_fake_quant(kc, 4, True, "per_token")
+    v8 = FQ.int_fake_quant(vh, 8, True, "per_channel")
+    l8 = [w8] * HQ if isinstance(w8, int) else w8
+    l4 = [w4] * HQ if isinstance(w4, int) else w4
+    # rows: start, sink edge, the first blocks whose 8-bit / 4-bit windows leave the sink, edges of 128-row blocks, the end
+    rows = [0, 127, 128, 255, 256, 383, 8192 + 255, 8192 + 256, 8192 + 384, 32768 + 127, 32768 + 256, 32768 + 511, 65535, 65536, 100000, N - 1]
+    worst = 0.0
+    for h in (0, 1, 2, 3, 6, 7, 27):
+        kvh = h // (HQ // HKV)
+        for i in rows:
+            qrow = q[0, i, h].cpu()[None, None, None]
+            q8 = A.fold_scale(FQ.int_fake_quant(qrow, 8, True, "per_token")[0, 0], D).double()[0]
+            q4 = A.fold_scale(FQ.int_fake_quant(qrow, 4, True, "per_token")[0, 0], D).double()[0]
+            qs = i // 128 * 128
+            ranges = A.kv_ranges(qs, qs + 128, sink=256, w8=l8[h], w4=l4[h])
+            ref, nkeys = _mixed_row_reference(q8, q4, k8[0, kvh].double(), k4[0, kvh].double(), v8[0, kvh].double(), ranges, i)
+            err = float((out[0, i, h].cpu().double() - ref).abs().max())
+            big = float(ref.abs().max())
+            assert err <= 4e-3 * big + 2.0 ** -8 * big + 1e-6, (h, i, err, big, nkeys)     # fp16 P and V, bf16 output
+            worst = max(worst, err / max(big, 1e-30))
+    print(f"  worst relative row error {worst:.2e}", flush=True)
+
+
+def test_decode_128k_batch_1_ragged_against_closed_form():
+    """Config 3 at batch 1 with its own ragged length (uniform in [96K, 128K]) in a 131072-token cache."""
+    from longcontext_sqattn_paddle_amd.sqattn.attn_triton_decode import attn_decode
+
+    print("case decode 128K b1 ragged", flush=True)
+    q, kc, vc, lens = inputs.decode_inputs(1, HQ, HKV, 131072, D, seed=32)      # 100 923 valid tokens
+    n = int(lens[0])
+    assert 98304 <= n < 131072
+    out, lse = attn_decode(q.to(DEV), kc.to(DEV), vc.to(DEV), "NHD", torch.float32, return_lse=True, seqlens=lens.to(DEV))
+    torch.cuda.synchronize()
+    ref, ref_lse = A.exact_attention(A.fold_scale(q.permute(0, 2, 1, 3), D), kc[:, :n].permute(0, 2, 1, 3), vc[:, :n].permute(0, 2, 1, 3),
+                                     causal=False, score_scale=math.log(2.0))
+    got = out[0].cpu().double().view(HQ, D)
+    rms = float(ref.pow(2).mean().sqrt())
+    assert float((got - ref[0, :, 0]).abs().max()) <= 2e-4 * rms + 1e-6
+    assert torch.allclose(lse[0].cpu().double().view(HQ), ref_lse[0, :, 0], atol=2e-4)
+    # rows behind the valid prefix must not matter: poison them and run again
+    kd, vd = kc.to(DEV), vc.to(DEV)
+    kd[:, n:] = float("nan")
+    vd[:, n:] = float("nan")
+    out2 = attn_decode(q.to(DEV), kd, vd, "NHD", torch.float32, seqlens=lens.to(DEV))
+    torch.cuda.synchronize()
+    assert torch.equal(out, out2)
+
+
 def test_decode_128k_batch_4_ragged_against_closed_form():
-    """Config 3 names batch sizes 1, 4 and 8; 1 and 8 are covered in tests/test_gpu_decode.py."""
+    """Config 3 names batch sizes 1, 4 and 8; 8 is covered in tests/test_gpu_decode.py, 1 above."""
     from longcontext_sqattn_paddle_amd.sqattn.attn_triton_decode import attn_decode
 
     print("case decode 128K b4 ragged", flush=True)

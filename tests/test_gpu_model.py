@@ -235,3 +235,111 @@ def test_end_to_end_configuration_sizes_three_layers_one_million_tokens():
     ref, _ = A.exact_attention(A.fold_scale(qh, 128), kf, vf, causal=False, score_scale=math.log(2.0))
     err = float((dense.cpu().view(28, 128).double() - ref[0, :, 0]).abs().max())
     assert err <= 2e-4 * float(ref.pow(2).mean().sqrt()) + 1e-6, err
+
+
+def _decode_closed_form(q, key_rows, value_rows, groups):
+    """Exact softmax attention of one query token, float64, one kv head at a time (a 28-head tensor of a million double
+    rows does not fit comfortably): q [Hq, D] bf16 (unscaled), key_rows / value_rows [Hkv][n, D] -> [Hq, D]."""
+    from oracle import attention as A
+
+    Hq, D = q.shape
+    qf = A.fold_scale(q, D).double()                                   # carries log2e / sqrt(D), rounded as the kernel folds it
+    out = torch.empty(Hq, D, dtype=torch.float64)
+    for kvh in range(Hq // groups):
+        k, v = key_rows[kvh].double(), value_rows[kvh].double()
+        s = k @ qf[kvh * groups:(kvh + 1) * groups].T                  # [n, groups], base-2 logits
+        p = torch.exp2(s - s.max(dim=0, keepdim=True).values)
+        out[kvh * groups:(kvh + 1) * groups] = (p.T @ v) / p.sum(dim=0)[:, None]
+    return out
+
+
+def test_end_to_end_configuration_as_written_28_layers_one_million_tokens_128_steps():
+    """The benchmark's end-to-end configuration as written: the 28-layer Qwen2.5-7B-shaped decoder (random weights, hidden
+    3584, 28/4 heads of 128, bf16), one prompt of 1 048 576 seeded random tokens prefilled through the runtime (MLP in
+    8192-token chunks; exact attention in the first and last layer, the SQAttn closure with the reference's shipped
+    windows -- ratio 0.1 / 0.1, sink 256 -- in layers 1..26, as `process_model` binds them), the whole 60 GB KV cache
+    resident, k-means clustering of every layer's keys (1024 clusters per kv head, 10 iterations), then 128 greedy tokens
+    with the decode step replayed from a HIP graph over the 4096-token selection.
+    Checked: token count and range, cache lengths; the tokens of the first 16 steps again from the eager loop (the cache
+    rewound to the prompt) equal the graph's; and, against the float64 closed form on the cache rows the step really
+    holds, a middle layer's attention over its selection list and its dense decode attention over all cached tokens."""
+    import time
+    import types
+
+    from longcontext_sqattn_paddle_amd.model_hub.qwen import QwenConfig, QwenModel
+    from longcontext_sqattn_paddle_amd.sqattn.attn_replacer import process_model
+    from longcontext_sqattn_paddle_amd.sqattn.attn_triton_decode import attn_decode
+
+    N, new = 1 << 20, 128
+    free_gib = torch.cuda.mem_get_info()[0] / 2.0 ** 30
+    need_gib = 150.0      # 60 GiB of cache (x 1.3 headroom the cache object asks for) + 17 GiB of weights + activations of a 1M-token layer
+    print(f"case model 28 layers x 1M tokens x {new} steps; free HBM {free_gib:.0f} GiB", flush=True)
+    if free_gib < need_gib:
+        pytest.skip(f"needs {need_gib:.0f} GiB of free HBM for the resident cache, the weights and a layer's activations; {free_gib:.0f} GiB are free")
+    cfg = QwenConfig()
+    model = QwenModel("Qwen2.5-7B-shaped", N + new + 32, torch.bfloat16, DEV, "SQAttn", config=cfg, seed=1)
+    args = types.SimpleNamespace(qk_qtype="int", v_qtype="int", use_relative_distance=True)
+    windows = {i: {"bit8": 0.1, "bit4": 0.1, "sink": 256} for i in range(1, cfg.num_hidden_layers - 1)}
+    process_model(model, "SQAttn", windows, args)
+    model.enable_kv_selection(num_centroids=1024, topk=4096, num_iters=10)
+    ids = torch.randint(0, cfg.vocab_size, (1, N), device=DEV, generator=torch.Generator(device=DEV).manual_seed(2))
+    inner, t0 = model.layer_prefill, time.time()
+
+    def layer_prefill(layer_idx, start_bdx, hidden_states):      # a progress line every four layers: the prefill takes a minute or two
+        out = inner(layer_idx, start_bdx, hidden_states)
+        if layer_idx % 4 == 3:
+            torch.cuda.synchronize()
+            print(f"  layer {layer_idx + 1} of {cfg.num_hidden_layers} prefilled at {time.time() - t0:.0f} s", flush=True)
+        return out
+
+    model.layer_prefill = layer_prefill
+    out = model.generate("SQAttn", ids, None, new, verbose=False, use_graph=True)
+    torch.cuda.synchronize()
+    print(f"  prefill {model.prefill_latency:.1f} s, clustering {model.cluster_latency:.2f} s, decode {model.decode_latency * 1e3:.2f} ms/step "
+          f"(HIP graph), total {time.time() - t0:.1f} s", flush=True)
+    assert len(out) == 1 and len(out[0]) == new and all(0 <= t < cfg.vocab_size for t in out[0])
+    cache, sel = model.kv_cache, model.kv_selection
+    assert cache.valid_length.cpu().tolist() == [N + new - 1] and cache.context == N + new - 1
+    assert len(sel.layers) == cfg.num_hidden_layers and all(int(st["cluster_size"].sum()) == 4 * N for st in sel.layers)
+
+    # ---- the first 16 steps again, eagerly, from the cache rewound to the prompt: same tokens as the graph's
+    # (a step's K/V rows are rewritten with the values they already hold; the selection lists depend on the lengths only)
+    cache.valid_length.fill_(N)
+    cache._host_valid = [N]
+    cache.context = N
+    tok = torch.tensor([[out[0][0]]], device=DEV)
+    eager = []
+    for _ in range(16):
+        tok = model.decode_forward(tok).argmax(dim=-1)
+        eager.append(int(tok))
+    torch.cuda.synchronize()
+    assert eager == out[0][1:17], (eager, out[0][1:17])
+    assert cache.valid_length.cpu().tolist() == [N + 16]
+
+    # ---- a middle layer's attention over the selection list, by hand
+    layer_id = 13
+    g = torch.Generator().manual_seed(3)
+    q = torch.randn(1, 1, 28, 128, generator=g).to(torch.bfloat16).to(DEV)
+    sel.begin_step(cache.attend_length)
+    got = sel.attend(layer_id, q, cache.key_cache[layer_id], cache.value_cache[layer_id], 7)
+    torch.cuda.synchronize()
+    n_list = int(sel.list_len[0])
+    assert n_list == 4096 + int(cache.attend_length[0]) - N
+    lists = sel.ids[:, :n_list]
+    assert int(lists[:, :4096].max()) < N and int(lists[:, :4096].min()) >= 0
+    assert torch.equal(lists[0, 4096:].cpu(), torch.arange(N, N + n_list - 4096, dtype=torch.int32))
+    rows = lists.long()
+    ref = _decode_closed_form(q.cpu()[0, 0], [cache.key_cache[layer_id][0, rows[h], h].cpu() for h in range(4)],
+                              [cache.value_cache[layer_id][0, rows[h], h].cpu() for h in range(4)], 7)
+    err = float((got.float().cpu().view(28, 128).double() - ref).abs().max())
+    assert err <= 2.0 ** -8 * float(ref.abs().max()) + 1e-6, err           # the slot returns bf16: half a unit in the last place
+    # ---- and its dense decode attention over the whole cache
+    L = int(cache.attend_length[0])
+    dense = attn_decode(q, cache.key_cache[layer_id], cache.value_cache[layer_id], "NHD", torch.float32, seqlens=cache.attend_length)
+    torch.cuda.synchronize()
+    ref = _decode_closed_form(q.cpu()[0, 0], [cache.key_cache[layer_id][0, :L, h].cpu() for h in range(4)],
+                              [cache.value_cache[layer_id][0, :L, h].cpu() for h in range(4)], 7)
+    err = float((dense.cpu().view(28, 128).double() - ref).abs().max())
+    assert err <= 2e-4 * float(ref.pow(2).mean().sqrt()) + 1e-6, err
+    del model, cache, sel
+    torch.cuda.empty_cache()

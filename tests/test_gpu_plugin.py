@@ -256,3 +256,35 @@ def test_integer_qk_closure_configurations_drawn_at_random():
         assert _cos(o, r) >= 0.99999, case
         assert float((o - r).abs().max()) <= 2 ** -7 * float(r.abs().max()) + 2e-3 * rms, case
 
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_delayed_sdpa_wrapper_quantised_branch_on_the_device(dtype):
+    """The masked-SDPA emulation of the mixed-precision windows (attn_replacer.py:36-190) with its operands on the GPU:
+    key centring, the five fake-quantisers, the [L, 2L] mask (scalar and per-head windows) and SDPA over
+    [8-bit keys ; 4-bit keys], against the oracle's float64 restatement.  Tolerance: fp32 operands 1e-3 absolute (the
+    library's SDPA accumulates in fp32, and the key mean's summation order may move an element across a rounding boundary
+    of its quantiser; a wrong mask or operand shows at 1e-2 and more); bf16 operands cosine >= 0.9995 and 3e-2 of the largest output (bf16 scores)."""
+    from longcontext_sqattn_paddle_amd.sqattn.attn_replacer import construct_mix_bit_mask, delayed_sdpa_wrapper
+    from oracle import plugin
+
+    print(f"case delayed_sdpa_wrapper on the device, {dtype}", flush=True)
+    g = torch.Generator().manual_seed(5)
+    q, k, v = (torch.randn(2, 3, 80, 64, generator=g).to(dtype) for _ in range(3))
+    k = (k.float() + 0.7).to(dtype)
+    args = types.SimpleNamespace(quant=True, qk_qtype="int", v_qtype="int", vis_attn=False)
+    for w8, w4, sink in ((6, 10, 4), ([4, 9, 80], [8, 0, 5], 2), (1, 0, 0)):
+        out = delayed_sdpa_wrapper(0, w8, w4, sink, args)(None, q.to(DEV), k.to(DEV), v.to(DEV), None, scaling=1.0)
+        torch.cuda.synchronize()
+        assert out.is_cuda and out.shape == (2, 80, 3 * 64)
+        ref = plugin.masked_sdpa_emulation(q, k, v, bit8_window=w8, bit4_window=w4, sink=sink)
+        got = out.cpu().view(2, 80, 3, 64).permute(0, 2, 1, 3).double()
+        if dtype == torch.float32:
+            assert float((got - ref).abs().max()) < 1e-3, (w8, w4)
+        else:
+            assert _cos(got, ref) >= 0.9995 and float((got - ref).abs().max()) <= 3e-2 * float(ref.abs().max()), (w8, w4)
+        assert torch.equal(construct_mix_bit_mask(80, w8, w4, sink, DEV).cpu(), plugin.mix_bit_mask(80, w8, w4, sink))
+    # the plain branch on the device: SDPA with the caller's mask
+    plain = delayed_sdpa_wrapper(0, 0, 0, 0, types.SimpleNamespace(quant=False))(None, q.to(DEV), k.to(DEV), v.to(DEV), None, tensor_layout="HND")
+    want = torch.nn.functional.scaled_dot_product_attention(q.double(), k.double(), v.double(), is_causal=True).transpose(1, 2).reshape(2, 80, 192)
+    assert float((plain.cpu().double() - want).abs().max()) <= (1e-4 if dtype == torch.float32 else 3e-2 * float(want.abs().max()))
