@@ -190,7 +190,8 @@ def time_plugin(torch, qkv, steps=3):
         del q8, k8, v8, o, kc, ks, v8b
         torch.cuda.empty_cache()
     # the absolute-window launch (sqattn/attn_triton_mix_bad.py:285-426, args.use_relative_distance false): 128-row query
-    # blocks, the 4-bit window range on its own 4-bit fake-quantised operands -- the one launch that runs 4-wave workgroups
+    # blocks, the 4-bit window range on its own 4-bit fake-quantised operands (two query blocks per workgroup, the tiles on
+    # which they want different operand sets walked twice)
     from longcontext_sqattn_paddle_amd.sqattn.attn_triton_mix_bad import attn_hierarchical_window
 
     w8, w4, sink = 8192, 32768, 256
@@ -206,7 +207,7 @@ def time_plugin(torch, qkv, steps=3):
     out["absolute_w8_8192_w4_32768_sink_256"] = {
         "window_tokens": [w8, w4], "flops": flops, "fraction_of_full_causal_flops": round(flops / (4.0 * N * N * D * Hq / 2), 4),
         "plugin_call_ms": round(call_ms, 3), "kernel_ms": round(kern_ms, 3),
-        "roofline": {"bound": "mfma", "kernel": "prefill_kernel (sink + absolute windows, separate 4-bit operands, 4-wave workgroups, fp16 P.V)",
+        "roofline": {"bound": "mfma", "kernel": "prefill_kernel (sink + absolute windows, separate 4-bit operands: two 128-row query blocks per 8-wave workgroup, fp16 P.V)",
                      "achieved": round(tf, 1), "peak": PEAK_MFMA_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / PEAK_MFMA_BF16_TFLOPS, 4)}}
     del q8, q4, k8, k4, v8, o
     torch.cuda.empty_cache()

@@ -393,7 +393,11 @@ __device__ __forceinline__ void quant_pack4(float p0, float p1, float p2, float 
 
 // One workgroup = WAVES waves x 32 query rows of one q-head (2 waves per SIMD when WAVES == 8, so that one
 // wave's MFMA phase overlaps the other's softmax phase).  MODE as in quant_pack8.
-template <bool BF16, int WAVES, int MODE>
+// DUAL (WAVES == 8, absolute windows with their own 4-bit operands, block_m == 128): the workgroup holds two query blocks,
+// A = waves 0..3 and B = waves 4..7, whose 4-bit ranges end 128 keys apart.  On the up to two tiles in between -- 8-bit
+// for A, 4-bit for B -- the blocks want different K tiles, so those tiles are walked twice: once as they are (B skips
+// them), once as 4-bit copies right behind (A skips those).  Everywhere else the blocks agree, or only one of them visits.
+template <bool BF16, int WAVES, int MODE, bool DUAL = false>
 __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
   constexpr int NT = WAVES * 64;
   constexpr int CH = (kBN * kD * 2 / 16) / NT;  // 16-byte chunks per thread and tile operand
@@ -460,12 +464,30 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
     segA_hi = 0;
     segB_lo = 0;
   }
-  // separate 4-bit operands only ever run with WAVES*32 == block_m <= 128 (all waves agree on a tile's operand set)
-  const bool distinct4 = (WAVES < 8) && a.q4 != nullptr;
-
+  // separate 4-bit operands run with WAVES*32 == block_m (all waves agree on a tile's operand set), or as DUAL
+  const bool distinct4 = (WAVES < 8 || DUAL) && a.q4 != nullptr;
+  // The tiles that are copied from the 4-bit key, [t4_lo, t4_hi): the 4-bit range of the workgroup's first query block.
+  // DUAL: tiles [c_lo, c_lo + n_dup), from where block A's 4-bit range ends to where block B's ends (128 keys later, unless
+  // the sink cuts both), are walked twice -- first as 4-bit copies for B, then as they are for A.
+  int t4_lo = wr.r4_lo, t4_hi = wr.r4_hi, c_lo = 0, n_dup = 0;
+  if constexpr (DUAL) {
+    const WaveRanges wa = wave_ranges(a, a.q_offset + row_wg0, head);
+    t4_lo = wa.r4_lo;
+    t4_hi = wa.r4_hi;
+    if (row_wg0 + 4 * ROWS < a.Nq) {
+      const int qeA = (a.q_offset + row_wg0) / a.block_m * a.block_m + a.block_m, qeB = qeA + a.block_m;
+      const int left8A = max(a.sink, qeA - a.w8[head]), left8B = max(a.sink, qeB - a.w8[head]), left4B = max(a.sink, qeB - a.w4[head]);
+      if (left4B < left8B && left8A < left8B) {
+        c_lo = left8A / kBN;
+        n_dup = (left8B - left8A) / kBN;
+        if (t4_hi <= t4_lo) t4_lo = c_lo;   // block A has no 4-bit range of its own (the sink cuts it): the copies are all there is
+        t4_hi = c_lo;                        // (where A has one, it ends at c_lo anyway)
+      }
+    }
+  }
   // ---- Q~ fragments (B operand of S^T = K.Q~^T): lane (column = query row c32, k-group g)
   uint4 qf[8];
-  auto load_q = [&](const void* qbase) {
+  auto load_q = [&](const void* qbase) __attribute__((always_inline)) {
     const uint16_t* qp = (const uint16_t*)qbase + (int64_t)b * a.q_sb + (int64_t)head * a.q_sh;
     const int row = max(min(row_w0 + c32, a.Nq - 1), 0);
     const uint16_t* rp = qp + (int64_t)row * a.q_sn + 8 * g;
@@ -577,18 +599,21 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
   // ---- tile staging: global -> LDS directly (no registers), CH wave instructions of 64 x 16 bytes per operand.
   // K and V^T have their own double buffers because the K tile runs one step ahead of the V^T tile (below).
   typedef __attribute__((address_space(3))) void* lds_ptr_t;
-  auto tile_uses4 = [&](int j) { return distinct4 && j >= wr.r4_lo && j < wr.r4_hi; };
   const int64_t k_head_off = (int64_t)b * a.k_sb + (int64_t)kvh * a.k_sh;
   char* const kbase_lds = smem;                     // 4 x 16 KB
   char* const vbase_lds = smem + 4 * kKTileBytes;   // 4 x 16 KB (8 KB used per buffer in the fp8 mode)
-  auto stage_k16 = [&](int j, int stage) {
+  auto stage_k16 = [&](int j, int stage, bool use4) {
     char* kbuf = kbase_lds + stage * kKTileBytes;
-    const uint16_t* kb = (const uint16_t*)(tile_uses4(j) ? a.k4 : a.k) + k_head_off;
+    const uint16_t* kb = (const uint16_t*)(use4 ? a.k4 : a.k) + k_head_off;
+    // DUAL runs this form for the first and the last few tiles only (stage_k_full in between): its per-lane addresses, for
+    // two key tensors, are formed here and not hoisted into registers the tile loop has no room for
+    int ln = lane;
+    if constexpr (DUAL) asm volatile("; clamped tile copy" : "+v"(ln));
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
       const int q = wave * CH + c;                       // wave instruction index 0..15 -> 1 KB of the tile
-      const int kr = 4 * q + (lane >> 4);                // K row in the tile
-      const int kc = (lane & 15) ^ (kr & 15);            // global chunk that lands in this lane's slot
+      const int kr = 4 * q + (ln >> 4);                  // K row in the tile
+      const int kc = (ln & 15) ^ (kr & 15);              // global chunk that lands in this lane's slot
       const int n = min(j * kBN + kr, a.Nk - 1);
       __builtin_amdgcn_global_load_lds((const void*)(kb + (int64_t)n * a.k_sn + 8 * kc), (lds_ptr_t)(kbuf + q * 1024), 16, 0, 0);
     }
@@ -611,9 +636,9 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
       __builtin_amdgcn_global_load_lds((const void*)(a.k_scale + (((int64_t)b * a.Hkv + kvh) * a.nT + j) * kBN + lane),
                                        (lds_ptr_t)(kbuf + kBN * kD), 4, 0, 0);
   };
-  auto stage_k = [&](int j, int stage) {
+  auto stage_k = [&](int j, int stage, bool use4) {
     if constexpr (kQK8) stage_k8(j, stage);
-    else stage_k16(j, stage);
+    else stage_k16(j, stage, use4);
   };
   auto stage_v = [&](int j, int stage) {
     char* vbuf = vbase_lds + stage * kVTileBytes;
@@ -648,9 +673,12 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
     kvoff[c] = (uint32_t)(kr * (int)a.k_sn + 8 * kc) * 2u;
   }
   const char* const k_bytes = (const char*)a.k + k_head_off * 2;
+  // (the 4-bit key as a byte distance from the 8-bit one: a choice between two integers, where a choice between the two
+  // captured pointers made the compiler keep this lambda's captures in memory)
+  const int64_t k4_delta = DUAL ? (int64_t)((const char*)a.k4 - (const char*)a.k) : 0;
   const uint32_t k_tile_bytes = (uint32_t)(kBN * a.k_sn * 2);
-  auto stage_k_full = [&](int j, int stage) {
-    const char* base = k_bytes + (uint64_t)(uint32_t)j * k_tile_bytes;
+  auto stage_k_full = [&](int j, int stage, bool use4) {
+    const char* base = k_bytes + ((DUAL && use4) ? k4_delta : (int64_t)0) + (uint64_t)(uint32_t)j * k_tile_bytes;
     char* kbuf = kbase_lds + stage * kKTileBytes;
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
@@ -1038,35 +1066,72 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
   // waves drift apart by up to a tile, which lets one wave's matrix phase overlap another's vector phase.
   // The schedule is addressed by a flat step index t = 0 .. nTot-1: the sink tiles [0, nA) first, then the tiles
   // [segB_lo, segB_hi).  The ring buffer of step t is t & 3.
+  // DUAL: the 4-bit copies of tiles [c_lo, c_lo + n_dup) sit at steps [d1 - n_dup, d1), where those tiles would sit
+  // anyway; the tiles themselves and everything behind them move up by n_dup steps.  The steps whose K tile comes from
+  // the 4-bit key then form one interval [u4_lo, u4_hi): block A's 4-bit range and, right behind it, the copies.
   const int nA = segA_hi, shiftB = segB_lo - segA_hi;
-  const int nTot = max(nA + segB_hi - segB_lo, 0);
-  auto tile_of = [&](int t) { return t < nA ? t : t + shiftB; };
+  const int d1 = (DUAL && n_dup > 0) ? c_lo - shiftB + n_dup : (1 << 30);
+  const int nTot = max(nA + segB_hi - segB_lo, 0) + n_dup;
+  auto tile_of = [&](int t) {
+    if (t < nA) return t;
+    if constexpr (DUAL) return t + shiftB - (t >= d1 ? n_dup : 0);
+    return t + shiftB;
+  };
+  const int u4_lo = t4_lo - shiftB, u4_hi = t4_hi - shiftB + n_dup;
+  // (a wave only ever visits steps whose operand set is the one it wants, so this also tells it which Q~ set a step takes)
+  auto step_uses4 = [&](int t) { return distinct4 && t >= u4_lo && t < u4_hi; };
   // steps whose K tile is complete (only the very last tile of the sequence can be partial)
   const int nFull = (nTot > 0 && (tile_of(nTot - 1) + 1) * kBN > a.Nk) ? nTot - 1 : nTot;
   // this wave's tiles in step space: [0, fa) (sink) and [fb, fe] (window up to its diagonal tile); from step fm
   // on the causal mask applies.  A wave without rows visits nothing.
+  // DUAL: for block A's waves every tile from c_lo on is its moved-up original, and they skip the copies; for block B's
+  // waves the tiles below c_lo + n_dup are the copies, and they skip the originals.
+  const int thr = wave < 4 ? c_lo : c_lo + n_dup;
+  auto step_of = [&](int j) { return j - shiftB + ((DUAL && j >= thr) ? n_dup : 0); };   // a tile of segment B
   const int fa = wave_active ? wr.sink_hi : 0;
-  const int fb = wave_active ? wr.win_lo - shiftB : (1 << 30);
-  const int fe = wr.diag_hi - shiftB, fm = wr.diag_lo - shiftB;
-  auto visits_step = [&](int t) { return t < fa || (t >= fb && t <= fe); };
+  const int fb = wave_active ? step_of(wr.win_lo) : (1 << 30);
+  const int fe = step_of(wr.diag_hi), fm = step_of(wr.diag_lo);
+  const int sk_lo = (DUAL && n_dup > 0) ? (wave < 4 ? d1 - n_dup : d1) : 0;
+  auto visits_step = [&](int t) {
+    const bool in = t < fa || (t >= fb && t <= fe);
+    if constexpr (DUAL) return in && (unsigned)(t - sk_lo) >= (unsigned)n_dup;
+    return in;
+  };
 
   if (0 < nTot) {
-    stage_k(tile_of(0), 0);
+    stage_k(tile_of(0), 0, step_uses4(0));
     stage_v(tile_of(0), 0);
   }
   if (1 < nTot) {
-    stage_k(tile_of(1), 1);
+    stage_k(tile_of(1), 1, step_uses4(1));
     stage_v(tile_of(1), 1);
   }
-  if (2 < nTot) stage_k(tile_of(2), 2);
+  if (2 < nTot) stage_k(tile_of(2), 2, step_uses4(2));
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
-  auto switch_q = [&](int jt) {
-    if constexpr (WAVES < 8) {
+  // Q~ fragments of the other operand set, one 16-byte piece at a time (a handful of switches per wave: no need for all
+  // eight loads in flight, and the registers they would take are the tile step's).  The 8-bit quantiser of load_q does
+  // not apply: a launch with its own 4-bit operands gets both sets quantised by the caller (q_quant == 0, checked on the host).
+  auto reload_q = [&](const void* qbase) __attribute__((always_inline)) {
+    // (the lane index is laundered so that the row addresses are formed here, at one of a wave's two or three switches,
+    // and not hoisted out of the tile loop into registers that loop has no room for)
+    int ln = lane;
+    asm volatile("; operand set switch" : "+v"(ln));
+    const uint16_t* qp = (const uint16_t*)qbase + (int64_t)b * a.q_sb + (int64_t)head * a.q_sh;
+    const int row = max(min(row_w0 + (ln & 31), a.Nq - 1), 0);
+    const uint16_t* rp = qp + (int64_t)row * a.q_sn + 8 * (ln >> 5);
+#pragma unroll
+    for (int kk = 0; kk < 8; ++kk) {
+      const uint4 raw = *(const uint4*)(rp + 16 * kk);
+      qf[kk] = make_uint4(scale_pair<BF16>(raw.x, a.sm), scale_pair<BF16>(raw.y, a.sm), scale_pair<BF16>(raw.z, a.sm), scale_pair<BF16>(raw.w, a.sm));
+    }
+  };
+  auto switch_q = [&](int t) __attribute__((always_inline)) {   // t: a step this wave visits
+    if constexpr (WAVES < 8 || DUAL) {
       if (distinct4) {  // switch the Q~ operand set when entering/leaving the 4-bit window range
-        const bool want4 = tile_uses4(jt);
+        const bool want4 = step_uses4(t);
         if (want4 != q_is4) {
-          load_q(want4 ? a.q4 : a.q);
+          reload_q(want4 ? a.q4 : a.q);
           q_is4 = want4;
         }
       }
@@ -1075,7 +1140,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
   f32x16_t Sa[2], Sb[2];
   bool vis_cur = nTot > 0 && visits_step(0);
   if (vis_cur) {
-    switch_q(tile_of(0));
+    switch_q(0);
     qk_tile(kbase_lds, Sa);
     if constexpr (!kPlain) {
       mfma_settle(Sa[0], Sa[1]);
@@ -1090,25 +1155,25 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
       if (t + 4 < nFull) {
         const int j2 = tile_of(t + 2), j3 = tile_of(t + 3), j4 = tile_of(t + 4);
         if constexpr (WAVES == 8 && !kQK8) {
-          stage_k_full(j3, (t + 3) & 3);
-          stage_k_full(j4, t & 3);
+          stage_k_full(j3, (t + 3) & 3, DUAL && step_uses4(t + 3));
+          stage_k_full(j4, t & 3, DUAL && step_uses4(t + 4));
         } else {
-          stage_k(j3, (t + 3) & 3);
-          stage_k(j4, t & 3);
+          stage_k(j3, (t + 3) & 3, step_uses4(t + 3));
+          stage_k(j4, t & 3, step_uses4(t + 4));
         }
         stage_v(j2, (t + 2) & 3);
         stage_v(j3, (t + 3) & 3);
       } else {
-        if (t + 3 < nTot) stage_k(tile_of(t + 3), (t + 3) & 3);
-        if (t + 4 < nTot) stage_k(tile_of(t + 4), t & 3);
+        if (t + 3 < nTot) stage_k(tile_of(t + 3), (t + 3) & 3, step_uses4(t + 3));
+        if (t + 4 < nTot) stage_k(tile_of(t + 4), t & 3, step_uses4(t + 4));
         if (t + 2 < nTot) stage_v(tile_of(t + 2), (t + 2) & 3);
         if (t + 3 < nTot) stage_v(tile_of(t + 3), (t + 3) & 3);
       }
     }
     const bool vis_nxt = visits_step(t + 1);
     const char* knext = kbase_lds + ((t + 1) & 3) * kKTileBytes;
-    if constexpr (WAVES < 8) {
-      if (vis_nxt) switch_q(tile_of(t + 1));
+    if constexpr (WAVES < 8 || DUAL) {
+      if (vis_nxt) switch_q(t + 1);
     }
     if (vis_cur) {
       // Q.K^T of the next tile is computed even if this wave will not use it (the buffer then holds an older
@@ -1291,7 +1356,9 @@ int prefill_impl(const DLTensor* q, const DLTensor* k, const DLTensor* v, const 
                  "sq_prefill_fwd: head %d: a 4-bit window wider than an 8-bit window smaller than block_m reads future keys "
                  "in the reference and is not supported", h);
     }
-    if (q4) waves = p->block_m / 32;  // all waves of a workgroup must agree on the operand set of a tile
+    // separate 4-bit operands: a workgroup of one 64-row query block (two waves), or, for 128-row blocks, of two blocks
+    // that walk the few tiles on which they disagree twice (DUAL)
+    if (q4 && p->block_m == 64) waves = 2;
   } else {
     SQ_REQUIRE(p->window_mode == SQ_WINDOW_NONE, SQ_EINVAL, "sq_prefill_fwd: window_mode %d not supported", p->window_mode);
     SQ_REQUIRE(!q4, SQ_EINVAL, "sq_prefill_fwd: q4/k4 only apply to window mode");
@@ -1381,6 +1448,7 @@ int prefill_impl(const DLTensor* q, const DLTensor* k, const DLTensor* v, const 
   const int rows_wg = waves * 32;
   local.nQB = (int)((Nq + rows_wg - 1) / rows_wg);
   SQ_REQUIRE(p->q_quant == 0 || p->q_quant == 8, SQ_EINVAL, "sq_prefill_fwd: q_quant must be 0 or 8 (got %d)", (int)p->q_quant);
+  SQ_REQUIRE(!(p->q_quant && q4), SQ_EINVAL, "sq_prefill_fwd: q_quant applies to launches without a separate 4-bit operand set");
   local.q_quant = p->q_quant;
   local.q_offset = (int)p->q_offset;
   local.p_quant = p->p_quant;
@@ -1422,6 +1490,21 @@ int prefill_impl(const DLTensor* q, const DLTensor* k, const DLTensor* v, const 
                                (int)smem));                                                                      \
     hipLaunchKernelGGL((prefill_kernel<BF, W, M>), dim3(blocks), dim3(W * 64), smem, st, local);                 \
   } while (0)
+#define SQ_LAUNCH_PREFILL_DUAL(BF, M)                                                                                  \
+  do {                                                                                                                \
+    SQ_HIP(hipFuncSetAttribute((const void*)prefill_kernel<BF, 8, M, true>, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                               (int)smem));                                                                           \
+    hipLaunchKernelGGL((prefill_kernel<BF, 8, M, true>), dim3(blocks), dim3(8 * 64), smem, st, local);                \
+  } while (0)
+#define SQ_LAUNCH_DUAL(BF)                                          \
+  do {                                                              \
+    switch (p->p_quant) {                                           \
+      case SQ_P_NONE: SQ_LAUNCH_PREFILL_DUAL(BF, 0); break;          \
+      case SQ_P_E4M3_STATIC: SQ_LAUNCH_PREFILL_DUAL(BF, 1); break;   \
+      case SQ_P_E4M3_BLOCK: SQ_LAUNCH_PREFILL_DUAL(BF, 2); break;    \
+      default: SQ_LAUNCH_PREFILL_DUAL(BF, 3); break;                 \
+    }                                                               \
+  } while (0)
 #define SQ_LAUNCH_MODE(BF, W)                                   \
   do {                                                          \
     if (k_scale) {                                              \
@@ -1437,13 +1520,15 @@ int prefill_impl(const DLTensor* q, const DLTensor* k, const DLTensor* v, const 
       default: SQ_LAUNCH_PREFILL(BF, W, 3); break;               \
     }                                                           \
   } while (0)
-  if (waves == 8) {
+  if (waves == 8 && q4) {
+    if (bf) SQ_LAUNCH_DUAL(true); else SQ_LAUNCH_DUAL(false);
+  } else if (waves == 8) {
     if (bf) SQ_LAUNCH_MODE(true, 8); else SQ_LAUNCH_MODE(false, 8);
-  } else if (waves == 4) {
-    if (bf) SQ_LAUNCH_MODE(true, 4); else SQ_LAUNCH_MODE(false, 4);
   } else {
     if (bf) SQ_LAUNCH_MODE(true, 2); else SQ_LAUNCH_MODE(false, 2);
   }
+#undef SQ_LAUNCH_DUAL
+#undef SQ_LAUNCH_PREFILL_DUAL
 #undef SQ_LAUNCH_MODE
 #undef SQ_LAUNCH_PREFILL
   SQ_HIP(hipGetLastError());
