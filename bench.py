@@ -690,6 +690,30 @@ def time_kmeans(torch, iters=10):
     us = e0.elapsed_time(e1) / iters * 1e3
     flops = 2.0 * N * C * D * G
     nbytes = G * (N * D * 2 + N * 4 + C * D * 2 * 2 + C * 4)   # keys read once, assignment written, centroids read and written, counts
+    # the iteration loop as segment_k_means runs it: three steps that re-sum every row, the third leaving the exact sums
+    # in the workspace, then steps that only apply the tokens that changed cluster (sq_kmeans_train_stateful).  Each key
+    # set has its own assignment and workspace (the carried state), and the two alternate as above.
+    from longcontext_sqattn_paddle_amd import _native as NV
+
+    state = [(torch.empty(G, N, dtype=torch.int32, device=dev), _workspace(G, N, C, dev)) for _ in sets]
+    run10, carried = [], []
+    for rep in range(3):
+        cents = [s_[0].index_select(1, idx0).contiguous() for s_ in sets]
+        torch.cuda.synchronize()
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+        ev[0].record()
+        for it in range(10):
+            if it == 3:
+                ev[1].record()
+            st = NV.KMEANS_STATELESS if it < 2 else (NV.KMEANS_KEEP_SUMS if it == 2 else NV.KMEANS_APPLY_CHANGES)
+            for k in range(2):
+                _triton_k_means_train(sets[k][0], cents[k], max_idx=state[k][0], workspace=state[k][1], state=st)
+        ev[2].record()
+        torch.cuda.synchronize()
+        run10.append(ev[0].elapsed_time(ev[2]) / 20 * 1e3)
+        carried.append(ev[1].elapsed_time(ev[2]) / 14 * 1e3)
+    us_run10, us_carried = sorted(run10)[1], sorted(carried)[1]
+    del state
     # the configuration as written: 10 Lloyd iterations (9 normalised + the final one), value sums, reverse index, then top-k
     full = []
     for i in range(4):
@@ -711,7 +735,7 @@ def time_kmeans(torch, iters=10):
     e1.record()
     torch.cuda.synchronize()
     assert int(out.min()) >= 0 and int(out.max()) < N
-    return us, flops, nbytes, e0.elapsed_time(e1) / 20 * 1e3, sorted(full[1:])[1]
+    return us, flops, nbytes, e0.elapsed_time(e1) / 20 * 1e3, sorted(full[1:])[1], us_run10, us_carried
 
 
 def time_prepass(torch, N, want4, iters=10, skip_query=False):
@@ -949,14 +973,20 @@ def main():
         log(f"[bench] end to end: {result['e2e_runs']}")
     if not args.no_kmeans:
         settle()
-        us, kflops, kbytes, topk_us, full_ms = time_kmeans(torch)
+        us, kflops, kbytes, topk_us, full_ms, us_run10, us_carried = time_kmeans(torch)
         t_mfma, t_hbm = kflops / PEAK_MFMA_BF16_TFLOPS / 1e6, kbytes / PEAK_HBM_GBS / 1e3
         result["kmeans"] = {"us_per_iteration": round(us, 1), "TFLOP_per_s": round(kflops / us / 1e6, 1),
                             "frac_of_bf16_mfma_peak": round(kflops / us / 1e6 / PEAK_MFMA_BF16_TFLOPS, 4),
                             "GB_per_s": round(kbytes / us / 1e3, 1), "frac_of_hbm_peak": round(kbytes / us / 1e3 / PEAK_HBM_GBS, 4),
                             "bound_us": round(max(t_mfma, t_hbm), 1), "frac_of_bound": round(max(t_mfma, t_hbm) / us, 4),
                             "bytes": kbytes, "flops": kflops,
-                            "shape": "4 heads x 131072 tokens x 128, 1024 centroids, one Lloyd iteration, two key sets alternating",
+                            "shape": "4 heads x 131072 tokens x 128, 1024 centroids, one Lloyd iteration that re-sums every row, two key sets alternating",
+                            "us_per_iteration_carried_sums": round(us_carried, 1),
+                            "frac_of_bound_carried_sums": round(max(t_mfma, t_hbm) / us_carried, 4),
+                            "us_per_iteration_mean_of_the_10_iteration_run": round(us_run10, 1),
+                            "carried_sums_note": "the loop of segment_k_means: iterations 1-3 re-sum every row, 4-10 apply only the tokens that changed "
+                                                 "cluster to the exact sums kept in the workspace (same centroids bit for bit); iterations 4-10 alone, "
+                                                 "and the mean over all ten",
                             "segment_k_means_10_iterations_ms": round(full_ms, 3),
                             "segment_k_means_note": "10 iterations + value sums + reverse index, host wall clock including its one host "
                                                     "synchronisation (the reference's Cnt.max().item(), cache_hub/kmeans.py:195)",

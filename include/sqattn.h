@@ -21,6 +21,7 @@
  *   sq_decode_noalloc_init    no reference counterpart: its one-off set-up, for callers that record HIP graphs
  *   sq_decode_selected_fwd    no reference counterpart: the same decode over the tokens sq_topk_select picked
  *   sq_kmeans_train           cache_hub/kmeans.py:127-196 (assign launch :147-173, update launch :175-193)
+ *   sq_kmeans_train_stateful  the same step inside the iteration loop of segment_k_means (cache_hub/kmeans.py:356-368)
  *   sq_reverse_index          cache_hub/kmeans.py:233-262
  *   sq_index_add              cache_hub/kmeans.py:307-329
  *   sq_topk_select            no reference counterpart (defined by this build's benchmark configuration)
@@ -205,6 +206,24 @@ size_t sq_kmeans_workspace_bytes(int64_t groups, int64_t num_tokens, int64_t num
  */
 int sq_kmeans_train(const DLTensor* data, DLTensor* centroids, DLTensor* idx, DLTensor* cnt,
                     DLTensor* workspace, int32_t normalize, void* stream);
+
+/*
+ * The same Lloyd step for a run of iterations over the same data (the loop of segment_k_means, cache_hub/kmeans.py:356-368),
+ * with the exact cluster sums carried in the workspace from one call to the next.  After the first few iterations hardly
+ * any token changes its cluster, and re-summing every row in every iteration reads the keys a second time for nothing.
+ *   SQ_KMEANS_STATELESS      what sq_kmeans_train does; nothing is kept;
+ *   SQ_KMEANS_KEEP_SUMS      the same step, and the clusters' exact fp64 sums and sizes stay in the workspace;
+ *   SQ_KMEANS_APPLY_CHANGES  idx must hold the previous call's assignment and the workspace the sums that call left
+ *                            (KEEP_SUMS or APPLY_CHANGES, same data, same shapes, nothing else run on the workspace's
+ *                            tail in between -- sq_reverse_index, sq_index_add and sq_topk_select leave it alone):
+ *                            the tokens whose cluster changes are subtracted from their old cluster's sum and added to
+ *                            their new one's, and the centroids are formed from the sums.
+ * The sums are exact, so every mode gives the same centroids, idx and cnt, bit for bit; APPLY_CHANGES costs the assign
+ * pass plus work in proportion to the tokens that moved (slower than a re-sum only when most of them move).
+ */
+enum { SQ_KMEANS_STATELESS = 0, SQ_KMEANS_KEEP_SUMS = 1, SQ_KMEANS_APPLY_CHANGES = 2 };
+int sq_kmeans_train_stateful(const DLTensor* data, DLTensor* centroids, DLTensor* idx, DLTensor* cnt,
+                             DLTensor* workspace, int32_t normalize, int32_t state, void* stream);
 
 /* clusters[g,c,0:cnt] = token ids with idx == c in ascending order (rest 0); cluster_size = counts. */
 int sq_reverse_index(const DLTensor* idx, DLTensor* clusters, DLTensor* cluster_size, DLTensor* workspace,

@@ -19,6 +19,7 @@ SQ_OK, SQ_EINVAL, SQ_ESHAPE, SQ_EDEVICE, SQ_EDTYPE, SQ_EUNSUPPORTED, SQ_EHIP, SQ
 LAYOUT = {"HND": 0, "NHD": 1}
 P_NONE, P_E4M3_STATIC, P_E4M3_BLOCK, P_E4M3_STATIC_FAST, P_E4M3_FP8_PV, P_E4M3_MX_FP8_PV = 0, 1, 2, 3, 4, 5
 WINDOW_NONE, WINDOW_SIZES = 0, 1
+KMEANS_STATELESS, KMEANS_KEEP_SUMS, KMEANS_APPLY_CHANGES = 0, 1, 2
 QTYPE = {"int": 0, "e4m3": 1, "e5m2": 2}
 
 
@@ -95,6 +96,7 @@ SYMBOLS = {
     "sq_decode_selected_fwd": (ctypes.c_int, [_P] * 8 + [ctypes.POINTER(DecodeParams), ctypes.c_void_p]),
     "sq_kmeans_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int64] * 4),
     "sq_kmeans_train": (ctypes.c_int, [_P, _P, _P, _P, _P, ctypes.c_int32, ctypes.c_void_p]),
+    "sq_kmeans_train_stateful": (ctypes.c_int, [_P, _P, _P, _P, _P, ctypes.c_int32, ctypes.c_int32, ctypes.c_void_p]),
     "sq_reverse_index": (ctypes.c_int, [_P, _P, _P, _P, ctypes.c_void_p]),
     "sq_index_add": (ctypes.c_int, [_P, _P, _P, _P, ctypes.c_void_p]),
     "sq_topk_select": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, ctypes.c_int32, ctypes.c_void_p]),

@@ -25,9 +25,12 @@ def _workspace(G: int, num_tokens: int, num_centroids: int, device) -> torch.Ten
 
 
 def _triton_k_means_train(data, centroids, max_idx=None, normalize_centroids=True, return_indices=False,
-                          workspace: Optional[torch.Tensor] = None):
+                          workspace: Optional[torch.Tensor] = None, state: int = N.KMEANS_STATELESS):
     """One Lloyd step, centroids updated in place (kmeans.py:127-196).  With `return_indices` also returns
-    the assignment and the largest cluster size (a host sync, like the reference's `.item()`, :195)."""
+    the assignment and the largest cluster size (a host sync, like the reference's `.item()`, :195).
+    `state` (extension, for a run of steps over the same data with the same `max_idx` and `workspace`):
+    `N.KMEANS_KEEP_SUMS` leaves the clusters' exact sums in the workspace, `N.KMEANS_APPLY_CHANGES` forms the new
+    centroids from those sums and the tokens that changed cluster instead of re-summing every row (same bits)."""
     _require(data, "data")
     batch_size, num_tokens, dim = data.shape
     num_centroids = centroids.shape[1]
@@ -38,7 +41,8 @@ def _triton_k_means_train(data, centroids, max_idx=None, normalize_centroids=Tru
     if workspace is None:
         workspace = _workspace(batch_size, num_tokens, num_centroids, data.device)
     b = [N.dl(t) for t in (data, centroids, max_idx, data_cnt, workspace)]
-    N.check(N.lib().sq_kmeans_train(*[N.ptr(x) for x in b], 1 if normalize_centroids else 0, N.current_stream(data.device)))
+    N.check(N.lib().sq_kmeans_train_stateful(*[N.ptr(x) for x in b], 1 if normalize_centroids else 0, int(state),
+                                             N.current_stream(data.device)))
     if return_indices:
         return centroids, max_idx, int(data_cnt.max().item())
     return centroids
@@ -69,9 +73,16 @@ def triton_index_add(value, max_idx, num_centroids: int, workspace: Optional[tor
     return out
 
 
+FULL_RESUM_STEPS = 3   # Lloyd steps that re-sum every row before the sums are carried (most tokens still move in them)
+
+
 def segment_k_means(key, value, num_centroids: int, num_iters: int = 10, num_segments: int = 1):
     """kmeans.py:332-375: strided initial centroids, `num_iters-1` normalised steps on the segmented data,
-    one un-normalised step on the whole data, then value sums and the reverse index."""
+    one un-normalised step on the whole data, then value sums and the reverse index.
+
+    From the fourth step on the exact cluster sums are carried from step to step and only the tokens that changed
+    cluster are re-added (`sq_kmeans_train_stateful`): the same centroids bit for bit, without reading the keys a second
+    time per step.  With one segment the final step runs on the same tensors and continues that way."""
     _require(key, "key")
     num_groups, num_tokens, head_dim = key.shape
     centroid_indices = torch.arange(num_centroids, dtype=torch.float32, device=key.device) * (num_tokens / num_centroids)
@@ -85,14 +96,22 @@ def segment_k_means(key, value, num_centroids: int, num_iters: int = 10, num_seg
     centroids = centroids.reshape((-1, num_centroids_per_segment, head_dim)).contiguous()
     max_idx = torch.empty((data.shape[0], data.shape[1]), dtype=torch.int32, device=data.device)
     ws = _workspace(data.shape[0], data.shape[1], num_centroids_per_segment, key.device)
-    for _ in range(num_iters - 1):
+    carried = False
+    for it in range(num_iters - 1):
+        state = N.KMEANS_STATELESS if it < FULL_RESUM_STEPS - 1 else (N.KMEANS_APPLY_CHANGES if carried else N.KMEANS_KEEP_SUMS)
         centroids = _triton_k_means_train(data, centroids, max_idx=max_idx, normalize_centroids=True,
-                                          return_indices=False, workspace=ws)
-    data = key.reshape((-1, num_tokens, head_dim))
-    centroids = centroids.reshape((-1, num_centroids, head_dim))
-    ws = _workspace(num_groups, num_tokens, num_centroids, key.device)
-    centroids, max_idx, max_cluster_size = _triton_k_means_train(data, centroids, normalize_centroids=False,
-                                                                  return_indices=True, workspace=ws)
+                                          return_indices=False, workspace=ws, state=state)
+        carried = state != N.KMEANS_STATELESS
+    if num_segments == 1 and carried and data.shape[1] == num_tokens:
+        # the same tensors, the same workspace: the last (un-normalised) step continues from the carried sums
+        centroids, max_idx, max_cluster_size = _triton_k_means_train(data, centroids, max_idx=max_idx, normalize_centroids=False,
+                                                                      return_indices=True, workspace=ws, state=N.KMEANS_APPLY_CHANGES)
+    else:
+        data = key.reshape((-1, num_tokens, head_dim))
+        centroids = centroids.reshape((-1, num_centroids, head_dim))
+        ws = _workspace(num_groups, num_tokens, num_centroids, key.device)
+        centroids, max_idx, max_cluster_size = _triton_k_means_train(data, centroids, normalize_centroids=False,
+                                                                      return_indices=True, workspace=ws)
     value_sum = triton_index_add(value.reshape((-1, num_tokens, head_dim)), max_idx, num_centroids, workspace=ws)
     clusters, cluster_size = triton_reverse_index(max_idx, num_centroids, max_cluster_size, workspace=ws)
     return centroids, value_sum, clusters, cluster_size

@@ -30,6 +30,8 @@ struct AssignArgs {
   int32_t* idx;          // [G,N]
   int64_t d_sg, d_sn, c_sg, c_sc, i_sg;
   int32_t N, C;
+  double* keep_sum;      // TRACK: [G,C,128] the clusters' exact sums, carried from the previous step
+  int32_t* keep_cnt;     // TRACK: [G,C] and their sizes
 };
 
 constexpr int kAssignWaves = 4;   // x 64 tokens; two workgroups per CU put two waves on every SIMD
@@ -40,8 +42,18 @@ constexpr int kAssignWaves = 4;   // x 64 tokens; two workgroups per CU put two 
 // (global_load_lds, unpadded rows, 16-byte chunks XOR-swizzled by row so that the MFMA operand reads are conflict
 // free), double buffered with one barrier per block; the arg-max over one half block's scores runs underneath the
 // MFMAs of the next half block (see `phase` below).
+// TRACK: the sums that are carried across iterations.  After the first few Lloyd iterations hardly any token changes its
+// cluster (configuration 4: 1 % in the fourth iteration, 0.1 % in the tenth), yet a full re-sum reads every row again.
+// The sums are exact (fp64 of bf16 values), so they can be carried: `idx` holds the previous iteration's assignment on
+// entry, and a token whose cluster changes is subtracted from its old cluster's sum and added to its new one's, in any
+// order, by fp64 atomics that round nothing -- the result is the sum a full re-sum would give, bit for bit.  The
+// workgroup lists its movers in LDS and applies them itself at the end (one channel per thread, the first 128 threads
+// adding, the others subtracting); kmeans_update_kernel then turns sums and sizes into centroids.
+template <bool TRACK>
 __global__ __launch_bounds__(kAssignWaves * 64, 1) void kmeans_assign_kernel(AssignArgs a) {
   __shared__ __attribute__((aligned(16))) char smem[2 * kCB * 256];
+  __shared__ int32_t s_chg_n;
+  __shared__ uint2 s_chg[TRACK ? kTileTok : 1];   // (token, old cluster << 16 | new cluster)
   typedef __attribute__((address_space(3))) void* lds_ptr_t;
   const int g_id = blockIdx.y;
   const int tid = threadIdx.x, lane = tid & 63;
@@ -58,6 +70,15 @@ __global__ __launch_bounds__(kAssignWaves * 64, 1) void kmeans_assign_kernel(Ass
     const uint16_t* rp = db + (int64_t)n * a.d_sn + 8 * g;
 #pragma unroll
     for (int kk = 0; kk < 8; ++kk) tf[tb][kk] = *(const uint4*)(rp + 16 * kk);
+  }
+  int old_idx[2] = {-1, -1};
+  if constexpr (TRACK) {   // requested now, needed at the very end
+    if (tid == 0) s_chg_n = 0;   // (the block loop below passes at least one barrier before anyone adds to it)
+#pragma unroll
+    for (int tb = 0; tb < 2; ++tb) {
+      const int n = tok0 + 32 * tb + c32;
+      if (n < a.N) old_idx[tb] = a.idx[(int64_t)g_id * a.i_sg + n];
+    }
   }
   const uint16_t* cb = a.cent + (int64_t)g_id * a.c_sg;
   // per-lane source of the wave's four 1 KB copies of a block (4 centroid rows each), as a byte offset from the block's
@@ -210,6 +231,37 @@ __global__ __launch_bounds__(kAssignWaves * 64, 1) void kmeans_assign_kernel(Ass
     const int n = tok0 + 32 * tb + c32;
     // cluster sizes come out of the counting sort that follows (per-tile histograms), not out of global atomics
     if (g == 0 && n < a.N) a.idx[(int64_t)g_id * a.i_sg + n] = bidx;
+    if constexpr (TRACK) {
+      const bool changed = g == 0 && n < a.N && old_idx[tb] != bidx;
+      const unsigned long long m = __ballot(changed);
+      if (m != 0) {   // wave-uniform
+        int base = 0;
+        if (lane == 0) base = atomicAdd(&s_chg_n, __popcll(m));
+        base = __shfl(base, 0);
+        if (changed) {
+          const int pos = base + __popcll(m & ((1ull << lane) - 1ull));
+          s_chg[pos] = make_uint2((uint32_t)n, ((uint32_t)old_idx[tb] << 16) | (uint32_t)bidx);
+        }
+      }
+    }
+  }
+  if constexpr (TRACK) {
+    __syncthreads();
+    const int n_chg = s_chg_n;
+    if (n_chg == 0) return;
+    const int ch = tid & (kD - 1);
+    const bool adds = tid < kD;
+    const uint16_t* drow = db + ch;
+    double* sg = a.keep_sum + (int64_t)g_id * a.C * kD + ch;
+    int32_t* cg = a.keep_cnt + (int64_t)g_id * a.C;
+    for (int i = 0; i < n_chg; ++i) {
+      const uint2 e = s_chg[i];
+      const int c = adds ? (int)(e.y & 0xffffu) : (int)(e.y >> 16);
+      if (c >= a.C) continue;   // (an old assignment that is no cluster: nothing to take it out of)
+      const double x = (double)bf16_bits_to_f32(drow[(int64_t)e.x * a.d_sn]);
+      unsafeAtomicAdd(sg + (int64_t)c * kD, adds ? x : -x);
+      if (ch == 0) atomicAdd(cg + c, adds ? 1 : -1);
+    }
   }
 }
 
@@ -441,7 +493,32 @@ struct SumArgs {
   int32_t* cnt;           // [G,C] cluster sizes, or null
   int64_t s_sg, s_sn, d_sg, d_sc;
   int32_t N, C, nT, mode; // mode 0: plain sum cast to bf16; 1: mean; 2: mean + L2 normalise (1,2: only where cnt > 0)
+  double* keep_sum;       // [G,C,128] or null: the exact sums, left for the iterations that only apply changes
+  int32_t* keep_cnt;      // [G,C] or null
 };
+
+// From a cluster's exact sum (channel t of thread t < 128) and size to its stored row: sum rounded once to fp32, mean
+// (kmeans.py:121), optional L2 normalisation with the squared norm summed in fp64 in a fixed tree (:122-123), bf16
+// store only where the cluster has tokens (:120, 124).  Shared by the full re-sum and by the update from kept sums, so
+// the two give the same bits.  All threads of the workgroup call it (it has barriers); ss_red: 128 doubles of LDS.
+__device__ __forceinline__ void finish_cluster(double s, int cnt, int mode, double* ss_red, int t, uint16_t* dst_row, int32_t* cnt_out) {
+  float x = 0.f;
+  if (t < kD) {
+    x = (float)s;                                   // exact sum rounded once to fp32
+    if (mode >= 1) x = x / (float)cnt;
+    ss_red[t] = (double)x * (double)x;
+  }
+  __syncthreads();
+  if (mode == 2) {
+    for (int d = kD / 2; d > 0; d >>= 1) {
+      if (t < d) ss_red[t] += ss_red[t + d];
+      __syncthreads();
+    }
+    if (t < kD) x = x / sqrtf((float)ss_red[0]);
+  }
+  if (t < kD && (mode == 0 || cnt > 0)) dst_row[t] = (uint16_t)f32_to_bf16_bits(x);
+  if (cnt_out && t == 0) *cnt_out = cnt;
+}
 
 constexpr int kSumRows = 4;   // rows in flight per thread (8: slower, 2: the same)
 constexpr int kListCap = 2048;   // token ids staged in LDS at a time
@@ -525,26 +602,33 @@ __global__ __launch_bounds__(256) void cluster_sum_kernel(SumArgs a) {
     for (int e = 0; e < 8; ++e) red[wave][8 * o + e] = acc[e];
   }
   __syncthreads();
-  float x = 0.f;
+  double s = 0;
   if (t < kD) {
-    double s = extra;
+    s = extra;
 #pragma unroll
     for (int rr = 0; rr < 4; ++rr) s += red[rr][t];
-    x = (float)s;                                   // exact sum rounded once to fp32
-    if (a.mode >= 1) x = x / (float)cnt;            // kmeans.py:121
-    ss_red[t] = (double)x * (double)x;
+    if (a.keep_sum) a.keep_sum[((int64_t)g * a.C + c) * kD + t] = s;
   }
-  __syncthreads();
-  if (a.mode == 2) {
-    for (int d = kD / 2; d > 0; d >>= 1) {
-      if (t < d) ss_red[t] += ss_red[t + d];
-      __syncthreads();
-    }
-    if (t < kD) x = x / sqrtf((float)ss_red[0]);    // kmeans.py:122-123
-  }
-  if (t < kD && (a.mode == 0 || cnt > 0))           // empty clusters keep the old centroid (kmeans.py:120,124)
-    a.dst[(int64_t)g * a.d_sg + (int64_t)c * a.d_sc + t] = (uint16_t)f32_to_bf16_bits(x);
-  if (a.cnt && t == 0) a.cnt[(int64_t)g * a.C + c] = cnt;
+  if (a.keep_cnt && t == 0) a.keep_cnt[(int64_t)g * a.C + c] = cnt;
+  finish_cluster(s, cnt, a.mode, ss_red, t, a.dst + (int64_t)g * a.d_sg + (int64_t)c * a.d_sc, a.cnt ? a.cnt + (int64_t)g * a.C + c : nullptr);
+}
+
+// ------------------------------------------------------------------------- centroids from the carried sums
+struct UpdateArgs {
+  const double* sum;      // [G,C,128]
+  const int32_t* cnt;     // [G,C]
+  uint16_t* dst;          // centroids [G,C,128] bf16
+  int32_t* cnt_out;       // [G,C]
+  int64_t d_sg, d_sc;
+  int32_t C, mode;
+};
+
+__global__ __launch_bounds__(kD) void kmeans_update_kernel(UpdateArgs a) {
+  __shared__ double ss_red[kD];
+  const int c = blockIdx.x, g = blockIdx.y, t = threadIdx.x;
+  const double s = a.sum[((int64_t)g * a.C + c) * kD + t];
+  const int cnt = a.cnt[(int64_t)g * a.C + c];
+  finish_cluster(s, cnt, a.mode, ss_red, t, a.dst + (int64_t)g * a.d_sg + (int64_t)c * a.d_sc, a.cnt_out + (int64_t)g * a.C + c);
 }
 
 // ---------------------------------------------------------------------------------- top-k selection
@@ -959,9 +1043,12 @@ __global__ __launch_bounds__(1024) void topk_select_kernel(TopkArgs a) {
 
 struct WsLayout {
   size_t off_bytes, hist_bytes, order_bytes, score_bytes, start_bytes, total_bytes, rec_bytes;
+  size_t sum_bytes, cnt_bytes;   // the sums and sizes carried from step to step (sq_kmeans_train_stateful)
   int nT, C;
   size_t rec_offset() const { return off_bytes + hist_bytes + order_bytes + score_bytes + start_bytes + total_bytes; }
-  size_t all() const { return rec_offset() + rec_bytes; }
+  size_t sum_offset() const { return rec_offset() + rec_bytes; }
+  size_t cnt_offset() const { return sum_offset() + sum_bytes; }
+  size_t all() const { return cnt_offset() + cnt_bytes; }
 };
 
 WsLayout ws_layout(int64_t G, int64_t N, int64_t C) {
@@ -976,6 +1063,8 @@ WsLayout ws_layout(int64_t G, int64_t N, int64_t C) {
   w.start_bytes = up((size_t)G * C * 4);
   w.total_bytes = up((size_t)G * C * 4);
   w.rec_bytes = up((size_t)G * ((N + kBigTile - 1) / kBigTile) * kSlots * kD * 8);
+  w.sum_bytes = up((size_t)G * C * kD * 8);
+  w.cnt_bytes = up((size_t)G * C * 4);
   return w;
 }
 
@@ -1046,7 +1135,7 @@ int run_group(const DLTensor* idx, const DLTensor* src, char* wsp, const WsLayou
 }
 
 // sums of `src` rows per cluster after run_group
-int run_cluster_sum(const DLTensor* src, char* wsp, const WsLayout& w, DLTensor* dst, int32_t* cnt, int mode, hipStream_t st) {
+int run_cluster_sum(const DLTensor* src, char* wsp, const WsLayout& w, DLTensor* dst, int32_t* cnt, int mode, hipStream_t st, bool keep = false) {
   const int64_t G = src->shape[0], N = src->shape[1];
   SumArgs s;
   s.src = (const uint16_t*)data_of(src);
@@ -1063,6 +1152,8 @@ int run_cluster_sum(const DLTensor* src, char* wsp, const WsLayout& w, DLTensor*
   s.C = w.C;
   s.nT = (int)((N + kBigTile - 1) / kBigTile);
   s.mode = mode;
+  s.keep_sum = keep ? (double*)(wsp + w.sum_offset()) : nullptr;
+  s.keep_cnt = keep ? (int32_t*)(wsp + w.cnt_offset()) : nullptr;
   hipLaunchKernelGGL(cluster_sum_kernel, dim3((unsigned)w.C, (unsigned)G), dim3(256), 0, st, s);
   SQ_HIP(hipGetLastError());
   return SQ_OK;
@@ -1095,23 +1186,25 @@ extern "C" size_t sq_kmeans_workspace_bytes(int64_t groups, int64_t num_tokens, 
   return ws_layout(groups, num_tokens, num_centroids).all();
 }
 
-extern "C" int sq_kmeans_train(const DLTensor* data, DLTensor* centroids, DLTensor* idx, DLTensor* cnt, DLTensor* workspace,
-                               int32_t normalize, void* stream) {
-  SQ_REQUIRE(data && centroids && idx && cnt, SQ_EINVAL, "sq_kmeans_train: data, centroids, idx and cnt must be non-null");
+namespace {
+int kmeans_train_impl(const DLTensor* data, DLTensor* centroids, DLTensor* idx, DLTensor* cnt, DLTensor* workspace,
+                      int32_t normalize, int32_t state, void* stream, const char* who) {
+  SQ_REQUIRE(data && centroids && idx && cnt, SQ_EINVAL, "%s: data, centroids, idx and cnt must be non-null", who);
+  SQ_REQUIRE(state >= SQ_KMEANS_STATELESS && state <= SQ_KMEANS_APPLY_CHANGES, SQ_EINVAL, "%s: state %d not supported", who, (int)state);
   const int dev = data->device.device_id;
   int rc;
   if ((rc = check_gnd(data, "data", dev)) || (rc = check_gnd(centroids, "centroids", dev)) || (rc = check_i32(idx, "idx", 2, dev)) ||
       (rc = check_i32(cnt, "cnt", 2, dev)))
     return rc;
   const int64_t G = data->shape[0], N = data->shape[1], C = centroids->shape[1];
-  SQ_REQUIRE(G > 0 && N > 0 && C > 0, SQ_ESHAPE, "sq_kmeans_train: empty tensor");
+  SQ_REQUIRE(G > 0 && N > 0 && C > 0, SQ_ESHAPE, "%s: empty tensor", who);
   SQ_REQUIRE(centroids->shape[0] == G && idx->shape[0] == G && idx->shape[1] == N && cnt->shape[0] == G && cnt->shape[1] == C,
-             SQ_ESHAPE, "sq_kmeans_train: shapes of data/centroids/idx/cnt disagree");
+             SQ_ESHAPE, "%s: shapes of data/centroids/idx/cnt disagree", who);
   SQ_REQUIRE(C % 32 == 0, SQ_ESHAPE, "num_centroids %% 32 != 0 (num_centroids = %lld)", (long long)C);
-  SQ_REQUIRE(C <= kMaxC, SQ_EUNSUPPORTED, "sq_kmeans_train: more than %d centroids", kMaxC);
-  SQ_REQUIRE(N < (1ll << 31) - 65536, SQ_EUNSUPPORTED, "sq_kmeans_train: too many tokens");
+  SQ_REQUIRE(C <= kMaxC, SQ_EUNSUPPORTED, "%s: more than %d centroids", who, kMaxC);
+  SQ_REQUIRE(N < (1ll << 31) - 65536, SQ_EUNSUPPORTED, "%s: too many tokens", who);
   const WsLayout w = ws_layout(G, N, C);
-  if ((rc = check_ws(workspace, w.all(), dev, "sq_kmeans_train")) || (rc = check_current_device(dev, "sq_kmeans_train"))) return rc;
+  if ((rc = check_ws(workspace, w.all(), dev, who)) || (rc = check_current_device(dev, who))) return rc;
   hipStream_t st = (hipStream_t)stream;
   char* wsp = data_of(workspace);
 
@@ -1126,10 +1219,40 @@ extern "C" int sq_kmeans_train(const DLTensor* data, DLTensor* centroids, DLTens
   a.i_sg = stride_of(idx, 0);
   a.N = (int)N;
   a.C = (int)C;
-  hipLaunchKernelGGL(kmeans_assign_kernel, dim3((unsigned)((N + kTileTok - 1) / kTileTok), (unsigned)G), dim3(kAssignWaves * 64), 0, st, a);
+  a.keep_sum = (double*)(wsp + w.sum_offset());
+  a.keep_cnt = (int32_t*)(wsp + w.cnt_offset());
+  const dim3 agrid((unsigned)((N + kTileTok - 1) / kTileTok), (unsigned)G);
+  const int mode = normalize ? 2 : 1;
+  if (state == SQ_KMEANS_APPLY_CHANGES) {
+    hipLaunchKernelGGL(kmeans_assign_kernel<true>, agrid, dim3(kAssignWaves * 64), 0, st, a);
+    UpdateArgs u;
+    u.sum = a.keep_sum;
+    u.cnt = a.keep_cnt;
+    u.dst = (uint16_t*)data_of(centroids);
+    u.cnt_out = (int32_t*)data_of(cnt);
+    u.d_sg = stride_of(centroids, 0);
+    u.d_sc = stride_of(centroids, 1);
+    u.C = (int)C;
+    u.mode = mode;
+    hipLaunchKernelGGL(kmeans_update_kernel, dim3((unsigned)C, (unsigned)G), dim3(kD), 0, st, u);
+    SQ_HIP(hipGetLastError());
+    return SQ_OK;
+  }
+  hipLaunchKernelGGL(kmeans_assign_kernel<false>, agrid, dim3(kAssignWaves * 64), 0, st, a);
   SQ_HIP(hipGetLastError());
   if ((rc = run_group(idx, data, wsp, w, st))) return rc;
-  return run_cluster_sum(data, wsp, w, centroids, (int32_t*)data_of(cnt), normalize ? 2 : 1, st);   // cnt = cluster sizes
+  return run_cluster_sum(data, wsp, w, centroids, (int32_t*)data_of(cnt), mode, st, state == SQ_KMEANS_KEEP_SUMS);   // cnt = cluster sizes
+}
+}  // namespace
+
+extern "C" int sq_kmeans_train(const DLTensor* data, DLTensor* centroids, DLTensor* idx, DLTensor* cnt, DLTensor* workspace,
+                               int32_t normalize, void* stream) {
+  return kmeans_train_impl(data, centroids, idx, cnt, workspace, normalize, SQ_KMEANS_STATELESS, stream, "sq_kmeans_train");
+}
+
+extern "C" int sq_kmeans_train_stateful(const DLTensor* data, DLTensor* centroids, DLTensor* idx, DLTensor* cnt, DLTensor* workspace,
+                                        int32_t normalize, int32_t state, void* stream) {
+  return kmeans_train_impl(data, centroids, idx, cnt, workspace, normalize, state, stream, "sq_kmeans_train_stateful");
 }
 
 extern "C" int sq_reverse_index(const DLTensor* idx, DLTensor* clusters, DLTensor* cluster_size, DLTensor* workspace, void* stream) {

@@ -241,3 +241,74 @@ def test_kmeans_configurations_drawn_at_random():
         rc, rs = KM.reverse_index(idx, C, max_cnt)
         assert torch.equal(size.cpu(), rs) and torch.equal(clusters.cpu(), rc), case
         assert torch.equal(vsum.cpu(), KM.index_add(value, idx, C)), case
+
+
+@pytest.mark.parametrize("G,N,C,modes", [(2, 5000, 64, 20), (1, 40000, 1024, 300), (3, 777, 32, 5)])
+def test_carried_sums_give_the_bits_of_the_full_resum(G, N, C, modes):
+    """`sq_kmeans_train_stateful`: a run of Lloyd steps whose cluster sums are carried in the workspace (one step that
+    keeps them, then steps that only apply the tokens that changed cluster) against the same run with every step
+    re-summing every row.  The sums are exact, so centroids, assignment and sizes must be equal bit for bit after every
+    step -- normalised and un-normalised steps, empty clusters, N not a multiple of the 256-token tile, and a step in
+    which nothing moves."""
+    from longcontext_sqattn_paddle_amd import _native as NV
+    from longcontext_sqattn_paddle_amd.cache_hub.kmeans import _triton_k_means_train, _workspace
+
+    print(f"case k-means carried sums G={G} N={N} C={C}", flush=True)
+    key, _ = inputs.kmeans_inputs(G, N, 128, n_modes=modes, seed=70 + C)
+    data = key.to(DEV)
+    sel = KM.init_centroid_indices(N, C).to(DEV)
+    ca, cb = data.index_select(1, sel).contiguous(), data.index_select(1, sel).contiguous()
+    ia = torch.empty(G, N, dtype=torch.int32, device=DEV)
+    ib = torch.full((G, N), -7, dtype=torch.int32, device=DEV)
+    wa, wb = _workspace(G, N, C, DEV), _workspace(G, N, C, DEV)
+    wb.fill_(0x5A)      # whatever the workspace held before must not matter
+    moved = []
+    for step in range(9):
+        norm = step != 5                                   # one un-normalised step in the middle of the run
+        state = NV.KMEANS_STATELESS if step == 0 else (NV.KMEANS_KEEP_SUMS if step == 1 else NV.KMEANS_APPLY_CHANGES)
+        prev = ib.clone()
+        _, _, max_a = _triton_k_means_train(data, ca, max_idx=ia, normalize_centroids=norm, return_indices=True, workspace=wa)
+        _, _, max_b = _triton_k_means_train(data, cb, max_idx=ib, normalize_centroids=norm, return_indices=True, workspace=wb, state=state)
+        torch.cuda.synchronize()
+        moved.append(int((prev != ib).sum()))
+        assert torch.equal(ia, ib), step
+        assert torch.equal(ca.view(torch.int16), cb.view(torch.int16)), step
+        assert max_a == max_b, step
+    print(f"  tokens that changed cluster per step: {moved}", flush=True)
+    # a step in which nothing moves (the same centroids again cannot be had, but the same assignment can: feed the
+    # centroids of the stateless run, which are equal, and repeat until the assignment is stable or 20 steps have passed)
+    for _ in range(20):
+        prev = ib.clone()
+        _triton_k_means_train(data, ca, max_idx=ia, normalize_centroids=True, workspace=wa)
+        _triton_k_means_train(data, cb, max_idx=ib, normalize_centroids=True, workspace=wb, state=NV.KMEANS_APPLY_CHANGES)
+        torch.cuda.synchronize()
+        assert torch.equal(ia, ib) and torch.equal(ca.view(torch.int16), cb.view(torch.int16))
+        if torch.equal(prev, ib):
+            break
+    # the sizes the carried state reports are the histogram of the assignment
+    cnt = torch.empty(G, C, dtype=torch.int32, device=DEV)
+    b = [NV.dl(t) for t in (data, cb, ib, cnt, wb)]
+    NV.check(NV.lib().sq_kmeans_train_stateful(*[NV.ptr(x) for x in b], 1, NV.KMEANS_APPLY_CHANGES, NV.current_stream(data.device)))
+    torch.cuda.synchronize()
+    for g in range(G):
+        assert torch.equal(cnt[g].cpu().long(), torch.bincount(ib[g].cpu().long(), minlength=C))
+
+
+def test_segment_k_means_with_carried_sums_equals_stateless_steps():
+    """`segment_k_means` carries the sums from its fourth step on; written out with stateless steps only it must return
+    the same centroids, value sums, clusters and sizes (one segment, where the last step continues the carried run, and
+    two, where it starts over on the unsegmented data)."""
+    from longcontext_sqattn_paddle_amd.cache_hub import kmeans as HK
+
+    key, value = inputs.kmeans_inputs(2, 6000, 128, n_modes=40, seed=81)
+    key, value = key.to(DEV), value.to(DEV)
+    for segments in (1, 2):
+        got = HK.segment_k_means(key, value, 64, num_iters=8, num_segments=segments)
+        saved, HK.FULL_RESUM_STEPS = HK.FULL_RESUM_STEPS, 1 << 30       # every step stateless
+        try:
+            want = HK.segment_k_means(key, value, 64, num_iters=8, num_segments=segments)
+        finally:
+            HK.FULL_RESUM_STEPS = saved
+        torch.cuda.synchronize()
+        for a, b in zip(got, want):
+            assert a.shape == b.shape and torch.equal(a.view(torch.int16) if a.dtype == torch.bfloat16 else a, b.view(torch.int16) if b.dtype == torch.bfloat16 else b), segments
