@@ -214,7 +214,7 @@ def time_plugin(torch, qkv, steps=3):
     return out
 
 
-def time_decode(torch, B, L, iters=10, warmup=5, rounds=7):
+def time_decode(torch, B, L, iters=10, warmup=5, rounds=7, preheat=None):
     from longcontext_sqattn_paddle_amd.sqattn.attn_triton_decode import DecodePlan
 
     dev = torch.device("cuda:0")
@@ -236,6 +236,8 @@ def time_decode(torch, B, L, iters=10, warmup=5, rounds=7):
     torch.cuda.synchronize()
     samples = []
     for _ in range(rounds):   # median over rounds of `iters` back-to-back calls (HIP events on the launch stream)
+        if preheat is not None:   # queued on the same stream right in front of the timed calls
+            preheat()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record(stream)
         for i in range(iters):
@@ -888,9 +890,6 @@ def main():
     if not args.no_plugin:
         result["plugin"] = time_plugin(torch, qkv)
         log(f"[bench] plugin closure: {result['plugin']}")
-    del qkv
-    torch.cuda.empty_cache()
-
     def settle():
         # The prefill legs above run the matrix cores at the chip's power limit for several seconds; a leg measured
         # right behind them inherits that state (the 1M-token decode reads 322 us then and 307 - 312 us from an idle
@@ -900,16 +899,36 @@ def main():
 
     result["settle_s"] = args.settle
     if not args.no_decode:
-        settle()
+        # Every decode leg is timed under two conditions: from a chip that has idled for `settle` seconds, and "hot",
+        # right behind half a second of prefill attention at the power limit (what a serving loop that interleaves
+        # prefill and decode sees).
+        ws_heat = None
+
+        def heat():
+            nonlocal ws_heat
+            from longcontext_sqattn_paddle_amd.sqattn._prefill import prefill_workspace
+            from longcontext_sqattn_paddle_amd.sqattn.attn_triton import attn_causal
+
+            if ws_heat is None:
+                ws_heat = (prefill_workspace(1, 4, N, qkv[0].device), torch.empty_like(qkv[0]))
+            for _ in range(6):
+                attn_causal(qkv[0], qkv[1], qkv[2], "HND", torch.bfloat16, p_quant=args.p_quant, workspace=ws_heat[0], out=ws_heat[1])
+
         dec = {}
         for name, B, L in (("1M_b1", 1, 1048576), ("128K_b1", 1, 131072), ("128K_b4", 4, 131072), ("128K_b8", 8, 131072)):
+            settle()
             us, nbytes = time_decode(torch, B, L)
+            us_hot, _ = time_decode(torch, B, L, preheat=heat)
             gbs = nbytes / us / 1e3
             dec[name] = {"us_per_call": round(us, 2), "GB_per_s": round(gbs, 1), "frac_of_hbm_peak": round(gbs / PEAK_HBM_GBS, 4),
+                         "us_per_call_hot": round(us_hot, 2), "frac_of_hbm_peak_hot": round(nbytes / us_hot / 1e3 / PEAK_HBM_GBS, 4),
                          "bytes": nbytes}
-            log(f"[bench] decode {name}: {us:.1f} us, {gbs:.0f} GB/s")
+            log(f"[bench] decode {name}: {us:.1f} us, {gbs:.0f} GB/s; right behind prefill work {us_hot:.1f} us")
             torch.cuda.empty_cache()
+        dec["note"] = ("us_per_call: after settle_s seconds of idle time; us_per_call_hot: timed immediately behind six prefill attention "
+                       "calls (0.45 s at the power limit)")
         result["decode"] = dec
+        ws_heat = None
         sel = {}
         for name, B, L, k, run in (("4096_of_128K_b1", 1, 131072, 4096, 1), ("4096_of_128K_b8", 8, 131072, 4096, 1),
                                    ("65536_of_1M_b1", 1, 1048576, 65536, 1), ("65536_of_1M_b1_runs_of_64", 1, 1048576, 65536, 64),
@@ -919,6 +938,8 @@ def main():
             log(f"[bench] decode over selected tokens {name}: {us:.1f} us, {nbytes / us / 1e3:.0f} GB/s")
             torch.cuda.empty_cache()
         result["decode_selected"] = sel
+    del qkv
+    torch.cuda.empty_cache()
     if not args.no_prepass:
         settle()
         pre = {}

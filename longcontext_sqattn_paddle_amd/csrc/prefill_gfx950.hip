@@ -580,12 +580,18 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
   // cinit = kC - m_run (kC = log2(448) in MODE 3, else 0), so the MFMA chain delivers S - m_run + kC and, as
   // long as the running maximum does not move, p (or 448 p) is a bare exp2 of the accumulator.
   constexpr float kC = (MODE >= 3 && MODE <= 5) ? kLog2_448 : 0.f;
-  // Lazy re-centring (MODE 5): a row maximum may rise up to kLazy (in log2 units) above the reference before the
-  // accumulators are rescaled; the block scale absorbs any power of two (its exponent then exceeds 127), while the
-  // fp32 accumulators and the denominator carry the common factor until the division at the end.  A row is shifted
-  // only when its own maximum passes the limit, so its arithmetic does not depend on the other rows of the wave.
-  // The other modes keep the reference's rounding points (fp16 P, static e4m3 scale) and re-centre at once.
-  constexpr float kLazy = (MODE == 5) ? 16.f : 0.f;
+  // Lazy re-centring (MODE 5 and MODE 0): a row maximum may rise up to kLazy (in log2 units) above the reference before
+  // the accumulators are rescaled.  MODE 5: the block scale absorbs any power of two (its exponent then exceeds 127),
+  // while the fp32 accumulators and the denominator carry the common factor until the division at the end.  MODE 0: p
+  // is rounded to fp16, which has the same ten mantissa bits at 2^8 as at 1, so p = 2^(s - reference) up to 2^8 is the
+  // same probability with the same relative rounding error (2^-11) as the reference's 2^(s - running maximum) <= 1 --
+  // not the same bits, and small probabilities keep more of their bits than there.  A row is shifted only when its own
+  // maximum passes the limit, so its arithmetic does not depend on the other rows of the wave.  With re-centring at once,
+  // one row of the wave's 32 finding a new maximum sends the whole wave through the rescale path (some 110 vector
+  // instructions): about 32 (1 + ln(tiles / 32)) times per wave, which is 8 % of the tiles of a 131072-key causal row
+  // and 40 % of the 214 tiles of a sink + 10 % window.  The e4m3 modes with the static scale (1, 3, 4) need p <= 1 for
+  // their grid and re-centre at once.
+  constexpr float kLazy = (MODE == 5) ? 16.f : (MODE == 0 ? 8.f : 0.f);
   constexpr float kMove = kC + kLazy;
   float m_run = 0.f;       // reference point of the exponent; the first visited tile replaces it by the row maximum
   float l_run = 0.f;       // this lane's share of the denominator (times 448 in MODE 3)

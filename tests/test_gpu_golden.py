@@ -30,7 +30,7 @@ def test_prefill_fixture():
         d = (out.double().cpu() - ref).abs()
         rms = float(ref.pow(2).mean().sqrt())
         if band is None:
-            return float(d.max()) <= 2e-3 * rms
+            return float(d.max()) <= 2e-3 * rms + 2.0 ** -11 * float(ref.abs().max())   # (fp16 p relative to a lazily moved reference point)
         # a probability within an ulp of an e4m3 boundary may land on the neighbouring grid value
         return float(d.flatten().kthvalue(int(0.999 * d.numel())).values) <= band * rms and float(d.max()) <= 0.25 * rms
 
@@ -50,7 +50,7 @@ def test_prefill_fixture():
     out, lse = run_prefill(q, k, v, tensor_layout="HND", output_dtype=torch.float32, return_lse=True, p_quant=0, window=window)
     torch.cuda.synchronize()
     ref = torch.from_numpy(z["out_window"]).double()
-    assert float((out.double().cpu() - ref).abs().max()) <= 2e-3 * float(ref.pow(2).mean().sqrt())
+    assert float((out.double().cpu() - ref).abs().max()) <= 2e-3 * float(ref.pow(2).mean().sqrt()) + 2.0 ** -11 * float(ref.abs().max())
     assert np.allclose(lse.cpu().numpy(), z["lse_window"], atol=2e-4)
     out, lse = run_prefill(q, k, v, tensor_layout="HND", output_dtype=torch.float32, return_lse=True, p_quant=5, window=window)
     torch.cuda.synchronize()

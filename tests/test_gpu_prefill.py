@@ -1,7 +1,10 @@
 """GPU parity: prefill kernel (through the C ABI) against the CPU oracle.
 
 Stated tolerances.  Kernel vs the same-algorithm oracle (identical quantisation points; only v_exp_f32 and
-fp32 summation order differ): without P quantisation max|d| <= 2e-3 * rms(out); with e4m3 P a few
+fp32 summation order differ): without P quantisation max|d| <= 2e-3 * rms(out) + 2^-11 * max|out| -- the second term
+because the kernel rounds p to fp16 relative to a reference point that may trail the row's running maximum by up to
+2^8 (the same probability with the same relative rounding error 2^-11 as the reference's, but a dominant key no longer
+has p = 1 exactly); with e4m3 P a few
 probabilities sit within an ulp of a rounding boundary and flip to the neighbouring e4m3 value, so the
 check is cosine >= 0.99999, 99.9 % of elements within 2e-3 * rms and every element within 0.25 * rms.
 Kernel vs exact attention: cosine >= 0.999 (the bar of the benchmark configuration).
@@ -28,7 +31,7 @@ def _check(out, ref, quantised, q_tol=2e-3):
     rms = float(ref.pow(2).mean().sqrt())
     d = (out - ref).abs()
     if not quantised:
-        assert float(d.max()) <= 2e-3 * rms, (float(d.max()), rms)
+        assert float(d.max()) <= 2e-3 * rms + 2.0 ** -11 * float(ref.abs().max()), (float(d.max()), rms)
     else:
         assert _cos(out, ref) >= 0.99999
         assert float(torch.quantile(d.flatten()[:: max(1, d.numel() // 1000000)], 0.999)) <= q_tol * rms
