@@ -25,9 +25,22 @@ PEAK_MFMA_FP8_TFLOPS = 5000.0    # MI355X dense fp8 MFMA
 # Q.K^T (half of the FLOPs) runs on the bf16 pipe, P.V (the other half) on the fp8 pipe in the default mode
 PEAK_MFMA_BLEND_TFLOPS = 1.0 / (0.5 / PEAK_MFMA_BF16_TFLOPS + 0.5 / PEAK_MFMA_FP8_TFLOPS)
 PEAK_HBM_GBS = 8000.0            # MI355X HBM3E
-# L2<->fabric bytes of one prefill_kernel launch at seq 131072, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a
-# 1 GiB copy (x2.000 / x1.000): 12.43 GB fetched + 0.94 GB written in P mode 5; mode 4 moves the same tiles (profiles/prefill_kernel_128k.md)
-PREFILL_TRAFFIC_BYTES_128K = 13.4e9
+
+
+def prefill_traffic_bytes(N, p_quant):
+    """L2<->fabric bytes of one prefill_kernel launch, from the committed rocprofv3 FETCH_SIZE / WRITE_SIZE summary of this
+    shape (profiles/prefill_kernel_128k.traffic.json: counters in KiB, each scaled by what the same counter read for a
+    1 GiB copy); None for shapes and P modes the summary does not cover."""
+    if N != 131072 or p_quant < 4:
+        return None
+    try:
+        with open(os.path.join(ROOT, "profiles", "prefill_kernel_128k.traffic.json")) as f:
+            t = json.load(f)
+        return (t["fetch_size_kib"] * t["fetch_scale"] + t["write_size_kib"] * t["write_scale"]) * 1024.0
+    except (OSError, KeyError, ValueError):
+        return None
+
+
 P_MODE_NOTE = {
     0: "no P quantisation",
     4: "e4m3 P with the static scale 448 and e4m3 V, fp8 MFMA P.V",
@@ -859,9 +872,9 @@ def main():
             "unit": "TFLOP/s",
             "frac": round(tflops / peak, 4),
             "frac_of_bf16_peak": round(tflops / PEAK_MFMA_BF16_TFLOPS, 4),
-            "traffic": PREFILL_TRAFFIC_BYTES_128K if (N == 131072 and args.p_quant >= 4) else None,
-            "traffic_note": "bytes per launch through the L2/fabric interface, a constant taken from the committed rocprofv3 FETCH_SIZE / "
-                            "WRITE_SIZE runs of this shape (profiles/prefill_kernel_128k.md), not re-measured by this run; null for other shapes",
+            "traffic": prefill_traffic_bytes(N, args.p_quant),
+            "traffic_note": "bytes per launch through the L2/fabric interface, read from the committed rocprofv3 FETCH_SIZE / WRITE_SIZE "
+                            "summary of this shape (profiles/prefill_kernel_128k.traffic.json), not re-measured by this run; null for other shapes",
             "numerics": "P mode 5 is build-defined (the reference multiplies fp16 P by fp16 V): see `variants` for the reference's own modes",
         },
     }

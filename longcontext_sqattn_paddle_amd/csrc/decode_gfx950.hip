@@ -67,9 +67,12 @@ constexpr int kMaxShareBatch = 32;
 // mode.  The split kernel (want_b < 0: finds the owner of workgroup w) and the combine kernel (want_b = its sequence)
 // both call this, so they agree by construction.
 // Every wave computes the whole table at once, one sequence per lane (B <= 32): one load, an integer prefix sum by
-// shuffles (lengths in units of 32 tokens, so that 32 sequences of 2^31 tokens fit 32 bits), one 64-bit integer
-// division per lane -- exact arithmetic, so the two kernels cannot disagree whatever flags they are compiled with.  A
-// loop over the sequences with a load and a division in every round took longer than the rest of the combine kernel.
+// shuffles (lengths in units of 32 tokens, so that 32 sequences of 2^31 tokens fit 32 bits), one 32-bit integer division
+// per lane -- exact arithmetic, so the two kernels cannot disagree whatever flags they are compiled with.  For the
+// division the prefix and the total are shifted right until the total is below 2^20 (the product with W - B < 2^12 then
+// fits 32 bits; a 64-bit division is a software routine that cost the combine kernel 3 us at batch 8): the shares stay
+// monotone and add up to W exactly, and proportional to 2^-20.  A loop over the sequences with a load and a division
+// in every round took longer than the rest of the combine kernel.
 __device__ __forceinline__ void share_of(const int32_t* seqlens, int B, int Lmax, int W, int want_b, int w, int& b, int& base, int& n) {
   const int lane = threadIdx.x & 63;
   const uint32_t len = lane < B ? ((uint32_t)min(max(seqlens[lane], 0), Lmax) + 31u) >> 5 : 0u;
@@ -80,7 +83,9 @@ __device__ __forceinline__ void share_of(const int32_t* seqlens, int B, int Lmax
     if (lane >= d) cum += v;
   }
   const uint32_t total = __shfl(cum, B - 1);
-  const int e1 = total > 0u ? (int)((uint64_t)(uint32_t)(W - B) * cum / total) : 0;   // W - B exactly for the last sequence
+  const int sh = max(0, 12 - (int)__builtin_clz(total | 1u));       // total >> sh < 2^20
+  const uint32_t ts = total >> sh;
+  const int e1 = ts > 0u ? (int)((uint32_t)(W - B) * (cum >> sh) / ts) : 0;   // W - B exactly for the last sequence
   int e0 = __shfl_up(e1, 1);
   if (lane == 0) e0 = 0;
   const int bs = lane + e0, ni = 1 + e1 - e0;

@@ -144,8 +144,9 @@ def test_delayed_sdpa_wrapper_quantised_branch_matches_the_oracle():
 def test_decode_shares_by_length_add_up():
     """The rule by which the decode kernels deal the W workgroups of a ragged batch to its sequences (csrc/decode_gfx950.hip,
     share_of): every sequence one workgroup, the other W - B by cumulative rounding down of (W - B) * prefix / total in
-    64-bit integers, the lengths counted in units of 32 tokens.  Replayed in Python integers: the shares are positive, add
-    up to W exactly, stay within one of a sequence's proportional share, and follow the lengths."""
+    32-bit integers, the lengths counted in units of 32 tokens and prefix and total shifted right until the total is
+    below 2^20.  Replayed in Python integers: the product fits 32 bits, the shares are positive, add up to W exactly, stay
+    within one (plus 2^-19 of W - B) of a sequence's proportional share, and follow the lengths."""
     import numpy as np
 
     rng = np.random.default_rng(11)
@@ -165,8 +166,10 @@ def test_decode_shares_by_length_add_up():
         units = (lens.astype(np.uint64) + 31) >> 5
         cum = np.cumsum(units).astype(np.uint32)           # fits 32 bits: 32 sequences of 2^26 units
         total = cum[-1]
-        assert (W - B) * int(total) < 2 ** 64              # the kernel's product fits its 64-bit integer
-        e1 = np.array([(W - B) * int(c) // int(total) for c in cum], dtype=np.int64) if total > 0 else np.zeros(B, np.int64)
+        sh = max(0, int(total).bit_length() - 20)
+        ts = int(total) >> sh
+        assert ts < 2 ** 20 and (W - B) * ts < 2 ** 32       # the kernel's product fits its 32-bit integer
+        e1 = np.array([(W - B) * (int(c) >> sh) // ts for c in cum], dtype=np.int64) if ts > 0 else np.zeros(B, np.int64)
         e0 = np.concatenate([[0], e1[:-1]])
         n = 1 + e1 - e0
         base = np.arange(B) + e0
@@ -174,7 +177,7 @@ def test_decode_shares_by_length_add_up():
         if total > 0:
             assert int(n.sum()) == W and int(base[-1] + n[-1]) == W
             want = (W - B) * units.astype(np.float64) / float(total)
-            assert (np.abs((n - 1) - want) < 1.0 + 1e-9).all()
+            assert (np.abs((n - 1) - want) < 1.0 + (W - B) * 2.0 ** -19 + 1e-9).all()
         else:
             assert (n == 1).all()
         assert (base[1:] == base[:-1] + n[:-1]).all()
