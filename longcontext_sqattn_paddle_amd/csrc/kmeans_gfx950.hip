@@ -5,9 +5,10 @@
 //   _triton_reverse_index_kernel :199-262, _triton_index_add_kernel :265-329.
 // The reference scatters every token into its cluster sum with fp32 atomics (16.8 M atomics per head and
 // iteration at 131072 x 128).  Here the assignment is a dense bf16 MFMA contraction with an arg-max
-// epilogue in registers, tokens are then counting-sorted by cluster (deterministic, ascending inside a
-// cluster) and every cluster is summed by one workgroup in fp64, which is exact for bf16 data and therefore
-// independent of order.  The same sort yields the reverse index.
+// epilogue in registers, tokens are then grouped by cluster tile by tile and every cluster is summed by one
+// workgroup in fp64, which is exact for bf16 data and therefore independent of order -- and of how the sums were
+// arrived at: a run of iterations may keep them in the workspace and apply only the tokens that changed cluster
+// (sq_kmeans_train_stateful).  A counting sort in ascending token order yields the reverse index.
 #include "common.hpp"
 
 namespace sq {

@@ -186,7 +186,8 @@ def test_absolute_windows_with_4bit_operands_128k(w8, w4):
     """The absolute-window launch with separate 4-bit operands (attn_triton_mix_bad.py:285-426) at the prefill benchmark
     shape, through the closure `mp_triton_wrapper` builds for `use_relative_distance = False`: 128-row query blocks, the
     4-bit range really multiplied with the 4-bit fake-quantised query and key.  It is the one configuration that runs
-    the 4-wave workgroups; here their 64-bit tile bases, the switch of the query operand set at the edges of the 4-bit
+    the workgroups of two query blocks (the tiles on which the blocks want different key operands walked twice); here
+    their 64-bit tile bases, the switch of the query operand set at the edges of the 4-bit
     range and the per-head windows (one head with both windows equal, one with a 128-token 8-bit window, one wider than
     the sequence) run at N = 131072.  Sampled rows against the float64 closed form over the oracle's key ranges on the
     oracle's fake-quantised operands."""

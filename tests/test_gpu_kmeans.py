@@ -177,6 +177,68 @@ def test_topk_select_shared_score_phase_repeated():
         assert torch.equal(o.cpu(), want[i % 2]), i
 
 
+def _shared_phase_case(seed):
+    B, Hkv, groups, N, C, k = 1, 4, 7, 8192, 1024, 1000
+    g = torch.Generator().manual_seed(seed)
+    idx = torch.randint(0, C, (B * Hkv, N), generator=g, dtype=torch.int32)
+    msize = int(torch.stack([torch.bincount(idx[i].long(), minlength=C) for i in range(B * Hkv)]).max())
+    clusters, size = KM.reverse_index(idx, C, msize)
+    cent = torch.randn(B * Hkv, C, 128, generator=g).bfloat16()
+    q = torch.randn(B, Hkv * groups, 128, generator=g).bfloat16()
+    return q, cent, clusters, size, k, groups
+
+
+@pytest.mark.parametrize("fill", ["ones", "random", "finished", "other_shape"])
+def test_topk_select_arrival_words_need_no_initialisation(fill):
+    """The arrival words of the shared score phase live in the caller's workspace and are never cleared by the host.
+    Whatever the memory holds -- all bits set, random words, the word a finished call leaves, or the words of a call
+    with another number of heads -- the first call over it must select what the oracle selects."""
+    from longcontext_sqattn_paddle_amd.cache_hub.kmeans import _workspace, topk_select
+
+    q, cent, clusters, size, k, groups = _shared_phase_case(83)
+    G, C = cent.shape[0], cent.shape[1]
+    want = KM.topk_select(q, cent, clusters, size, k, groups)
+    ws = _workspace(G, 1, C, DEV)
+    words = ws[: ws.numel() // 4 * 4].view(torch.int32)
+    if fill == "ones":
+        ws.fill_(0xFF)
+    elif fill == "random":
+        words.copy_(torch.randint(-2**31, 2**31 - 1, (words.numel(),), generator=torch.Generator().manual_seed(5),
+                                  dtype=torch.int64).to(torch.int32).to(DEV))
+    elif fill == "finished":
+        topk_select(q.to(DEV), cent.to(DEV), clusters.to(DEV), size.to(DEV), k, groups, workspace=ws)
+    else:   # a call over 2 of the 4 heads first, then all 4 over the same memory
+        topk_select(q[:, : 2 * groups].to(DEV), cent[:2].to(DEV), clusters[:2].to(DEV), size[:2].to(DEV), k, groups,
+                    workspace=ws)
+    for _ in range(3):
+        got = topk_select(q.to(DEV), cent.to(DEV), clusters.to(DEV), size.to(DEV), k, groups, workspace=ws)
+        torch.cuda.synchronize()
+        assert torch.equal(got.cpu(), want)
+
+
+def test_topk_select_two_workspaces_on_two_streams():
+    """Calls that use different workspaces share nothing: two selections with different queries run on two streams at
+    the same time, 200 times, and each must equal its own oracle result."""
+    from longcontext_sqattn_paddle_amd.cache_hub.kmeans import _workspace, topk_select
+
+    cases = [_shared_phase_case(s) for s in (85, 86)]
+    want = [KM.topk_select(*c) for c in cases]
+    dev = [[x.to(DEV) if torch.is_tensor(x) else x for x in c] for c in cases]
+    G, C = cases[0][1].shape[0], cases[0][1].shape[1]
+    wss = [_workspace(G, 1, C, DEV) for _ in cases]
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    torch.cuda.synchronize()
+    outs = [[], []]
+    for _ in range(200):
+        for i in (0, 1):
+            with torch.cuda.stream(streams[i]):
+                outs[i].append(topk_select(*dev[i], workspace=wss[i]))
+    torch.cuda.synchronize()
+    for i in (0, 1):
+        for o in outs[i]:
+            assert torch.equal(o.cpu(), want[i])
+
+
 def test_full_size_properties():
     """Benchmark shape (4 heads x 131072 tokens x 128, 1024 centroids): size-independent invariants plus an
     oracle check on a token sample."""
