@@ -530,45 +530,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
   typedef __attribute__((ext_vector_type(16))) int i32x16_t;
   i32x4_t qc[4] = {};
   float q_scale = 0.f;
-  if constexpr (kQK8) {
-    const uint16_t* qp = (const uint16_t*)a.q + (int64_t)b * a.q_sb + (int64_t)head * a.q_sh;
-    const int row = max(min(row_w0 + c32, a.Nq - 1), 0);
-    const uint16_t* rp = qp + (int64_t)row * a.q_sn + 16 * g;
-    uint4 raw[4][2];
-#pragma unroll
-    for (int kk = 0; kk < 4; ++kk) {
-      raw[kk][0] = *(const uint4*)(rp + 32 * kk);
-      raw[kk][1] = *(const uint4*)(rp + 32 * kk + 8);
-    }
-    float amax = 0.f;
-#pragma unroll
-    for (int kk = 0; kk < 4; ++kk)
-#pragma unroll
-      for (int hf = 0; hf < 2; ++hf) {
-        const uint32_t w[4] = {raw[kk][hf].x, raw[kk][hf].y, raw[kk][hf].z, raw[kk][hf].w};
-#pragma unroll
-        for (int j = 0; j < 4; ++j) amax = fmaxf(amax, fmaxf(fabsf(elem16<BF16>(w[j] & 0xffffu)), fabsf(elem16<BF16>(w[j] >> 16))));
-      }
-    amax = fmaxf(xor32_max(amax), 1e-5f);
-    const Divisor scale = make_divisor(amax / 127.f);
-    auto code = [&](float x) {   // clamp(round(x / scale), -128, 127), fake_quant.py:114-116
-      const float t = divide(x, scale);
-      return (uint32_t)((int)fminf(fmaxf(copysignf(floorf(fabsf(t) + 0.5f), t) + 0.0f, -128.f), 127.f) & 0xff);
-    };
-#pragma unroll
-    for (int kk = 0; kk < 4; ++kk)
-#pragma unroll
-      for (int hf = 0; hf < 2; ++hf) {
-        const uint32_t w[4] = {raw[kk][hf].x, raw[kk][hf].y, raw[kk][hf].z, raw[kk][hf].w};
-#pragma unroll
-        for (int j = 0; j < 2; ++j)   // four elements (two words) per code word
-          qc[kk][2 * hf + j] = (int)(code(elem16<BF16>(w[2 * j] & 0xffffu)) | (code(elem16<BF16>(w[2 * j] >> 16)) << 8) |
-                                     (code(elem16<BF16>(w[2 * j + 1] & 0xffffu)) << 16) | (code(elem16<BF16>(w[2 * j + 1] >> 16)) << 24));
-      }
-    q_scale = scale.d * a.sm;
-  } else {
-    load_q(a.q);
-  }
+  // (the query rows are loaded further down, behind the first tile copies, so that both travel at the same time)
   bool q_is4 = false;
 
   f32x16_t O[4];
@@ -1113,6 +1075,46 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
     stage_v(tile_of(1), 1);
   }
   if (2 < nTot) stage_k(tile_of(2), 2, step_uses4(2));
+  // the wave's query rows, requested while the first tiles are on their way
+  if constexpr (kQK8) {
+    const uint16_t* qp = (const uint16_t*)a.q + (int64_t)b * a.q_sb + (int64_t)head * a.q_sh;
+    const int row = max(min(row_w0 + c32, a.Nq - 1), 0);
+    const uint16_t* rp = qp + (int64_t)row * a.q_sn + 16 * g;
+    uint4 raw[4][2];
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      raw[kk][0] = *(const uint4*)(rp + 32 * kk);
+      raw[kk][1] = *(const uint4*)(rp + 32 * kk + 8);
+    }
+    float amax = 0.f;
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk)
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf) {
+        const uint32_t w[4] = {raw[kk][hf].x, raw[kk][hf].y, raw[kk][hf].z, raw[kk][hf].w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) amax = fmaxf(amax, fmaxf(fabsf(elem16<BF16>(w[j] & 0xffffu)), fabsf(elem16<BF16>(w[j] >> 16))));
+      }
+    amax = fmaxf(xor32_max(amax), 1e-5f);
+    const Divisor scale = make_divisor(amax / 127.f);
+    auto code = [&](float x) {   // clamp(round(x / scale), -128, 127), fake_quant.py:114-116
+      const float t = divide(x, scale);
+      return (uint32_t)((int)fminf(fmaxf(copysignf(floorf(fabsf(t) + 0.5f), t) + 0.0f, -128.f), 127.f) & 0xff);
+    };
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk)
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf) {
+        const uint32_t w[4] = {raw[kk][hf].x, raw[kk][hf].y, raw[kk][hf].z, raw[kk][hf].w};
+#pragma unroll
+        for (int j = 0; j < 2; ++j)   // four elements (two words) per code word
+          qc[kk][2 * hf + j] = (int)(code(elem16<BF16>(w[2 * j] & 0xffffu)) | (code(elem16<BF16>(w[2 * j] >> 16)) << 8) |
+                                     (code(elem16<BF16>(w[2 * j + 1] & 0xffffu)) << 16) | (code(elem16<BF16>(w[2 * j + 1] >> 16)) << 24));
+      }
+    q_scale = scale.d * a.sm;
+  } else {
+    load_q(a.q);
+  }
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
   // Q~ fragments of the other operand set, one 16-byte piece at a time (a handful of switches per wave: no need for all
