@@ -555,6 +555,17 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
   // their grid and re-centre at once.
   constexpr float kLazy = (MODE == 5) ? 16.f : (MODE == 0 ? 8.f : 0.f);
   constexpr float kMove = kC + kLazy;
+  // MODE 5 takes neither the block scale nor the decision to move the reference from the row's maximum of the tile but
+  // from the row's SUM of the tile's probabilities, which the denominator needs anyway: the maximum tree (26 vector
+  // instructions per tile) goes.  The probabilities of a tile are formed against the standing reference without looking
+  // at the scores first; a row whose sum then exceeds 2^kLazy moves its reference up by a whole number of binades
+  // (exact rescaling, also of the tile just packed, through the scale operand of its MFMA), and a row whose sum is not
+  // finite -- a score more than 2^100 above everything the row has seen -- has the tile recomputed from the key rows in
+  // memory against the tile's own maximum (redo_tile).  The scale needs the whole tile's sum, so the tile's P.V product
+  // is deferred by one visited step: the conversions to e4m3 run under the P.V MFMAs of the tile before.
+  constexpr bool kDefer = MODE == 5;
+  constexpr float kSumLimit = 448.f * 65536.f;   // 2^kLazy in units of the probabilities as formed (times 448)
+  constexpr float kRedoLimit = 1.329227995784916e36f;   // 2^120: beyond it (or not a number) the tile is formed again
   float m_run = 0.f;       // reference point of the exponent; the first visited tile replaces it by the row maximum
   float l_run = 0.f;       // this lane's share of the denominator (times 448 in MODE 3)
   bool first = true;       // wave-uniform: no tile visited yet
@@ -677,6 +688,11 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
   typedef __attribute__((ext_vector_type(8))) int i32x8_t;
   i32x8_t P8 = {0, 0, 0, 0, 0, 0, 0, 0};   // MODE 4: e4m3 probabilities of the current tile (registers reused tile after tile)
   int P8w[8] = {0, 0, 0, 0, 0, 0, 0, 0};   // MODE 5: the same as eight scalars
+  // MODE 5 multiplies a tile's probabilities with V one visited step later (kDefer): P8w holds the pending tile.  A step's
+  // four P.V MFMAs consume it between the Q.K^T MFMAs of the next tile, before the current tile is packed into the same
+  // registers at the end of the step.  It is zero while nothing is pending, so those MFMAs then add nothing.
+  int e_pend = 127;    // E8M0 exponent of the pending tile's block scale
+  int pend_t = -1;     // step of the pending tile (wave-uniform), -1: none
   const int vsw = (c32 >> 1) & 7;    // swizzle of this lane's V^T rows (32 bd + c32)
 
   // S^T = K . Q~^T + Cinit for one tile: 16 MFMAs that nothing below depends on until the next step
@@ -744,11 +760,84 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
   auto block_exp = [](float t) { return (int)__builtin_ceilf(__builtin_amdgcn_fmed3f(t + (127.f - kC), 67.f, 127.f + kLazy)); };
   int e_row = 127;
 
+  // Q~ fragments of the other operand set, one 16-byte piece at a time (a handful of switches per wave: no need for all
+  // eight loads in flight, and the registers they would take are the tile step's).  The 8-bit quantiser of load_q does
+  // not apply: a launch with its own 4-bit operands gets both sets quantised by the caller (q_quant == 0, checked on the host).
+  auto reload_q = [&](const void* qbase) __attribute__((always_inline)) {
+    // (the lane index is laundered so that the row addresses are formed here, at one of a wave's two or three switches,
+    // and not hoisted out of the tile loop into registers that loop has no room for)
+    int ln = lane;
+    asm volatile("; operand set switch" : "+v"(ln));
+    const uint16_t* qp = (const uint16_t*)qbase + (int64_t)b * a.q_sb + (int64_t)head * a.q_sh;
+    const int row = max(min(row_w0 + (ln & 31), a.Nq - 1), 0);
+    const uint16_t* rp = qp + (int64_t)row * a.q_sn + 8 * (ln >> 5);
+#pragma unroll
+    for (int kk = 0; kk < 8; ++kk) {
+      const uint4 raw = *(const uint4*)(rp + 16 * kk);
+      qf[kk] = make_uint4(scale_pair<BF16>(raw.x, a.sm), scale_pair<BF16>(raw.y, a.sm), scale_pair<BF16>(raw.z, a.sm), scale_pair<BF16>(raw.w, a.sm));
+    }
+  };
+  // kDefer, rare: the scores of tile j (step t) once more, from the key rows in memory instead of the LDS ring -- the same
+  // MFMAs in the same order, so the same bits.  One fragment at a time: this path may not raise the kernel's register count.
+  auto redo_tile = [&](int j, bool use4, bool masked, f32x16_t (&S)[2]) __attribute__((always_inline)) {
+    const char* kb = (const char*)a.k + (use4 ? (int64_t)((const char*)a.k4 - (const char*)a.k) : (int64_t)0) + k_head_off * 2;
+    int ln = lane;
+    asm volatile("; tile from memory" : "+v"(ln));
+    // (with separate 4-bit operands the fragments in qf may already belong to the next step's operand set)
+    bool other_q = false;
+    if constexpr (WAVES < 8 || DUAL) {
+      other_q = distinct4 && use4 != q_is4;
+      if (other_q) reload_q(use4 ? a.q4 : a.q);
+    }
+#pragma unroll
+    for (int bn = 0; bn < 2; ++bn) {
+      const int n = min(j * kBN + 32 * bn + (ln & 31), a.Nk - 1);
+      const char* rp = kb + ((int64_t)n * a.k_sn + 8 * (ln >> 5)) * 2;
+#pragma unroll
+      for (int kk = 0; kk < 8; ++kk) {
+        const uint4 ka = *(const uint4*)(rp + 32 * kk);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        S[bn] = mfma_qk32<BF16>(ka, qf[kk], kk == 0 ? Cinit : S[bn]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    if constexpr (WAVES < 8 || DUAL) {
+      if (other_q) reload_q(q_is4 ? a.q4 : a.q);
+    }
+    if (masked) {
+      const int rel = pos0 + (ln & 31) - j * kBN - 4 * (ln >> 5);
+#pragma unroll
+      for (int bn = 0; bn < 2; ++bn)
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+          if (32 * bn + 8 * (i >> 2) + (i & 3) > rel) S[bn][i] = -INFINITY;
+    }
+    mfma_settle(S[0], S[1]);
+  };
+  // kDefer: the P.V product of the pending tile on its own, for a wave that does not visit the step after it (or has
+  // reached the end): V^T fragments from the tile's ring buffer, four MFMAs, and the words back to zero.
+  auto flush_pv = [&](auto rg) __attribute__((always_inline)) {   // rg: ring position of the pending tile's step
+    constexpr int R = decltype(rg)::value;
+    // one fragment pair at a time: this path may not raise the kernel's register count
+    static_for<0, 4>([&](auto I) {
+      constexpr int bd = decltype(I)::value;
+      u32x4_t vlo = lds_read128<R * kVTileBytes + bd * 2048>(v8lo_base), vhi = lds_read128<R * kVTileBytes + bd * 2048>(v8hi_base);
+      lds_wait<0>(vlo, vhi);
+      const i32x8_t av = {(int)vlo[0], (int)vlo[1], (int)vlo[2], (int)vlo[3], (int)vhi[0], (int)vhi[1], (int)vhi[2], (int)vhi[3]};
+      const i32x8_t pb = {P8w[0], P8w[1], P8w[2], P8w[3], P8w[4], P8w[5], P8w[6], P8w[7]};
+      O[bd] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, pb, O[bd], 0, 0, 0, 0x7f7f7f7f, 0, e_pend);
+      __builtin_amdgcn_sched_barrier(0);
+    });
+#pragma unroll
+    for (int r = 0; r < 8; ++r) P8w[r] = 0;
+    pend_t = -1;
+  };
+
   // softmax update + P.V for the tile whose scores are in S.  Once the running maximum of this tile is settled,
   // the Q.K^T MFMAs of the following tile (K in knext, result in Snext) are issued in the same straight-line
   // block as the exponentials, conversions and P.V MFMAs, so that the matrix pipe and the vector ALU of this
   // wave work side by side.
-  auto softmax_pv = [&](auto rg, int j, int it, const char* vbuf, bool masked, f32x16_t (&S)[2], const char* knext, f32x16_t (&Snext)[2]) {
+  auto softmax_pv = [&](auto rg, int j, int it, bool use4, const char* vbuf, bool masked, f32x16_t (&S)[2], const char* knext, f32x16_t (&Snext)[2]) {
     constexpr int R = decltype(rg)::value;   // it & 3, known at compile time
     // MODE 4: the first K fragments of the next tile are requested before anything else, so that their LDS
     // latency passes under the row-maximum bookkeeping
@@ -777,7 +866,15 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
     // row maximum of S - m_run + kC; the row's other 32 keys live in lane^32
     float tmax;
     bool slow;
-    if constexpr (!kPlain) {
+    if constexpr (kDefer) {
+      // only a wave's first tile looks at its scores before exponentiating them: it sets the reference
+      slow = first;
+      tmax = 0.f;
+      if (__builtin_expect(first, 0)) {
+        mfma_settle(S[0], S[1]);
+        tmax = xor32_max(lane_max(S));
+      }
+    } else if constexpr (!kPlain) {
       if (masked) {
         tmax_row = xor32_max(lane_max(S));
         moved = __any(tmax_row > kMove);
@@ -812,6 +909,160 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) Cinit[i] = c;
       first = false;
+    }
+    if constexpr (kDefer) {
+      __builtin_amdgcn_s_setprio(0);
+      // Hand-scheduled tile step.  16 slots of {Q.K^T MFMA of the next tile, one LDS prefetch, two exponentials of the
+      // current tile and their addition to the row sum}; the row sum's exchange with the lane that holds the row's other
+      // 32 keys and the block exponent; then 4 slots of {fp8 P.V MFMA of the PENDING tile (the one visited before this
+      // one; its V^T tile is in ring buffer R - 1), two LDS prefetches, four packs of the current tile to e4m3}.
+      // LDS requests, in order: K fragments 0 .. 15 (kDepth ahead of their MFMA), then V^T fragments 0 .. 7 (lo and hi
+      // half of the rows of P.V slot r / 2): four in the last four Q.K^T slots, which request no K fragment any more, two
+      // more behind each of the first two P.V MFMAs -- two slots ahead of their use.
+      static_assert(kDepth == 4, "the wait counts below are those of K fragments requested four slots ahead");
+      constexpr int kVoff = ((R + 3) & 3) * kVTileBytes;
+      u32x4_t vlo[4], vhi[4];
+      auto vread = [&](auto RR) __attribute__((always_inline)) {
+        constexpr int rr = decltype(RR)::value;
+        if constexpr (rr & 1) vhi[rr >> 1] = lds_read128<kVoff + (rr >> 1) * 2048>(v8hi_base);
+        else vlo[rr >> 1] = lds_read128<kVoff + (rr >> 1) * 2048>(v8lo_base);
+      };
+      float ps[2] = {0.f, 0.f};
+      static_for<0, 16>([&](auto I) {
+        constexpr int i = decltype(I)::value;
+        constexpr int bn = i & 1, kk = i >> 1;
+        lds_wait<3>(kf[i]);     // behind it: K fragments i + 1 .. i + 3, or in the last slots V^T fragments in their place
+        __builtin_amdgcn_sched_barrier(0);
+        constexpr int sb = i >> 3, e = 2 * (i & 7);
+        const float p0 = __builtin_amdgcn_exp2f(S[sb][e]), p1 = __builtin_amdgcn_exp2f(S[sb][e + 1]);
+        S[sb][e] = p0;
+        S[sb][e + 1] = p1;
+        __builtin_amdgcn_sched_barrier(0);
+        const uint4 ka = make_uint4(kf[i][0], kf[i][1], kf[i][2], kf[i][3]);
+        if constexpr (kk == 0) Snext[bn] = mfma_qk32<BF16>(ka, qf[0], Cinit);
+        else Snext[bn] = mfma_qk32<BF16>(ka, qf[kk], Snext[bn]);
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (i + kDepth < 16) kread(std::integral_constant<int, i + kDepth>{});
+        else vread(std::integral_constant<int, i + kDepth - 16>{});
+        ps[i & 1] += p0;
+        ps[i & 1] += p1;
+        __builtin_amdgcn_sched_barrier(0);
+      });
+      // The row's sum of the tile, rs = 448 sum 2^(s - reference).  Block scale 2^-k with rs 2^-k in [128, 256): every
+      // scaled probability is below 256 (e4m3 reaches 448), the row's largest one at least 2.  The E8M0 exponent of 2^k is
+      // eb = frexp exponent + 119, kept in [67, 245]: the pack divides by 2^(eb - 127), the MFMA multiplies by it.
+      // (only rs_lane and eb stay live through the P.V slots: the rare paths below form the row sum again)
+      float rs_lane = ps[0] + ps[1];
+      int eb;
+      {
+        const float rs_row = xor32_sum(rs_lane);
+        eb = min(max(__builtin_amdgcn_frexp_expf(rs_row) + 119, 67), 245);
+        moved = __any(!(rs_row <= kSumLimit));
+      }
+      const float pack_scale = __int_as_float(eb << 23);
+      typedef __attribute__((ext_vector_type(2))) short i16x2_t;
+      int P8n[8];
+      auto pack_words = [&](auto BD, float sc) __attribute__((always_inline)) {   // words 2 bd, 2 bd + 1: S[bd >> 1][8 (bd & 1) .. + 7]
+        constexpr int bd = decltype(BD)::value;
+        constexpr int sb = bd >> 1, o = 8 * (bd & 1);
+        // (each pack writes one half of the word and keeps the other: the halves start out as whatever the register held)
+        int u0, u1;
+        asm volatile("" : "=v"(u0), "=v"(u1));
+        i16x2_t w0 = __builtin_bit_cast(i16x2_t, u0), w1 = __builtin_bit_cast(i16x2_t, u1);
+        w0 = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(w0, S[sb][o], S[sb][o + 1], sc, false);
+        w0 = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(w0, S[sb][o + 2], S[sb][o + 3], sc, true);
+        w1 = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(w1, S[sb][o + 4], S[sb][o + 5], sc, false);
+        w1 = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(w1, S[sb][o + 6], S[sb][o + 7], sc, true);
+        P8n[2 * bd] = __builtin_bit_cast(int, w0);
+        P8n[2 * bd + 1] = __builtin_bit_cast(int, w1);
+      };
+      static_for<0, 4>([&](auto I) {
+        constexpr int bd = decltype(I)::value;
+        lds_wait<(bd < 3) ? 2 : 0>(vlo[bd], vhi[bd]);   // the next pair is behind it, except for the last
+        __builtin_amdgcn_sched_barrier(0);
+        const i32x8_t av = {(int)vlo[bd][0], (int)vlo[bd][1], (int)vlo[bd][2], (int)vlo[bd][3],
+                            (int)vhi[bd][0], (int)vhi[bd][1], (int)vhi[bd][2], (int)vhi[bd][3]};
+        const i32x8_t pb = {P8w[0], P8w[1], P8w[2], P8w[3], P8w[4], P8w[5], P8w[6], P8w[7]};
+        O[bd] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, pb, O[bd], 0, 0, 0, 0x7f7f7f7f, 0, e_pend);
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (bd < 2) {
+          vread(std::integral_constant<int, 2 * bd + 4>{});
+          vread(std::integral_constant<int, 2 * bd + 5>{});
+        }
+        pack_words(I, pack_scale);
+        __builtin_amdgcn_sched_barrier(0);
+      });
+#pragma unroll
+      for (int r = 0; r < 8; ++r) P8w[r] = P8n[r];
+      __builtin_amdgcn_s_setprio(3);
+      if (__builtin_expect(moved, 0)) {   // one tile in thousands
+        asm volatile("; reference moves" ::: "memory");
+        float rs_row = xor32_sum(rs_lane);
+        int fe = __builtin_amdgcn_frexp_expf(rs_row);
+        if (__builtin_expect(__any(!(rs_row < kRedoLimit)), 0)) {
+          // A row's sum overflowed: its probabilities are lost.  The tile's scores are formed again from the key rows in
+          // memory (the K tile may have left the ring), such a row takes the tile's maximum as its new reference, and the
+          // tile is exponentiated, summed and packed once more for all rows (rows that were fine get the bits they had).
+          const bool redo = !(rs_row < kRedoLimit);
+          redo_tile(j, use4, masked, S);
+          const float tm = xor32_max(lane_max(S));
+          const float d = redo ? tm - kC : 0.f;
+          const float alpha = __builtin_amdgcn_exp2f(-d);
+          m_run += d;
+          l_run *= alpha;
+#pragma unroll
+          for (int bd = 0; bd < 4; ++bd) O[bd] *= alpha;
+          float q0 = 0.f, q1 = 0.f;
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            S[0][i] = __builtin_amdgcn_exp2f(S[0][i] - d);
+            S[1][i] = __builtin_amdgcn_exp2f(S[1][i] - d);
+          }
+          // the additions in the order of the slots above: slot i takes S[i >> 3][2 (i & 7)] and its neighbour
+#pragma unroll
+          for (int i = 0; i < 16; i += 2) {
+            q0 += S[i >> 3][2 * (i & 7)];
+            q0 += S[i >> 3][2 * (i & 7) + 1];
+            q1 += S[(i + 1) >> 3][2 * ((i + 1) & 7)];
+            q1 += S[(i + 1) >> 3][2 * ((i + 1) & 7) + 1];
+          }
+          rs_lane = q0 + q1;
+          rs_row = xor32_sum(rs_lane);
+          fe = __builtin_amdgcn_frexp_expf(rs_row);
+          eb = min(max(fe + 119, 67), 245);
+          const float sc = __int_as_float(eb << 23);
+          static_for<0, 4>([&](auto I) { pack_words(I, sc); });
+#pragma unroll
+          for (int r = 0; r < 8; ++r) P8w[r] = P8n[r];
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            Snext[0][i] -= d;
+            Snext[1][i] -= d;
+          }
+        }
+        // rows whose sum passed the limit: the reference goes up by n binades, rs 2^-n in [256, 512)
+        const int n = (rs_row > kSumLimit) ? fe - 9 : 0;
+        const float down = __int_as_float((127 - n) << 23);
+        const float nf = (float)n;
+        m_run += nf;
+        l_run *= down;
+        rs_lane *= down;
+#pragma unroll
+        for (int bd = 0; bd < 4; ++bd) O[bd] *= down;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          Snext[0][i] -= nf;
+          Snext[1][i] -= nf;
+        }
+        eb = max(eb - n, 1);
+        const float c = kC - m_run;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) Cinit[i] = c;
+      }
+      l_run += rs_lane;
+      e_pend = eb;
+      pend_t = it;
+      return;
     }
     if constexpr (kPV8) {
       // MODE 5: the pack divides by 2^-k, the MFMA multiplies this lane's 32 values by 2^-k again (E8M0 scale in
@@ -1066,15 +1317,22 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
     return in;
   };
 
+  // kDefer: a tile's V^T is needed one step after its K (the P.V product runs a visited step late), so its copy starts
+  // a step later as well and the buffer is refilled a step later: V^T(t) is read in step t + 1, or in a flush before the
+  // workgroup has left step t + 1
   if (0 < nTot) {
     stage_k(tile_of(0), 0, step_uses4(0));
     stage_v(tile_of(0), 0);
   }
   if (1 < nTot) {
     stage_k(tile_of(1), 1, step_uses4(1));
-    stage_v(tile_of(1), 1);
+    if constexpr (!kDefer) stage_v(tile_of(1), 1);
   }
   if (2 < nTot) stage_k(tile_of(2), 2, step_uses4(2));
+  if constexpr (kDefer) {
+    // ring buffer 3 is read by step 0's P.V MFMAs, which have zeros for probabilities: it must hold finite numbers
+    for (int i = tid; i < kVTileBytes / 16; i += NT) *(uint4*)(vbase_lds + 3 * kVTileBytes + 16 * i) = make_uint4(0, 0, 0, 0);
+  }
   // the wave's query rows, requested while the first tiles are on their way
   if constexpr (kQK8) {
     const uint16_t* qp = (const uint16_t*)a.q + (int64_t)b * a.q_sb + (int64_t)head * a.q_sh;
@@ -1117,23 +1375,6 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
   }
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
-  // Q~ fragments of the other operand set, one 16-byte piece at a time (a handful of switches per wave: no need for all
-  // eight loads in flight, and the registers they would take are the tile step's).  The 8-bit quantiser of load_q does
-  // not apply: a launch with its own 4-bit operands gets both sets quantised by the caller (q_quant == 0, checked on the host).
-  auto reload_q = [&](const void* qbase) __attribute__((always_inline)) {
-    // (the lane index is laundered so that the row addresses are formed here, at one of a wave's two or three switches,
-    // and not hoisted out of the tile loop into registers that loop has no room for)
-    int ln = lane;
-    asm volatile("; operand set switch" : "+v"(ln));
-    const uint16_t* qp = (const uint16_t*)qbase + (int64_t)b * a.q_sb + (int64_t)head * a.q_sh;
-    const int row = max(min(row_w0 + (ln & 31), a.Nq - 1), 0);
-    const uint16_t* rp = qp + (int64_t)row * a.q_sn + 8 * (ln >> 5);
-#pragma unroll
-    for (int kk = 0; kk < 8; ++kk) {
-      const uint4 raw = *(const uint4*)(rp + 16 * kk);
-      qf[kk] = make_uint4(scale_pair<BF16>(raw.x, a.sm), scale_pair<BF16>(raw.y, a.sm), scale_pair<BF16>(raw.z, a.sm), scale_pair<BF16>(raw.w, a.sm));
-    }
-  };
   auto switch_q = [&](int t) __attribute__((always_inline)) {   // t: a step this wave visits
     if constexpr (WAVES < 8 || DUAL) {
       if (distinct4) {  // switch the Q~ operand set when entering/leaving the 4-bit window range
@@ -1150,7 +1391,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
   if (vis_cur) {
     switch_q(0);
     qk_tile(kbase_lds, Sa);
-    if constexpr (!kPlain) {
+    if constexpr (!kPlain && !kDefer) {
       mfma_settle(Sa[0], Sa[1]);
       tmax_row = xor32_max(lane_max(Sa));
       moved = __any(tmax_row > kMove);
@@ -1169,13 +1410,23 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
           stage_k(j3, (t + 3) & 3, step_uses4(t + 3));
           stage_k(j4, t & 3, step_uses4(t + 4));
         }
-        stage_v(j2, (t + 2) & 3);
-        stage_v(j3, (t + 3) & 3);
+        if constexpr (kDefer) {
+          stage_v(tile_of(t + 1), (t + 1) & 3);
+          stage_v(j2, (t + 2) & 3);
+        } else {
+          stage_v(j2, (t + 2) & 3);
+          stage_v(j3, (t + 3) & 3);
+        }
       } else {
         if (t + 3 < nTot) stage_k(tile_of(t + 3), (t + 3) & 3, step_uses4(t + 3));
         if (t + 4 < nTot) stage_k(tile_of(t + 4), t & 3, step_uses4(t + 4));
-        if (t + 2 < nTot) stage_v(tile_of(t + 2), (t + 2) & 3);
-        if (t + 3 < nTot) stage_v(tile_of(t + 3), (t + 3) & 3);
+        if constexpr (kDefer) {
+          if (t + 1 < nTot) stage_v(tile_of(t + 1), (t + 1) & 3);
+          if (t + 2 < nTot) stage_v(tile_of(t + 2), (t + 2) & 3);
+        } else {
+          if (t + 2 < nTot) stage_v(tile_of(t + 2), (t + 2) & 3);
+          if (t + 3 < nTot) stage_v(tile_of(t + 3), (t + 3) & 3);
+        }
       }
     }
     const bool vis_nxt = visits_step(t + 1);
@@ -1186,11 +1437,11 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
     if (vis_cur) {
       // Q.K^T of the next tile is computed even if this wave will not use it (the buffer then holds an older
       // tile or nothing meaningful; the result is dropped): the common path stays free of branches
-      softmax_pv(rg, tile_of(t), t, vbase_lds + (t & 3) * kVTileBytes, t >= fm, Scur, knext, Snxt);
+      softmax_pv(rg, tile_of(t), t, step_uses4(t), vbase_lds + (t & 3) * kVTileBytes, t >= fm, Scur, knext, Snxt);
     } else {
       if (vis_nxt) {
         qk_tile(knext, Snxt);
-        if constexpr (!kPlain) {
+        if constexpr (!kPlain && !kDefer) {
           mfma_settle(Snxt[0], Snxt[1]);
           tmax_row = xor32_max(lane_max(Snxt));
           moved = __any(tmax_row > kMove);
@@ -1206,6 +1457,11 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
       __builtin_amdgcn_s_waitcnt(0);   // this wave's share of the tiles staged at the start of the pair has landed
       __syncthreads();
     }
+    if constexpr (kDefer) {
+      // the wave leaves its range: the last tile's P.V product now (its V^T tile has landed -- it was staged for the next
+      // step -- and the buffer is not refilled before the end of that step)
+      if (__builtin_expect(pend_t >= 0 && !vis_nxt, 0)) flush_pv(rg);
+    }
     vis_cur = vis_nxt;
   };
   // both steps of a pair always run (the second one idles when the number of steps is odd), so that every wave
@@ -1219,6 +1475,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
 
   // ---- epilogue: out = acc / l (attn_triton.py:208-209), lse2 = log2(l) + m (:210-213)
   if (!wave_active) return;
+  // (kDefer: nothing is pending here -- the step after a wave's last visited step is never visited, so that step flushed)
   const float l = xor32_sum(l_run);
   const int row = row_w0 + c32;
   if (row >= a.Nq) return;

@@ -29,7 +29,8 @@ MASK_ADD = -1000000.0  # additive causal mask (attn_triton.py:71)
 
 P_NONE, P_STATIC448, P_BLOCK_ABSMAX, P_STATIC448_GRID = 0, 1, 2, 3
 P_MX_ROW = 5   # e4m3 with one power-of-two scale per query row and 64-key tile (block-scaled fp8 MFMA operand)
-MX_LAZY = 16.0  # P_MX_ROW: a row's reference point follows its maximum only once the maximum leads by more than this (log2)
+MX_LAZY = 16.0  # P_MX_ROW: a row's reference point moves only once the row's sum of a block's probabilities exceeds 2^this
+MX_REDO = 2.0 ** 120   # P_MX_ROW: a block sum (times 448) at or beyond this, or not a number, has the block formed again
 
 
 # --------------------------------------------------------------------------- helpers
@@ -98,14 +99,14 @@ def _quant_p(p: torch.Tensor, mode: int, group_rows: int = 64) -> torch.Tensor:
     if mode == P_STATIC448_GRID:   # the e4m3 grid of mode 1 without the fp16 rounding of p/448 (fp8 operand of an fp8 MFMA)
         return (p * 448.0).to(torch.float8_e4m3fn).float() / 448.0
     if mode == P_MX_ROW:
-        # build-defined: scale 2^k per row of the tile with k = floor(-log2(row maximum)) in [-MX_LAZY, 60], so that the
-        # row's largest scaled probability lies in (224, 448]; the dequantised value is e4m3(p*448*2^k) / (448*2^k).
-        # (p is taken relative to a reference that may trail the row maximum by up to MX_LAZY, see _RowState.update.)
-        a = p.max(dim=1, keepdim=True).values
-        k = torch.floor(-torch.log2(a)).clamp(-MX_LAZY, 60.0)
-        k = torch.where(a > 0, k, torch.full_like(k, 60.0))
-        sc = torch.exp2(k) * 448.0
-        return (p * sc).to(torch.float8_e4m3fn).float() / sc
+        # build-defined: scale 2^k per row of the tile, taken from the row's SUM rs = sum(448 p) (fp32), which the
+        # denominator needs anyway: with rs = f 2^E, f in [1/2, 1) (frexp), k = 8 - E clamped to [-118, 60], so that
+        # rs 2^k lies in [128, 256): every scaled probability is below 256 (e4m3 reaches 448) and the row's largest one
+        # at least 2.  The dequantised value is e4m3(448 p 2^k) / (448 2^k).
+        # (p is taken relative to a reference that may trail the row maximum, see _RowState.update.)
+        p448 = p * 448.0
+        k = mx_row_exponent(p448.sum(dim=1, keepdim=True))
+        return (p448 * torch.exp2(k)).to(torch.float8_e4m3fn).float() / (torch.exp2(k) * 448.0)
     if mode == P_BLOCK_ABSMAX:
         out = torch.empty_like(p)
         for r0 in range(0, p.shape[0], group_rows):
@@ -122,6 +123,12 @@ def _quant_p(p: torch.Tensor, mode: int, group_rows: int = 64) -> torch.Tensor:
     raise ValueError(f"unknown p_quant mode {mode}")
 
 
+def mx_row_exponent(rs448: torch.Tensor) -> torch.Tensor:
+    """P_MX_ROW: the block scale's exponent k (as fp32) for rows whose probabilities, times 448, sum to `rs448`."""
+    e = torch.frexp(rs448.float()).exponent.float()      # rs448 in [2^(e-1), 2^e); 0 for a zero sum
+    return (8.0 - e).clamp(-118.0, 60.0)
+
+
 class _RowState:
     """Online-softmax state of a tile of query rows (attn_triton.py:165-167)."""
 
@@ -133,14 +140,9 @@ class _RowState:
     def update(self, s: torch.Tensor, vblk: torch.Tensor, p_quant: int, group_rows: int):
         """One KV-block step (attn_triton.py:72-84). `s` fp32 [rows, cols], `vblk` fp32 [cols, D]
         holding fp16-representable values."""
-        m_new = torch.maximum(self.m, s.max(dim=1).values)
         if p_quant == P_MX_ROW:
-            # build-defined: the reference point m is not the running maximum itself.  It is set by the first block and
-            # afterwards replaced by a row's block maximum only when that exceeds it by more than MX_LAZY; until then
-            # p = 2^(s - m) may exceed 1 (the block scale of _quant_p absorbs the factor) and l, acc carry the same factor,
-            # which cancels in finish().  Mathematically the same softmax; the e4m3 grid points differ.
-            keep = (self.m > float("-inf")) & ~(m_new - self.m > MX_LAZY)
-            m_new = torch.where(keep, self.m, m_new)
+            return self._update_mx_row(s, vblk)
+        m_new = torch.maximum(self.m, s.max(dim=1).values)
         p = torch.exp2(s - m_new[:, None])
         alpha = torch.exp2(self.m - m_new)
         self.l = self.l * alpha + p.sum(dim=1)
@@ -148,6 +150,34 @@ class _RowState:
         pq = _quant_p(p, p_quant, group_rows)
         self.acc = self.acc + pq @ vblk
         self.m = m_new
+
+    def _update_mx_row(self, s: torch.Tensor, vblk: torch.Tensor):
+        """Build-defined (no reference counterpart): the reference point m of a row is not its running maximum and no
+        maximum is looked at.  The first block sets m to its row maximum.  Afterwards a block's probabilities are formed
+        against the standing m, p = 2^(s - m), whatever the scores are (p may exceed 1: the block scale of `_quant_p`
+        absorbs any power of two, and l, acc carry the common factor, which cancels in finish()); the block's sum decides
+        what follows:
+          * rs = sum(448 p) > 448 2^MX_LAZY: after the block has been added, m goes up by the whole number n = E - 9
+            (rs in [2^(E-1), 2^E)), l and acc are multiplied by 2^-n (exactly), so that the block's sum becomes [256, 512);
+          * rs >= MX_REDO or not a number (a score 2^100 above everything before it): the row takes the block's maximum
+            as m first (l and acc rescaled as in the reference's step) and the block is formed again.
+        Mathematically the same softmax; the e4m3 grid points differ."""
+        blockmax = s.max(dim=1).values
+        first = self.m == float("-inf")
+        m = torch.where(first, blockmax, self.m)
+        rs = (torch.exp2(s - m[:, None]) * 448.0).sum(dim=1)
+        redo = ~(rs < MX_REDO)
+        m = torch.where(redo, blockmax, m)
+        alpha = torch.where(m == self.m, torch.ones_like(m), torch.exp2(self.m - m))
+        p = torch.exp2(s - m[:, None])
+        rs = (p * 448.0).sum(dim=1)
+        self.l = self.l * alpha + p.sum(dim=1)
+        self.acc = self.acc * alpha[:, None] + _quant_p(p, P_MX_ROW) @ vblk
+        n = torch.where(rs > 448.0 * 2.0 ** MX_LAZY, torch.frexp(rs).exponent.float() - 9.0, torch.zeros_like(rs))
+        down = torch.exp2(-n)
+        self.l = self.l * down
+        self.acc = self.acc * down[:, None]
+        self.m = m + n
 
     def finish(self):
         out = self.acc / self.l[:, None]

@@ -93,7 +93,7 @@ def test_block_scaled_p_keeps_small_probabilities_the_static_scale_flushes():
     """Attention sink: key 0 outscores every other key by about 2^17, so all later tiles hold probabilities near
     2^-17 whose 448-fold lies in the subnormal range of e4m3 (steps of 2^-9) and partly rounds to zero under the
     static scale (modes 3 and 4), although the 8192 of them together carry a few percent of the row.  The per-row
-    block scale of mode 5 moves each tile's row maximum to (224, 448], i.e. back to three mantissa bits."""
+    block scale of mode 5 moves each tile's row sum to [128, 256), i.e. its probabilities back to three mantissa bits."""
     from longcontext_sqattn_paddle_amd.sqattn.attn_triton import attn_causal
 
     N, D = 8192, 128
@@ -116,6 +116,46 @@ def test_block_scaled_p_keeps_small_probabilities_the_static_scale_flushes():
         errs[mode] = float((out.cpu().double()[:, :, N // 2:] - exact[:, :, N // 2:]).pow(2).mean().sqrt())
     print("rms error vs exact attention, rows N/2..N:", errs, flush=True)
     assert errs[5] <= 0.5 * errs[4]
+
+
+@pytest.mark.parametrize("step_up,jump", [(6.0, 40.0), (0.0, 140.0), (3.0, 17.0)])
+def test_block_scaled_p_reference_moves_and_overflows(step_up, jump):
+    """Mode 5 forms a tile's probabilities against the standing reference point without looking at the scores first.
+    Scores that climb by `step_up` (log2) per 64-key tile push the row sums past 2^16 every few tiles (the reference then
+    moves up by whole binades, which rescales the tile packed just before as well); one key that leads everything before
+    it by `jump` does the same in one step, and by 140 it overflows 2^(s - reference): the tile is formed again from the
+    key rows in memory.  Against the oracle's restatement of the same rule, and against exact attention."""
+    from longcontext_sqattn_paddle_amd.sqattn.attn_triton import attn_causal
+
+    N, D = 1536, 128
+    print(f"case prefill mode 5 reference moves step_up={step_up} jump={jump}", flush=True)
+    g = torch.Generator().manual_seed(91)
+    q = torch.randn(1, 4, N, D, generator=g) * 0.5
+    k = torch.randn(1, 2, N, D, generator=g) * 0.5
+    v = torch.randn(1, 2, N, D, generator=g)
+    ramp = torch.arange(N, dtype=torch.float32) / 64.0 * step_up
+    ramp[700:] += jump          # key 700 sits in the middle of a tile, 1000 on a tile that is a diagonal tile for some rows
+    ramp[1000:] += jump / 2
+    q[..., 0] = 1.0
+    k[:, :, :, 0] = (ramp * (D ** 0.5 / 1.44269504))[None, None]
+    q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
+    ref, lse_ref = A.prefill_blockwise(q, k, v, p_quant=A.P_MX_ROW, v_quant="e4m3_channel", out_dtype=torch.float32)
+    out, lse = attn_causal(q.to(DEV), k.to(DEV), v.to(DEV), "HND", torch.float32, return_lse=True, p_quant=5)
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(out).all()) and bool(torch.isfinite(lse).all())
+    # The scores here reach 200 and more (log2), so their fp32 rounding (1e-4, and the MFMA adds the products in another
+    # order than the oracle) moves a probability by 1e-4 relative -- enough to send one in a thousand across an e4m3
+    # rounding boundary, a step of 6 %.  Rows like these hang on a dozen leading keys each, so such a flip shows in the
+    # row (up to 0.1 rms) where on random data it disappears: a few percent of the rows differ visibly, none grossly.
+    err = (out.cpu().double() - ref.double()).abs()
+    rms = float(ref.double().pow(2).mean().sqrt())
+    assert float(torch.quantile(err.flatten()[:: 7], 0.90)) <= 5e-3 * rms
+    assert float(err.max()) <= 0.25 * rms
+    assert _cos(out.cpu(), ref) >= 0.9995
+    assert torch.allclose(lse.cpu(), lse_ref, atol=2e-4, rtol=1e-6)       # the log-sum-exp has no quantised quantity in it
+    exact, lse_exact = A.exact_attention(q, k, v)
+    assert _cos(out.cpu(), exact) >= 0.999
+    assert torch.allclose(lse.cpu(), lse_exact.float(), atol=2e-2, rtol=5e-3)
 
 
 def test_nhd_layout_bf16_out_and_gqa_7():

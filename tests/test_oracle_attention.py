@@ -139,37 +139,50 @@ def test_fp8_error_levels_against_exact():
 
 
 def test_block_scaled_p_quantiser_properties():
-    """`P_MX_ROW` (build-defined, no reference counterpart) pinned by what the definition fixes:
-    rows whose maximum lies in (1/2, 1] get scale 1 and equal the static-scale grid; multiplying a row by 2^-j
-    multiplies its result by exactly 2^-j (the scale absorbs it) until the clamp at 2^60; every element within 2^6
-    of its row maximum keeps three mantissa bits (relative error <= 2^-4); a zero row stays zero."""
+    """`P_MX_ROW` (build-defined, no reference counterpart) pinned by what the definition fixes: the scale 2^k comes from
+    the row's sum rs = sum(448 p) = f 2^E (f in [1/2, 1)), k = 8 - E.  Rows whose sum lies in [2/7, 4/7) (rs in [128, 256))
+    get scale 1 and equal the static-scale grid; multiplying a row by 2^-j multiplies its result by exactly 2^-j (the scale
+    absorbs it) until the clamp at 2^60; every scaled probability stays below 256; every element that is at least 2^-13
+    of the row's sum keeps three mantissa bits (relative error <= 2^-4); a zero row stays zero."""
     g = torch.Generator().manual_seed(11)
-    p = torch.rand(16, 64, generator=g) * 0.9 + 1e-3
-    p[:, 5] = torch.linspace(0.5001, 1.0, 16)          # row maximum in (1/2, 1]
+    p = torch.rand(16, 64, generator=g) + 1e-3
+    p = p / p.sum(dim=1, keepdim=True) * torch.linspace(0.29, 0.57, 16)[:, None]      # row sums in [2/7, 4/7)
+    assert bool(((p * 448).sum(dim=1) >= 128).all()) and bool(((p * 448).sum(dim=1) < 256).all())
     base = A._quant_p(p, A.P_MX_ROW)
     assert torch.equal(base, A._quant_p(p, A.P_STATIC448_GRID))
-    for j in (1, 7, 16, 40, 59):
+    for j in (1, 7, 16, 40, 52):
         assert torch.equal(A._quant_p(p * 2.0 ** -j, A.P_MX_ROW), base * 2.0 ** -j), j
-    # the scale is 2^k with k = floor(-log2(max)): a maximum of exactly 2^-9 takes k = 9 and is kept exactly
+        assert torch.equal(A._quant_p(p * 2.0 ** j, A.P_MX_ROW), base * 2.0 ** j), j       # sums far above 1 as well
+    # the exponent itself, at both ends of a binade and at the clamps
+    rs = torch.tensor([128.0, 255.99, 256.0, 0.875, 2.0 ** 100, 2.0 ** -70, 0.0])
+    assert A.mx_row_exponent(rs).tolist() == [0.0, 0.0, -1.0, 8.0, -93.0, 60.0, 8.0]
+    # a lone probability of 2^-9: rs = 0.875, k = 8, scaled value 224 is on the grid and is kept exactly
     one = torch.zeros(1, 64)
     one[0, 0] = 2.0 ** -9
     assert float(A._quant_p(one, A.P_MX_ROW)[0, 0]) == 2.0 ** -9
+    # a single dominant probability is scaled to [128, 256): never saturates (e4m3 reaches 448)
+    for top in (1.0, 0.57, 3.99, 2.0 ** 15.9):
+        row = torch.full((1, 64), 1e-9)
+        row[0, 3] = top
+        qrow = A._quant_p(row, A.P_MX_ROW)
+        assert abs(float(qrow[0, 3]) / top - 1.0) <= 2.0 ** -4
     # beyond the clamp the scale stays 2^60 and small values fall off the grid as under any fixed scale
     tiny = torch.full((1, 64), 2.0 ** -80)
     assert float(A._quant_p(tiny, A.P_MX_ROW).abs().max()) == 0.0
-    # precision: elements down to 2^-6 of the row maximum are e4m3 normals
+    # precision: elements down to 2^-13 of the row's sum are e4m3 normals
     p2 = torch.rand(32, 64, generator=g) * 2.0 ** -14
     p2[:, 0] = 2.0 ** -14
     q2 = A._quant_p(p2, A.P_MX_ROW)
-    big = p2 >= 2.0 ** -20
+    big = p2 >= p2.sum(dim=1, keepdim=True) * 2.0 ** -13
+    assert float(big.float().mean()) > 0.9
     assert float(((q2 - p2).abs() / p2)[big].max()) <= 2.0 ** -4
     assert float(((A._quant_p(p2, A.P_STATIC448_GRID) - p2).abs() / p2)[big].max()) > 0.2   # what the static scale loses
     assert torch.equal(A._quant_p(torch.zeros(2, 64), A.P_MX_ROW), torch.zeros(2, 64))
 
 
 def test_block_scaled_p_reference_point_is_lazy_but_the_softmax_is_not():
-    """`P_MX_ROW` keeps a row's reference point until the row maximum leads it by more than `MX_LAZY`.  What that must
-    not change: the log-sum-exp (no quantised quantity enters it) and the output up to e4m3 noise, also when the
+    """`P_MX_ROW` keeps a row's reference point until the row's sum of a block's probabilities exceeds 2^`MX_LAZY`.  What
+    that must not change: the log-sum-exp (no quantised quantity enters it) and the output up to e4m3 noise, also when the
     maxima rise block after block by more than the limit in total and, for some rows, in one step."""
     N, D = 512, 64
     g = torch.Generator().manual_seed(21)
@@ -190,7 +203,9 @@ def test_block_scaled_p_reference_point_is_lazy_but_the_softmax_is_not():
     assert torch.allclose(lse, lse_eager, atol=2e-4, rtol=1e-6)
     cos = lambda a, b: float((a.double() * b.double()).sum() / (a.double().norm() * b.double().norm()))
     assert cos(out, exact) >= 0.9995
-    assert cos(out, exact) >= cos(eager, exact) - 1e-4   # no worse than the static scale with its eager reference
+    # (the static scale with its eager reference represents a row's dominant probability, exactly 1, without error -- 448 is
+    # on the grid -- which rows like these, with one leading key each, profit from; the block scale rounds it like any value)
+    assert cos(out, exact) >= cos(eager, exact) - 3e-4
 
 
 def test_window_invariants_and_explicit_mask():
@@ -515,39 +530,54 @@ def test_decode_fp8_p_matches_scalar_bruteforce():
 def _scalar_mx_row(scores, vals):
     """Independent per-row scalar restatement of the `P_MX_ROW` state: scores [blocks][64] (fp32, base-2 logits of one
     query row), vals [blocks][64] (one output channel).  Written from the definition, not from the oracle's tensors:
-      * reference point r: the first block's maximum; a later block's maximum replaces it only when it exceeds r by more
-        than 16, otherwise r stays;
-      * p = 2^(s - r); the denominator sums p as it is; the block scale is 2^k, k = floor(-log2(max p)) clamped to
-        [-16, 60]; the product uses e4m3(p 448 2^k) / (448 2^k);
-      * when r moves by d, numerator and denominator are multiplied by 2^-d first."""
+      * reference point r: the first block's maximum;
+      * p = 2^(s - r) whatever the scores; the denominator sums p as it is; with rs = sum(448 p) in [2^(E-1), 2^E) the
+        block scale is 2^k, k = 8 - E clamped to [-118, 60]; the product uses e4m3(448 p 2^k) / (448 2^k);
+      * after a block with rs > 448 2^16, r goes up by n = E - 9 and numerator and denominator are multiplied by 2^-n;
+      * a block whose rs is not below 2^120 is formed again with r = the block's maximum, numerator and denominator
+        multiplied by 2^(old r - new r) first."""
     f32 = np.float32
     r, num, den = None, 0.0, f32(0.0)
-    moves = []
+    moves, redone = [], 0
+
+    def form(s, r):
+        with np.errstate(over="ignore"):
+            p = np.exp2((np.asarray(s, dtype=f32) - r).astype(np.float64)).astype(f32)
+            rs = (p * f32(448.0)).sum(dtype=f32)
+        return p, rs
+
     for s, v in zip(scores, vals):
-        mx = f32(max(s))
         if r is None:
-            r = mx
-        elif float(mx) - float(r) > 16.0:
-            alpha = f32(np.exp2(np.float64(r) - np.float64(mx)))
+            r = f32(max(s))
+        p, rs = form(s, r)
+        if not rs < f32(2.0 ** 120):
+            new_r = f32(max(s))
+            alpha = f32(np.exp2(np.float64(r) - np.float64(new_r)))
             num, den = num * float(alpha), f32(den * alpha)
-            moves.append(float(mx) - float(r))
-            r = mx
-        p = np.exp2((np.asarray(s, dtype=f32) - r).astype(np.float64)).astype(f32)
+            r = new_r
+            redone += 1
+            p, rs = form(s, r)
         den = f32(den + p.sum(dtype=f32))
-        kk = min(max(np.floor(-np.log2(np.float64(p.max()))), -16.0), 60.0)
+        E = int(np.frexp(np.float64(rs))[1]) if rs > 0 else 0
+        kk = min(max(8 - E, -118), 60)
         sc = 448.0 * 2.0 ** kk
         pq = _e4m3_scalar((p.astype(np.float64) * sc).astype(np.float32).astype(np.float64)) / sc
         num = num + float(np.dot(pq, np.asarray(v, dtype=np.float64)))
-    return num / float(den), float(np.log2(np.float64(den)) + np.float64(r)), moves
+        if rs > f32(448.0 * 2.0 ** 16):
+            n = E - 9
+            num, den, r = num * 2.0 ** -n, f32(den * f32(2.0 ** -n)), f32(r + f32(n))
+            moves.append(n)
+    return num / float(den), float(np.log2(np.float64(den)) + np.float64(r)), moves, redone
 
 
 def test_lazy_reference_point_matches_scalar_row_loop():
-    """`_RowState.update` in `P_MX_ROW` against the scalar loop above, on rows whose maximum rises in one block by 15.9
-    (the reference point stays: p up to 2^15.9, block exponent -15), by 16.1 (it moves) and by 40 (it moves), then falls
-    back; one row per case plus a row that creeps up by 6 per block (moves once the lead passes 16)."""
+    """`_RowState.update` in `P_MX_ROW` against the scalar loop above, on rows in which one key of the third block leads
+    everything before it by 15.0 (block sum below 2^16: the reference point stays), by 16.5 and by 40 (it moves up by a
+    whole number of binades), and by 140 (2^(s - r) overflows: the block is formed again against its own maximum); one
+    more row creeps up by 6 per block (the sum passes 2^16 at the third step)."""
     g = torch.Generator().manual_seed(71)
     blocks, D = 6, 4
-    rises = [15.9, 16.1, 40.0, None]
+    rises = [15.0, 16.5, 40.0, 140.0, None]
     S = torch.randn(len(rises), blocks, 64, generator=g) * 2.0 - 3.0
     for i, rise in enumerate(rises):
         top0 = float(S[i, 0].max())
@@ -562,15 +592,22 @@ def test_lazy_reference_point_matches_scalar_row_loop():
     for b in range(blocks):
         st.update(S[:, b].contiguous(), V[b], A.P_MX_ROW, 64)
     out, lse = st.finish()
-    expect_moves = [0, 1, 1, None]
+    # n = E - 9 with the block's sum 448 2^rise (1 + small) = 2^(8.807 + rise) in [2^(E-1), 2^E): rise 16.5 -> E = 26, 40 -> E = 49;
+    # the creeping row reaches 2^18 in its fourth block (2^6 and 2^12 before): E = 27
+    expect = [([], 0), ([17], 0), ([40], 0), ([], 1), ([18], 0)]
     for i, rise in enumerate(rises):
         for d in range(D):
-            ref, lref, moves = _scalar_mx_row(S[i].numpy(), V[:, :, d].numpy())
+            ref, lref, moves, redone = _scalar_mx_row(S[i].numpy(), V[:, :, d].numpy())
             assert abs(float(out[i, d]) - ref) <= 2e-5 * max(abs(ref), 1.0), (i, d, float(out[i, d]), ref)
         assert abs(float(lse[i]) - lref) <= 2e-5 * max(abs(lref), 1.0)
-        if expect_moves[i] is not None:
-            assert len(moves) == expect_moves[i], (rise, moves)
-        else:
-            assert len(moves) == 1 and abs(moves[0] - 18.0) < 1e-4      # leads of 6 and 12 are tolerated, 18 is not
-    # the row that rose by 15.9 really kept its reference point: its m is still the first block's maximum
-    assert float(st.m[0]) == float(S[0, 0].max()) and float(st.m[1]) == float(S[1, 2, 11])
+        assert (moves, redone) == expect[i], (rise, moves, redone)
+    # and against the exact softmax of the same scores: the lazily followed reference point changes no value
+    for i in range(len(rises)):
+        s = S[i].reshape(-1).double()
+        w = torch.softmax(s * math.log(2.0), dim=0)
+        exact = w @ V.reshape(-1, D).double()
+        assert torch.allclose(out[i].double(), exact, atol=3e-2 * float(exact.abs().max()) + 1e-3)
+        assert abs(float(lse[i]) - float(torch.logsumexp(s * math.log(2.0), 0) / math.log(2.0))) < 1e-4
+    # the row that rose by 15.0 really kept its reference point, the one that overflowed sits on its block maximum
+    assert float(st.m[0]) == float(S[0, 0].max()) and float(st.m[3]) == float(S[3, 2, 11])
+    assert float(st.m[1]) == float(S[1, 0].max() + 17.0)      # (the sum in fp32, as the state holds it)
