@@ -31,7 +31,7 @@ def prefill_traffic_bytes(N, p_quant):
     """L2<->fabric bytes of one prefill_kernel launch, from the committed rocprofv3 FETCH_SIZE / WRITE_SIZE summary of this
     shape (profiles/prefill_kernel_128k.traffic.json: counters in KiB, each scaled by what the same counter read for a
     1 GiB copy); None for shapes and P modes the summary does not cover."""
-    if N != 131072 or p_quant < 4:
+    if N != 131072 or p_quant != 5:
         return None
     try:
         with open(os.path.join(ROOT, "profiles", "prefill_kernel_128k.traffic.json")) as f:

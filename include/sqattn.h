@@ -83,8 +83,11 @@ enum {
                          /* channel, from a pre-pass): P.V runs on the fp8 matrix pipe.  No reference */
                          /* counterpart (it keeps V in fp16, attn_triton.py:83); prefill only         */
   SQ_P_E4M3_MX_FP8_PV = 5 /* as FP8_PV with a block scale on P: one power of two per query row and     */
-                         /* 64-key tile, 2^k with k = floor(-log2(largest p of the row in the tile)),  */
-                         /* carried in the scale operand of the block-scaled fp8 MFMA; prefill only   */
+                         /* 64-key tile, taken from the row's sum of the tile's probabilities (scaled */
+                         /* sum in [128, 256), every scaled probability below 256), carried in the    */
+                         /* scale operand of the block-scaled fp8 MFMA; the row's reference point is  */
+                         /* set by its first tile and moves, by whole binades, when a tile's sum      */
+                         /* exceeds 2^16; prefill only                                                */
 };
 
 enum { SQ_WINDOW_NONE = 0, SQ_WINDOW_SIZES = 1 };

@@ -952,14 +952,10 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
       // scaled probability is below 256 (e4m3 reaches 448), the row's largest one at least 2.  The E8M0 exponent of 2^k is
       // eb = frexp exponent + 119, kept in [67, 245]: the pack divides by 2^(eb - 127), the MFMA multiplies by it.
       // (only rs_lane and eb stay live through the P.V slots: the rare paths below form the row sum again)
+      // (this chain of dependent instructions sits behind the first P.V MFMA, not in front of it)
       float rs_lane = ps[0] + ps[1];
-      int eb;
-      {
-        const float rs_row = xor32_sum(rs_lane);
-        eb = min(max(__builtin_amdgcn_frexp_expf(rs_row) + 119, 67), 245);
-        moved = __any(!(rs_row <= kSumLimit));
-      }
-      const float pack_scale = __int_as_float(eb << 23);
+      int eb = 127;
+      float pack_scale = 1.f;
       typedef __attribute__((ext_vector_type(2))) short i16x2_t;
       int P8n[8];
       auto pack_words = [&](auto BD, float sc) __attribute__((always_inline)) {   // words 2 bd, 2 bd + 1: S[bd >> 1][8 (bd & 1) .. + 7]
@@ -988,6 +984,12 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
         if constexpr (bd < 2) {
           vread(std::integral_constant<int, 2 * bd + 4>{});
           vread(std::integral_constant<int, 2 * bd + 5>{});
+        }
+        if constexpr (bd == 0) {
+          const float rs_row = xor32_sum(rs_lane);
+          eb = min(max(__builtin_amdgcn_frexp_expf(rs_row) + 119, 67), 245);
+          moved = __any(!(rs_row <= kSumLimit));
+          pack_scale = __int_as_float(eb << 23);
         }
         pack_words(I, pack_scale);
         __builtin_amdgcn_sched_barrier(0);
