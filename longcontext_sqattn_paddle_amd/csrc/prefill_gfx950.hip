@@ -542,29 +542,29 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
   // cinit = kC - m_run (kC = log2(448) in MODE 3, else 0), so the MFMA chain delivers S - m_run + kC and, as
   // long as the running maximum does not move, p (or 448 p) is a bare exp2 of the accumulator.
   constexpr float kC = (MODE >= 3 && MODE <= 5) ? kLog2_448 : 0.f;
-  // Lazy re-centring (MODE 5 and MODE 0): a row maximum may rise up to kLazy (in log2 units) above the reference before
-  // the accumulators are rescaled.  MODE 5: the block scale absorbs any power of two (its exponent then exceeds 127),
-  // while the fp32 accumulators and the denominator carry the common factor until the division at the end.  MODE 0: p
-  // is rounded to fp16, which has the same ten mantissa bits at 2^8 as at 1, so p = 2^(s - reference) up to 2^8 is the
-  // same probability with the same relative rounding error (2^-11) as the reference's 2^(s - running maximum) <= 1 --
-  // not the same bits, and small probabilities keep more of their bits than there.  A row is shifted only when its own
-  // maximum passes the limit, so its arithmetic does not depend on the other rows of the wave.  With re-centring at once,
-  // one row of the wave's 32 finding a new maximum sends the whole wave through the rescale path (some 110 vector
-  // instructions): about 32 (1 + ln(tiles / 32)) times per wave, which is 8 % of the tiles of a 131072-key causal row
-  // and 40 % of the 214 tiles of a sink + 10 % window.  The e4m3 modes with the static scale (1, 3, 4) need p <= 1 for
-  // their grid and re-centre at once.
-  constexpr float kLazy = (MODE == 5) ? 16.f : (MODE == 0 ? 8.f : 0.f);
+  // Lazy re-centring (the modes whose P is a plain fp16 number: MODE 0, and MODE 6, which differs from it in the Q.K^T
+  // product only): a row maximum may rise up to kLazy (in log2 units) above the reference before the accumulators are
+  // rescaled.  p is rounded to fp16, which has the same ten mantissa bits at 2^8 as at 1, so p = 2^(s - reference) up to
+  // 2^8 is the same probability with the same relative rounding error (2^-11) as the reference's
+  // 2^(s - running maximum) <= 1 -- not the same bits, and small probabilities keep more of their bits than there; the
+  // fp32 accumulators and the denominator carry the common factor until the division at the end.  A row is shifted only
+  // when its own maximum passes the limit, so its arithmetic does not depend on the other rows of the wave.  With
+  // re-centring at once, one row of the wave's 32 finding a new maximum sends the whole wave through the rescale path
+  // (some 110 vector instructions): about 32 (1 + ln(tiles / 32)) times per wave, which is 8 % of the tiles of a
+  // 131072-key causal row and 40 % of the 214 tiles of a sink + 10 % window.  The e4m3 modes with the static scale (1, 3,
+  // 4) need p <= 1 for their grid and re-centre at once; MODE 5 has a rule of its own (kDefer below).
+  constexpr float kLazy = (MODE == 0 || MODE == 6) ? 8.f : 0.f;
   constexpr float kMove = kC + kLazy;
   // MODE 5 takes neither the block scale nor the decision to move the reference from the row's maximum of the tile but
   // from the row's SUM of the tile's probabilities, which the denominator needs anyway: the maximum tree (26 vector
   // instructions per tile) goes.  The probabilities of a tile are formed against the standing reference without looking
-  // at the scores first; a row whose sum then exceeds 2^kLazy moves its reference up by a whole number of binades
+  // at the scores first; a row whose sum then exceeds 2^16 moves its reference up by a whole number of binades
   // (exact rescaling, also of the tile just packed, through the scale operand of its MFMA), and a row whose sum is not
   // finite -- a score more than 2^100 above everything the row has seen -- has the tile recomputed from the key rows in
   // memory against the tile's own maximum (redo_tile).  The scale needs the whole tile's sum, so the tile's P.V product
   // is deferred by one visited step: the conversions to e4m3 run under the P.V MFMAs of the tile before.
   constexpr bool kDefer = MODE == 5;
-  constexpr float kSumLimit = 448.f * 65536.f;   // 2^kLazy in units of the probabilities as formed (times 448)
+  constexpr float kSumLimit = 448.f * 65536.f;   // 2^16 in units of the probabilities as formed (times 448)
   constexpr float kRedoLimit = 1.329227995784916e36f;   // 2^120: beyond it (or not a number) the tile is formed again
   float m_run = 0.f;       // reference point of the exponent; the first visited tile replaces it by the row maximum
   float l_run = 0.f;       // this lane's share of the denominator (times 448 in MODE 3)
@@ -687,10 +687,13 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
     vxr[m] = smem_addr + 4 * kKTileBytes + ((c32 * kVStride + ((g ^ ((c32 >> 1) & 7)) << 4)) ^ (m << 5));
   typedef __attribute__((ext_vector_type(8))) int i32x8_t;
   i32x8_t P8 = {0, 0, 0, 0, 0, 0, 0, 0};   // MODE 4: e4m3 probabilities of the current tile (registers reused tile after tile)
-  int P8w[8] = {0, 0, 0, 0, 0, 0, 0, 0};   // MODE 5: the same as eight scalars
-  // MODE 5 multiplies a tile's probabilities with V one visited step later (kDefer): P8w holds the pending tile.  A step's
-  // four P.V MFMAs consume it between the Q.K^T MFMAs of the next tile, before the current tile is packed into the same
-  // registers at the end of the step.  It is zero while nothing is pending, so those MFMAs then add nothing.
+  // MODE 5 multiplies a tile's probabilities with V one visited step later (kDefer): P8w holds the pending tile, which the
+  // step's four P.V MFMAs consume while the current tile is packed, underneath them, into registers its probabilities
+  // leave; it takes the current tile over at the end of the step.  It is zero while nothing is pending, so those MFMAs
+  // then add nothing.  (Eight scalars, not a vector: the pack builtin takes the word it half-overwrites as two shorts,
+  // and with the words kept as elements of a vector every element's old value came out as element 0's -- a wrong fold of
+  // the element extraction with the cast.)
+  int P8w[8] = {0, 0, 0, 0, 0, 0, 0, 0};
   int e_pend = 127;    // E8M0 exponent of the pending tile's block scale
   int pend_t = -1;     // step of the pending tile (wave-uniform), -1: none
   const int vsw = (c32 >> 1) & 7;    // swizzle of this lane's V^T rows (32 bd + c32)
@@ -754,11 +757,6 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
   // whether any row's maximum moved; both computed one step ahead, under the P.V MFMAs
   float tmax_row = 0.f;
   bool moved = false;
-  // MODE 5: block scale of a row's 64 probabilities in a tile, 2^k with k = floor(log2 448 - t) in [0, 60] for the
-  // row maximum t of the scores (which carry log2 448); kept as the E8M0 exponent 127 - k = ceil(t + 127 - log2 448)
-  // of 2^-k.  Computed one step ahead like tmax_row, again after a shift of the reference.
-  auto block_exp = [](float t) { return (int)__builtin_ceilf(__builtin_amdgcn_fmed3f(t + (127.f - kC), 67.f, 127.f + kLazy)); };
-  int e_row = 127;
 
   // Q~ fragments of the other operand set, one 16-byte piece at a time (a handful of switches per wave: no need for all
   // eight loads in flight, and the registers they would take are the tile step's).  The 8-bit quantiser of load_q does
@@ -878,7 +876,6 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
       if (masked) {
         tmax_row = xor32_max(lane_max(S));
         moved = __any(tmax_row > kMove);
-        if constexpr (MODE == 5) e_row = block_exp(tmax_row);
       }
       tmax = tmax_row;   // came out of the previous step's P.V phase
       slow = first || moved;
@@ -898,7 +895,6 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
       const float alpha = first ? 0.f : __builtin_amdgcn_exp2f(-d);
       m_run += d;
       l_run *= alpha;
-      if constexpr (MODE == 5) e_row = block_exp(tmax - d);
 #pragma unroll
       for (int bn = 0; bn < 2; ++bn)
 #pragma unroll
@@ -1066,11 +1062,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
       pend_t = it;
       return;
     }
-    if constexpr (kPV8) {
-      // MODE 5: the pack divides by 2^-k, the MFMA multiplies this lane's 32 values by 2^-k again (E8M0 scale in
-      // byte 0 of the operand).  MODE 4: k = 0.
-      const int mfma_scale_b = (MODE == 5) ? e_row : 0x7f7f7f7f;
-      const float pack_scale = __int_as_float(mfma_scale_b << 23);
+    if constexpr (kPV8) {   // MODE 4 (MODE 5 has returned above)
       __builtin_amdgcn_s_setprio(0);
       // Hand-scheduled tile step.  16 slots of {Q.K^T MFMA of the next tile, one LDS prefetch, two exponentials
       // and one e4m3 pack of the current tile}, then 4 slots of {fp8 P.V MFMA, two LDS prefetches, 8 additions of
@@ -1105,16 +1097,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
           if constexpr (rr & 1) vhi[rr >> 1] = lds_read128<kVoff + (rr >> 1) * 2048>(vhi_addr);
           else vlo[rr >> 1] = lds_read128<kVoff + (rr >> 1) * 2048>(vlo_addr);
         }
-        if constexpr (MODE == 5) {
-          typedef __attribute__((ext_vector_type(2))) short i16x2_t;
-          // The half of the word that is not written comes from the first operand.  With the words kept as elements
-          // of a vector, every element's old value came out as element 0's (a wrong fold of the element extraction
-          // with the cast to two shorts), hence eight scalars here.
-          P8w[r] = __builtin_bit_cast(int, __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(__builtin_bit_cast(i16x2_t, P8w[r]), p0, p1,
-                                                                                  pack_scale, (i & 1) != 0));
-        } else {
-          P8[r] = __builtin_amdgcn_cvt_pk_fp8_f32(p0, p1, P8[r], (i & 1) != 0);
-        }
+        P8[r] = __builtin_amdgcn_cvt_pk_fp8_f32(p0, p1, P8[r], (i & 1) != 0);
         __builtin_amdgcn_sched_barrier(0);
       });
       // P.V slots: the vector ALU is nearly idle under the four K=64 MFMAs, so the row sum of this tile and the
@@ -1134,12 +1117,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
         __builtin_amdgcn_sched_barrier(0);
         const i32x8_t av = {(int)vlo[bd][0], (int)vlo[bd][1], (int)vlo[bd][2], (int)vlo[bd][3],
                             (int)vhi[bd][0], (int)vhi[bd][1], (int)vhi[bd][2], (int)vhi[bd][3]};
-        if constexpr (MODE == 5) {
-          const i32x8_t pb = {P8w[0], P8w[1], P8w[2], P8w[3], P8w[4], P8w[5], P8w[6], P8w[7]};
-          O[bd] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, pb, O[bd], 0, 0, 0, 0x7f7f7f7f, 0, mfma_scale_b);
-        } else {
-          O[bd] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, P8, O[bd], 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
-        }
+        O[bd] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, P8, O[bd], 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
         __builtin_amdgcn_sched_barrier(0);
         if constexpr (issued < 8) {
           vlo[issued / 2] = lds_read128<kVoff + (issued / 2) * 2048>(vlo_addr);
@@ -1163,7 +1141,6 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
       tmax_row = xor32_max(max3_of4(cm[0], cm[1], cm[2], cm[3]));
       l_run += ps[0] + ps[1];
       moved = __any(tmax_row > kMove);
-      if constexpr (MODE == 5) e_row = block_exp(tmax_row);
       __builtin_amdgcn_s_setprio(3);
       return;
     }
@@ -1397,7 +1374,6 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
       mfma_settle(Sa[0], Sa[1]);
       tmax_row = xor32_max(lane_max(Sa));
       moved = __any(tmax_row > kMove);
-      if constexpr (MODE == 5) e_row = block_exp(tmax_row);
     }
   }
   __syncthreads();   // ring buffer 0 is about to be refilled: every wave has read K(step 0) out of it
@@ -1447,7 +1423,6 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
           mfma_settle(Snxt[0], Snxt[1]);
           tmax_row = xor32_max(lane_max(Snxt));
           moved = __any(tmax_row > kMove);
-          if constexpr (MODE == 5) e_row = block_exp(tmax_row);
         }
       }
       if constexpr (MODE == 2) {
