@@ -933,6 +933,8 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
         const float p0 = __builtin_amdgcn_exp2f(S[sb][e]), p1 = __builtin_amdgcn_exp2f(S[sb][e + 1]);
         S[sb][e] = p0;
         S[sb][e + 1] = p1;
+        ps[i & 1] += p0;
+        ps[i & 1] += p1;
         __builtin_amdgcn_sched_barrier(0);
         const uint4 ka = make_uint4(kf[i][0], kf[i][1], kf[i][2], kf[i][3]);
         if constexpr (kk == 0) Snext[bn] = mfma_qk32<BF16>(ka, qf[0], Cinit);
@@ -940,8 +942,6 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
         __builtin_amdgcn_sched_barrier(0);
         if constexpr (i + kDepth < 16) kread(std::integral_constant<int, i + kDepth>{});
         else vread(std::integral_constant<int, i + kDepth - 16>{});
-        ps[i & 1] += p0;
-        ps[i & 1] += p1;
         __builtin_amdgcn_sched_barrier(0);
       });
       // The row's sum of the tile, rs = 448 sum 2^(s - reference).  Block scale 2^-k with rs 2^-k in [128, 256): every
