@@ -1154,6 +1154,9 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
       // {P.V MFMA, one LDS prefetch, two additions of the row sum, later two steps of the next tile's row maximum}.
       // P.V slot s multiplies V^T rows 32 (s & 3) .. +31 with the keys of group m = s >> 2 (8 keys per lane), whose
       // probabilities are the B operand words Pw[m][0..3].
+      // Order inside a slot, held by scheduling barriers: the wait, the MFMA, the LDS request, then the vector work (1.2 %
+      // faster than the order the compiler chose, and 3 % faster than the vector work in front of the MFMA -- the other
+      // way round than in the fp8 steps, whose slots carry more vector work per MFMA).
       __builtin_amdgcn_s_setprio(0);
       const uint32_t vlane = smem_addr + 4 * kKTileBytes + (it & 3) * kVTileBytes + c32 * kVStride + ((g ^ vsw) << 4);
       u32x4_t vf[16];
@@ -1173,11 +1176,14 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
         constexpr int i = decltype(I)::value;
         constexpr int bn = i & 1, kk = i >> 1;
         lds_wait<kDepth - 1>(kf[i]);
+        __builtin_amdgcn_sched_barrier(0);
         const uint4 ka = make_uint4(kf[i][0], kf[i][1], kf[i][2], kf[i][3]);
         if constexpr (kk == 0) Snext[bn] = mfma_qk32<BF16>(ka, qf[0], Cinit);
         else Snext[bn] = mfma_qk32<BF16>(ka, qf[kk], Snext[bn]);
+        __builtin_amdgcn_sched_barrier(0);
         if constexpr (i + kDepth < 16) kread(std::integral_constant<int, i + kDepth>{});
         else vread(std::integral_constant<int, i + kDepth - 16>{});
+        __builtin_amdgcn_sched_barrier(0);
         constexpr int sb = i >> 3, e = 2 * (i & 7);
         S[sb][e] = __builtin_amdgcn_exp2f(S[sb][e]);
         S[sb][e + 1] = __builtin_amdgcn_exp2f(S[sb][e + 1]);
@@ -1201,9 +1207,12 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_kernel(PrefillArgs a) {
         constexpr int m = sl >> 2, bd = sl & 3;
         constexpr int issued = (kDepth + sl < 16) ? kDepth + sl : 16;   // V^T requests issued before this slot
         lds_wait<issued - sl - 1>(vf[sl]);
+        __builtin_amdgcn_sched_barrier(0);
         const uint4 av = make_uint4(vf[sl][0], vf[sl][1], vf[sl][2], vf[sl][3]);
         O[bd] = mfma_pv32(av, make_uint4(Pw[m][0], Pw[m][1], Pw[m][2], Pw[m][3]), O[bd]);
+        __builtin_amdgcn_sched_barrier(0);
         if constexpr (issued < 16) vread(std::integral_constant<int, issued>{});
+        __builtin_amdgcn_sched_barrier(0);
         if constexpr (sl == 0) pack_unit(std::integral_constant<int, 7>{});
         ps[0] += S[sl >> 3][2 * (sl & 7)];
         ps[1] += S[sl >> 3][2 * (sl & 7) + 1];
