@@ -5,6 +5,7 @@ the size limit.  "Allocates nothing" is checked against the driver's own count o
 (`hipMemGetInfo`, which also sees a `hipMalloc` made inside the library), not only against torch's allocator; and the
 call is recorded into a HIP graph after `sq_decode_noalloc_init` and replayed."""
 import ctypes
+import gc
 
 import pytest
 import torch
@@ -50,12 +51,23 @@ def test_noalloc_decode_equals_workspace_decode_twice_second_smaller():
         assert rc == 0, msg
         assert lib.sq_decode_noalloc_init() == 0, lib.sq_last_error().decode()   # the one-off look-up, outside the measured call
         torch.cuda.synchronize()
-        before, free_before = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
-        rc, msg = _call("sq_decode_fwd_noalloc", q, k, v, sl, out_b, lse_b, 0)
+        # Tensors of earlier tests that only a collection of reference cycles frees must not be freed between the two
+        # readings (after a long run of other tests that was tens of GB): collect now, and keep the collector off
+        # for the measured call.  torch's count is its cumulative number of allocations, which a free cannot change.
+        gc.collect()
+        gc.disable()
+        try:
+            n_before = torch.cuda.memory_stats()["allocation.all.allocated"]
+            before, free_before = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
+            rc, msg = _call("sq_decode_fwd_noalloc", q, k, v, sl, out_b, lse_b, 0)
+            torch.cuda.synchronize()
+            n_after = torch.cuda.memory_stats()["allocation.all.allocated"]
+            after, free_after = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
+        finally:
+            gc.enable()
         assert rc == 0, msg
-        torch.cuda.synchronize()
-        assert torch.cuda.memory_allocated() == before
-        assert torch.cuda.mem_get_info()[0] == free_before      # the driver's count: no hipMalloc inside the library either
+        assert n_after == n_before and after == before
+        assert free_after == free_before      # the driver's count: no hipMalloc inside the library either
         assert bool(torch.isfinite(out_b).all())
         assert torch.equal(out_a, out_b) and torch.equal(lse_a, lse_b)
 
